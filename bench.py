@@ -1,0 +1,246 @@
+#!/usr/bin/env python3
+"""Benchmark of the fused score + SPEC-RL verify path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c2|c3|c4|c1]
+
+One step = one pass of vrl_fused_score_verify (row kernel + verify kernel, through
+the C ABI, outputs preallocated) over the whole synthetic batch, logits resident
+in HBM. Prints one JSON line: whole-job verified tokens/s, the HBM roofline of
+the row kernel (algorithmic bytes / average kernel time from HIP events on the
+launch stream), and the same computation in torch on the host cores (bounded sample).
+"""
+
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import statistics
+import sys
+import time
+
+import torch
+
+REPO = os.path.dirname(os.path.abspath(__file__))
+if REPO not in sys.path:
+    sys.path.insert(0, REPO)
+
+from verl_amd import _lib, synthetic  # noqa: E402
+from verl_amd import spec_verify as sv  # noqa: E402
+from verl_amd import torch_functional as vf  # noqa: E402
+
+HBM_PEAK_GBPS = 8000.0
+METRIC = "verified tokens/sec + achieved HBM GB/s (% of peak), vocab 152k bf16, 1 GPU"
+
+
+def algorithmic_bytes_per_token(V: int, esize: int, with_temperature: bool, with_verify: bool) -> int:
+    """Logits once + label (8) + log-prob out (4) + entropy out (4) [+ temperature (4)];
+    verify adds old log-prob (4), log u (4), mask (1), accept out (1)."""
+    b = V * esize + 8 + 4 + 4 + (4 if with_temperature else 0)
+    if with_verify:
+        b += 4 + 4 + 1 + 1
+    return b
+
+
+class Step:
+    """Preallocated buffers and the raw ABI calls for one workload."""
+
+    def __init__(self, w: synthetic.Workload, dev, seed: int, n_rows: int | None = None):
+        self.w = w
+        self.dev = dev
+        B, T = w.B, w.T
+        if n_rows is not None:  # micro-batch of whole padded sequences
+            B = max(1, n_rows // T)
+            w = w.scaled(B=B)
+            self.w = w
+        d = synthetic.make_padded(w, dev, seed)
+        self.logits = d["logits"].view(-1, w.V)
+        self.labels = d["labels"].view(-1).contiguous()
+        self.mask = d["mask"].contiguous()
+        self.mask8 = self.mask.view(torch.uint8)
+        self.log_u = d["log_u"].contiguous()
+        self.temp = None if d["temperature"] is None else d["temperature"].view(-1).contiguous()
+        self.n = self.logits.shape[0]
+        self.B, self.T = w.B, w.T
+        self.n_valid = int(self.mask.sum().item())
+        self.off = sv.thresh_offset_from_lenience(w.lenience)
+        f32 = dict(dtype=torch.float32, device=dev)
+        self.lp = torch.empty(self.n, **f32)
+        self.h = torch.empty(self.n, **f32)
+        self.flag = torch.zeros(1, dtype=torch.int32, device=dev)
+        self.accept = torch.empty(self.n, dtype=torch.uint8, device=dev)
+        self.first = torch.empty(self.B, dtype=torch.int32, device=dev)
+        self.prefix = torch.empty(self.B, dtype=torch.int32, device=dev)
+        self.near = torch.empty(self.B, dtype=torch.int32, device=dev)
+        self.ids = self.labels
+        self.out_ids = torch.empty_like(self.ids)
+        self.out_mask = torch.empty(self.n, dtype=torch.uint8, device=dev)
+        self.lib = _lib.load()
+        self.dt = _lib.VRL_BF16 if w.dtype == torch.bfloat16 else _lib.VRL_F32
+        self.stream = torch.cuda.current_stream(dev).cuda_stream
+        # old log-probs = new (from the kernel) + drift
+        self.score()
+        torch.cuda.synchronize()
+        self.lp_old = synthetic.drift_old_logprobs(self.lp, w, seed).contiguous()
+
+    def _tp(self):
+        return None if self.temp is None else self.temp.data_ptr()
+
+    def score(self):
+        st = self.lib.vrl_rowscore(self.logits.data_ptr(), self.dt, self.n, self.w.V, self.logits.stride(0),
+                                   self.labels.data_ptr(), self._tp(), self.lp.data_ptr(), self.h.data_ptr(),
+                                   self.flag.data_ptr(), self.stream)
+        _lib.check("vrl_rowscore", st)
+
+    def fused(self):
+        st = self.lib.vrl_fused_score_verify(
+            self.logits.data_ptr(), self.dt, self.n, self.w.V, self.logits.stride(0), self.labels.data_ptr(),
+            self._tp(), self.lp.data_ptr(), self.h.data_ptr(), self.flag.data_ptr(),
+            self.lp_old.data_ptr(), self.log_u.data_ptr(), self.mask8.data_ptr(), None, self.B, self.T,
+            self.off, 1e-6, self.accept.data_ptr(), self.first.data_ptr(), self.prefix.data_ptr(),
+            self.near.data_ptr(), self.ids.data_ptr(), 0, self.out_ids.data_ptr(), self.out_mask.data_ptr(),
+            self.stream)
+        _lib.check("vrl_fused_score_verify", st)
+
+    def check_against_torch(self, rows: int = 1024):
+        """Guard: the first rows against torch's fp32 ops on the GPU (not timed)."""
+        z = self.logits[:rows].float()
+        if self.temp is not None:
+            z = z / self.temp[:rows].clamp(min=1e-8).unsqueeze(-1)
+        lse = torch.logsumexp(z, -1)
+        ref_lp = z.gather(-1, self.labels[:rows, None]).squeeze(-1) - lse
+        ref_h = lse - (torch.softmax(z, -1) * z).sum(-1)
+        e1 = (self.lp[:rows] - ref_lp).abs().max().item()
+        e2 = (self.h[:rows] - ref_h).abs().max().item()
+        tol = 1e-5 if self.w.dtype == torch.float32 else 2e-3
+        if not (e1 <= tol and e2 <= tol):
+            raise SystemExit(f"bench: kernel disagrees with torch fp32 (logprob {e1}, entropy {e2}, tol {tol})")
+        if int(self.flag.item()) != 0:
+            raise SystemExit("bench: label out of range flagged")
+        return e1, e2
+
+
+def cpu_baseline(step: Step, budget_s: float = 20.0):
+    """The torch restatement of the reference composition on the host cores, on a slice of the same batch."""
+    from oracle import scoring, verify as overify  # checker/baseline only
+
+    w = step.w
+    rows = min(step.n, 1024)
+    x = step.logits[:rows].cpu()
+    lab = step.labels[:rows].cpu()
+    temp = None if step.temp is None else step.temp[:rows].cpu()
+    old = step.lp_old[:rows].cpu().view(1, rows)
+    lu = step.log_u.view(-1)[:rows].cpu().view(1, rows)
+    mk = step.mask.view(-1)[:rows].cpu().view(1, rows)
+
+    def once():
+        t0 = time.perf_counter()
+        lp, h = scoring.score_reference(x, lab, temp)
+        overify.verify(lp.float().view(1, rows), old, lu, mk, step.off)
+        return time.perf_counter() - t0
+
+    first = once()
+    reps = max(1, min(5, int(budget_s / max(first, 1e-3)) - 1))
+    times = [first] + [once() for _ in range(reps)]
+    best = statistics.median(times)
+    return {
+        "value": rows / best,
+        "unit": "tokens/s",
+        "cores": torch.get_num_threads(),
+        "kind": "port",
+        "sample": f"{rows} rows of the same batch (V={w.V}, {str(w.dtype).replace('torch.', '')}), "
+                  f"median of {len(times)} runs, torch {torch.__version__} on {os.cpu_count()} logical CPUs",
+    }
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--workload", default="c2", choices=["c1", "c2", "c3", "c4"])
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build runs on one GPU only (rows are independent; see DESIGN.md for how it would shard); "
+              f"--gpus {args.gpus} is not supported", file=sys.stderr)
+        sys.exit(2)
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible; the HIP path has no CPU fallback", file=sys.stderr)
+        sys.exit(2)
+
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    w = synthetic.WORKLOADS[args.workload]
+    n_rows = w.micro_batch_tokens  # c3: one 8192-token micro-batch per step
+    step = Step(w, dev, seed=1000 * int(args.workload[1]), n_rows=n_rows)
+    err_lp, err_h = step.check_against_torch()
+
+    for _ in range(args.warmup):
+        step.fused()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step.fused()
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    ms_per_step = wall * 1e3 / args.steps
+    tokens_per_s = step.n_valid * args.steps / wall
+
+    # Row kernel alone, one HIP event pair per launch on the launch stream.
+    evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(args.steps)]
+    for a, b in evs:
+        a.record()
+        step.score()
+        b.record()
+    torch.cuda.synchronize()
+    kern_ms = [a.elapsed_time(b) for a, b in evs]
+    avg_kern_ms = sum(kern_ms) / len(kern_ms)
+    esize = 2 if w.dtype == torch.bfloat16 else 4
+    bytes_score = algorithmic_bytes_per_token(w.V, esize, step.temp is not None, False) * step.n
+    achieved = bytes_score / (avg_kern_ms * 1e-3) / 1e9
+    bytes_fused = algorithmic_bytes_per_token(w.V, esize, step.temp is not None, True) * step.n
+
+    out = {
+        "metric": METRIC,
+        "value": tokens_per_s,
+        "unit": "tokens/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": ms_per_step,
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "bf16" if w.dtype == torch.bfloat16 else "f32",
+        "data": "synthetic",
+        "config": {
+            "workload": step.w.name,
+            "rows_per_step": step.n,
+            "valid_tokens_per_step": step.n_valid,
+            "vocab": w.V,
+            "lenience": w.lenience,
+            "temperature": w.temperature,
+            "step": "vrl_fused_score_verify (row kernel + verify kernel), logits resident in HBM",
+        },
+        "hbm_gbps_fused_step": bytes_fused / (ms_per_step * 1e-3) / 1e9,
+        "roofline": {
+            "bound": "hbm",
+            "achieved": achieved,
+            "peak": HBM_PEAK_GBPS,
+            "unit": "GB/s",
+            "frac": achieved / HBM_PEAK_GBPS,
+            "traffic": None,
+            "kernel": "rowscore_kernel",
+            "avg_kernel_ms": avg_kern_ms,
+            "algorithmic_bytes_per_launch": bytes_score,
+        },
+        "parity_guard": {"rows": 1024, "max_abs_err_logprob": err_lp, "max_abs_err_entropy": err_h},
+    }
+    if not args.no_cpu_baseline:
+        out["cpu_baseline"] = cpu_baseline(step)
+    print(json.dumps(out), flush=True)
+
+
+if __name__ == "__main__":
+    main()

@@ -1,0 +1,141 @@
+/*
+ * vrl.h — C ABI of libvrl_hip.so: per-token scoring of LLM logits and the
+ * SPEC-RL draft-verify step on one MI355X (gfx950).
+ *
+ * Conventions shared by every entry point
+ *   - Every pointer named below is a DEVICE pointer into memory the caller
+ *     owns (hipMalloc / torch allocator). The library allocates nothing,
+ *     frees nothing and keeps no pointer after the call returns.
+ *   - `stream` is a hipStream_t passed as void* (NULL = the null stream).
+ *     Kernels are enqueued on it and the call returns without synchronising.
+ *   - Return value: VRL_OK, or a negative VRL_ERR_* found on the host before
+ *     anything was enqueued (nothing has been launched in that case).
+ *     Errors that only the device can see (a label outside [0, vocab)) are
+ *     OR-ed into *err_flag (device int32, caller zeroes it, caller reads it
+ *     after synchronising).
+ *   - Nothing throws or aborts across this boundary.
+ *   - Row space: logits are (n_rows, vocab), row r starts at element
+ *     r * row_stride. Per-token arrays (labels, temperature, outputs, and
+ *     for verify logp/mask/accept) are indexed by the same r.
+ *   - Sequence space: sequence b owns rows [cu_seqlens[b], cu_seqlens[b+1])
+ *     when cu_seqlens != NULL (packed layout, B+1 int64 entries), else rows
+ *     [b*T, (b+1)*T) (padded (B, T) layout).
+ */
+#ifndef VRL_H_
+#define VRL_H_
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define VRL_ABI_VERSION 1
+
+/* status codes */
+#define VRL_OK 0
+#define VRL_ERR_NULL (-1)      /* a required pointer is NULL */
+#define VRL_ERR_DTYPE (-2)     /* dtype is not one of VRL_F32 / VRL_BF16 */
+#define VRL_ERR_SHAPE (-3)     /* negative count, vocab <= 0, stride < vocab, too many rows */
+#define VRL_ERR_ALIGN (-4)     /* pointer not aligned to its element size */
+#define VRL_ERR_HIP (-5)       /* the HIP runtime refused the launch; see vrl_last_hip_error */
+#define VRL_ERR_ARG (-6)       /* inconsistent optional arguments */
+
+/* logits element types */
+#define VRL_F32 0
+#define VRL_BF16 1
+
+/* bits of *err_flag */
+#define VRL_FLAG_LABEL_OOB 1   /* some label was < 0 or >= vocab; that row's logprob is NaN */
+
+/*
+ * vrl_rowscore — one HBM pass over (n_rows, vocab) logits producing, per row,
+ *   logprob[r] = z[label[r]] - logsumexp(z),  entropy[r] = logsumexp(z) - sum(softmax(z) * z)
+ * with z = logits[r, :] / max(temperature[r], 1e-8) (z = logits[r, :] when
+ * temperature == NULL), accumulated in fp32, written as fp32.
+ *
+ * Replaces, in the reference:
+ *   verl/utils/torch_functional.py:73-107   logprobs_from_logits (dispatch)
+ *   verl/utils/torch_functional.py:173-207  logprobs_from_logits_v2
+ *   verl/utils/torch_functional.py:155-170  logprobs_from_logits_naive
+ *   verl/utils/torch_functional.py:231-245  entropy_from_logits
+ *   verl/utils/torch_functional.py:248-270  entropy_from_logits_with_chunking
+ *   verl/workers/engine/fsdp/transformer_impl.py:1357  division by per-token temperature
+ *
+ * out_logprob == NULL skips the label gather (labels may then be NULL);
+ * out_entropy == NULL skips the entropy store. At least one must be given.
+ * Rows containing -inf logits give NaN entropy (0 * -inf), as torch does.
+ */
+int vrl_rowscore(const void* logits, int dtype, int64_t n_rows, int64_t vocab, int64_t row_stride,
+                 const int64_t* labels, const float* temperature, float* out_logprob,
+                 float* out_entropy, int32_t* err_flag, void* stream);
+
+/*
+ * vrl_spec_verify — SPEC-RL draft verification over B sequences.
+ * For token i of sequence b:
+ *   d = logp_new[i] - logp_old[i];  tau = log_u[i] + thresh_offset      (fp32, no contraction)
+ *   valid = mask ? mask[i] != 0 : 1
+ *   accept[i] = valid && d >= tau            (NaN compares false => reject)
+ *   first_reject[b] = smallest in-sequence position with valid && !(d >= tau);
+ *                     when there is none, one past the last valid position
+ *                     (= number of valid tokens for a right-padded mask)
+ *   prefix_len[b]   = number of valid tokens at positions < first_reject[b]
+ *   near_count[b]   = number of valid tokens with |d - tau| < near_eps
+ * Optional truncated draft (all three or none): for positions >= first_reject
+ *   out_ids = pad_id, out_mask = 0; below it they copy draft_ids / mask.
+ *
+ * No function in the reference computes this (its recipe/ submodule is not
+ * vendored: .gitmodules:1-3). Layout, mask and sign conventions follow
+ *   verl/trainer/ppo/rollout_corr_helper.py:197-233,262-268,849
+ *   verl/trainer/ppo/ray_trainer.py:120-135 (response_mask = attention_mask[:, -T:])
+ * which is where a caller would slot it in (ray_trainer.py:1647-1660).
+ */
+int vrl_spec_verify(const float* logp_new, const float* logp_old, const float* log_u,
+                    const uint8_t* mask, const int64_t* cu_seqlens, int64_t B, int64_t T,
+                    float thresh_offset, float near_eps, uint8_t* accept, int32_t* first_reject,
+                    int32_t* prefix_len, int32_t* near_count, const int64_t* draft_ids,
+                    int64_t pad_id, int64_t* out_ids, uint8_t* out_mask, void* stream);
+
+/*
+ * vrl_truncate_draft — apply an already known first_reject[b] to a draft:
+ * positions >= first_reject[b] get pad_id / mask 0, the rest are copied.
+ * Same provenance as vrl_spec_verify (no reference counterpart); the nearest
+ * reference step is the mask rewrite at verl/trainer/ppo/rollout_corr_helper.py:1061.
+ */
+int vrl_truncate_draft(const int64_t* draft_ids, const uint8_t* mask, const int64_t* cu_seqlens,
+                       int64_t B, int64_t T, const int32_t* first_reject, int64_t pad_id,
+                       int64_t* out_ids, uint8_t* out_mask, void* stream);
+
+/*
+ * vrl_fused_score_verify — vrl_rowscore followed on the same stream by
+ * vrl_spec_verify fed with the log-probs just written (logp_new = out_logprob,
+ * which is therefore required). Row space and sequence space are as above:
+ * n_rows must equal cu_seqlens[B] (packed) or B*T (padded); the host checks
+ * only the padded case, cu_seqlens lives on the device.
+ *
+ * Replaces the composition at
+ *   verl/workers/engine/fsdp/transformer_impl.py:1353-1399 (divide, entropy, log-probs)
+ * plus the verify step described under vrl_spec_verify.
+ */
+int vrl_fused_score_verify(const void* logits, int dtype, int64_t n_rows, int64_t vocab,
+                           int64_t row_stride, const int64_t* labels, const float* temperature,
+                           float* out_logprob, float* out_entropy, int32_t* err_flag,
+                           const float* logp_old, const float* log_u, const uint8_t* mask,
+                           const int64_t* cu_seqlens, int64_t B, int64_t T, float thresh_offset,
+                           float near_eps, uint8_t* accept, int32_t* first_reject,
+                           int32_t* prefix_len, int32_t* near_count, const int64_t* draft_ids,
+                           int64_t pad_id, int64_t* out_ids, uint8_t* out_mask, void* stream);
+
+/* Text for a VRL_* status code; never NULL. */
+const char* vrl_strerror(int status);
+
+/* hipGetErrorString of the last launch this thread saw refused ("" if none). */
+const char* vrl_last_hip_error(void);
+
+/* VRL_ABI_VERSION the library was built with. */
+int vrl_abi_version(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* VRL_H_ */

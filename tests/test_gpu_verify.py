@@ -1,0 +1,165 @@
+"""The HIP verify kernel (through the C ABI) against the CPU statement of the rule: bit-exact."""
+
+import math
+
+import numpy as np
+import pytest
+import torch
+
+from verl_amd import spec_verify as sv
+from verl_amd import synthetic
+from oracle import c_oracle, verify as overify
+
+pytestmark = pytest.mark.gpu
+
+
+def _same(res, ref, with_draft=False):
+    assert np.array_equal(res.accept.cpu().numpy().astype(np.uint8), np.asarray(ref["accept"]).astype(np.uint8))
+    for k in ("first_reject", "prefix_len", "near_count"):
+        assert np.array_equal(getattr(res, k).cpu().numpy(), np.asarray(ref[k])), k
+    if with_draft:
+        assert np.array_equal(res.out_ids.cpu().numpy(), np.asarray(ref["out_ids"]))
+        assert np.array_equal(res.out_mask.cpu().numpy().astype(np.uint8), np.asarray(ref["out_mask"]).astype(np.uint8))
+
+
+def _inputs(dev, B, T, seed, drift=0.3, lengths=None):
+    g = torch.Generator(device=dev).manual_seed(seed)
+    ln = -torch.rand(B, T, generator=g, device=dev) * 5
+    lo = ln + torch.randn(B, T, generator=g, device=dev) * drift
+    lu = torch.log(torch.rand(B, T, generator=g, device=dev))
+    ids = torch.randint(0, 150000, (B, T), generator=g, device=dev)
+    if lengths is None:
+        lengths = torch.randint(0, T + 1, (B,), generator=torch.Generator().manual_seed(seed))
+    mask = synthetic.right_pad_mask(lengths, T, dev)
+    return ln, lo, lu, mask, ids
+
+
+@pytest.mark.parametrize("B,T", [(1, 1), (3, 63), (4, 64), (5, 65), (8, 512), (7, 1000), (2, 5000)])
+@pytest.mark.parametrize("off", [0.0, 0.5, -0.5])
+def test_padded_matches_oracles(dev, B, T, off):
+    ln, lo, lu, mask, ids = _inputs(dev, B, T, seed=B * 1000 + T)
+    res = sv.spec_verify(ln, lo, mask, log_u=lu, thresh_offset=off, draft_ids=ids, pad_id=-7)
+    _same(res, overify.verify(ln, lo, lu, mask, off, draft_ids=ids, pad_id=-7), with_draft=True)
+    _same(res, c_oracle.spec_verify(ln, lo, lu, mask, off, draft_ids=ids, pad_id=-7), with_draft=True)
+    if B * T <= 4096:
+        _same(res, overify.verify_loops(ln, lo, lu, mask, off, draft_ids=ids, pad_id=-7), with_draft=True)
+
+
+def test_mask_dtypes_and_no_mask(dev):
+    ln, lo, lu, mask, ids = _inputs(dev, 6, 200, seed=5)
+    ref = overify.verify(ln, lo, lu, mask, 0.0)
+    for m in (mask, mask.long(), mask.float(), mask.to(torch.uint8), mask.int() * 3):
+        _same(sv.spec_verify(ln, lo, m, log_u=lu), ref)
+    _same(sv.spec_verify(ln, lo, None, log_u=lu), overify.verify(ln, lo, lu, None, 0.0))
+
+
+def test_masks_with_holes(dev):
+    # multi-turn style masks: tool-output tokens inside the response are masked out
+    ln, lo, lu, _, ids = _inputs(dev, 9, 333, seed=6)
+    g = torch.Generator(device=dev).manual_seed(60)
+    mask = torch.rand(9, 333, generator=g, device=dev) < 0.6
+    mask[0] = False           # no valid token at all
+    mask[1, :] = True
+    res = sv.spec_verify(ln, lo, mask, log_u=lu, draft_ids=ids)
+    _same(res, c_oracle.spec_verify(ln, lo, lu, mask, 0.0, draft_ids=ids), with_draft=True)
+    _same(res, overify.verify_loops(ln, lo, lu, mask, 0.0, draft_ids=ids), with_draft=True)
+    assert res.first_reject[0].item() == 0 and res.prefix_len[0].item() == 0
+
+
+def test_packed_layout_ragged_lengths(dev):
+    lengths = torch.tensor([0, 1, 63, 64, 65, 300, 0, 2049, 17, 256])
+    cu = synthetic.pack_by_lengths(lengths)
+    N = int(cu[-1])
+    g = torch.Generator(device=dev).manual_seed(8)
+    ln = -torch.rand(N, generator=g, device=dev) * 4
+    lo = ln + torch.randn(N, generator=g, device=dev) * 0.2
+    lu = torch.log(torch.rand(N, generator=g, device=dev))
+    mask = torch.rand(N, generator=g, device=dev) < 0.9
+    ids = torch.randint(0, 1000, (N,), generator=g, device=dev)
+    for m in (None, mask):
+        res = sv.spec_verify(ln, lo, m, log_u=lu, thresh_offset=0.25, cu_seqlens=cu.to(dev), draft_ids=ids, pad_id=1)
+        _same(res, c_oracle.spec_verify(ln, lo, lu, m, 0.25, cu_seqlens=cu, draft_ids=ids, pad_id=1), with_draft=True)
+        _same(res, overify.verify(ln, lo, lu, m, 0.25, cu_seqlens=cu, draft_ids=ids, pad_id=1), with_draft=True)
+
+
+def test_exact_rows(dev):
+    # hand-computed: d = -1.0 everywhere, log u = -2.0 / -0.5 / -1.0 (boundary)
+    ln = torch.full((3, 6), -2.0, device=dev)
+    lo = torch.full((3, 6), -1.0, device=dev)
+    lu = torch.tensor([[-2.0] * 6, [-2.0, -2.0, -0.5, -2.0, -0.5, -2.0], [-1.0] * 6], device=dev)
+    mask = torch.tensor([[1, 1, 1, 1, 0, 0], [1, 1, 1, 1, 1, 1], [1, 1, 1, 0, 0, 0]], device=dev)
+    res = sv.spec_verify(ln, lo, mask, log_u=lu, near_eps=1e-6)
+    assert res.accept.int().tolist() == [[1, 1, 1, 1, 0, 0], [1, 1, 0, 1, 0, 1], [1, 1, 1, 0, 0, 0]]
+    assert res.first_reject.tolist() == [4, 2, 3]
+    assert res.prefix_len.tolist() == [4, 2, 3]
+    assert res.near_count.tolist() == [0, 0, 3]          # d == tau exactly on the valid tokens of row 2
+    # lenience: literal adds log(l) to the threshold, relax subtracts it
+    strict = sv.spec_verify(ln, lo, mask, log_u=lu, lenience=math.e, lenience_mode="literal")
+    assert strict.first_reject.tolist() == [4, 2, 0]     # tau = log u + 1: rows 0 (=-1, boundary) still accept
+    loose = sv.spec_verify(ln, lo, mask, log_u=lu, lenience=math.e, lenience_mode="relax")
+    assert loose.first_reject.tolist() == [4, 6, 3]
+
+
+def test_special_values(dev):
+    nan, inf = float("nan"), float("inf")
+    ln = torch.tensor([[-1.0, nan, -1.0, -1.0], [-1.0, -1.0, -inf, -1.0], [-1.0, -1.0, -1.0, -1.0]], device=dev)
+    lo = torch.full((3, 4), -1.0, device=dev)
+    lu = torch.tensor([[-1.0, -1.0, -1.0, -1.0], [-inf, -inf, -inf, -1.0], [-1.0, nan, -inf, -1.0]], device=dev)
+    res = sv.spec_verify(ln, lo, None, log_u=lu)
+    # NaN d rejects; u = 0 accepts any finite d; d = -inf vs tau = -inf accepts (>=); NaN tau rejects
+    assert res.accept.int().tolist() == [[1, 0, 1, 1], [1, 1, 1, 1], [1, 0, 1, 1]]
+    assert res.first_reject.tolist() == [1, 4, 1]
+    _same(res, c_oracle.spec_verify(ln, lo, lu, None, 0.0))
+    _same(res, overify.verify_loops(ln, lo, lu, None, 0.0))
+
+
+def test_seeded_uniforms_reproduce(dev):
+    ln, lo, _, mask, _ = _inputs(dev, 4, 100, seed=12)
+    a = sv.spec_verify(ln, lo, mask, seed=1234)
+    b = sv.spec_verify(ln, lo, mask, seed=1234)
+    c = sv.spec_verify(ln, lo, mask, seed=1235)
+    assert torch.equal(a.log_u, b.log_u) and torch.equal(a.accept, b.accept)
+    assert not torch.equal(a.log_u, c.log_u)
+    _same(a, overify.verify(ln, lo, a.log_u, mask, 0.0))
+    with pytest.raises(ValueError):
+        sv.spec_verify(ln, lo, mask)
+    with pytest.raises(ValueError):
+        sv.spec_verify(ln, lo, mask, seed=1, log_u=a.log_u)
+
+
+def test_truncate_draft_standalone_and_idempotent(dev):
+    ln, lo, lu, mask, ids = _inputs(dev, 5, 77, seed=13)
+    res = sv.spec_verify(ln, lo, mask, log_u=lu, draft_ids=ids, pad_id=9)
+    ids2, mask2 = sv.truncate_draft(ids, mask, res.first_reject, pad_id=9)
+    assert torch.equal(ids2, res.out_ids) and torch.equal(mask2, res.out_mask)
+    ids3, mask3 = sv.truncate_draft(ids2, mask2, res.first_reject, pad_id=9)
+    assert torch.equal(ids3, ids2) and torch.equal(mask3, mask2)
+
+
+def test_empty_shapes(dev):
+    z = torch.empty(0, 5, device=dev)
+    res = sv.spec_verify(z, z, None, log_u=z)
+    assert res.accept.shape == (0, 5) and res.first_reject.shape == (0,)
+    z = torch.empty(3, 0, device=dev)
+    res = sv.spec_verify(z, z, None, log_u=z)
+    assert res.first_reject.tolist() == [0, 0, 0] and res.prefix_len.tolist() == [0, 0, 0]
+
+
+def test_c5_imbalance_verify_only_full_size(dev):
+    """512 sequences, lengths log-uniform in [32, 16384], Student-t drift: packed layout, whole workload."""
+    w = synthetic.WORKLOADS["c5"]
+    lengths = synthetic.draw_lengths(w, seed=5002)
+    cu = synthetic.pack_by_lengths(lengths)
+    N = int(cu[-1])
+    g = torch.Generator(device=dev).manual_seed(5000)
+    ln = -torch.rand(N, generator=g, device=dev) * 6
+    lo = synthetic.drift_old_logprobs(ln, w, seed=5000)
+    lu = torch.log(torch.rand(N, generator=g, device=dev))
+    off = sv.thresh_offset_from_lenience(w.lenience)
+    assert off == 0.5
+    res = sv.spec_verify(ln, lo, None, log_u=lu, thresh_offset=off, cu_seqlens=cu.to(dev))
+    ref = c_oracle.spec_verify(ln, lo, lu, None, off, cu_seqlens=cu)
+    _same(res, ref)
+    _same(res, overify.verify(ln, lo, lu, None, off, cu_seqlens=cu))
+    assert (res.first_reject.cpu() <= lengths).all()
+    assert res.first_reject.float().mean().item() < lengths.float().mean().item()   # early rejections do happen

@@ -1,0 +1,148 @@
+// SPEC-RL draft verification: one workgroup per sequence.
+//
+// Per token: d = logp_new - logp_old, tau = log_u + thresh_offset, both single
+// fp32 operations (no multiply, so nothing can be contracted), accept iff the
+// token is valid and d >= tau. Each wavefront turns its 64 predicates into a
+// ballot; the first set bit of the first non-empty "rejected" ballot is that
+// wavefront's earliest rejection, and the minimum over wavefronts (through
+// LDS) is the sequence's. Counts come from popcounts of ballots, so every
+// per-sequence result is produced without atomics and is deterministic.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace vrl {
+
+constexpr int kNoReject = 0x7fffffff;
+
+struct SeqSpan {
+  int64_t start;
+  int64_t len;
+};
+
+__device__ __forceinline__ SeqSpan seq_span(const int64_t* cu_seqlens, int64_t b, int64_t T) {
+  SeqSpan s;
+  if (cu_seqlens != nullptr) {
+    s.start = cu_seqlens[b];
+    s.len = cu_seqlens[b + 1] - s.start;
+    if (s.len < 0) s.len = 0;
+  } else {
+    s.start = b * T;
+    s.len = T;
+  }
+  return s;
+}
+
+template <int WAVES>
+__device__ __forceinline__ void truncate_span(const SeqSpan sp, int first, const int64_t* draft_ids,
+                                              const uint8_t* mask, int64_t pad_id, int64_t* out_ids,
+                                              uint8_t* out_mask) {
+  constexpr int NTHR = WAVES * 64;
+  for (int64_t i = threadIdx.x; i < sp.len; i += NTHR) {
+    const bool keep = i < first;
+    const int64_t g = sp.start + i;
+    out_ids[g] = keep ? draft_ids[g] : pad_id;
+    const uint8_t mv = (mask != nullptr) ? static_cast<uint8_t>(mask[g] != 0) : static_cast<uint8_t>(1);
+    out_mask[g] = keep ? mv : static_cast<uint8_t>(0);
+  }
+}
+
+// grid.x = B, block = WAVES*64. No thread leaves before the last barrier.
+template <int WAVES>
+__global__ __launch_bounds__(WAVES * 64) void spec_verify_kernel(
+    const float* __restrict__ logp_new, const float* __restrict__ logp_old,
+    const float* __restrict__ log_u, const uint8_t* __restrict__ mask,
+    const int64_t* __restrict__ cu_seqlens, int64_t T, float thresh_offset, float near_eps,
+    uint8_t* __restrict__ accept, int32_t* __restrict__ first_reject,
+    int32_t* __restrict__ prefix_len, int32_t* __restrict__ near_count,
+    const int64_t* __restrict__ draft_ids, int64_t pad_id, int64_t* __restrict__ out_ids,
+    uint8_t* __restrict__ out_mask) {
+  constexpr int NTHR = WAVES * 64;
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = tid >> 6;
+  const int64_t b = blockIdx.x;
+  const SeqSpan sp = seq_span(cu_seqlens, b, T);
+
+  // wave-uniform running results
+  int first = kNoReject;  // earliest rejected position seen by this wavefront
+  int last_valid = 0;     // one past the last valid position seen by this wavefront
+  int near = 0;
+
+  for (int64_t base = 0; base < sp.len; base += NTHR) {
+    const int64_t i = base + tid;
+    bool valid = false, ok = false, close = false;
+    if (i < sp.len) {
+      const int64_t g = sp.start + i;
+      const float d = logp_new[g] - logp_old[g];
+      const float tau = log_u[g] + thresh_offset;
+      valid = (mask != nullptr) ? (mask[g] != 0) : true;
+      ok = d >= tau;
+      close = valid && (__builtin_fabsf(d - tau) < near_eps);
+      accept[g] = static_cast<uint8_t>(valid && ok);
+    }
+    const unsigned long long rej = __ballot(valid && !ok);
+    const unsigned long long val = __ballot(valid);
+    const unsigned long long nr = __ballot(close);
+    const int wbase = static_cast<int>(base) + wave * 64;
+    if (rej != 0ull && first == kNoReject) first = wbase + __builtin_ctzll(rej);
+    if (val != 0ull) last_valid = wbase + 64 - __builtin_clzll(val);
+    near += __builtin_popcountll(nr);
+  }
+
+  __shared__ int sm_first[WAVES];
+  __shared__ int sm_last[WAVES];
+  __shared__ int sm_near[WAVES];
+  __shared__ int sm_cnt[WAVES];
+  if (lane == 0) {
+    sm_first[wave] = first;
+    sm_last[wave] = last_valid;
+    sm_near[wave] = near;
+  }
+  __syncthreads();
+  int f = kNoReject, lv = 0, nc = 0;
+#pragma unroll
+  for (int w = 0; w < WAVES; ++w) {
+    f = min(f, sm_first[w]);
+    lv = max(lv, sm_last[w]);
+    nc += sm_near[w];
+  }
+  if (f == kNoReject) f = lv;
+
+  // valid tokens strictly before the first rejection
+  int cnt = 0;
+  if (mask != nullptr) {
+    for (int64_t base = 0; base < f; base += NTHR) {
+      const int64_t i = base + tid;
+      const bool v = (i < f) && (mask[sp.start + i] != 0);
+      cnt += __builtin_popcountll(__ballot(v));
+    }
+  }
+  if (lane == 0) sm_cnt[wave] = cnt;
+  __syncthreads();
+  if (tid == 0) {
+    int total = f;
+    if (mask != nullptr) {
+      total = 0;
+#pragma unroll
+      for (int w = 0; w < WAVES; ++w) total += sm_cnt[w];
+    }
+    first_reject[b] = f;
+    prefix_len[b] = total;
+    near_count[b] = nc;
+  }
+  if (out_ids != nullptr) truncate_span<WAVES>(sp, f, draft_ids, mask, pad_id, out_ids, out_mask);
+}
+
+template <int WAVES>
+__global__ __launch_bounds__(WAVES * 64) void truncate_draft_kernel(
+    const int64_t* __restrict__ draft_ids, const uint8_t* __restrict__ mask,
+    const int64_t* __restrict__ cu_seqlens, int64_t T, const int32_t* __restrict__ first_reject,
+    int64_t pad_id, int64_t* __restrict__ out_ids, uint8_t* __restrict__ out_mask) {
+  const int64_t b = blockIdx.x;
+  const SeqSpan sp = seq_span(cu_seqlens, b, T);
+  truncate_span<WAVES>(sp, first_reject[b], draft_ids, mask, pad_id, out_ids, out_mask);
+}
+
+}  // namespace vrl

@@ -1,0 +1,183 @@
+// C ABI of libvrl_hip.so: argument checks on the host, then kernel launches on
+// the caller's stream. Declarations and the reference interfaces each entry
+// point replaces are in include/vrl.h.
+#include "vrl.h"
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <string.h>
+
+#include "rowscore_kernels.h"
+#include "verify_kernels.h"
+
+namespace {
+
+thread_local char g_hip_error[256] = {0};
+
+int launch_status() {
+  const hipError_t e = hipGetLastError();
+  if (e == hipSuccess) return VRL_OK;
+  const char* msg = hipGetErrorString(e);
+  strncpy(g_hip_error, msg ? msg : "unknown HIP error", sizeof(g_hip_error) - 1);
+  g_hip_error[sizeof(g_hip_error) - 1] = 0;
+  return VRL_ERR_HIP;
+}
+
+bool aligned(const void* p, uintptr_t a) { return (reinterpret_cast<uintptr_t>(p) & (a - 1)) == 0; }
+
+constexpr int64_t kMaxGrid = 0x7fffffffLL;
+
+// Workgroup shape of the row kernel: wavefronts per row and 128-bit loads per
+// lane and batch.
+constexpr int kRowWaves = 4;
+constexpr int kRowUnroll = 4;
+
+int check_rowscore(const void* logits, int dtype, int64_t n_rows, int64_t vocab, int64_t row_stride,
+                   const int64_t* labels, const float* temperature, const float* out_logprob,
+                   const float* out_entropy, const int32_t* err_flag) {
+  if (dtype != VRL_F32 && dtype != VRL_BF16) return VRL_ERR_DTYPE;
+  if (n_rows < 0 || vocab <= 0 || row_stride < vocab || n_rows > kMaxGrid) return VRL_ERR_SHAPE;
+  if (out_logprob == nullptr && out_entropy == nullptr) return VRL_ERR_ARG;
+  if (n_rows == 0) return VRL_OK;
+  if (logits == nullptr) return VRL_ERR_NULL;
+  if (out_logprob != nullptr && (labels == nullptr || err_flag == nullptr)) return VRL_ERR_NULL;
+  const uintptr_t esize = (dtype == VRL_F32) ? 4 : 2;
+  if (!aligned(logits, esize) || !aligned(labels, 8) || !aligned(temperature, 4) ||
+      !aligned(out_logprob, 4) || !aligned(out_entropy, 4) || !aligned(err_flag, 4))
+    return VRL_ERR_ALIGN;
+  return VRL_OK;
+}
+
+template <int DT, bool EXACT>
+void launch_rowscore(const void* logits, int64_t n_rows, int64_t vocab, int64_t row_stride,
+                     const int64_t* labels, const float* temperature, float* out_logprob,
+                     float* out_entropy, int32_t* err_flag, hipStream_t stream) {
+  const dim3 grid(static_cast<unsigned>(n_rows));
+  const dim3 block(kRowWaves * 64);
+  vrl::rowscore_kernel<DT, kRowWaves, kRowUnroll, EXACT, true><<<grid, block, 0, stream>>>(
+      logits, vocab, row_stride, labels, temperature, out_logprob, out_entropy, err_flag);
+}
+
+int check_verify(const float* logp_new, const float* logp_old, const float* log_u, const uint8_t* mask,
+                 const int64_t* cu_seqlens, int64_t B, int64_t T, const uint8_t* accept,
+                 const int32_t* first_reject, const int32_t* prefix_len, const int32_t* near_count,
+                 const int64_t* draft_ids, const int64_t* out_ids, const uint8_t* out_mask) {
+  (void)mask;
+  if (B < 0 || T < 0 || B > kMaxGrid || T > kMaxGrid) return VRL_ERR_SHAPE;
+  const bool any_trunc = (draft_ids != nullptr) || (out_ids != nullptr) || (out_mask != nullptr);
+  const bool all_trunc = (draft_ids != nullptr) && (out_ids != nullptr) && (out_mask != nullptr);
+  if (any_trunc && !all_trunc) return VRL_ERR_ARG;
+  if (B == 0) return VRL_OK;
+  if (first_reject == nullptr || prefix_len == nullptr || near_count == nullptr) return VRL_ERR_NULL;
+  // A padded layout with T == 0 has no tokens: the kernel only writes the per-sequence zeros.
+  const bool has_tokens = (cu_seqlens != nullptr) || (T > 0);
+  if (has_tokens && (logp_new == nullptr || logp_old == nullptr || log_u == nullptr || accept == nullptr))
+    return VRL_ERR_NULL;
+  if (!aligned(logp_new, 4) || !aligned(logp_old, 4) || !aligned(log_u, 4) || !aligned(cu_seqlens, 8) ||
+      !aligned(first_reject, 4) || !aligned(prefix_len, 4) || !aligned(near_count, 4) ||
+      !aligned(draft_ids, 8) || !aligned(out_ids, 8))
+    return VRL_ERR_ALIGN;
+  return VRL_OK;
+}
+
+constexpr int kVerifyWaves = 4;
+
+}  // namespace
+
+extern "C" {
+
+int vrl_rowscore(const void* logits, int dtype, int64_t n_rows, int64_t vocab, int64_t row_stride,
+                 const int64_t* labels, const float* temperature, float* out_logprob,
+                 float* out_entropy, int32_t* err_flag, void* stream) {
+  const int st = check_rowscore(logits, dtype, n_rows, vocab, row_stride, labels, temperature,
+                                out_logprob, out_entropy, err_flag);
+  if (st != VRL_OK || n_rows == 0) return st;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  if (dtype == VRL_F32) {
+    if (temperature != nullptr)
+      launch_rowscore<VRL_F32, true>(logits, n_rows, vocab, row_stride, labels, temperature,
+                                     out_logprob, out_entropy, err_flag, s);
+    else
+      launch_rowscore<VRL_F32, false>(logits, n_rows, vocab, row_stride, labels, temperature,
+                                      out_logprob, out_entropy, err_flag, s);
+  } else {
+    launch_rowscore<VRL_BF16, false>(logits, n_rows, vocab, row_stride, labels, temperature,
+                                     out_logprob, out_entropy, err_flag, s);
+  }
+  return launch_status();
+}
+
+int vrl_spec_verify(const float* logp_new, const float* logp_old, const float* log_u,
+                    const uint8_t* mask, const int64_t* cu_seqlens, int64_t B, int64_t T,
+                    float thresh_offset, float near_eps, uint8_t* accept, int32_t* first_reject,
+                    int32_t* prefix_len, int32_t* near_count, const int64_t* draft_ids,
+                    int64_t pad_id, int64_t* out_ids, uint8_t* out_mask, void* stream) {
+  const int st = check_verify(logp_new, logp_old, log_u, mask, cu_seqlens, B, T, accept, first_reject,
+                              prefix_len, near_count, draft_ids, out_ids, out_mask);
+  if (st != VRL_OK || B == 0) return st;
+  vrl::spec_verify_kernel<kVerifyWaves>
+      <<<dim3(static_cast<unsigned>(B)), dim3(kVerifyWaves * 64), 0, static_cast<hipStream_t>(stream)>>>(
+          logp_new, logp_old, log_u, mask, cu_seqlens, T, thresh_offset, near_eps, accept,
+          first_reject, prefix_len, near_count, draft_ids, pad_id, out_ids, out_mask);
+  return launch_status();
+}
+
+int vrl_truncate_draft(const int64_t* draft_ids, const uint8_t* mask, const int64_t* cu_seqlens,
+                       int64_t B, int64_t T, const int32_t* first_reject, int64_t pad_id,
+                       int64_t* out_ids, uint8_t* out_mask, void* stream) {
+  if (B < 0 || T < 0 || B > kMaxGrid || T > kMaxGrid) return VRL_ERR_SHAPE;
+  if (B == 0 || (cu_seqlens == nullptr && T == 0)) return VRL_OK;
+  if (draft_ids == nullptr || first_reject == nullptr || out_ids == nullptr || out_mask == nullptr)
+    return VRL_ERR_NULL;
+  if (!aligned(draft_ids, 8) || !aligned(out_ids, 8) || !aligned(cu_seqlens, 8) ||
+      !aligned(first_reject, 4))
+    return VRL_ERR_ALIGN;
+  vrl::truncate_draft_kernel<kVerifyWaves>
+      <<<dim3(static_cast<unsigned>(B)), dim3(kVerifyWaves * 64), 0, static_cast<hipStream_t>(stream)>>>(
+          draft_ids, mask, cu_seqlens, T, first_reject, pad_id, out_ids, out_mask);
+  return launch_status();
+}
+
+int vrl_fused_score_verify(const void* logits, int dtype, int64_t n_rows, int64_t vocab,
+                           int64_t row_stride, const int64_t* labels, const float* temperature,
+                           float* out_logprob, float* out_entropy, int32_t* err_flag,
+                           const float* logp_old, const float* log_u, const uint8_t* mask,
+                           const int64_t* cu_seqlens, int64_t B, int64_t T, float thresh_offset,
+                           float near_eps, uint8_t* accept, int32_t* first_reject,
+                           int32_t* prefix_len, int32_t* near_count, const int64_t* draft_ids,
+                           int64_t pad_id, int64_t* out_ids, uint8_t* out_mask, void* stream) {
+  // Check both halves before anything is enqueued.
+  if (out_logprob == nullptr && n_rows > 0) return VRL_ERR_NULL;
+  int st = check_rowscore(logits, dtype, n_rows, vocab, row_stride, labels, temperature, out_logprob,
+                          out_entropy, err_flag);
+  if (st != VRL_OK) return st;
+  st = check_verify(out_logprob, logp_old, log_u, mask, cu_seqlens, B, T, accept, first_reject,
+                    prefix_len, near_count, draft_ids, out_ids, out_mask);
+  if (st != VRL_OK) return st;
+  if (cu_seqlens == nullptr && n_rows != B * T) return VRL_ERR_SHAPE;
+  st = vrl_rowscore(logits, dtype, n_rows, vocab, row_stride, labels, temperature, out_logprob,
+                    out_entropy, err_flag, stream);
+  if (st != VRL_OK) return st;
+  return vrl_spec_verify(out_logprob, logp_old, log_u, mask, cu_seqlens, B, T, thresh_offset, near_eps,
+                         accept, first_reject, prefix_len, near_count, draft_ids, pad_id, out_ids,
+                         out_mask, stream);
+}
+
+const char* vrl_strerror(int status) {
+  switch (status) {
+    case VRL_OK: return "ok";
+    case VRL_ERR_NULL: return "a required pointer is NULL";
+    case VRL_ERR_DTYPE: return "unsupported logits dtype (expected VRL_F32 or VRL_BF16)";
+    case VRL_ERR_SHAPE: return "bad shape (negative count, vocab <= 0, row_stride < vocab, or too many rows)";
+    case VRL_ERR_ALIGN: return "pointer is not aligned to its element size";
+    case VRL_ERR_HIP: return "the HIP runtime refused the kernel launch";
+    case VRL_ERR_ARG: return "inconsistent optional arguments";
+    default: return "unknown vrl status";
+  }
+}
+
+const char* vrl_last_hip_error(void) { return g_hip_error; }
+
+int vrl_abi_version(void) { return VRL_ABI_VERSION; }
+
+}  // extern "C"

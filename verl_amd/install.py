@@ -1,0 +1,120 @@
+"""Put the HIP scoring path behind verl's own function names.
+
+What gets replaced (verl/utils/torch_functional.py):
+    logprobs_from_logits :73, logprobs_from_logits_v2 :173, logprobs_from_logits_naive :155,
+    entropy_from_logits :231, entropy_from_logits_with_chunking :248
+and every copy of those names that an already imported ``verl.*`` module bound
+with ``from verl.utils.torch_functional import ...`` (the engines do so at
+verl/workers/engine/fsdp/transformer_impl.py:66 and siblings; the reference's
+own tests patch exactly that bound name,
+tests/workers/test_distillation_topk_symmetry_on_cpu.py:143-146).
+
+A replaced function sends GPU tensors of a supported dtype under no_grad to
+the HIP kernel. Anything else (CPU tensors on the driver, fp16/fp64, tensors
+that need a backward) is handed to the function it replaced, i.e. verl's own
+code, and counted in ``stats()``: this package adds no second implementation.
+"""
+
+from __future__ import annotations
+
+import functools
+import importlib
+import sys
+from typing import Callable, Dict, List, Tuple
+
+import torch
+
+from . import torch_functional as _amd
+
+TARGET_MODULE = "verl.utils.torch_functional"
+PATCHED_NAMES = (
+    "logprobs_from_logits",
+    "logprobs_from_logits_v2",
+    "logprobs_from_logits_naive",
+    "entropy_from_logits",
+    "entropy_from_logits_with_chunking",
+)
+
+_originals: Dict[str, Callable] = {}
+_rebound: List[Tuple[object, str, Callable]] = []
+_stats = {"hip_calls": 0, "passed_to_verl": 0}
+
+
+def _eligible(logits) -> bool:
+    return (
+        isinstance(logits, torch.Tensor)
+        and logits.is_cuda
+        and logits.dtype in (torch.float32, torch.bfloat16)
+        and logits.dim() >= 1
+        and logits.shape[-1] > 0
+        and not (torch.is_grad_enabled() and logits.requires_grad)
+    )
+
+
+def _make_shim(name: str, original: Callable) -> Callable:
+    ours = getattr(_amd, name)
+
+    @functools.wraps(original)
+    def shim(logits, *args, **kwargs):
+        if _eligible(logits):
+            _stats["hip_calls"] += 1
+            return ours(logits, *args, **kwargs)
+        _stats["passed_to_verl"] += 1
+        return original(logits, *args, **kwargs)
+
+    shim.__verl_amd_original__ = original
+    return shim
+
+
+def stats() -> dict:
+    """Calls served by the HIP kernel vs handed back to verl since install()."""
+    return dict(_stats)
+
+
+def install(target_module: str = TARGET_MODULE) -> List[str]:
+    """Patch ``target_module`` and re-bind the names in already imported ``verl.*`` modules.
+
+    Returns the fully qualified names that were replaced. Calling it twice is a no-op.
+    """
+    if _originals:
+        return []
+    mod = importlib.import_module(target_module)
+    replaced = []
+    shims = {}
+    for name in PATCHED_NAMES:
+        original = getattr(mod, name, None)
+        if original is None:
+            continue
+        shim = _make_shim(name, original)
+        _originals[name] = original
+        shims[name] = shim
+        setattr(mod, name, shim)
+        replaced.append(f"{target_module}.{name}")
+    root = target_module.split(".")[0] + "."
+    for mod_name, other in list(sys.modules.items()):
+        if other is None or other is mod or not mod_name.startswith(root):
+            continue
+        for name, shim in shims.items():
+            if getattr(other, name, None) is _originals[name]:
+                setattr(other, name, shim)
+                _rebound.append((other, name, _originals[name]))
+                replaced.append(f"{mod_name}.{name}")
+    _installed_in.append(mod)
+    return replaced
+
+
+_installed_in: List[object] = []
+
+
+def uninstall() -> None:
+    """Undo install()."""
+    for other, name, original in _rebound:
+        setattr(other, name, original)
+    _rebound.clear()
+    for mod in _installed_in:
+        for name, original in _originals.items():
+            setattr(mod, name, original)
+    _installed_in.clear()
+    _originals.clear()
+    _stats["hip_calls"] = 0
+    _stats["passed_to_verl"] = 0

@@ -1,0 +1,195 @@
+"""Per-token scoring on MI355X behind the names of verl.utils.torch_functional.
+
+Same names, argument meaning and leading-shape handling as the reference
+functions (verl/utils/torch_functional.py:73-107, 155-207, 231-270); the work
+is done by the HIP row kernel through the C ABI (include/vrl.h). Inputs must
+live on the GPU: there is no CPU or eager-torch path in this module, and a
+missing libvrl_hip.so raises.
+
+Differences from the reference that a caller can observe:
+  * results are fp32 for bf16 inputs too (the reference's non-fp32 branch
+    returns the input dtype, :199-206; its flash-attn branch returns fp32);
+  * a label outside [0, vocab) raises IndexError after the kernel ran
+    (torch.gather device-asserts);
+  * inputs that require grad raise NotImplementedError (forward-only).
+"""
+
+from __future__ import annotations
+
+from typing import Optional, Union
+
+import torch
+
+from . import _lib
+
+__all__ = [
+    "logprobs_from_logits",
+    "logprobs_from_logits_v2",
+    "logprobs_from_logits_naive",
+    "entropy_from_logits",
+    "entropy_from_logits_with_chunking",
+    "fused_logprob_entropy",
+]
+
+_DTYPE_CODES = {torch.float32: _lib.VRL_F32, torch.bfloat16: _lib.VRL_BF16}
+
+
+def _ptr(t: Optional[torch.Tensor]) -> Optional[int]:
+    return None if t is None else t.data_ptr()
+
+
+def _check_logits(logits: torch.Tensor, what: str) -> None:
+    if not isinstance(logits, torch.Tensor):
+        raise TypeError(f"{what}: logits must be a torch.Tensor, got {type(logits).__name__}")
+    if not logits.is_cuda:
+        raise RuntimeError(
+            f"{what}: logits are on {logits.device}; verl_amd only runs on the GPU (HIP kernels), "
+            "it has no CPU implementation"
+        )
+    if logits.dtype not in _DTYPE_CODES:
+        raise TypeError(f"{what}: logits dtype {logits.dtype} is not supported (float32 and bfloat16 are)")
+    if logits.dim() < 1 or logits.shape[-1] == 0:
+        raise ValueError(f"{what}: logits need a non-empty last (vocab) dimension, got shape {tuple(logits.shape)}")
+    if torch.is_grad_enabled() and logits.requires_grad:
+        raise NotImplementedError(
+            f"{what}: logits require grad, but this is the forward-only scoring path "
+            "(call it under torch.no_grad(), as the reference's compute_log_prob does)"
+        )
+
+
+def _rows_2d(logits: torch.Tensor) -> torch.Tensor:
+    """(..., V) -> (N, V) with unit stride along V; a view whenever torch allows one."""
+    V = logits.shape[-1]
+    if logits.dim() == 2:
+        x = logits
+    else:
+        x = logits.reshape(-1, V)
+    if x.stride(-1) != 1 or (x.shape[0] > 1 and x.stride(0) < V):
+        x = x.contiguous()
+    return x
+
+
+def _temperature_rows(temperature, lead_shape, n_rows, device) -> Optional[torch.Tensor]:
+    if temperature is None:
+        return None
+    if isinstance(temperature, (int, float)):
+        return torch.full((n_rows,), float(temperature), dtype=torch.float32, device=device)
+    t = temperature.to(device=device, dtype=torch.float32)
+    if t.numel() == 1:
+        return t.reshape(1).expand(n_rows).contiguous()
+    if t.numel() != n_rows:
+        raise ValueError(
+            f"temperature has {t.numel()} entries, expected one per token ({n_rows}) for logits leading shape {tuple(lead_shape)}"
+        )
+    return t.reshape(n_rows).contiguous()
+
+
+def rowscore(
+    logits: torch.Tensor,
+    labels: Optional[torch.Tensor],
+    temperature: Union[None, float, torch.Tensor] = None,
+    *,
+    want_logprob: bool = True,
+    want_entropy: bool = True,
+    check_labels: bool = True,
+    what: str = "rowscore",
+):
+    """Launch vrl_rowscore; returns (logprob | None, entropy | None), each fp32 of shape logits.shape[:-1]."""
+    _check_logits(logits, what)
+    if not (want_logprob or want_entropy):
+        raise ValueError(f"{what}: nothing to compute")
+    lead = logits.shape[:-1]
+    V = logits.shape[-1]
+    x = _rows_2d(logits)
+    n = x.shape[0]
+    dev = x.device
+
+    lab = None
+    if want_logprob:
+        if labels is None:
+            raise ValueError(f"{what}: labels are required for log-probs")
+        if tuple(labels.shape) != tuple(lead):
+            raise ValueError(f"{what}: labels shape {tuple(labels.shape)} does not match logits leading shape {tuple(lead)}")
+        if labels.dtype.is_floating_point or labels.dtype == torch.bool:
+            raise TypeError(f"{what}: labels must be an integer tensor, got {labels.dtype}")
+        lab = labels.to(device=dev, dtype=torch.int64).reshape(n).contiguous()
+
+    temp = _temperature_rows(temperature, lead, n, dev)
+    out_lp = torch.empty(n, dtype=torch.float32, device=dev) if want_logprob else None
+    out_h = torch.empty(n, dtype=torch.float32, device=dev) if want_entropy else None
+    flag = torch.zeros(1, dtype=torch.int32, device=dev) if want_logprob else None
+
+    if n > 0:
+        lib = _lib.load()
+        with torch.cuda.device(dev):
+            stream = torch.cuda.current_stream(dev).cuda_stream
+            st = lib.vrl_rowscore(
+                x.data_ptr(), _DTYPE_CODES[x.dtype], n, V, x.stride(0) if n > 1 else V,
+                _ptr(lab), _ptr(temp), _ptr(out_lp), _ptr(out_h), _ptr(flag), stream,
+            )
+        _lib.check("vrl_rowscore", st)
+        if want_logprob and check_labels and (int(flag.item()) & _lib.VRL_FLAG_LABEL_OOB):
+            raise IndexError(f"{what}: a label is outside [0, {V})")
+
+    lp = out_lp.reshape(lead) if want_logprob else None
+    h = out_h.reshape(lead) if want_entropy else None
+    return lp, h
+
+
+def logprobs_from_logits(logits: torch.Tensor, labels: torch.Tensor, inplace_backward: bool = True) -> torch.Tensor:
+    """log softmax(logits)[labels], shape logits.shape[:-1], fp32.
+
+    Mirrors verl/utils/torch_functional.py:73-107. ``inplace_backward`` only
+    matters to the reference's flash-attn backward and is accepted and ignored.
+    """
+    del inplace_backward
+    return rowscore(logits, labels, want_entropy=False, what="logprobs_from_logits")[0]
+
+
+def logprobs_from_logits_v2(logits: torch.Tensor, labels: torch.Tensor) -> torch.Tensor:
+    """Same result as logprobs_from_logits (verl/utils/torch_functional.py:173-207)."""
+    return rowscore(logits, labels, want_entropy=False, what="logprobs_from_logits_v2")[0]
+
+
+def logprobs_from_logits_naive(logits: torch.Tensor, labels: torch.Tensor) -> torch.Tensor:
+    """Same result as logprobs_from_logits (verl/utils/torch_functional.py:155-170)."""
+    return rowscore(logits, labels, want_entropy=False, what="logprobs_from_logits_naive")[0]
+
+
+def entropy_from_logits(logits: torch.Tensor) -> torch.Tensor:
+    """logsumexp(logits) - sum(softmax(logits) * logits) over the last dim, fp32.
+
+    Mirrors verl/utils/torch_functional.py:231-245.
+    """
+    return rowscore(logits, None, want_logprob=False, what="entropy_from_logits")[1]
+
+
+def entropy_from_logits_with_chunking(logits: torch.Tensor, chunk_size: int = 2048) -> torch.Tensor:
+    """Same value as entropy_from_logits (verl/utils/torch_functional.py:248-270).
+
+    The reference chunks rows to bound the size of its softmax temporaries; the
+    row kernel has no temporaries, so ``chunk_size`` is validated and unused.
+    """
+    if int(chunk_size) <= 0:
+        raise ValueError(f"chunk_size must be positive, got {chunk_size}")
+    return rowscore(logits, None, want_logprob=False, what="entropy_from_logits_with_chunking")[1]
+
+
+def fused_logprob_entropy(
+    logits: torch.Tensor,
+    labels: torch.Tensor,
+    temperature: Union[None, float, torch.Tensor] = None,
+    *,
+    check_labels: bool = True,
+):
+    """(log-probs, entropy) of softmax(logits / temperature) in one pass over the logits.
+
+    Replaces the three steps of the reference's engine
+    (verl/workers/engine/fsdp/transformer_impl.py:1357 divide, :1364-1376 entropy,
+    :1395-1399 log-probs). ``temperature`` is a float, or a tensor with one entry
+    per token (same leading shape as ``labels``), clamped below at 1e-8 like the
+    reference. For fp32 logits the quotient is rounded per element exactly like
+    ``logits / temperature``; for bf16 logits it is formed in fp32 from the bf16
+    values (the reference rounds the quotient back to bf16).
+    """
+    return rowscore(logits, labels, temperature, check_labels=check_labels, what="fused_logprob_entropy")
