@@ -26,7 +26,7 @@ if REPO not in sys.path:
     sys.path.insert(0, REPO)
 
 from verl_amd import _lib, synthetic  # noqa: E402
-from verl_amd import spec_verify as sv  # noqa: E402
+from verl_amd import spec_rl as sv  # noqa: E402
 from verl_amd import torch_functional as vf  # noqa: E402
 
 HBM_PEAK_GBPS = 8000.0
@@ -112,9 +112,11 @@ class Step:
         ref_h = lse - (torch.softmax(z, -1) * z).sum(-1)
         e1 = (self.lp[:rows] - ref_lp).abs().max().item()
         e2 = (self.h[:rows] - ref_h).abs().max().item()
-        tol = 1e-5 if self.w.dtype == torch.float32 else 2e-3
-        if not (e1 <= tol and e2 <= tol):
-            raise SystemExit(f"bench: kernel disagrees with torch fp32 (logprob {e1}, entropy {e2}, tol {tol})")
+        # A coarse guard, not the parity test: torch's own fp32 entropy on the GPU is up to ~1.3e-5 from the
+        # exact value at V ~ 128k (tests/_parity.py measures it against the fp64 oracle), hence 5e-5 there.
+        tol_lp, tol_h = (1e-5, 5e-5) if self.w.dtype == torch.float32 else (2e-3, 2e-3)
+        if not (e1 <= tol_lp and e2 <= tol_h):
+            raise SystemExit(f"bench: kernel disagrees with torch fp32 (logprob {e1} > {tol_lp} or entropy {e2} > {tol_h})")
         if int(self.flag.item()) != 0:
             raise SystemExit("bench: label out of range flagged")
         return e1, e2
@@ -162,7 +164,7 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     args = ap.parse_args()
     if args.gpus != 1:
-        print("bench.py: this build runs on one GPU only (rows are independent; see DESIGN.md for how it would shard); "
+        print("bench.py: this build runs on one GPU only; "
               f"--gpus {args.gpus} is not supported", file=sys.stderr)
         sys.exit(2)
     if not torch.cuda.is_available():

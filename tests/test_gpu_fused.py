@@ -5,10 +5,11 @@ import numpy as np
 import pytest
 import torch
 
-from verl_amd import spec_verify as sv
+from verl_amd import spec_rl as sv
 from verl_amd import synthetic
 from verl_amd import torch_functional as vf
 from oracle import c_oracle, scoring, verify as overify
+from _parity import assert_scores_match
 
 pytestmark = pytest.mark.gpu
 
@@ -28,8 +29,7 @@ def _run(dev, name, B, T, seed, packed=False):
                                        thresh_offset=off, draft_ids=ids, pad_id=0)
     tol = 1e-5 if w.dtype == torch.float32 else 2e-3
     valid = mask.cpu()
-    assert (lp.cpu() - ref_lp)[valid].abs().max().item() <= tol
-    assert (h.cpu() - ref_h)[valid].abs().max().item() <= tol
+    assert_scores_match(lp, h, logits, labels, temp, valid=mask)
 
     # (i) verify fed the kernel's own log-probs must equal the rule applied to those log-probs, bit for bit
     own = overify.verify(lp, logp_old, log_u, mask, off, draft_ids=ids, pad_id=0)

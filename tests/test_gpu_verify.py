@@ -6,7 +6,7 @@ import numpy as np
 import pytest
 import torch
 
-from verl_amd import spec_verify as sv
+from verl_amd import spec_rl as sv
 from verl_amd import synthetic
 from oracle import c_oracle, verify as overify
 

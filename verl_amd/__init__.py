@@ -12,7 +12,7 @@ Setting ``VERL_USE_EXTERNAL_MODULES=verl_amd.plugin`` makes verl import
 """
 
 from .install import install, uninstall
-from .spec_verify import (
+from .spec_rl import (
     VerifyResult,
     draw_log_uniforms,
     fused_score_verify,
