@@ -1,0 +1,139 @@
+"""The C ABI without a GPU: the library loads, exports exactly what include/vrl.h declares, and every
+argument error is caught on the host before anything could be launched."""
+
+import ctypes
+import os
+import re
+
+import pytest
+
+from verl_amd import _lib
+
+HEADER = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "include", "vrl.h")
+
+
+def _declarations():
+    text = open(HEADER).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    decls = {}
+    for m in re.finditer(r"\b(?:int|const char\*)\s+(vrl_\w+)\s*\(([^)]*)\)\s*;", text):
+        args = m.group(2).strip()
+        n = 0 if args in ("", "void") else len(args.split(","))
+        decls[m.group(1)] = n
+    return decls
+
+
+@pytest.fixture(scope="module")
+def lib():
+    return _lib.load()
+
+
+def test_header_and_binding_declare_the_same_entry_points():
+    decls = _declarations()
+    assert set(decls) == set(_lib.SIGNATURES), (sorted(decls), sorted(_lib.SIGNATURES))
+    for name, nargs in decls.items():
+        assert len(_lib.SIGNATURES[name][1]) == nargs, name
+
+
+def test_library_exports_every_declared_symbol(lib):
+    raw = ctypes.CDLL(_lib.LIB_PATH)
+    for name in _declarations():
+        assert hasattr(raw, name), name
+    assert lib.vrl_abi_version() == _lib.ABI_VERSION
+    m = re.search(r"#define VRL_ABI_VERSION (\d+)", open(HEADER).read())
+    assert int(m.group(1)) == _lib.ABI_VERSION
+
+
+def test_status_codes_match_header_and_have_text(lib):
+    text = open(HEADER).read()
+    for name in ("VRL_OK", "VRL_ERR_NULL", "VRL_ERR_DTYPE", "VRL_ERR_SHAPE", "VRL_ERR_ALIGN", "VRL_ERR_HIP", "VRL_ERR_ARG"):
+        m = re.search(rf"#define {name} \(?(-?\d+)\)?", text)
+        assert int(m.group(1)) == getattr(_lib, name), name
+        assert lib.vrl_strerror(getattr(_lib, name)).decode() not in ("", "unknown vrl status")
+    assert lib.vrl_strerror(-99).decode() == "unknown vrl status"
+    assert lib.vrl_last_hip_error().decode() == ""
+
+
+# Fake, suitably aligned "device pointers": every call below must return before touching them.
+P = 0x10000
+
+
+def test_rowscore_argument_errors(lib):
+    f = lib.vrl_rowscore
+    ok = dict(logits=P, dtype=_lib.VRL_BF16, n=4, V=100, stride=100, labels=P, temp=None, lp=P, h=P, flag=P)
+
+    def call(**kw):
+        a = {**ok, **kw}
+        return f(a["logits"], a["dtype"], a["n"], a["V"], a["stride"], a["labels"], a["temp"], a["lp"], a["h"], a["flag"], None)
+
+    assert call(dtype=7) == _lib.VRL_ERR_DTYPE
+    assert call(n=-1) == _lib.VRL_ERR_SHAPE
+    assert call(V=0) == _lib.VRL_ERR_SHAPE
+    assert call(stride=99) == _lib.VRL_ERR_SHAPE
+    assert call(n=2**31) == _lib.VRL_ERR_SHAPE
+    assert call(lp=None, h=None) == _lib.VRL_ERR_ARG
+    assert call(logits=None) == _lib.VRL_ERR_NULL
+    assert call(labels=None) == _lib.VRL_ERR_NULL
+    assert call(flag=None) == _lib.VRL_ERR_NULL
+    assert call(logits=P + 1) == _lib.VRL_ERR_ALIGN
+    assert call(dtype=_lib.VRL_F32, logits=P + 2) == _lib.VRL_ERR_ALIGN
+    assert call(labels=P + 4) == _lib.VRL_ERR_ALIGN
+    assert call(lp=P + 2) == _lib.VRL_ERR_ALIGN
+    assert call(temp=P + 1) == _lib.VRL_ERR_ALIGN
+    # nothing to do is not an error, and needs no pointers
+    assert f(None, _lib.VRL_F32, 0, 100, 100, None, None, None, P, None, None) == _lib.VRL_OK
+
+
+def test_verify_argument_errors(lib):
+    f = lib.vrl_spec_verify
+
+    def call(ln=P, lo=P, lu=P, mask=None, cu=None, B=2, T=8, accept=P, first=P, prefix=P, near=P, ids=None, out_ids=None, out_mask=None):
+        return f(ln, lo, lu, mask, cu, B, T, 0.0, 1e-6, accept, first, prefix, near, ids, 0, out_ids, out_mask, None)
+
+    assert call(B=-1) == _lib.VRL_ERR_SHAPE
+    assert call(T=-1) == _lib.VRL_ERR_SHAPE
+    assert call(ln=None) == _lib.VRL_ERR_NULL
+    assert call(lu=None) == _lib.VRL_ERR_NULL
+    assert call(accept=None) == _lib.VRL_ERR_NULL
+    assert call(first=None) == _lib.VRL_ERR_NULL
+    assert call(ids=P) == _lib.VRL_ERR_ARG                      # draft without outputs
+    assert call(ids=P, out_ids=P) == _lib.VRL_ERR_ARG
+    assert call(lo=P + 2) == _lib.VRL_ERR_ALIGN
+    assert call(cu=P + 4) == _lib.VRL_ERR_ALIGN
+    assert call(B=0, ln=None, lo=None, lu=None, accept=None, first=None, prefix=None, near=None) == _lib.VRL_OK
+
+
+def test_truncate_and_fused_argument_errors(lib):
+    t = lib.vrl_truncate_draft
+    assert t(P, None, None, -1, 4, P, 0, P, P, None) == _lib.VRL_ERR_SHAPE
+    assert t(None, None, None, 2, 4, P, 0, P, P, None) == _lib.VRL_ERR_NULL
+    assert t(P, None, None, 2, 4, None, 0, P, P, None) == _lib.VRL_ERR_NULL
+    assert t(P + 4, None, None, 2, 4, P, 0, P, P, None) == _lib.VRL_ERR_ALIGN
+    assert t(None, None, None, 0, 4, None, 0, None, None, None) == _lib.VRL_OK
+
+    f = lib.vrl_fused_score_verify
+
+    def call(n=16, B=2, T=8, lp=P, dtype=_lib.VRL_BF16, cu=None, lo=P):
+        return f(P, dtype, n, 100, 100, P, None, lp, P, P, lo, P, None, cu, B, T, 0.0, 1e-6, P, P, P, P, None, 0, None, None, None)
+
+    assert call(lp=None) == _lib.VRL_ERR_NULL                  # verify needs the log-probs
+    assert call(dtype=3) == _lib.VRL_ERR_DTYPE
+    assert call(n=15) == _lib.VRL_ERR_SHAPE                     # padded layout: n_rows must be B*T
+    assert call(lo=None) == _lib.VRL_ERR_NULL
+    assert call(B=-2) == _lib.VRL_ERR_SHAPE
+
+
+def test_missing_library_is_a_loud_error(tmp_path):
+    with pytest.raises(_lib.VrlLibraryError, match="does not exist"):
+        _lib.load(str(tmp_path / "libvrl_hip.so"))
+    bogus = tmp_path / "bogus.so"
+    bogus.write_bytes(b"not an elf")
+    with pytest.raises(_lib.VrlLibraryError, match="cannot load"):
+        _lib.load(str(bogus))
+
+
+def test_check_raises_with_text():
+    with pytest.raises(_lib.VrlCallError, match="vocab") as ei:
+        _lib.check("vrl_rowscore", _lib.VRL_ERR_SHAPE)
+    assert ei.value.status == _lib.VRL_ERR_SHAPE
+    _lib.check("vrl_rowscore", _lib.VRL_OK)

@@ -11,7 +11,7 @@ Setting ``VERL_USE_EXTERNAL_MODULES=verl_amd.plugin`` makes verl import
 ``install()``.
 """
 
-from .install import install, uninstall
+from .hook import install, uninstall
 from .spec_rl import (
     VerifyResult,
     draw_log_uniforms,

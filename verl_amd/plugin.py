@@ -5,6 +5,6 @@ verl imports every module named in that variable while ``import verl`` runs
 module has bound ``logprobs_from_logits`` by name.
 """
 
-from .install import install
+from .hook import install
 
 install()
