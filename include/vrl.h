@@ -47,10 +47,13 @@ extern "C" {
 
 /* bits of *err_flag */
 #define VRL_FLAG_LABEL_OOB 1   /* some label was < 0 or >= vocab; that row's logprob is NaN */
+#define VRL_FLAG_SLICE_RANGE 2 /* vrl_response_slice: a sequence had no prompt token or a bad response length */
 
 /*
  * vrl_rowscore — one HBM pass over (n_rows, vocab) logits producing, per row,
- *   logprob[r] = z[label[r]] - logsumexp(z),  entropy[r] = logsumexp(z) - sum(softmax(z) * z)
+ *   logprob[r]   = z[label[r]] - logsumexp(z)
+ *   entropy[r]   = logsumexp(z) - sum(softmax(z) * z)
+ *   sum_pi_sq[r] = sum(softmax(z)^2) = exp(logsumexp(2z) - 2 logsumexp(z))
  * with z = logits[r, :] / max(temperature[r], 1e-8) (z = logits[r, :] when
  * temperature == NULL), accumulated in fp32, written as fp32.
  *
@@ -60,15 +63,46 @@ extern "C" {
  *   verl/utils/torch_functional.py:155-170  logprobs_from_logits_naive
  *   verl/utils/torch_functional.py:231-245  entropy_from_logits
  *   verl/utils/torch_functional.py:248-270  entropy_from_logits_with_chunking
+ *   verl/utils/torch_functional.py:690-704  calculate_sum_pi_squared_from_logits
  *   verl/workers/engine/fsdp/transformer_impl.py:1357  division by per-token temperature
  *
- * out_logprob == NULL skips the label gather (labels may then be NULL);
- * out_entropy == NULL skips the entropy store. At least one must be given.
+ * Each output pointer may be NULL to skip that output (labels may be NULL when
+ * out_logprob is); at least one must be given.
  * Rows containing -inf logits give NaN entropy (0 * -inf), as torch does.
  */
 int vrl_rowscore(const void* logits, int dtype, int64_t n_rows, int64_t vocab, int64_t row_stride,
                  const int64_t* labels, const float* temperature, float* out_logprob,
-                 float* out_entropy, int32_t* err_flag, void* stream);
+                 float* out_entropy, float* out_sum_pi_sq, int32_t* err_flag, void* stream);
+
+/*
+ * vrl_rowscore_split — the same results for FEW rows: n_splits workgroups share
+ * each row and a second small kernel merges their partial results, so that a
+ * batch of tens or hundreds of rows still occupies the whole chip.
+ * `partials` is caller-owned scratch of n_rows * n_splits * 4 floats; its
+ * contents before and after the call are meaningless. n_splits in [1, 64];
+ * n_splits == 1 is vrl_rowscore. vrl_rowscore_split_plan returns the n_splits
+ * this library would pick for a shape (1 = do not split), so a caller can size
+ * the scratch before the call. Same reference counterparts as vrl_rowscore.
+ */
+int vrl_rowscore_split(const void* logits, int dtype, int64_t n_rows, int64_t vocab, int64_t row_stride,
+                       const int64_t* labels, const float* temperature, float* out_logprob,
+                       float* out_entropy, float* out_sum_pi_sq, int32_t* err_flag, int n_splits,
+                       float* partials, void* stream);
+int vrl_rowscore_split_plan(int dtype, int64_t n_rows, int64_t vocab);
+
+/*
+ * vrl_response_slice — packed per-token values (total_nnz,) -> padded (B, T_out)
+ * response block: out[b, j] = values[cu_seqlens[b+1] - response_lens[b] - 1 + j]
+ * for j < response_lens[b], else 0 (the model output at a position scores the
+ * NEXT token, hence the shift by one). Sets VRL_FLAG_SLICE_RANGE and writes a
+ * zero row when a sequence has no prompt token, or response_lens[b] is outside
+ * [0, T_out].
+ *
+ * Replaces verl/workers/utils/padding.py:97-141 (no_padding_2_padding) for fp32
+ * per-token vectors; fixture: tests/models/test_fsdp_no_padding_on_gpu.py:180-201.
+ */
+int vrl_response_slice(const float* values, const int64_t* cu_seqlens, const int64_t* response_lens,
+                       int64_t B, int64_t T_out, float* out, int32_t* err_flag, void* stream);
 
 /*
  * vrl_spec_verify — SPEC-RL draft verification over B sequences.
@@ -119,8 +153,8 @@ int vrl_truncate_draft(const int64_t* draft_ids, const uint8_t* mask, const int6
  */
 int vrl_fused_score_verify(const void* logits, int dtype, int64_t n_rows, int64_t vocab,
                            int64_t row_stride, const int64_t* labels, const float* temperature,
-                           float* out_logprob, float* out_entropy, int32_t* err_flag,
-                           const float* logp_old, const float* log_u, const uint8_t* mask,
+                           float* out_logprob, float* out_entropy, float* out_sum_pi_sq,
+                           int32_t* err_flag, const float* logp_old, const float* log_u, const uint8_t* mask,
                            const int64_t* cu_seqlens, int64_t B, int64_t T, float thresh_offset,
                            float near_eps, uint8_t* accept, int32_t* first_reject,
                            int32_t* prefix_len, int32_t* near_count, const int64_t* draft_ids,

@@ -64,7 +64,7 @@ def test_rowscore_argument_errors(lib):
 
     def call(**kw):
         a = {**ok, **kw}
-        return f(a["logits"], a["dtype"], a["n"], a["V"], a["stride"], a["labels"], a["temp"], a["lp"], a["h"], a["flag"], None)
+        return f(a["logits"], a["dtype"], a["n"], a["V"], a["stride"], a["labels"], a["temp"], a["lp"], a["h"], a.get("q"), a["flag"], None)
 
     assert call(dtype=7) == _lib.VRL_ERR_DTYPE
     assert call(n=-1) == _lib.VRL_ERR_SHAPE
@@ -81,7 +81,36 @@ def test_rowscore_argument_errors(lib):
     assert call(lp=P + 2) == _lib.VRL_ERR_ALIGN
     assert call(temp=P + 1) == _lib.VRL_ERR_ALIGN
     # nothing to do is not an error, and needs no pointers
-    assert f(None, _lib.VRL_F32, 0, 100, 100, None, None, None, P, None, None) == _lib.VRL_OK
+    assert call(q=P + 2) == _lib.VRL_ERR_ALIGN
+    assert f(None, _lib.VRL_F32, 0, 100, 100, None, None, None, P, None, None, None) == _lib.VRL_OK
+
+
+def test_split_and_slice_argument_errors(lib):
+    f = lib.vrl_rowscore_split
+
+    def call(n=4, splits=4, partials=P, lp=P, dtype=_lib.VRL_BF16):
+        return f(P, dtype, n, 100000, 100000, P, None, lp, P, None, P, splits, partials, None)
+
+    assert call(splits=0) == _lib.VRL_ERR_ARG
+    assert call(splits=65) == _lib.VRL_ERR_ARG
+    assert call(partials=None) == _lib.VRL_ERR_NULL
+    assert call(partials=P + 2) == _lib.VRL_ERR_ALIGN
+    assert call(dtype=9) == _lib.VRL_ERR_DTYPE
+    assert call(n=0, partials=None) == _lib.VRL_OK
+    plan = lib.vrl_rowscore_split_plan
+    assert plan(_lib.VRL_BF16, 8192, 151936) == 1          # enough rows: one workgroup per row
+    assert plan(_lib.VRL_BF16, 2048, 151936) == 1
+    assert 2 <= plan(_lib.VRL_BF16, 256, 151936) <= 64
+    assert plan(_lib.VRL_BF16, 1, 151936) >= 16
+    assert plan(_lib.VRL_F32, 16, 1000) == 1                # rows too short to cut
+    assert plan(7, 16, 151936) == 1 and plan(_lib.VRL_F32, 0, 10) == 1
+
+    g = lib.vrl_response_slice
+    assert g(P, P, P, -1, 4, P, P, None) == _lib.VRL_ERR_SHAPE
+    assert g(None, P, P, 2, 4, P, P, None) == _lib.VRL_ERR_NULL
+    assert g(P, P, P, 2, 4, P, None, None) == _lib.VRL_ERR_NULL
+    assert g(P, P + 4, P, 2, 4, P, P, None) == _lib.VRL_ERR_ALIGN
+    assert g(None, None, None, 0, 4, None, None, None) == _lib.VRL_OK
 
 
 def test_verify_argument_errors(lib):
@@ -114,7 +143,7 @@ def test_truncate_and_fused_argument_errors(lib):
     f = lib.vrl_fused_score_verify
 
     def call(n=16, B=2, T=8, lp=P, dtype=_lib.VRL_BF16, cu=None, lo=P):
-        return f(P, dtype, n, 100, 100, P, None, lp, P, P, lo, P, None, cu, B, T, 0.0, 1e-6, P, P, P, P, None, 0, None, None, None)
+        return f(P, dtype, n, 100, 100, P, None, lp, P, None, P, lo, P, None, cu, B, T, 0.0, 1e-6, P, P, P, P, None, 0, None, None, None)
 
     assert call(lp=None) == _lib.VRL_ERR_NULL                  # verify needs the log-probs
     assert call(dtype=3) == _lib.VRL_ERR_DTYPE

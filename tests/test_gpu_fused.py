@@ -71,7 +71,7 @@ def test_fused_packed_layout(dev):
     ref_lp, _ = scoring.score_fp32(logits.cpu(), labels.cpu())
     logp_old = ref_lp.to(dev) + torch.randn(N, generator=g, device=dev) * 0.3
     lp, h, res = sv.fused_score_verify(logits, labels, logp_old, None, log_u=log_u, cu_seqlens=cu.to(dev))
-    lp2, h2 = vf.fused_logprob_entropy(logits, labels)
+    lp2, h2 = vf.fused_logprob_entropy(logits, labels, n_splits=1)
     assert torch.equal(lp, lp2) and torch.equal(h, h2)
     own = c_oracle.spec_verify(lp, logp_old, log_u, None, 0.0, cu_seqlens=cu)
     assert np.array_equal(res.accept.cpu().numpy().astype(np.uint8), own["accept"])
@@ -82,7 +82,8 @@ def test_fused_packed_layout(dev):
 def test_fused_equals_two_calls(dev):
     w = synthetic.WORKLOADS["c2"].scaled(B=3, T=40, V=20011)
     d = synthetic.make_padded(w, dev, seed=5)
-    lp, h = vf.fused_logprob_entropy(d["logits"], d["labels"])
+    # the fused entry point scores with one workgroup per row; ask the two-call path for the same
+    lp, h = vf.fused_logprob_entropy(d["logits"], d["labels"], n_splits=1)
     old = synthetic.drift_old_logprobs(lp, w, 5)
     lp2, h2, res = sv.fused_score_verify(d["logits"], d["labels"], old, d["mask"], log_u=d["log_u"])
     two = sv.spec_verify(lp, old, d["mask"], log_u=d["log_u"])

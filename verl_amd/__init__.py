@@ -12,6 +12,7 @@ Setting ``VERL_USE_EXTERNAL_MODULES=verl_amd.plugin`` makes verl import
 """
 
 from .hook import install, uninstall
+from .layout import response_slice, roll_labels
 from .spec_rl import (
     VerifyResult,
     draw_log_uniforms,
@@ -21,6 +22,7 @@ from .spec_rl import (
     truncate_draft,
 )
 from .torch_functional import (
+    calculate_sum_pi_squared_from_logits,
     entropy_from_logits,
     entropy_from_logits_with_chunking,
     fused_logprob_entropy,
@@ -40,6 +42,9 @@ __all__ = [
     "spec_verify",
     "thresh_offset_from_lenience",
     "truncate_draft",
+    "response_slice",
+    "roll_labels",
+    "calculate_sum_pi_squared_from_logits",
     "entropy_from_logits",
     "entropy_from_logits_with_chunking",
     "fused_logprob_entropy",

@@ -25,6 +25,7 @@ VRL_F32 = 0
 VRL_BF16 = 1
 
 VRL_FLAG_LABEL_OOB = 1
+VRL_FLAG_SLICE_RANGE = 2
 
 ABI_VERSION = 1
 
@@ -36,7 +37,10 @@ _F32 = _c.c_float
 
 # name -> (restype, argtypes); mirrors include/vrl.h one to one.
 SIGNATURES = {
-    "vrl_rowscore": (_INT, [_P, _INT, _I64, _I64, _I64, _P, _P, _P, _P, _P, _P]),
+    "vrl_rowscore": (_INT, [_P, _INT, _I64, _I64, _I64, _P, _P, _P, _P, _P, _P, _P]),
+    "vrl_rowscore_split": (_INT, [_P, _INT, _I64, _I64, _I64, _P, _P, _P, _P, _P, _P, _INT, _P, _P]),
+    "vrl_rowscore_split_plan": (_INT, [_INT, _I64, _I64]),
+    "vrl_response_slice": (_INT, [_P, _P, _P, _I64, _I64, _P, _P, _P]),
     "vrl_spec_verify": (
         _INT,
         [_P, _P, _P, _P, _P, _I64, _I64, _F32, _F32, _P, _P, _P, _P, _P, _I64, _P, _P, _P],
@@ -44,7 +48,7 @@ SIGNATURES = {
     "vrl_truncate_draft": (_INT, [_P, _P, _P, _I64, _I64, _P, _I64, _P, _P, _P]),
     "vrl_fused_score_verify": (
         _INT,
-        [_P, _INT, _I64, _I64, _I64, _P, _P, _P, _P, _P]
+        [_P, _INT, _I64, _I64, _I64, _P, _P, _P, _P, _P, _P]
         + [_P, _P, _P, _P, _I64, _I64, _F32, _F32, _P, _P, _P, _P, _P, _I64, _P, _P, _P],
     ),
     "vrl_strerror": (_c.c_char_p, [_INT]),

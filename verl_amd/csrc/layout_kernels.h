@@ -1,0 +1,28 @@
+// Packed per-token values -> padded (B, T_out) response block, shifted left by
+// one token: the model output at position p scores token p+1, so the response
+// tokens of a sequence that ends at row `end` with `r` response tokens are
+// scored by rows [end - r - 1, end - 1).
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace vrl {
+
+// grid.x = B, block = 256. Sequence b owns packed rows [cu[b], cu[b+1]).
+__global__ __launch_bounds__(256) void response_slice_kernel(
+    const float* __restrict__ values, const int64_t* __restrict__ cu_seqlens,
+    const int64_t* __restrict__ response_lens, int64_t T_out, float* __restrict__ out, int32_t* err_flag) {
+  const int64_t b = blockIdx.x;
+  const int64_t begin = cu_seqlens[b];
+  const int64_t end = cu_seqlens[b + 1];
+  const int64_t r = response_lens[b];
+  const int64_t first = end - r - 1;
+  // the reference asserts prompt_len > 0 (first >= begin) and pads up to T_out (r <= T_out)
+  const bool ok = (r >= 0) && (r <= T_out) && (first >= begin);
+  if (!ok && threadIdx.x == 0) atomicOr(err_flag, 2);
+  float* dst = out + b * T_out;
+  for (int64_t j = threadIdx.x; j < T_out; j += 256) dst[j] = (ok && j < r) ? values[first + j] : 0.f;
+}
+
+}  // namespace vrl

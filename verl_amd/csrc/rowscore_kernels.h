@@ -10,8 +10,12 @@
 //   alpha = 2^(m - M);  s' = alpha*s;  t' = alpha*(t + (m - M)*s).
 // At the end  logsumexp = ln2*(M + log2 S),  logprob = ln2*((y_label - M) - log2 S),
 // entropy = ln2*(log2 S - T/S)  (the shift cancels, nothing large is subtracted).
+// The optional sum of squared probabilities carries q = sum 2^(2(y-m)), merged with
+// alpha^2, and ends as Q/S^2.
 //
-// Mapping. One workgroup of WAVES wavefronts owns one row. A register batch is
+// Mapping. One workgroup of WAVES wavefronts owns one row (or, when there are
+// too few rows to fill the chip, one slice of a row; a second small kernel then
+// merges the slices). A register batch is
 // U 128-bit loads per lane; wave w of the group reads the w-th contiguous
 // U KiB slice of each WAVES*U KiB block of the row, so every load instruction
 // is one fully coalesced 1 KiB request and a lane's U loads differ only in the
@@ -39,6 +43,7 @@ struct Part {
   float m;  // shift, log2 domain; -inf while nothing finite has been seen
   float s;  // sum 2^(y-m)
   float t;  // sum 2^(y-m)*(y-m)
+  float q;  // sum 2^(2(y-m)), only maintained when the sum of squared probabilities is asked for
 };
 
 // Bring p to the shift M >= p.m. A partial that has seen nothing finite
@@ -49,6 +54,7 @@ __device__ __forceinline__ void rescale(Part& p, float M) {
   const float alpha = dead ? 0.f : hw_exp2(dm);
   p.t = alpha * (p.t + dm * p.s);
   p.s = alpha * p.s;
+  p.q = (alpha * alpha) * p.q;
   p.m = M;
 }
 
@@ -115,7 +121,7 @@ struct Scale {
 };
 
 // ---- one register batch --------------------------------------------------
-template <int N, bool EXACT>
+template <int N, bool EXACT, bool WANT_Q>
 __device__ __forceinline__ void accumulate(Part& a, float* x, const Scale<EXACT>& sc) {
   if constexpr (EXACT) {
 #pragma unroll
@@ -130,16 +136,18 @@ __device__ __forceinline__ void accumulate(Part& a, float* x, const Scale<EXACT>
   }
   // While only -inf has been seen the shift must stay finite: -inf - (-inf) is NaN.
   const float sub = (a.m == neg_inf()) ? 0.f : a.m;
-  float ps = 0.f, pt = 0.f;
+  float ps = 0.f, pt = 0.f, pq = 0.f;
 #pragma unroll
   for (int i = 0; i < N; ++i) {
     const float d = __builtin_fmaf(x[i], sc.c, -sub);
     const float e = hw_exp2(d);
     ps += e;
     pt = __builtin_fmaf(e, d, pt);
+    if constexpr (WANT_Q) pq = __builtin_fmaf(e, e, pq);
   }
   a.s += ps;
   a.t += pt;
+  if constexpr (WANT_Q) a.q += pq;
 }
 
 // ---- wavefront reductions (DPP within rows of 16 lanes, readlane across) ---
@@ -175,56 +183,34 @@ __device__ __forceinline__ u32x4 load_vec(const u32x4* p) {
   }
 }
 
-// ---- the kernel ------------------------------------------------------------
-// grid.x = n_rows, block = WAVES*64 threads. All threads of a block reach the
-// reductions and the barrier (no early exit), so EXEC is full for the DPP ops.
-template <int DT, int WAVES, int U, bool EXACT, bool NT>
-__global__ __launch_bounds__(WAVES * 64) void rowscore_kernel(
-    const void* __restrict__ logits, int64_t vocab, int64_t row_stride,
-    const int64_t* __restrict__ labels, const float* __restrict__ temperature,
-    float* __restrict__ out_logprob, float* __restrict__ out_entropy, int32_t* err_flag) {
+// ---- a workgroup reduces elements [e_lo, e_hi) of one row -------------------
+// Every thread of the workgroup must call this (it contains a barrier and DPP
+// operations that need a full EXEC mask). The result is valid in thread 0.
+template <int DT, int WAVES, int U, bool EXACT, bool NT, bool WANT_Q>
+__device__ __forceinline__ Part block_reduce_range(const char* rowp, int64_t e_lo, int64_t e_hi,
+                                                   const Scale<EXACT>& sc) {
   using E = Elem<DT>;
   constexpr int NTHR = WAVES * 64;
   constexpr int PV = E::kPerVec;
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = tid >> 6;
-  const int64_t row = blockIdx.x;
-  const char* rowp = static_cast<const char*>(logits) + row * row_stride * E::kBytes;
 
-  Scale<EXACT> sc;
-  sc.T = 1.f;
-  sc.r = 1.f;
-  sc.c = kLog2e;
-  if (temperature != nullptr) {
-    float T = temperature[row];
-    T = (T < kMinTemperature) ? kMinTemperature : T;  // NaN stays NaN, as torch.clamp keeps it
-    sc.T = T;
-    sc.r = 1.0f / T;
-    sc.c = EXACT ? kLog2e : kLog2e / T;
-  }
-
-  // Label logit: one extra element load by thread 0, issued before the stream.
-  float xl = 0.f;
-  bool label_ok = true;
-  if (out_logprob != nullptr && tid == 0) {
-    const int64_t lab = labels[row];
-    label_ok = (lab >= 0) && (lab < vocab);
-    xl = label_ok ? E::load1(rowp, lab) : quiet_nan();
-  }
-
-  // Split the row into [head scalars][16-byte vectors][tail scalars].
-  const uintptr_t addr = reinterpret_cast<uintptr_t>(rowp);
+  // Split the range into [head scalars][16-byte vectors][tail scalars].
+  const int64_t count = e_hi - e_lo;
+  const char* basep = rowp + e_lo * E::kBytes;
+  const uintptr_t addr = reinterpret_cast<uintptr_t>(basep);
   int64_t head = static_cast<int64_t>(((16u - (addr & 15u)) & 15u) / E::kBytes);
-  if (head > vocab) head = vocab;
-  const int64_t nvec = (vocab - head) / PV;
+  if (head > count) head = count;
+  const int64_t nvec = (count - head) / PV;
   const int64_t tail0 = head + nvec * PV;
-  const u32x4* vp = reinterpret_cast<const u32x4*>(rowp + head * E::kBytes);
+  const u32x4* vp = reinterpret_cast<const u32x4*>(basep + head * E::kBytes);
 
   Part a;
   a.m = neg_inf();
   a.s = 0.f;
   a.t = 0.f;
+  a.q = 0.f;
 
   constexpr int64_t kBatchVecs = static_cast<int64_t>(NTHR) * U;
   const int64_t nfull = nvec / kBatchVecs;
@@ -236,21 +222,21 @@ __global__ __launch_bounds__(WAVES * 64) void rowscore_kernel(
     float x[U * PV];
 #pragma unroll
     for (int u = 0; u < U; ++u) E::unpack(v[u], x + u * PV);
-    accumulate<U * PV, EXACT>(a, x, sc);
+    accumulate<U * PV, EXACT, WANT_Q>(a, x, sc);
   }
   for (int64_t k = nfull * kBatchVecs + tid; k < nvec; k += NTHR) {
     const u32x4 v = load_vec<NT>(vp + k);
     float x[PV];
     E::unpack(v, x);
-    accumulate<PV, EXACT>(a, x, sc);
+    accumulate<PV, EXACT, WANT_Q>(a, x, sc);
   }
   {
-    const int64_t nscalar = head + (vocab - tail0);  // < 2*PV <= 16
+    const int64_t nscalar = head + (count - tail0);  // < 2*PV <= 16
     if (tid < nscalar) {
       const int64_t idx = (tid < head) ? tid : tail0 + (tid - head);
       float x[1];
-      x[0] = E::load1(rowp, idx);
-      accumulate<1, EXACT>(a, x, sc);
+      x[0] = E::load1(basep, idx);
+      accumulate<1, EXACT, WANT_Q>(a, x, sc);
     }
   }
 
@@ -261,62 +247,187 @@ __global__ __launch_bounds__(WAVES * 64) void rowscore_kernel(
   w.m = wm;
   w.s = wave_sum(a.s);
   w.t = wave_sum(a.t);
+  w.q = WANT_Q ? wave_sum(a.q) : 0.f;
 
   if constexpr (WAVES > 1) {
-    __shared__ float sm[WAVES][3];
+    __shared__ float sm[WAVES][4];
     if (lane == 0) {
       sm[wave][0] = w.m;
       sm[wave][1] = w.s;
       sm[wave][2] = w.t;
+      sm[wave][3] = w.q;
     }
     __syncthreads();
     if (tid == 0) {
       float M = sm[0][0];
 #pragma unroll
       for (int i = 1; i < WAVES; ++i) M = __builtin_fmaxf(M, sm[i][0]);
-      float S = 0.f, Tt = 0.f;
+      float S = 0.f, Tt = 0.f, Q = 0.f;
 #pragma unroll
       for (int i = 0; i < WAVES; ++i) {
         Part p;
         p.m = sm[i][0];
         p.s = sm[i][1];
         p.t = sm[i][2];
+        p.q = sm[i][3];
         rescale(p, M);
         S += p.s;
         Tt += p.t;
+        Q += p.q;
       }
       w.m = M;
       w.s = S;
       w.t = Tt;
+      w.q = Q;
     }
   }
+  return w;
+}
 
-  if (tid == 0) {
-    float lp, H;
-    if (w.m == neg_inf()) {
-      // empty row or every logit -inf: logsumexp = -inf, x - (-inf) and softmax are NaN in torch
-      lp = quiet_nan();
-      H = quiet_nan();
-    } else if (w.m == pos_inf()) {
-      // a +inf logit: logsumexp = +inf
-      lp = (sc.pre(xl) * sc.c == pos_inf()) ? quiet_nan() : neg_inf();
-      H = quiet_nan();
-    } else {
-      const double S = static_cast<double>(w.s);
-      const double l2s = log2(S);
-      const double yl = static_cast<double>(sc.pre(xl)) * static_cast<double>(sc.c) - static_cast<double>(w.m);
-      lp = static_cast<float>(kLn2d * (yl - l2s));
-      H = static_cast<float>(kLn2d * (l2s - static_cast<double>(w.t) / S));
-    }
-    if (out_logprob != nullptr) {
-      if (!label_ok) {
-        lp = quiet_nan();
-        atomicOr(err_flag, 1);
-      }
-      out_logprob[row] = lp;
-    }
-    if (out_entropy != nullptr) out_entropy[row] = H;
+template <bool EXACT>
+__device__ __forceinline__ Scale<EXACT> make_scale(const float* temperature, int64_t row) {
+  Scale<EXACT> sc;
+  sc.T = 1.f;
+  sc.r = 1.f;
+  sc.c = kLog2e;
+  if (temperature != nullptr) {
+    float T = temperature[row];
+    T = (T < kMinTemperature) ? kMinTemperature : T;  // NaN stays NaN, as torch.clamp keeps it
+    sc.T = T;
+    sc.r = 1.0f / T;
+    sc.c = EXACT ? kLog2e : kLog2e / T;
   }
+  return sc;
+}
+
+// Label logit: one extra element load, issued before the row is streamed.
+template <int DT>
+__device__ __forceinline__ float load_label_logit(const char* rowp, const int64_t* labels, int64_t row,
+                                                  int64_t vocab, bool& label_ok) {
+  const int64_t lab = labels[row];
+  label_ok = (lab >= 0) && (lab < vocab);
+  return label_ok ? Elem<DT>::load1(rowp, lab) : quiet_nan();
+}
+
+// One thread turns the row's (M, S, T, Q) into the outputs. The last step is
+// done in double: it runs once per row and keeps the result's error at the
+// level of the fp32 accumulation.
+template <bool EXACT, bool WANT_Q>
+__device__ __forceinline__ void finalize_row(const Part& w, float xl, bool label_ok, const Scale<EXACT>& sc,
+                                             int64_t row, float* out_logprob, float* out_entropy,
+                                             float* out_sum_pi_sq, int32_t* err_flag) {
+  float lp, H, sps;
+  if (w.m == neg_inf()) {
+    // empty row or every logit -inf: logsumexp = -inf, x - (-inf) and softmax are NaN in torch
+    lp = quiet_nan();
+    H = quiet_nan();
+    sps = quiet_nan();
+  } else if (w.m == pos_inf()) {
+    // a +inf logit: logsumexp = +inf
+    lp = (sc.pre(xl) * sc.c == pos_inf()) ? quiet_nan() : neg_inf();
+    H = quiet_nan();
+    sps = quiet_nan();
+  } else {
+    const double S = static_cast<double>(w.s);
+    const double l2s = log2(S);
+    const double yl = static_cast<double>(sc.pre(xl)) * static_cast<double>(sc.c) - static_cast<double>(w.m);
+    lp = static_cast<float>(kLn2d * (yl - l2s));
+    H = static_cast<float>(kLn2d * (l2s - static_cast<double>(w.t) / S));
+    sps = static_cast<float>(static_cast<double>(w.q) / (S * S));
+  }
+  if (out_logprob != nullptr) {
+    if (!label_ok) {
+      lp = quiet_nan();
+      atomicOr(err_flag, 1);
+    }
+    out_logprob[row] = lp;
+  }
+  if (out_entropy != nullptr) out_entropy[row] = H;
+  if constexpr (WANT_Q) {
+    if (out_sum_pi_sq != nullptr) out_sum_pi_sq[row] = sps;
+  }
+}
+
+// ---- one workgroup per row ---------------------------------------------------
+// grid.x = n_rows, block = WAVES*64 threads; no thread exits early.
+template <int DT, int WAVES, int U, bool EXACT, bool NT, bool WANT_Q>
+__global__ __launch_bounds__(WAVES * 64) void rowscore_kernel(
+    const void* __restrict__ logits, int64_t vocab, int64_t row_stride,
+    const int64_t* __restrict__ labels, const float* __restrict__ temperature,
+    float* __restrict__ out_logprob, float* __restrict__ out_entropy,
+    float* __restrict__ out_sum_pi_sq, int32_t* err_flag) {
+  const int64_t row = blockIdx.x;
+  const char* rowp = static_cast<const char*>(logits) + row * row_stride * Elem<DT>::kBytes;
+  const Scale<EXACT> sc = make_scale<EXACT>(temperature, row);
+  float xl = 0.f;
+  bool label_ok = true;
+  if (out_logprob != nullptr && threadIdx.x == 0) xl = load_label_logit<DT>(rowp, labels, row, vocab, label_ok);
+  const Part w = block_reduce_range<DT, WAVES, U, EXACT, NT, WANT_Q>(rowp, 0, vocab, sc);
+  if (threadIdx.x == 0)
+    finalize_row<EXACT, WANT_Q>(w, xl, label_ok, sc, row, out_logprob, out_entropy, out_sum_pi_sq, err_flag);
+}
+
+// ---- few rows: several workgroups per row ------------------------------------
+// grid.x = n_rows * n_splits. Workgroup (row, k) reduces elements
+// [k*slice, min((k+1)*slice, vocab)) and stores its partial (M, S, T, Q) at
+// partials[(row*n_splits + k)*4 ...]; rowscore_merge_kernel finishes the rows.
+template <int DT, int WAVES, int U, bool EXACT, bool NT, bool WANT_Q>
+__global__ __launch_bounds__(WAVES * 64) void rowscore_split_kernel(
+    const void* __restrict__ logits, int64_t vocab, int64_t row_stride,
+    const float* __restrict__ temperature, int n_splits, int64_t slice, float* __restrict__ partials) {
+  const int64_t row = blockIdx.x / n_splits;
+  const int k = static_cast<int>(blockIdx.x % n_splits);
+  const char* rowp = static_cast<const char*>(logits) + row * row_stride * Elem<DT>::kBytes;
+  const Scale<EXACT> sc = make_scale<EXACT>(temperature, row);
+  int64_t lo = k * slice;
+  int64_t hi = lo + slice;
+  if (lo > vocab) lo = vocab;
+  if (hi > vocab) hi = vocab;
+  const Part w = block_reduce_range<DT, WAVES, U, EXACT, NT, WANT_Q>(rowp, lo, hi, sc);
+  if (threadIdx.x == 0) {
+    float* dst = partials + (row * n_splits + k) * 4;
+    dst[0] = w.m;
+    dst[1] = w.s;
+    dst[2] = w.t;
+    dst[3] = w.q;
+  }
+}
+
+// grid.x = ceil(n_rows / 64), block = 64: one lane per row merges that row's
+// n_splits partials in index order (deterministic) and writes the outputs.
+template <int DT, bool EXACT, bool WANT_Q>
+__global__ __launch_bounds__(64) void rowscore_merge_kernel(
+    const void* __restrict__ logits, int64_t n_rows, int64_t vocab, int64_t row_stride,
+    const int64_t* __restrict__ labels, const float* __restrict__ temperature, int n_splits,
+    const float* __restrict__ partials, float* __restrict__ out_logprob, float* __restrict__ out_entropy,
+    float* __restrict__ out_sum_pi_sq, int32_t* err_flag) {
+  const int64_t row = static_cast<int64_t>(blockIdx.x) * 64 + threadIdx.x;
+  if (row >= n_rows) return;
+  const char* rowp = static_cast<const char*>(logits) + row * row_stride * Elem<DT>::kBytes;
+  const Scale<EXACT> sc = make_scale<EXACT>(temperature, row);
+  float xl = 0.f;
+  bool label_ok = true;
+  if (out_logprob != nullptr) xl = load_label_logit<DT>(rowp, labels, row, vocab, label_ok);
+  const float* src = partials + row * n_splits * 4;
+  float M = src[0];
+  for (int k = 1; k < n_splits; ++k) M = __builtin_fmaxf(M, src[k * 4]);
+  Part w;
+  w.m = M;
+  w.s = 0.f;
+  w.t = 0.f;
+  w.q = 0.f;
+  for (int k = 0; k < n_splits; ++k) {
+    Part p;
+    p.m = src[k * 4 + 0];
+    p.s = src[k * 4 + 1];
+    p.t = src[k * 4 + 2];
+    p.q = src[k * 4 + 3];
+    rescale(p, M);
+    w.s += p.s;
+    w.t += p.t;
+    w.q += p.q;
+  }
+  finalize_row<EXACT, WANT_Q>(w, xl, label_ok, sc, row, out_logprob, out_entropy, out_sum_pi_sq, err_flag);
 }
 
 }  // namespace vrl

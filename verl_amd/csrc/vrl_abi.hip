@@ -7,6 +7,7 @@
 #include <stdint.h>
 #include <string.h>
 
+#include "layout_kernels.h"
 #include "rowscore_kernels.h"
 #include "verify_kernels.h"
 
@@ -27,35 +28,99 @@ bool aligned(const void* p, uintptr_t a) { return (reinterpret_cast<uintptr_t>(p
 
 constexpr int64_t kMaxGrid = 0x7fffffffLL;
 
-// Workgroup shape of the row kernel: wavefronts per row and 128-bit loads per
-// lane and batch.
-constexpr int kRowWaves = 4;
-constexpr int kRowUnroll = 4;
+// Workgroup shape of the row kernel (wavefronts per row, 128-bit loads per lane
+// and batch), chosen by measurement on MI355X at 8192 x 151936.
+template <int DT>
+struct RowShape;
+template <>
+struct RowShape<VRL_F32> {
+  static constexpr int kWaves = 4, kUnroll = 4;
+};
+template <>
+struct RowShape<VRL_BF16> {
+  static constexpr int kWaves = 8, kUnroll = 8;
+};
+// Shape of a workgroup that reduces one slice of a row (split path).
+constexpr int kSplitWaves = 4;
+constexpr int kSplitUnroll = 2;
+constexpr int kMaxSplits = 64;
 
 int check_rowscore(const void* logits, int dtype, int64_t n_rows, int64_t vocab, int64_t row_stride,
                    const int64_t* labels, const float* temperature, const float* out_logprob,
-                   const float* out_entropy, const int32_t* err_flag) {
+                   const float* out_entropy, const float* out_sum_pi_sq, const int32_t* err_flag) {
   if (dtype != VRL_F32 && dtype != VRL_BF16) return VRL_ERR_DTYPE;
   if (n_rows < 0 || vocab <= 0 || row_stride < vocab || n_rows > kMaxGrid) return VRL_ERR_SHAPE;
-  if (out_logprob == nullptr && out_entropy == nullptr) return VRL_ERR_ARG;
+  if (out_logprob == nullptr && out_entropy == nullptr && out_sum_pi_sq == nullptr) return VRL_ERR_ARG;
   if (n_rows == 0) return VRL_OK;
   if (logits == nullptr) return VRL_ERR_NULL;
   if (out_logprob != nullptr && (labels == nullptr || err_flag == nullptr)) return VRL_ERR_NULL;
   const uintptr_t esize = (dtype == VRL_F32) ? 4 : 2;
   if (!aligned(logits, esize) || !aligned(labels, 8) || !aligned(temperature, 4) ||
-      !aligned(out_logprob, 4) || !aligned(out_entropy, 4) || !aligned(err_flag, 4))
+      !aligned(out_logprob, 4) || !aligned(out_entropy, 4) || !aligned(out_sum_pi_sq, 4) ||
+      !aligned(err_flag, 4))
     return VRL_ERR_ALIGN;
   return VRL_OK;
 }
 
+struct RowArgs {
+  const void* logits;
+  int64_t n_rows, vocab, row_stride;
+  const int64_t* labels;
+  const float* temperature;
+  float* out_logprob;
+  float* out_entropy;
+  float* out_sum_pi_sq;
+  int32_t* err_flag;
+  int n_splits;     // 1: one workgroup per row
+  float* partials;  // split path only
+  hipStream_t stream;
+};
+
+int64_t split_slice_elems(int64_t vocab, int n_splits, int dtype) {
+  const int64_t per_vec = (dtype == VRL_F32) ? 4 : 8;
+  const int64_t batch = static_cast<int64_t>(kSplitWaves) * 64 * kSplitUnroll * per_vec;
+  const int64_t per_split = (vocab + n_splits - 1) / n_splits;
+  return ((per_split + batch - 1) / batch) * batch;
+}
+
+template <int DT, bool EXACT, bool WANT_Q>
+void launch_rows(const RowArgs& a) {
+  if (a.n_splits <= 1) {
+    constexpr int W = RowShape<DT>::kWaves, U = RowShape<DT>::kUnroll;
+    vrl::rowscore_kernel<DT, W, U, EXACT, true, WANT_Q>
+        <<<dim3(static_cast<unsigned>(a.n_rows)), dim3(W * 64), 0, a.stream>>>(
+            a.logits, a.vocab, a.row_stride, a.labels, a.temperature, a.out_logprob, a.out_entropy,
+            a.out_sum_pi_sq, a.err_flag);
+    return;
+  }
+  const int64_t slice = split_slice_elems(a.vocab, a.n_splits, DT);
+  vrl::rowscore_split_kernel<DT, kSplitWaves, kSplitUnroll, EXACT, true, WANT_Q>
+      <<<dim3(static_cast<unsigned>(a.n_rows * a.n_splits)), dim3(kSplitWaves * 64), 0, a.stream>>>(
+          a.logits, a.vocab, a.row_stride, a.temperature, a.n_splits, slice, a.partials);
+  vrl::rowscore_merge_kernel<DT, EXACT, WANT_Q>
+      <<<dim3(static_cast<unsigned>((a.n_rows + 63) / 64)), dim3(64), 0, a.stream>>>(
+          a.logits, a.n_rows, a.vocab, a.row_stride, a.labels, a.temperature, a.n_splits, a.partials,
+          a.out_logprob, a.out_entropy, a.out_sum_pi_sq, a.err_flag);
+}
+
 template <int DT, bool EXACT>
-void launch_rowscore(const void* logits, int64_t n_rows, int64_t vocab, int64_t row_stride,
-                     const int64_t* labels, const float* temperature, float* out_logprob,
-                     float* out_entropy, int32_t* err_flag, hipStream_t stream) {
-  const dim3 grid(static_cast<unsigned>(n_rows));
-  const dim3 block(kRowWaves * 64);
-  vrl::rowscore_kernel<DT, kRowWaves, kRowUnroll, EXACT, true><<<grid, block, 0, stream>>>(
-      logits, vocab, row_stride, labels, temperature, out_logprob, out_entropy, err_flag);
+void launch_rows_q(const RowArgs& a) {
+  if (a.out_sum_pi_sq != nullptr)
+    launch_rows<DT, EXACT, true>(a);
+  else
+    launch_rows<DT, EXACT, false>(a);
+}
+
+void launch_rows_any(int dtype, const RowArgs& a) {
+  if (dtype == VRL_F32) {
+    // fp32 logits with a temperature: per-element quotient rounded like `logits / temperature`
+    if (a.temperature != nullptr)
+      launch_rows_q<VRL_F32, true>(a);
+    else
+      launch_rows_q<VRL_F32, false>(a);
+  } else {
+    launch_rows_q<VRL_BF16, false>(a);
+  }
 }
 
 int check_verify(const float* logp_new, const float* logp_old, const float* log_u, const uint8_t* mask,
@@ -88,22 +153,61 @@ extern "C" {
 
 int vrl_rowscore(const void* logits, int dtype, int64_t n_rows, int64_t vocab, int64_t row_stride,
                  const int64_t* labels, const float* temperature, float* out_logprob,
-                 float* out_entropy, int32_t* err_flag, void* stream) {
+                 float* out_entropy, float* out_sum_pi_sq, int32_t* err_flag, void* stream) {
   const int st = check_rowscore(logits, dtype, n_rows, vocab, row_stride, labels, temperature,
-                                out_logprob, out_entropy, err_flag);
+                                out_logprob, out_entropy, out_sum_pi_sq, err_flag);
   if (st != VRL_OK || n_rows == 0) return st;
-  hipStream_t s = static_cast<hipStream_t>(stream);
-  if (dtype == VRL_F32) {
-    if (temperature != nullptr)
-      launch_rowscore<VRL_F32, true>(logits, n_rows, vocab, row_stride, labels, temperature,
-                                     out_logprob, out_entropy, err_flag, s);
-    else
-      launch_rowscore<VRL_F32, false>(logits, n_rows, vocab, row_stride, labels, temperature,
-                                      out_logprob, out_entropy, err_flag, s);
-  } else {
-    launch_rowscore<VRL_BF16, false>(logits, n_rows, vocab, row_stride, labels, temperature,
-                                     out_logprob, out_entropy, err_flag, s);
-  }
+  const RowArgs a{logits, n_rows, vocab, row_stride, labels, temperature, out_logprob, out_entropy,
+                  out_sum_pi_sq, err_flag, 1, nullptr, static_cast<hipStream_t>(stream)};
+  launch_rows_any(dtype, a);
+  return launch_status();
+}
+
+int vrl_rowscore_split_plan(int dtype, int64_t n_rows, int64_t vocab) {
+  if ((dtype != VRL_F32 && dtype != VRL_BF16) || n_rows <= 0 || vocab <= 0) return 1;
+  // One workgroup per row fills the chip from about a thousand rows on.
+  constexpr int64_t kTargetGroups = 2048;
+  if (n_rows >= kTargetGroups / 2) return 1;
+  int64_t want = (kTargetGroups + n_rows - 1) / n_rows;
+  // every slice keeps at least two register batches of the split workgroup
+  const int64_t per_vec = (dtype == VRL_F32) ? 4 : 8;
+  const int64_t batch = static_cast<int64_t>(kSplitWaves) * 64 * kSplitUnroll * per_vec;
+  const int64_t by_size = vocab / (2 * batch);
+  if (want > by_size) want = by_size;
+  if (want > kMaxSplits) want = kMaxSplits;
+  return want < 2 ? 1 : static_cast<int>(want);
+}
+
+int vrl_rowscore_split(const void* logits, int dtype, int64_t n_rows, int64_t vocab, int64_t row_stride,
+                       const int64_t* labels, const float* temperature, float* out_logprob,
+                       float* out_entropy, float* out_sum_pi_sq, int32_t* err_flag, int n_splits,
+                       float* partials, void* stream) {
+  const int st = check_rowscore(logits, dtype, n_rows, vocab, row_stride, labels, temperature,
+                                out_logprob, out_entropy, out_sum_pi_sq, err_flag);
+  if (st != VRL_OK) return st;
+  if (n_splits < 1 || n_splits > kMaxSplits) return VRL_ERR_ARG;
+  if (n_rows * n_splits > kMaxGrid) return VRL_ERR_SHAPE;
+  if (n_rows == 0) return VRL_OK;
+  if (n_splits > 1 && partials == nullptr) return VRL_ERR_NULL;
+  if (!aligned(partials, 4)) return VRL_ERR_ALIGN;
+  const RowArgs a{logits, n_rows, vocab, row_stride, labels, temperature, out_logprob, out_entropy,
+                  out_sum_pi_sq, err_flag, n_splits, partials, static_cast<hipStream_t>(stream)};
+  launch_rows_any(dtype, a);
+  return launch_status();
+}
+
+int vrl_response_slice(const float* values, const int64_t* cu_seqlens, const int64_t* response_lens,
+                       int64_t B, int64_t T_out, float* out, int32_t* err_flag, void* stream) {
+  if (B < 0 || T_out < 0 || B > kMaxGrid) return VRL_ERR_SHAPE;
+  if (B == 0 || T_out == 0) return VRL_OK;
+  if (values == nullptr || cu_seqlens == nullptr || response_lens == nullptr || out == nullptr ||
+      err_flag == nullptr)
+    return VRL_ERR_NULL;
+  if (!aligned(values, 4) || !aligned(cu_seqlens, 8) || !aligned(response_lens, 8) || !aligned(out, 4) ||
+      !aligned(err_flag, 4))
+    return VRL_ERR_ALIGN;
+  vrl::response_slice_kernel<<<dim3(static_cast<unsigned>(B)), dim3(256), 0, static_cast<hipStream_t>(stream)>>>(
+      values, cu_seqlens, response_lens, T_out, out, err_flag);
   return launch_status();
 }
 
@@ -140,8 +244,8 @@ int vrl_truncate_draft(const int64_t* draft_ids, const uint8_t* mask, const int6
 
 int vrl_fused_score_verify(const void* logits, int dtype, int64_t n_rows, int64_t vocab,
                            int64_t row_stride, const int64_t* labels, const float* temperature,
-                           float* out_logprob, float* out_entropy, int32_t* err_flag,
-                           const float* logp_old, const float* log_u, const uint8_t* mask,
+                           float* out_logprob, float* out_entropy, float* out_sum_pi_sq,
+                           int32_t* err_flag, const float* logp_old, const float* log_u, const uint8_t* mask,
                            const int64_t* cu_seqlens, int64_t B, int64_t T, float thresh_offset,
                            float near_eps, uint8_t* accept, int32_t* first_reject,
                            int32_t* prefix_len, int32_t* near_count, const int64_t* draft_ids,
@@ -149,14 +253,14 @@ int vrl_fused_score_verify(const void* logits, int dtype, int64_t n_rows, int64_
   // Check both halves before anything is enqueued.
   if (out_logprob == nullptr && n_rows > 0) return VRL_ERR_NULL;
   int st = check_rowscore(logits, dtype, n_rows, vocab, row_stride, labels, temperature, out_logprob,
-                          out_entropy, err_flag);
+                          out_entropy, out_sum_pi_sq, err_flag);
   if (st != VRL_OK) return st;
   st = check_verify(out_logprob, logp_old, log_u, mask, cu_seqlens, B, T, accept, first_reject,
                     prefix_len, near_count, draft_ids, out_ids, out_mask);
   if (st != VRL_OK) return st;
   if (cu_seqlens == nullptr && n_rows != B * T) return VRL_ERR_SHAPE;
   st = vrl_rowscore(logits, dtype, n_rows, vocab, row_stride, labels, temperature, out_logprob,
-                    out_entropy, err_flag, stream);
+                    out_entropy, out_sum_pi_sq, err_flag, stream);
   if (st != VRL_OK) return st;
   return vrl_spec_verify(out_logprob, logp_old, log_u, mask, cu_seqlens, B, T, thresh_offset, near_eps,
                          accept, first_reject, prefix_len, near_count, draft_ids, pad_id, out_ids,

@@ -2,7 +2,8 @@
 
 What gets replaced (verl/utils/torch_functional.py):
     logprobs_from_logits :73, logprobs_from_logits_v2 :173, logprobs_from_logits_naive :155,
-    entropy_from_logits :231, entropy_from_logits_with_chunking :248
+    entropy_from_logits :231, entropy_from_logits_with_chunking :248,
+    calculate_sum_pi_squared_from_logits :690
 and every copy of those names that an already imported ``verl.*`` module bound
 with ``from verl.utils.torch_functional import ...`` (the engines do so at
 verl/workers/engine/fsdp/transformer_impl.py:66 and siblings; the reference's
@@ -33,6 +34,7 @@ PATCHED_NAMES = (
     "logprobs_from_logits_naive",
     "entropy_from_logits",
     "entropy_from_logits_with_chunking",
+    "calculate_sum_pi_squared_from_logits",
 )
 
 _originals: Dict[str, Callable] = {}

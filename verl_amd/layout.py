@@ -1,0 +1,60 @@
+"""Layout steps either side of the scoring path, on the GPU.
+
+``roll_labels`` restates the one-line label construction of the reference's engine
+(verl/workers/engine/fsdp/transformer_impl.py:1177); ``response_slice`` replaces the
+per-sequence Python loop of verl/workers/utils/padding.py:97-141 with one kernel launch.
+"""
+
+from __future__ import annotations
+
+from typing import Optional
+
+import torch
+
+from . import _lib
+
+__all__ = ["roll_labels", "response_slice"]
+
+
+def roll_labels(input_ids_rmpad: torch.Tensor) -> torch.Tensor:
+    """Labels of the packed token axis: every position is scored against the NEXT token id.
+
+    The roll is over the whole packed axis, so the last token of a sequence gets the first id of the next
+    one; that position is never part of a response slice. Under sequence parallelism it must happen before
+    the per-rank split (tests/models/test_fused_kernels_ulysses_sp_on_cpu.py:69-90 in the reference).
+    """
+    return torch.roll(input_ids_rmpad, shifts=-1, dims=-1)
+
+
+def response_slice(values: torch.Tensor, cu_seqlens: torch.Tensor, response_lens: torch.Tensor,
+                   max_response_len: Optional[int] = None, check: bool = True) -> torch.Tensor:
+    """Packed per-token fp32 ``values`` (total_nnz,) -> ``(B, max_response_len)`` block of response positions.
+
+    Row b holds ``values[end_b - r_b - 1 : end_b - 1]`` (model output is shifted left by one token) padded
+    with zeros, where ``end_b = cu_seqlens[b+1]`` and ``r_b = response_lens[b]``. Like the reference it
+    requires every sequence to have a prompt token; with ``check`` a violation raises ValueError.
+    """
+    if not values.is_cuda:
+        raise RuntimeError(f"values is on {values.device}; verl_amd only runs on the GPU, it has no CPU implementation")
+    if values.dim() != 1:
+        raise ValueError(f"values must be 1-D (total_nnz,), got shape {tuple(values.shape)}")
+    dev = values.device
+    v = values.to(torch.float32).contiguous()
+    cu = cu_seqlens.to(device=dev, dtype=torch.int64).contiguous()
+    rl = response_lens.to(device=dev, dtype=torch.int64).contiguous()
+    B = rl.numel()
+    if cu.numel() != B + 1:
+        raise ValueError(f"cu_seqlens must have B+1 = {B + 1} entries, got {cu.numel()}")
+    if max_response_len is None or max_response_len < 0:
+        max_response_len = int(rl.max().item()) if B > 0 else 0
+    T = int(max_response_len)
+    out = torch.empty((B, T), dtype=torch.float32, device=dev)
+    flag = torch.zeros(1, dtype=torch.int32, device=dev)
+    lib = _lib.load()
+    with torch.cuda.device(dev):
+        st = lib.vrl_response_slice(v.data_ptr(), cu.data_ptr(), rl.data_ptr(), B, T, out.data_ptr(), flag.data_ptr(),
+                                    torch.cuda.current_stream(dev).cuda_stream)
+    _lib.check("vrl_response_slice", st)
+    if check and (int(flag.item()) & _lib.VRL_FLAG_SLICE_RANGE):
+        raise ValueError("response_slice: a sequence has no prompt token, or a response length outside [0, max_response_len]")
+    return out

@@ -265,7 +265,7 @@ def fused_score_verify(
         stream = torch.cuda.current_stream(dev).cuda_stream
         st = lib.vrl_fused_score_verify(
             x.data_ptr(), _DTYPE_CODES[x.dtype], n, V, x.stride(0) if n > 1 else V, lab.data_ptr(), _ptr(temp),
-            out_lp.data_ptr(), out_h.data_ptr(), flag.data_ptr(),
+            out_lp.data_ptr(), out_h.data_ptr(), None, flag.data_ptr(),
             lo.data_ptr(), lu.data_ptr(), _ptr(m8), _ptr(cu), B, T, off, float(near_eps),
             accept.data_ptr(), first.data_ptr(), prefix.data_ptr(), near.data_ptr(),
             _ptr(ids), int(pad_id), _ptr(out_ids), _ptr(out_mask), stream,

@@ -28,6 +28,7 @@ __all__ = [
     "logprobs_from_logits_naive",
     "entropy_from_logits",
     "entropy_from_logits_with_chunking",
+    "calculate_sum_pi_squared_from_logits",
     "fused_logprob_entropy",
 ]
 
@@ -91,12 +92,19 @@ def rowscore(
     *,
     want_logprob: bool = True,
     want_entropy: bool = True,
+    want_sum_pi_sq: bool = False,
     check_labels: bool = True,
+    n_splits: Optional[int] = None,
     what: str = "rowscore",
 ):
-    """Launch vrl_rowscore; returns (logprob | None, entropy | None), each fp32 of shape logits.shape[:-1]."""
+    """Launch the row kernel; returns (logprob | None, entropy | None) and, with ``want_sum_pi_sq``,
+    a third entry, each fp32 of shape logits.shape[:-1].
+
+    With few rows the work of one row is spread over ``n_splits`` workgroups (vrl_rowscore_split);
+    ``n_splits=None`` lets the library choose, 1 forces one workgroup per row.
+    """
     _check_logits(logits, what)
-    if not (want_logprob or want_entropy):
+    if not (want_logprob or want_entropy or want_sum_pi_sq):
         raise ValueError(f"{what}: nothing to compute")
     lead = logits.shape[:-1]
     V = logits.shape[-1]
@@ -117,22 +125,36 @@ def rowscore(
     temp = _temperature_rows(temperature, lead, n, dev)
     out_lp = torch.empty(n, dtype=torch.float32, device=dev) if want_logprob else None
     out_h = torch.empty(n, dtype=torch.float32, device=dev) if want_entropy else None
+    out_q = torch.empty(n, dtype=torch.float32, device=dev) if want_sum_pi_sq else None
     flag = torch.zeros(1, dtype=torch.int32, device=dev) if want_logprob else None
 
     if n > 0:
         lib = _lib.load()
+        dt = _DTYPE_CODES[x.dtype]
+        stride = x.stride(0) if n > 1 else V
+        splits = lib.vrl_rowscore_split_plan(dt, n, V) if n_splits is None else int(n_splits)
         with torch.cuda.device(dev):
             stream = torch.cuda.current_stream(dev).cuda_stream
-            st = lib.vrl_rowscore(
-                x.data_ptr(), _DTYPE_CODES[x.dtype], n, V, x.stride(0) if n > 1 else V,
-                _ptr(lab), _ptr(temp), _ptr(out_lp), _ptr(out_h), _ptr(flag), stream,
-            )
-        _lib.check("vrl_rowscore", st)
+            if splits > 1:
+                partials = torch.empty(n * splits * 4, dtype=torch.float32, device=dev)
+                st = lib.vrl_rowscore_split(
+                    x.data_ptr(), dt, n, V, stride, _ptr(lab), _ptr(temp), _ptr(out_lp), _ptr(out_h), _ptr(out_q),
+                    _ptr(flag), splits, partials.data_ptr(), stream,
+                )
+                _lib.check("vrl_rowscore_split", st)
+            else:
+                st = lib.vrl_rowscore(
+                    x.data_ptr(), dt, n, V, stride, _ptr(lab), _ptr(temp), _ptr(out_lp), _ptr(out_h), _ptr(out_q),
+                    _ptr(flag), stream,
+                )
+                _lib.check("vrl_rowscore", st)
         if want_logprob and check_labels and (int(flag.item()) & _lib.VRL_FLAG_LABEL_OOB):
             raise IndexError(f"{what}: a label is outside [0, {V})")
 
     lp = out_lp.reshape(lead) if want_logprob else None
     h = out_h.reshape(lead) if want_entropy else None
+    if want_sum_pi_sq:
+        return lp, h, out_q.reshape(lead)
     return lp, h
 
 
@@ -175,12 +197,23 @@ def entropy_from_logits_with_chunking(logits: torch.Tensor, chunk_size: int = 20
     return rowscore(logits, None, want_logprob=False, what="entropy_from_logits_with_chunking")[1]
 
 
+def calculate_sum_pi_squared_from_logits(logits: torch.Tensor) -> torch.Tensor:
+    """sum(softmax(logits)^2) over the last dim, fp32.
+
+    Mirrors verl/utils/torch_functional.py:690-704 (exp(logsumexp(2x) - 2 logsumexp(x))).
+    """
+    return rowscore(logits, None, want_logprob=False, want_entropy=False, want_sum_pi_sq=True,
+                    what="calculate_sum_pi_squared_from_logits")[2]
+
+
 def fused_logprob_entropy(
     logits: torch.Tensor,
     labels: torch.Tensor,
     temperature: Union[None, float, torch.Tensor] = None,
     *,
     check_labels: bool = True,
+    want_sum_pi_sq: bool = False,
+    n_splits: Optional[int] = None,
 ):
     """(log-probs, entropy) of softmax(logits / temperature) in one pass over the logits.
 
@@ -190,6 +223,9 @@ def fused_logprob_entropy(
     per token (same leading shape as ``labels``), clamped below at 1e-8 like the
     reference. For fp32 logits the quotient is rounded per element exactly like
     ``logits / temperature``; for bf16 logits it is formed in fp32 from the bf16
-    values (the reference rounds the quotient back to bf16).
+    values (the reference rounds the quotient back to bf16). With ``want_sum_pi_sq`` a third
+    tensor, sum(softmax^2), comes out of the same pass
+    (verl/workers/engine/fsdp/transformer_impl.py:1361-1362).
     """
-    return rowscore(logits, labels, temperature, check_labels=check_labels, what="fused_logprob_entropy")
+    return rowscore(logits, labels, temperature, check_labels=check_labels, want_sum_pi_sq=want_sum_pi_sq,
+                    n_splits=n_splits, what="fused_logprob_entropy")
