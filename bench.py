@@ -30,6 +30,10 @@ from verl_amd import spec_rl as sv  # noqa: E402
 from verl_amd import torch_functional as vf  # noqa: E402
 
 HBM_PEAK_GBPS = 8000.0
+# HBM bytes per row-kernel launch measured with rocprofv3 (--pmc FETCH_SIZE and --pmc WRITE_SIZE, one run each,
+# both scaled by what the same counter reads for a plain 1 GiB device copy: x1.999956 and x1.0). The workload
+# shapes are fixed, so the figure is a property of (kernel, shape); the counter summary is kept under profiles/.
+MEASURED_TRAFFIC_BYTES = {"c2": 19943708065, "c3": 2490920770, "c4": 67292648393}
 METRIC = "verified tokens/sec + achieved HBM GB/s (% of peak), vocab 152k bf16, 1 GPU"
 
 
@@ -43,26 +47,47 @@ def algorithmic_bytes_per_token(V: int, esize: int, with_temperature: bool, with
 
 
 class Step:
-    """Preallocated buffers and the raw ABI calls for one workload."""
+    """Preallocated buffers and the raw ABI calls for one workload.
 
-    def __init__(self, w: synthetic.Workload, dev, seed: int, n_rows: int | None = None):
-        self.w = w
+    Workloads whose logits fit in HBM at once (c1, c2, c4) are one padded (B, T) batch. A workload with
+    ``micro_batch_tokens`` (c3) is scored the way verl feeds it after padding removal: whole sequences packed
+    end to end until the token budget is full (the last one cut to fit), so every row is a valid token.
+    """
+
+    def __init__(self, w: synthetic.Workload, dev, seed: int):
         self.dev = dev
-        B, T = w.B, w.T
-        if n_rows is not None:  # micro-batch of whole padded sequences
-            B = max(1, n_rows // T)
-            w = w.scaled(B=B)
-            self.w = w
-        d = synthetic.make_padded(w, dev, seed)
-        self.logits = d["logits"].view(-1, w.V)
-        self.labels = d["labels"].view(-1).contiguous()
-        self.mask = d["mask"].contiguous()
-        self.mask8 = self.mask.view(torch.uint8)
-        self.log_u = d["log_u"].contiguous()
-        self.temp = None if d["temperature"] is None else d["temperature"].view(-1).contiguous()
+        if w.micro_batch_tokens is None:
+            d = synthetic.make_padded(w, dev, seed)
+            self.logits = d["logits"].view(-1, w.V)
+            self.labels = d["labels"].view(-1).contiguous()
+            self.mask8 = d["mask"].contiguous().view(torch.uint8).view(-1)
+            self.log_u = d["log_u"].contiguous().view(-1)
+            self.temp = None if d["temperature"] is None else d["temperature"].view(-1).contiguous()
+            self.B, self.T, self.cu = w.B, w.T, None
+            self.layout = f"padded {w.B}x{w.T}"
+        else:
+            budget = int(w.micro_batch_tokens)
+            lengths = synthetic.draw_lengths(w, seed + 2).tolist()
+            picked, total = [], 0
+            for L in lengths:
+                take = min(L, budget - total)
+                picked.append(take)
+                total += take
+                if total == budget:
+                    break
+            cu = synthetic.pack_by_lengths(torch.tensor(picked))
+            g = torch.Generator(device=dev).manual_seed(seed + 1)
+            self.labels = torch.randint(0, w.V, (total,), generator=g, device=dev, dtype=torch.int64)
+            self.log_u = torch.log(torch.rand(total, generator=g, device=dev, dtype=torch.float32))
+            self.logits = synthetic.make_logits(total, w.V, w.dtype, w.sigma, self.labels, dev, seed + 3,
+                                                boost=w.boost, boost_frac=w.boost_frac)
+            self.mask8 = torch.ones(total, dtype=torch.uint8, device=dev)
+            self.temp = None if w.temperature is None else torch.full((total,), float(w.temperature), device=dev)
+            self.B, self.T, self.cu = len(picked), 0, cu.to(dev)
+            self.layout = f"packed {len(picked)} sequences, {total} tokens"
+        self.w = w
         self.n = self.logits.shape[0]
-        self.B, self.T = w.B, w.T
-        self.n_valid = int(self.mask.sum().item())
+        self.n_valid = int(self.mask8.sum().item())
         self.off = sv.thresh_offset_from_lenience(w.lenience)
         f32 = dict(dtype=torch.float32, device=dev)
         self.lp = torch.empty(self.n, **f32)
@@ -96,7 +121,8 @@ class Step:
         st = self.lib.vrl_fused_score_verify(
             self.logits.data_ptr(), self.dt, self.n, self.w.V, self.logits.stride(0), self.labels.data_ptr(),
             self._tp(), self.lp.data_ptr(), self.h.data_ptr(), None, self.flag.data_ptr(),
-            self.lp_old.data_ptr(), self.log_u.data_ptr(), self.mask8.data_ptr(), None, self.B, self.T,
+            self.lp_old.data_ptr(), self.log_u.data_ptr(), self.mask8.data_ptr(),
+            None if self.cu is None else self.cu.data_ptr(), self.B, self.T,
             self.off, 1e-6, self.accept.data_ptr(), self.first.data_ptr(), self.prefix.data_ptr(),
             self.near.data_ptr(), self.ids.data_ptr(), 0, self.out_ids.data_ptr(), self.out_mask.data_ptr(),
             self.stream)
@@ -132,8 +158,8 @@ def cpu_baseline(step: Step, budget_s: float = 20.0):
     lab = step.labels[:rows].cpu()
     temp = None if step.temp is None else step.temp[:rows].cpu()
     old = step.lp_old[:rows].cpu().view(1, rows)
-    lu = step.log_u.view(-1)[:rows].cpu().view(1, rows)
-    mk = step.mask.view(-1)[:rows].cpu().view(1, rows)
+    lu = step.log_u[:rows].cpu().view(1, rows)
+    mk = step.mask8[:rows].cpu().view(1, rows)
 
     def once():
         t0 = time.perf_counter()
@@ -162,6 +188,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--workload", default="c2", choices=["c1", "c2", "c3", "c4"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="also run a plain device copy of known size (for scaling rocprofv3 byte counters)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on one GPU only; "
@@ -174,9 +202,18 @@ def main():
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
     w = synthetic.WORKLOADS[args.workload]
-    n_rows = w.micro_batch_tokens  # c3: one 8192-token micro-batch per step
-    step = Step(w, dev, seed=1000 * int(args.workload[1]), n_rows=n_rows)
+    step = Step(w, dev, seed=1000 * int(args.workload[1]))
     err_lp, err_h = step.check_against_torch()
+
+    if args.copy_calibration:
+        # A plain copy kernel of known size: reads 1 GiB, writes 1 GiB. Whatever FETCH_SIZE / WRITE_SIZE report
+        # for it is the scale that converts the same counters of the row kernel into bytes.
+        src = torch.empty(1 << 29, dtype=torch.int16, device=dev).fill_(3)
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
 
     for _ in range(args.warmup):
         step.fused()
@@ -218,12 +255,14 @@ def main():
         "data": "synthetic",
         "config": {
             "workload": step.w.name,
+            "layout": step.layout,
+            "launches_per_step": 2,
             "rows_per_step": step.n,
             "valid_tokens_per_step": step.n_valid,
             "vocab": w.V,
             "lenience": w.lenience,
             "temperature": w.temperature,
-            "step": "vrl_fused_score_verify (row kernel + verify kernel), logits resident in HBM",
+            "step": "vrl_fused_score_verify through the C ABI, logits resident in HBM",
         },
         "hbm_gbps_fused_step": bytes_fused / (ms_per_step * 1e-3) / 1e9,
         "roofline": {
@@ -232,7 +271,7 @@ def main():
             "peak": HBM_PEAK_GBPS,
             "unit": "GB/s",
             "frac": achieved / HBM_PEAK_GBPS,
-            "traffic": None,
+            "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload),
             "kernel": "rowscore_kernel",
             "avg_kernel_ms": avg_kern_ms,
             "algorithmic_bytes_per_launch": bytes_score,

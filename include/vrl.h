@@ -141,11 +141,17 @@ int vrl_truncate_draft(const int64_t* draft_ids, const uint8_t* mask, const int6
                        int64_t* out_ids, uint8_t* out_mask, void* stream);
 
 /*
- * vrl_fused_score_verify — vrl_rowscore followed on the same stream by
- * vrl_spec_verify fed with the log-probs just written (logp_new = out_logprob,
- * which is therefore required). Row space and sequence space are as above:
- * n_rows must equal cu_seqlens[B] (packed) or B*T (padded); the host checks
- * only the padded case, cu_seqlens lives on the device.
+ * vrl_fused_score_verify — scoring and verification of the same batch in one
+ * call: the results of vrl_rowscore, and of vrl_spec_verify fed with the
+ * log-probs just computed (logp_new = out_logprob, which is therefore required).
+ * Row space and sequence space are as above: n_rows must equal cu_seqlens[B]
+ * (packed) or B*T (padded); the host checks only the padded case, cu_seqlens
+ * lives on the device.
+ *
+ * Two launches on `stream`: the row kernel, then the verify kernel. (Doing the
+ * verification inside the row kernel, by the last workgroup of each sequence,
+ * was measured and is slower on MI355X: the agent-scope release each workgroup
+ * needs costs more than the second launch.)
  *
  * Replaces the composition at
  *   verl/workers/engine/fsdp/transformer_impl.py:1353-1399 (divide, entropy, log-probs)

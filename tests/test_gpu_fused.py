@@ -91,3 +91,17 @@ def test_fused_equals_two_calls(dev):
     assert torch.equal(res.accept, two.accept) and torch.equal(res.first_reject, two.first_reject)
     m = res.metrics(d["mask"])
     assert 0.0 <= m["spec/accept_rate"] <= 1.0 and m["spec/near_threshold_count"] >= 0
+
+
+def test_many_short_sequences(dev):
+    B, T, V = 300, 5, 1537
+    w = synthetic.WORKLOADS["c1"].scaled(B=B, T=T, V=V, lengths=("uniform", 0, 5))
+    d = synthetic.make_padded(w, dev, seed=31)
+    lp0, _ = vf.fused_logprob_entropy(d["logits"], d["labels"], n_splits=1)
+    old = synthetic.drift_old_logprobs(lp0, w, 31)
+    lp, h, res = sv.fused_score_verify(d["logits"], d["labels"], old, d["mask"], log_u=d["log_u"], draft_ids=d["labels"])
+    assert torch.equal(lp, lp0)
+    ref = overify.verify(lp, old, d["log_u"], d["mask"], 0.0, draft_ids=d["labels"])
+    assert np.array_equal(res.first_reject.cpu().numpy(), ref["first_reject"].numpy())
+    assert np.array_equal(res.accept.cpu().numpy().astype(np.uint8), ref["accept"].numpy())
+    assert np.array_equal(res.out_ids.cpu().numpy(), ref["out_ids"].numpy())

@@ -48,22 +48,34 @@ __device__ __forceinline__ void truncate_span(const SeqSpan sp, int first, const
   }
 }
 
-// grid.x = B, block = WAVES*64. No thread leaves before the last barrier.
+struct VerifyArgs {
+  const float* logp_new;
+  const float* logp_old;
+  const float* log_u;
+  const uint8_t* mask;
+  const int64_t* cu_seqlens;
+  int64_t B;
+  int64_t T;
+  float thresh_offset;
+  float near_eps;
+  uint8_t* accept;
+  int32_t* first_reject;
+  int32_t* prefix_len;
+  int32_t* near_count;
+  const int64_t* draft_ids;
+  int64_t pad_id;
+  int64_t* out_ids;
+  uint8_t* out_mask;
+};
+
+// The whole workgroup (WAVES*64 threads, all of them) verifies sequence b.
 template <int WAVES>
-__global__ __launch_bounds__(WAVES * 64) void spec_verify_kernel(
-    const float* __restrict__ logp_new, const float* __restrict__ logp_old,
-    const float* __restrict__ log_u, const uint8_t* __restrict__ mask,
-    const int64_t* __restrict__ cu_seqlens, int64_t T, float thresh_offset, float near_eps,
-    uint8_t* __restrict__ accept, int32_t* __restrict__ first_reject,
-    int32_t* __restrict__ prefix_len, int32_t* __restrict__ near_count,
-    const int64_t* __restrict__ draft_ids, int64_t pad_id, int64_t* __restrict__ out_ids,
-    uint8_t* __restrict__ out_mask) {
+__device__ __forceinline__ void verify_sequence(const VerifyArgs& v, int64_t b) {
   constexpr int NTHR = WAVES * 64;
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = tid >> 6;
-  const int64_t b = blockIdx.x;
-  const SeqSpan sp = seq_span(cu_seqlens, b, T);
+  const SeqSpan sp = seq_span(v.cu_seqlens, b, v.T);
 
   // wave-uniform running results
   int first = kNoReject;  // earliest rejected position seen by this wavefront
@@ -75,12 +87,12 @@ __global__ __launch_bounds__(WAVES * 64) void spec_verify_kernel(
     bool valid = false, ok = false, close = false;
     if (i < sp.len) {
       const int64_t g = sp.start + i;
-      const float d = logp_new[g] - logp_old[g];
-      const float tau = log_u[g] + thresh_offset;
-      valid = (mask != nullptr) ? (mask[g] != 0) : true;
+      const float d = v.logp_new[g] - v.logp_old[g];
+      const float tau = v.log_u[g] + v.thresh_offset;
+      valid = (v.mask != nullptr) ? (v.mask[g] != 0) : true;
       ok = d >= tau;
-      close = valid && (__builtin_fabsf(d - tau) < near_eps);
-      accept[g] = static_cast<uint8_t>(valid && ok);
+      close = valid && (__builtin_fabsf(d - tau) < v.near_eps);
+      v.accept[g] = static_cast<uint8_t>(valid && ok);
     }
     const unsigned long long rej = __ballot(valid && !ok);
     const unsigned long long val = __ballot(valid);
@@ -112,27 +124,33 @@ __global__ __launch_bounds__(WAVES * 64) void spec_verify_kernel(
 
   // valid tokens strictly before the first rejection
   int cnt = 0;
-  if (mask != nullptr) {
+  if (v.mask != nullptr) {
     for (int64_t base = 0; base < f; base += NTHR) {
       const int64_t i = base + tid;
-      const bool v = (i < f) && (mask[sp.start + i] != 0);
-      cnt += __builtin_popcountll(__ballot(v));
+      const bool m = (i < f) && (v.mask[sp.start + i] != 0);
+      cnt += __builtin_popcountll(__ballot(m));
     }
   }
   if (lane == 0) sm_cnt[wave] = cnt;
   __syncthreads();
   if (tid == 0) {
     int total = f;
-    if (mask != nullptr) {
+    if (v.mask != nullptr) {
       total = 0;
 #pragma unroll
       for (int w = 0; w < WAVES; ++w) total += sm_cnt[w];
     }
-    first_reject[b] = f;
-    prefix_len[b] = total;
-    near_count[b] = nc;
+    v.first_reject[b] = f;
+    v.prefix_len[b] = total;
+    v.near_count[b] = nc;
   }
-  if (out_ids != nullptr) truncate_span<WAVES>(sp, f, draft_ids, mask, pad_id, out_ids, out_mask);
+  if (v.out_ids != nullptr) truncate_span<WAVES>(sp, f, v.draft_ids, v.mask, v.pad_id, v.out_ids, v.out_mask);
+}
+
+// grid.x = B, block = WAVES*64. No thread leaves before the last barrier.
+template <int WAVES>
+__global__ __launch_bounds__(WAVES * 64) void spec_verify_kernel(const VerifyArgs v) {
+  verify_sequence<WAVES>(v, blockIdx.x);
 }
 
 template <int WAVES>
