@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the fused score + SPEC-RL verify path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c2|c3|c4|c1]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c2|c3|c4|c1|c5]
 
 One step = one pass of vrl_fused_score_verify (row kernel + verify kernel, through
 the C ABI, outputs preallocated) over the whole synthetic batch, logits resident
@@ -148,6 +148,88 @@ class Step:
         return e1, e2
 
 
+class VerifyOnlyStep:
+    """c5: 512 sequences with log-uniform lengths in [32, 16384], packed; only the verify kernel is timed
+    (its logits would be 408 GB, scored in 8192-token micro-batches like c3)."""
+
+    def __init__(self, w: synthetic.Workload, dev, seed: int):
+        self.w, self.dev = w, dev
+        lengths = synthetic.draw_lengths(w, seed + 2)
+        self.cu = synthetic.pack_by_lengths(lengths).to(dev)
+        self.B = lengths.numel()
+        self.n = int(lengths.sum())
+        self.n_valid = self.n
+        self.layout = f"packed {self.B} sequences, {self.n} tokens (verify only)"
+        g = torch.Generator(device=dev).manual_seed(seed + 1)
+        self.lp = -torch.rand(self.n, generator=g, device=dev) * 6
+        self.lp_old = synthetic.drift_old_logprobs(self.lp, w, seed).contiguous()
+        self.log_u = torch.log(torch.rand(self.n, generator=g, device=dev))
+        self.ids = torch.randint(0, w.V, (self.n,), generator=g, device=dev)
+        self.off = sv.thresh_offset_from_lenience(w.lenience)
+        self.accept = torch.empty(self.n, dtype=torch.uint8, device=dev)
+        self.first = torch.empty(self.B, dtype=torch.int32, device=dev)
+        self.prefix = torch.empty(self.B, dtype=torch.int32, device=dev)
+        self.near = torch.empty(self.B, dtype=torch.int32, device=dev)
+        self.out_ids = torch.empty_like(self.ids)
+        self.out_mask = torch.empty(self.n, dtype=torch.uint8, device=dev)
+        self.lib = _lib.load()
+        self.stream = torch.cuda.current_stream(dev).cuda_stream
+
+    def verify(self):
+        st = self.lib.vrl_spec_verify(
+            self.lp.data_ptr(), self.lp_old.data_ptr(), self.log_u.data_ptr(), None, self.cu.data_ptr(), self.B, 0,
+            self.off, 1e-6, self.accept.data_ptr(), self.first.data_ptr(), self.prefix.data_ptr(),
+            self.near.data_ptr(), self.ids.data_ptr(), 0, self.out_ids.data_ptr(), self.out_mask.data_ptr(), self.stream)
+        _lib.check("vrl_spec_verify", st)
+
+
+def bench_verify_only(args, dev):
+    """tokens/s of vrl_spec_verify alone on the c5 workload; 4+4+4 in, 1 out per token, plus the truncated draft
+    (8 in, 8+1 out) = 30 B/token with the draft, 14 B/token (13 + per-sequence outputs) without."""
+    w = synthetic.WORKLOADS["c5"]
+    step = VerifyOnlyStep(w, dev, seed=5000)
+    for _ in range(args.warmup):
+        step.verify()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step.verify()
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(args.steps)]
+    for a, b in evs:
+        a.record()
+        step.verify()
+        b.record()
+    torch.cuda.synchronize()
+    avg_ms = sum(a.elapsed_time(b) for a, b in evs) / len(evs)
+    bytes_launch = step.n * (4 + 4 + 4 + 1 + 8 + 8 + 1) + step.B * (12 + 8)
+    achieved = bytes_launch / (avg_ms * 1e-3) / 1e9
+    out = {
+        "metric": METRIC, "value": step.n * args.steps / wall, "unit": "tokens/s", "n_gpus": 1, "steps": args.steps,
+        "warmup": args.warmup, "ms_per_step": wall * 1e3 / args.steps, "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+        "config": {"workload": w.name, "layout": step.layout, "launches_per_step": 1, "tokens_per_step": step.n,
+                   "lenience": w.lenience, "step": "vrl_spec_verify with truncated draft, through the C ABI"},
+        "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                     "frac": achieved / HBM_PEAK_GBPS, "traffic": None, "kernel": "spec_verify_kernel",
+                     "avg_kernel_ms": avg_ms, "algorithmic_bytes_per_launch": bytes_launch},
+    }
+    if not args.no_cpu_baseline:
+        from oracle import verify as overify  # baseline only
+
+        ln, lo, lu, ids, cu = step.lp.cpu(), step.lp_old.cpu(), step.log_u.cpu(), step.ids.cpu(), step.cu.cpu()
+        times = []
+        for _ in range(3):
+            t0 = time.perf_counter()
+            overify.verify(ln, lo, lu, None, step.off, cu_seqlens=cu, draft_ids=ids)
+            times.append(time.perf_counter() - t0)
+        out["cpu_baseline"] = {"value": step.n / statistics.median(times), "unit": "tokens/s",
+                               "cores": torch.get_num_threads(), "kind": "port",
+                               "sample": f"the whole workload ({step.n} tokens), median of 3 runs of the vectorised torch statement of the rule"}
+    print(json.dumps(out), flush=True)
+
+
 def cpu_baseline(step: Step, budget_s: float = 20.0):
     """The torch restatement of the reference composition on the host cores, on a slice of the same batch."""
     from oracle import scoring, verify as overify  # checker/baseline only
@@ -186,7 +268,8 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
-    ap.add_argument("--workload", default="c2", choices=["c1", "c2", "c3", "c4"])
+    ap.add_argument("--workload", default="c2", choices=["c1", "c2", "c3", "c4", "c5"],
+                    help="c5 times the verify kernel alone (its logits do not fit; they are scored like c3)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run a plain device copy of known size (for scaling rocprofv3 byte counters)")
@@ -201,6 +284,9 @@ def main():
 
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
+    if args.workload == "c5":
+        bench_verify_only(args, dev)
+        return
     w = synthetic.WORKLOADS[args.workload]
     step = Step(w, dev, seed=1000 * int(args.workload[1]))
     err_lp, err_h = step.check_against_torch()

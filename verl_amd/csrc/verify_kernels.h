@@ -39,12 +39,19 @@ __device__ __forceinline__ void truncate_span(const SeqSpan sp, int first, const
                                               const uint8_t* mask, int64_t pad_id, int64_t* out_ids,
                                               uint8_t* out_mask) {
   constexpr int NTHR = WAVES * 64;
+  // Positions at or after the cut need no load at all.
+#pragma unroll 4
   for (int64_t i = threadIdx.x; i < sp.len; i += NTHR) {
     const bool keep = i < first;
     const int64_t g = sp.start + i;
-    out_ids[g] = keep ? draft_ids[g] : pad_id;
-    const uint8_t mv = (mask != nullptr) ? static_cast<uint8_t>(mask[g] != 0) : static_cast<uint8_t>(1);
-    out_mask[g] = keep ? mv : static_cast<uint8_t>(0);
+    int64_t id = pad_id;
+    uint8_t mv = 0;
+    if (keep) {
+      id = draft_ids[g];
+      mv = (mask != nullptr) ? static_cast<uint8_t>(mask[g] != 0) : static_cast<uint8_t>(1);
+    }
+    out_ids[g] = id;
+    out_mask[g] = mv;
   }
 }
 
@@ -82,25 +89,45 @@ __device__ __forceinline__ void verify_sequence(const VerifyArgs& v, int64_t b) 
   int last_valid = 0;     // one past the last valid position seen by this wavefront
   int near = 0;
 
-  for (int64_t base = 0; base < sp.len; base += NTHR) {
-    const int64_t i = base + tid;
-    bool valid = false, ok = false, close = false;
-    if (i < sp.len) {
-      const int64_t g = sp.start + i;
-      const float d = v.logp_new[g] - v.logp_old[g];
-      const float tau = v.log_u[g] + v.thresh_offset;
-      valid = (v.mask != nullptr) ? (v.mask[g] != 0) : true;
-      ok = d >= tau;
-      close = valid && (__builtin_fabsf(d - tau) < v.near_eps);
-      v.accept[g] = static_cast<uint8_t>(valid && ok);
+  // kChunks chunks of NTHR tokens per trip, all loads of a trip issued before any is used, so a long
+  // sequence costs len / (kChunks * NTHR) memory round trips instead of len / NTHR.
+  constexpr int kChunks = 4;
+  for (int64_t base = 0; base < sp.len; base += static_cast<int64_t>(NTHR) * kChunks) {
+    float ln[kChunks], lo[kChunks], lu[kChunks];
+    uint8_t mk[kChunks];
+    bool in[kChunks];
+#pragma unroll
+    for (int j = 0; j < kChunks; ++j) {
+      const int64_t i = base + static_cast<int64_t>(j) * NTHR + tid;
+      in[j] = i < sp.len;
+      ln[j] = lo[j] = lu[j] = 0.f;
+      mk[j] = 0;
+      if (in[j]) {
+        const int64_t g = sp.start + i;
+        ln[j] = v.logp_new[g];
+        lo[j] = v.logp_old[g];
+        lu[j] = v.log_u[g];
+        mk[j] = (v.mask != nullptr) ? v.mask[g] : static_cast<uint8_t>(1);
+      }
     }
-    const unsigned long long rej = __ballot(valid && !ok);
-    const unsigned long long val = __ballot(valid);
-    const unsigned long long nr = __ballot(close);
-    const int wbase = static_cast<int>(base) + wave * 64;
-    if (rej != 0ull && first == kNoReject) first = wbase + __builtin_ctzll(rej);
-    if (val != 0ull) last_valid = wbase + 64 - __builtin_clzll(val);
-    near += __builtin_popcountll(nr);
+#pragma unroll
+    for (int j = 0; j < kChunks; ++j) {
+      const int64_t cbase = base + static_cast<int64_t>(j) * NTHR;
+      if (cbase >= sp.len) break;  // uniform over the workgroup
+      const float d = ln[j] - lo[j];
+      const float tau = lu[j] + v.thresh_offset;
+      const bool valid = in[j] && (mk[j] != 0);
+      const bool ok = d >= tau;
+      const bool close = valid && (__builtin_fabsf(d - tau) < v.near_eps);
+      if (in[j]) v.accept[sp.start + cbase + tid] = static_cast<uint8_t>(valid && ok);
+      const unsigned long long rej = __ballot(valid && !ok);
+      const unsigned long long val = __ballot(valid);
+      const unsigned long long nr = __ballot(close);
+      const int wbase = static_cast<int>(cbase) + wave * 64;
+      if (rej != 0ull && first == kNoReject) first = wbase + __builtin_ctzll(rej);
+      if (val != 0ull) last_valid = wbase + 64 - __builtin_clzll(val);
+      near += __builtin_popcountll(nr);
+    }
   }
 
   __shared__ int sm_first[WAVES];

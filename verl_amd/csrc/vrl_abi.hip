@@ -148,7 +148,14 @@ int check_verify(const float* logp_new, const float* logp_old, const float* log_
   return VRL_OK;
 }
 
-constexpr int kVerifyWaves = 4;
+// Wavefronts per sequence for the verify/truncate kernels. A workgroup handles 4 * 64 * waves tokens per
+// memory round trip; long sequences want many wavefronts, a batch of many short ones wants few (idle
+// wavefronts still have to be launched). Packed layouts keep their lengths on the device, so the
+// choice there goes by the number of sequences.
+int verify_waves(const int64_t* cu_seqlens, int64_t B, int64_t T) {
+  if (cu_seqlens == nullptr) return T <= 256 ? 1 : (T <= 2048 ? 4 : 16);
+  return B <= 4096 ? 16 : 4;
+}
 
 }  // namespace
 
@@ -224,8 +231,13 @@ int vrl_spec_verify(const float* logp_new, const float* logp_old, const float* l
   if (st != VRL_OK || B == 0) return st;
   const vrl::VerifyArgs v{logp_new, logp_old, log_u, mask, cu_seqlens, B, T, thresh_offset, near_eps,
                           accept, first_reject, prefix_len, near_count, draft_ids, pad_id, out_ids, out_mask};
-  vrl::spec_verify_kernel<kVerifyWaves>
-      <<<dim3(static_cast<unsigned>(B)), dim3(kVerifyWaves * 64), 0, static_cast<hipStream_t>(stream)>>>(v);
+  const dim3 grid(static_cast<unsigned>(B));
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  switch (verify_waves(cu_seqlens, B, T)) {
+    case 1: vrl::spec_verify_kernel<1><<<grid, dim3(64), 0, s>>>(v); break;
+    case 4: vrl::spec_verify_kernel<4><<<grid, dim3(256), 0, s>>>(v); break;
+    default: vrl::spec_verify_kernel<16><<<grid, dim3(1024), 0, s>>>(v); break;
+  }
   return launch_status();
 }
 
@@ -239,9 +251,13 @@ int vrl_truncate_draft(const int64_t* draft_ids, const uint8_t* mask, const int6
   if (!aligned(draft_ids, 8) || !aligned(out_ids, 8) || !aligned(cu_seqlens, 8) ||
       !aligned(first_reject, 4))
     return VRL_ERR_ALIGN;
-  vrl::truncate_draft_kernel<kVerifyWaves>
-      <<<dim3(static_cast<unsigned>(B)), dim3(kVerifyWaves * 64), 0, static_cast<hipStream_t>(stream)>>>(
-          draft_ids, mask, cu_seqlens, T, first_reject, pad_id, out_ids, out_mask);
+  const dim3 grid(static_cast<unsigned>(B));
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  switch (verify_waves(cu_seqlens, B, T)) {
+    case 1: vrl::truncate_draft_kernel<1><<<grid, dim3(64), 0, s>>>(draft_ids, mask, cu_seqlens, T, first_reject, pad_id, out_ids, out_mask); break;
+    case 4: vrl::truncate_draft_kernel<4><<<grid, dim3(256), 0, s>>>(draft_ids, mask, cu_seqlens, T, first_reject, pad_id, out_ids, out_mask); break;
+    default: vrl::truncate_draft_kernel<16><<<grid, dim3(1024), 0, s>>>(draft_ids, mask, cu_seqlens, T, first_reject, pad_id, out_ids, out_mask); break;
+  }
   return launch_status();
 }
 
