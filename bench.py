@@ -114,13 +114,13 @@ class Step:
     def score(self):
         st = self.lib.vrl_rowscore(self.logits.data_ptr(), self.dt, self.n, self.w.V, self.logits.stride(0),
                                    self.labels.data_ptr(), self._tp(), self.lp.data_ptr(), self.h.data_ptr(), None,
-                                   self.flag.data_ptr(), self.stream)
+                                   None, self.flag.data_ptr(), self.stream)
         _lib.check("vrl_rowscore", st)
 
     def fused(self):
         st = self.lib.vrl_fused_score_verify(
             self.logits.data_ptr(), self.dt, self.n, self.w.V, self.logits.stride(0), self.labels.data_ptr(),
-            self._tp(), self.lp.data_ptr(), self.h.data_ptr(), None, self.flag.data_ptr(),
+            self._tp(), self.lp.data_ptr(), self.h.data_ptr(), None, None, self.flag.data_ptr(),
             self.lp_old.data_ptr(), self.log_u.data_ptr(), self.mask8.data_ptr(),
             None if self.cu is None else self.cu.data_ptr(), self.B, self.T,
             self.off, 1e-6, self.accept.data_ptr(), self.first.data_ptr(), self.prefix.data_ptr(),

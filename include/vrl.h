@@ -54,6 +54,7 @@ extern "C" {
  *   logprob[r]   = z[label[r]] - logsumexp(z)
  *   entropy[r]   = logsumexp(z) - sum(softmax(z) * z)
  *   sum_pi_sq[r] = sum(softmax(z)^2) = exp(logsumexp(2z) - 2 logsumexp(z))
+ *   lse[r]       = logsumexp(z)            (what vrl_rowscore_backward needs)
  * with z = logits[r, :] / max(temperature[r], 1e-8) (z = logits[r, :] when
  * temperature == NULL), accumulated in fp32, written as fp32.
  *
@@ -72,7 +73,8 @@ extern "C" {
  */
 int vrl_rowscore(const void* logits, int dtype, int64_t n_rows, int64_t vocab, int64_t row_stride,
                  const int64_t* labels, const float* temperature, float* out_logprob,
-                 float* out_entropy, float* out_sum_pi_sq, int32_t* err_flag, void* stream);
+                 float* out_entropy, float* out_sum_pi_sq, float* out_lse, int32_t* err_flag,
+                 void* stream);
 
 /*
  * vrl_rowscore_split — the same results for FEW rows: n_splits workgroups share
@@ -86,9 +88,28 @@ int vrl_rowscore(const void* logits, int dtype, int64_t n_rows, int64_t vocab, i
  */
 int vrl_rowscore_split(const void* logits, int dtype, int64_t n_rows, int64_t vocab, int64_t row_stride,
                        const int64_t* labels, const float* temperature, float* out_logprob,
-                       float* out_entropy, float* out_sum_pi_sq, int32_t* err_flag, int n_splits,
-                       float* partials, void* stream);
+                       float* out_entropy, float* out_sum_pi_sq, float* out_lse, int32_t* err_flag,
+                       int n_splits, float* partials, void* stream);
 int vrl_rowscore_split_plan(int dtype, int64_t n_rows, int64_t vocab);
+
+/*
+ * vrl_rowscore_backward — gradient of the row op with respect to the logits,
+ * one read of the logits and one write of the gradient (same dtype as the logits):
+ *   dlogits[r, v] = ( g_logprob[r] * (1[v == label[r]] - p)  -  g_entropy[r] * p * (log p + entropy[r]) ) / T[r]
+ * with p = exp(z_v - lse[r]), z = logits[r, :] / max(temperature[r], 1e-8). `lse` and
+ * `entropy` are the forward outputs. g_logprob or g_entropy may be NULL (that
+ * term is then absent; labels / entropy may be NULL with it). dlogits may be
+ * the logits buffer itself (in place). Elements whose p underflows to 0 get 0.
+ *
+ * Replaces what torch autograd builds for the compositions at
+ *   verl/workers/engine/fsdp/transformer_impl.py:1357-1399 under update_actor
+ *   (verl/workers/engine_workers.py:707-714, loss.backward() at fsdp/transformer_impl.py:739-743);
+ * the closed form is the reference's verl/utils/experimental/torch_functional.py:66-79.
+ */
+int vrl_rowscore_backward(const void* logits, int dtype, int64_t n_rows, int64_t vocab, int64_t row_stride,
+                          const int64_t* labels, const float* temperature, const float* lse,
+                          const float* entropy, const float* g_logprob, const float* g_entropy,
+                          void* dlogits, int64_t d_row_stride, void* stream);
 
 /*
  * vrl_response_slice — packed per-token values (total_nnz,) -> padded (B, T_out)
@@ -159,7 +180,7 @@ int vrl_truncate_draft(const int64_t* draft_ids, const uint8_t* mask, const int6
  */
 int vrl_fused_score_verify(const void* logits, int dtype, int64_t n_rows, int64_t vocab,
                            int64_t row_stride, const int64_t* labels, const float* temperature,
-                           float* out_logprob, float* out_entropy, float* out_sum_pi_sq,
+                           float* out_logprob, float* out_entropy, float* out_sum_pi_sq, float* out_lse,
                            int32_t* err_flag, const float* logp_old, const float* log_u, const uint8_t* mask,
                            const int64_t* cu_seqlens, int64_t B, int64_t T, float thresh_offset,
                            float near_eps, uint8_t* accept, int32_t* first_reject,

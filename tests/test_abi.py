@@ -64,7 +64,7 @@ def test_rowscore_argument_errors(lib):
 
     def call(**kw):
         a = {**ok, **kw}
-        return f(a["logits"], a["dtype"], a["n"], a["V"], a["stride"], a["labels"], a["temp"], a["lp"], a["h"], a.get("q"), a["flag"], None)
+        return f(a["logits"], a["dtype"], a["n"], a["V"], a["stride"], a["labels"], a["temp"], a["lp"], a["h"], a.get("q"), a.get("lse"), a["flag"], None)
 
     assert call(dtype=7) == _lib.VRL_ERR_DTYPE
     assert call(n=-1) == _lib.VRL_ERR_SHAPE
@@ -82,14 +82,16 @@ def test_rowscore_argument_errors(lib):
     assert call(temp=P + 1) == _lib.VRL_ERR_ALIGN
     # nothing to do is not an error, and needs no pointers
     assert call(q=P + 2) == _lib.VRL_ERR_ALIGN
-    assert f(None, _lib.VRL_F32, 0, 100, 100, None, None, None, P, None, None, None) == _lib.VRL_OK
+    assert call(lse=P + 1) == _lib.VRL_ERR_ALIGN
+    assert call(lp=None, h=None, labels=None, flag=None, lse=None) == _lib.VRL_ERR_ARG
+    assert f(None, _lib.VRL_F32, 0, 100, 100, None, None, None, P, None, None, None, None) == _lib.VRL_OK
 
 
 def test_split_and_slice_argument_errors(lib):
     f = lib.vrl_rowscore_split
 
     def call(n=4, splits=4, partials=P, lp=P, dtype=_lib.VRL_BF16):
-        return f(P, dtype, n, 100000, 100000, P, None, lp, P, None, P, splits, partials, None)
+        return f(P, dtype, n, 100000, 100000, P, None, lp, P, None, None, P, splits, partials, None)
 
     assert call(splits=0) == _lib.VRL_ERR_ARG
     assert call(splits=65) == _lib.VRL_ERR_ARG
@@ -104,6 +106,21 @@ def test_split_and_slice_argument_errors(lib):
     assert plan(_lib.VRL_BF16, 1, 151936) >= 16
     assert plan(_lib.VRL_F32, 16, 1000) == 1                # rows too short to cut
     assert plan(7, 16, 151936) == 1 and plan(_lib.VRL_F32, 0, 10) == 1
+
+    bw = lib.vrl_rowscore_backward
+
+    def back(dtype=_lib.VRL_BF16, n=4, V=100, stride=100, dstride=100, labels=P, lse=P, ent=P, gl=P, gh=P, dx=P, x=P):
+        return bw(x, dtype, n, V, stride, labels, None, lse, ent, gl, gh, dx, dstride, None)
+
+    assert back(dtype=5) == _lib.VRL_ERR_DTYPE
+    assert back(dstride=99) == _lib.VRL_ERR_SHAPE
+    assert back(gl=None, gh=None) == _lib.VRL_ERR_ARG
+    assert back(lse=None) == _lib.VRL_ERR_NULL
+    assert back(labels=None) == _lib.VRL_ERR_NULL
+    assert back(ent=None) == _lib.VRL_ERR_NULL
+    assert back(dx=None) == _lib.VRL_ERR_NULL
+    assert back(dx=P + 1) == _lib.VRL_ERR_ALIGN
+    assert back(n=0, x=None, dx=None, lse=None) == _lib.VRL_OK
 
     g = lib.vrl_response_slice
     assert g(P, P, P, -1, 4, P, P, None) == _lib.VRL_ERR_SHAPE
@@ -143,7 +160,7 @@ def test_truncate_and_fused_argument_errors(lib):
     f = lib.vrl_fused_score_verify
 
     def call(n=16, B=2, T=8, lp=P, dtype=_lib.VRL_BF16, cu=None, lo=P):
-        return f(P, dtype, n, 100, 100, P, None, lp, P, None, P, lo, P, None, cu, B, T, 0.0, 1e-6, P, P, P, P, None, 0, None, None, None)
+        return f(P, dtype, n, 100, 100, P, None, lp, P, None, None, P, lo, P, None, cu, B, T, 0.0, 1e-6, P, P, P, P, None, 0, None, None, None)
 
     assert call(lp=None) == _lib.VRL_ERR_NULL                  # verify needs the log-probs
     assert call(dtype=3) == _lib.VRL_ERR_DTYPE

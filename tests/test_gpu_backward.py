@@ -1,0 +1,132 @@
+"""Backward of the row op (vrl_rowscore_backward through torch.autograd) against torch's autograd of the
+oracle's composition on the same inputs.
+
+fp32 logits: absolute 2e-6 (gradient entries are bounded by |g_logprob| + |g_entropy| * (|log p| + H) / T).
+bf16 logits: the reference gradient is the fp32 autograd result rounded to bf16; the kernel computes in fp32 and
+rounds once, so the two agree to one bf16 ulp (2^-8 relative) plus the fp32 difference.
+"""
+
+import pytest
+import torch
+
+from verl_amd import torch_functional as vf
+from oracle import scoring
+
+pytestmark = pytest.mark.gpu
+
+
+def _reference_grad(x, lab, temp, w_lp, w_h):
+    xr = x.detach().float().requires_grad_(True)
+    lp, h = scoring.score_reference(xr, lab, temp)
+    loss = 0.0
+    if w_lp is not None:
+        loss = loss + (lp * w_lp).sum()
+    if w_h is not None:
+        loss = loss + (h * w_h).sum()
+    loss.backward()
+    return xr.grad
+
+
+def _ours(x, lab, temp, w_lp, w_h):
+    xo = x.detach().clone().requires_grad_(True)
+    lp, h = vf.fused_logprob_entropy(xo, lab, temp)
+    loss = 0.0
+    if w_lp is not None:
+        loss = loss + (lp * w_lp).sum()
+    if w_h is not None:
+        loss = loss + (h * w_h).sum()
+    loss.backward()
+    assert xo.grad.dtype == x.dtype and xo.grad.shape == x.shape
+    return xo.grad
+
+
+def _compare(got, ref, dtype, scale=4.0):
+    """``scale`` bounds the incoming gradients (|w| of a standard normal stays below 4 here). The exponent
+    x*c - lse*log2(e) is formed in fp32 at magnitude ~25, so p carries ~1e-6 relative error: 4e-6 * scale absolute."""
+    got, ref = got.float(), ref.float()
+    floor = 4e-6 * scale
+    if dtype == torch.float32:
+        assert (got - ref).abs().max().item() <= floor
+    else:
+        assert ((got - ref).abs() <= ref.abs() * 2.0 ** -7 + floor).all(), (got - ref).abs().max().item()
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("n,V", [(5, 1), (9, 7), (33, 1000), (17, 4099), (6, 32000), (4, 151936)])
+@pytest.mark.parametrize("which", ["both", "logprob", "entropy"])
+def test_gradient_matches_torch_autograd(dev, dtype, n, V, which):
+    g = torch.Generator(device=dev).manual_seed(n * 100 + V)
+    x = (torch.randn(n, V, generator=g, device=dev) * 3).to(dtype)
+    lab = torch.randint(0, V, (n,), generator=g, device=dev)
+    temp = torch.rand(n, generator=g, device=dev) + 0.5
+    w_lp = torch.randn(n, generator=g, device=dev) if which in ("both", "logprob") else None
+    w_h = torch.randn(n, generator=g, device=dev) if which in ("both", "entropy") else None
+    for t in (None, temp):
+        _compare(_ours(x, lab, t, w_lp, w_h), _reference_grad(x, lab, t, w_lp, w_h), dtype)
+
+
+def test_leading_dims_strided_rows_and_separate_functions(dev):
+    g = torch.Generator(device=dev).manual_seed(8)
+    base = torch.randn(3, 4, 1030, generator=g, device=dev)
+    lab = torch.randint(0, 1021, (3, 4), generator=g, device=dev)
+    w1 = torch.randn(3, 4, generator=g, device=dev)
+    w2 = torch.randn(3, 4, generator=g, device=dev)
+    # a strided, misaligned view: rows start 3 elements into each 1030-element row
+    leaf = base.clone().requires_grad_(True)
+    view = leaf[..., 3:1024]
+    lp = vf.logprobs_from_logits(view, lab, inplace_backward=False)
+    h = vf.entropy_from_logits(view)
+    ((lp * w1).sum() + (h * w2).sum()).backward()
+    ref_leaf = base.clone().requires_grad_(True)
+    rlp = scoring.logprobs_from_logits(ref_leaf[..., 3:1024], lab)
+    rh = scoring.entropy_from_logits(ref_leaf[..., 3:1024])
+    ((rlp * w1).sum() + (rh * w2).sum()).backward()
+    assert (leaf.grad - ref_leaf.grad).abs().max().item() <= 1.6e-5
+    assert leaf.grad[..., :3].abs().max().item() == 0
+
+
+def test_inplace_backward_writes_over_the_logits(dev):
+    g = torch.Generator(device=dev).manual_seed(9)
+    leaf = (torch.randn(64, 5000, generator=g, device=dev)).requires_grad_(True)
+    lab = torch.randint(0, 5000, (64,), generator=g, device=dev)
+    w = torch.randn(64, generator=g, device=dev)
+    z = leaf * 1.0                      # a non-leaf tensor, like `logits / temperature` in the engine
+    ptr = z.data_ptr()
+    lp = vf.logprobs_from_logits(z, lab)            # inplace_backward=True by default, as in the reference
+    (lp * w).sum().backward()
+    ref = _reference_grad(leaf, lab, None, w, None)
+    assert (leaf.grad - ref).abs().max().item() <= 1.6e-5
+    assert z.data_ptr() == ptr and (z.detach() - ref).abs().max().item() <= 1.6e-5   # z now holds its own gradient
+    # a leaf is never overwritten
+    leaf2 = leaf.detach().clone().requires_grad_(True)
+    keep = leaf2.detach().clone()
+    (vf.logprobs_from_logits(leaf2, lab) * w).sum().backward()
+    assert torch.equal(leaf2.detach(), keep) and (leaf2.grad - ref).abs().max().item() <= 1.6e-5
+
+
+def test_minus_inf_logits_and_unused_outputs(dev):
+    x = torch.randn(4, 300, device=dev)
+    x[0, :50] = float("-inf")
+    lab = torch.tensor([100, 1, 2, 3], device=dev)
+    xo = x.clone().requires_grad_(True)
+    lp, h = vf.fused_logprob_entropy(xo, lab)
+    lp.sum().backward()                      # entropy unused: its gradient is absent, not zero-filled
+    ref = _reference_grad(x, lab, None, torch.ones(4, device=dev), None)
+    assert torch.isfinite(xo.grad).all() and (xo.grad - ref).abs().max().item() <= 4e-6
+    assert xo.grad[0, :50].abs().max().item() == 0
+    # no grad requested: plain forward, no graph
+    with torch.no_grad():
+        lp2, _ = vf.fused_logprob_entropy(xo, lab)
+    assert not lp2.requires_grad and torch.equal(lp2, lp.detach())
+
+
+def test_full_vocab_bf16_c3_shape_slice(dev):
+    """256 rows of the c3 shape (V = 151936 bf16), both gradients, temperature 0.7."""
+    g = torch.Generator(device=dev).manual_seed(12)
+    n, V = 256, 151936
+    x = (torch.randn(n, V, generator=g, device=dev) * 3).bfloat16()
+    lab = torch.randint(0, V, (n,), generator=g, device=dev)
+    temp = torch.full((n,), 0.7, device=dev)
+    w1 = torch.randn(n, generator=g, device=dev)
+    w2 = torch.randn(n, generator=g, device=dev)
+    _compare(_ours(x, lab, temp, w1, w2), _reference_grad(x, lab, temp, w1, w2).bfloat16(), torch.bfloat16)

@@ -29,7 +29,7 @@ def test_split_path_matches_oracle_and_single_pass(dev, dtype, n, V):
             # a different summation tree, same numbers to fp32 rounding
             assert (got[0] - one[0]).abs().max().item() <= 4e-6
             assert (got[1] - one[1]).abs().max().item() <= 4e-6
-            assert ((got[2] - one[2]).abs() <= 1e-6 * one[2].abs() + 1e-12).all()
+            assert ((got[2] - one[2]).abs() <= 4e-6 * one[2].abs() + 1e-12).all()
     auto = vf.fused_logprob_entropy(x, lab)       # what the wrapper picks by itself
     assert_scores_match(auto[0], auto[1], x, lab, None, cpu_torch=False)
 

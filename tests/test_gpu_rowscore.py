@@ -191,14 +191,17 @@ def test_label_out_of_range_raises(dev):
     assert torch.isnan(lp[2]) and torch.isfinite(lp[[0, 1, 3]]).all()
 
 
-def test_rejects_cpu_and_grad_inputs(dev):
+def test_rejects_cpu_and_unsupported_inputs(dev):
     with pytest.raises(RuntimeError, match="no CPU implementation"):
         vf.logprobs_from_logits(torch.randn(2, 10), torch.zeros(2, dtype=torch.long))
     x = torch.randn(2, 10, device=dev, requires_grad=True)
-    with pytest.raises(NotImplementedError):
-        vf.entropy_from_logits(x)
+    assert vf.entropy_from_logits(x).requires_grad          # differentiable when the logits need it
     with torch.no_grad():
-        vf.entropy_from_logits(x)
+        assert not vf.entropy_from_logits(x).requires_grad
+    from verl_amd import spec_rl
+    with pytest.raises(NotImplementedError):                 # the verify step is forward-only
+        spec_rl.fused_score_verify(x, torch.zeros(2, dtype=torch.long, device=dev), torch.zeros(2, device=dev), seed=0,
+                                   cu_seqlens=torch.tensor([0, 2], device=dev))
     with pytest.raises(TypeError):
         vf.entropy_from_logits(torch.randn(2, 10, device=dev).half())
 

@@ -106,7 +106,7 @@ def test_install_patches_module_and_bound_names(fake_verl):
     assert tf.logprobs_from_logits.__verl_amd_original__ is orig
     assert inst.install() == []  # second call is a no-op
 
-    # CPU tensors, unsupported dtypes and tensors that need grad go to verl's own function
+    # CPU tensors and unsupported dtypes go to verl's own function
     x = torch.randn(2, 5)
     assert tf.logprobs_from_logits(x, torch.zeros(2, dtype=torch.long)) == ("verl", "logprobs_from_logits")
     assert eng.logprobs_from_logits(x, torch.zeros(2, dtype=torch.long), inplace_backward=False) == ("verl", "logprobs_from_logits")

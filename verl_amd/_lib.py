@@ -37,8 +37,9 @@ _F32 = _c.c_float
 
 # name -> (restype, argtypes); mirrors include/vrl.h one to one.
 SIGNATURES = {
-    "vrl_rowscore": (_INT, [_P, _INT, _I64, _I64, _I64, _P, _P, _P, _P, _P, _P, _P]),
-    "vrl_rowscore_split": (_INT, [_P, _INT, _I64, _I64, _I64, _P, _P, _P, _P, _P, _P, _INT, _P, _P]),
+    "vrl_rowscore": (_INT, [_P, _INT, _I64, _I64, _I64, _P, _P, _P, _P, _P, _P, _P, _P]),
+    "vrl_rowscore_split": (_INT, [_P, _INT, _I64, _I64, _I64, _P, _P, _P, _P, _P, _P, _P, _INT, _P, _P]),
+    "vrl_rowscore_backward": (_INT, [_P, _INT, _I64, _I64, _I64, _P, _P, _P, _P, _P, _P, _P, _I64, _P]),
     "vrl_rowscore_split_plan": (_INT, [_INT, _I64, _I64]),
     "vrl_response_slice": (_INT, [_P, _P, _P, _I64, _I64, _P, _P, _P]),
     "vrl_spec_verify": (
@@ -48,7 +49,7 @@ SIGNATURES = {
     "vrl_truncate_draft": (_INT, [_P, _P, _P, _I64, _I64, _P, _I64, _P, _P, _P]),
     "vrl_fused_score_verify": (
         _INT,
-        [_P, _INT, _I64, _I64, _I64, _P, _P, _P, _P, _P, _P]
+        [_P, _INT, _I64, _I64, _I64, _P, _P, _P, _P, _P, _P, _P]
         + [_P, _P, _P, _P, _I64, _I64, _F32, _F32, _P, _P, _P, _P, _P, _I64, _P, _P, _P],
     ),
     "vrl_strerror": (_c.c_char_p, [_INT]),

@@ -1,0 +1,162 @@
+// Backward of the row op: one read of the logits, one write of their gradient.
+//
+// With z = x / T, p = softmax(z), log p_v = z_v - lse, H the row's entropy and
+// (g_l, g_h) the incoming gradients of the label log-prob and of the entropy,
+//   d/dz_v = g_l * (1[v == label] - p_v) - g_h * p_v * (log p_v + H)
+//   d/dx_v = (d/dz_v) / T
+// which is the closed form the reference states at
+// verl/utils/experimental/torch_functional.py:66-79. In the log2 domain:
+//   u = fma(x, c, -lse*log2e);  p = v_exp_f32(u);  dx = p * fma(u, a, b)  (+ g_l/T at the label)
+// with a = -g_h*ln2/T and b = -(g_l + g_h*H)/T constant over the row.
+// lse and H come from the forward pass. The gradient has the logits' dtype and
+// may be written over the logits themselves (every element is read and then
+// written by the same lane).
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "rowscore_kernels.h"
+
+namespace vrl {
+
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+
+constexpr float kLn2f = 0.69314718055994530942f;
+
+template <int DT>
+struct ElemOut;
+
+template <>
+struct ElemOut<0> {
+  __device__ static __forceinline__ u32x4 pack(const float* y) {
+    u32x4 v;
+    v.x = __float_as_uint(y[0]);
+    v.y = __float_as_uint(y[1]);
+    v.z = __float_as_uint(y[2]);
+    v.w = __float_as_uint(y[3]);
+    return v;
+  }
+  __device__ static __forceinline__ void store1(char* rowp, int64_t idx, float y) {
+    reinterpret_cast<float*>(rowp)[idx] = y;
+  }
+};
+
+template <>
+struct ElemOut<1> {
+  __device__ static __forceinline__ uint32_t pack2(float lo, float hi) {
+    const f32x2 v = {lo, hi};
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2));  // round to nearest even
+  }
+  __device__ static __forceinline__ u32x4 pack(const float* y) {
+    u32x4 v;
+    v.x = pack2(y[0], y[1]);
+    v.y = pack2(y[2], y[3]);
+    v.z = pack2(y[4], y[5]);
+    v.w = pack2(y[6], y[7]);
+    return v;
+  }
+  __device__ static __forceinline__ void store1(char* rowp, int64_t idx, float y) {
+    reinterpret_cast<uint16_t*>(rowp)[idx] = static_cast<uint16_t>(pack2(y, 0.f) & 0xffffu);
+  }
+};
+
+struct RowGrad {
+  float c;     // log2e / T
+  float lse2;  // lse * log2e
+  float a;     // -g_h * ln2 / T
+  float b;     // -(g_l + g_h * H) / T
+  float lab;   // g_l / T, added at the label
+  __device__ __forceinline__ float operator()(float x) const {
+    const float u = __builtin_fmaf(x, c, -lse2);
+    const float p = hw_exp2(u);
+    // p == 0 (a -inf logit, or one far below the row's bulk) has zero gradient; without the
+    // select, u = -inf would give 0 * inf.
+    return (p == 0.f) ? 0.f : p * __builtin_fmaf(u, a, b);
+  }
+};
+
+// grid.x = n_rows, block = WAVES*64.
+template <int DT, int WAVES, int U>
+__global__ __launch_bounds__(WAVES * 64) void rowscore_backward_kernel(
+    const void* logits, int64_t vocab, int64_t row_stride, const int64_t* __restrict__ labels,
+    const float* __restrict__ temperature, const float* __restrict__ lse, const float* __restrict__ entropy,
+    const float* __restrict__ g_logprob, const float* __restrict__ g_entropy, void* dlogits,
+    int64_t d_row_stride) {
+  using E = Elem<DT>;
+  using O = ElemOut<DT>;
+  constexpr int NTHR = WAVES * 64;
+  constexpr int PV = E::kPerVec;
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = tid >> 6;
+  const int64_t row = blockIdx.x;
+  const char* rowp = static_cast<const char*>(logits) + row * row_stride * E::kBytes;
+  char* outp = static_cast<char*>(dlogits) + row * d_row_stride * E::kBytes;
+
+  float T = 1.f;
+  if (temperature != nullptr) {
+    T = temperature[row];
+    T = (T < kMinTemperature) ? kMinTemperature : T;
+  }
+  const float rT = 1.0f / T;
+  const float gl = (g_logprob != nullptr) ? g_logprob[row] : 0.f;
+  const float gh = (g_entropy != nullptr) ? g_entropy[row] : 0.f;
+  const float H = (g_entropy != nullptr) ? entropy[row] : 0.f;
+  RowGrad f;
+  f.c = kLog2e * rT;
+  f.lse2 = lse[row] * kLog2e;
+  f.a = -(gh * kLn2f) * rT;
+  f.b = -(gl + gh * H) * rT;
+  f.lab = gl * rT;
+  // a label outside [0, vocab) was reported by the forward pass; here it simply matches nothing
+  const int64_t label = (g_logprob != nullptr) ? labels[row] : -1;
+
+  // Vector path only when the input and output rows have the same 16-byte phase.
+  const uintptr_t ain = reinterpret_cast<uintptr_t>(rowp);
+  const uintptr_t aout = reinterpret_cast<uintptr_t>(outp);
+  const bool same_phase = ((ain ^ aout) & 15u) == 0;
+  int64_t head = same_phase ? static_cast<int64_t>(((16u - (ain & 15u)) & 15u) / E::kBytes) : vocab;
+  if (head > vocab) head = vocab;
+  const int64_t nvec = (vocab - head) / PV;
+  const int64_t tail0 = head + nvec * PV;
+  const u32x4* vin = reinterpret_cast<const u32x4*>(rowp + head * E::kBytes);
+  u32x4* vout = reinterpret_cast<u32x4*>(outp + head * E::kBytes);
+
+  auto do_vec = [&](int64_t k, const u32x4& v) {
+    float x[PV];
+    E::unpack(v, x);
+#pragma unroll
+    for (int i = 0; i < PV; ++i) x[i] = f(x[i]);
+    const int64_t rel = label - (head + k * PV);
+    if (rel >= 0 && rel < PV) {
+#pragma unroll
+      for (int i = 0; i < PV; ++i)
+        if (i == rel) x[i] += f.lab;
+    }
+    __builtin_nontemporal_store(O::pack(x), vout + k);
+  };
+
+  constexpr int64_t kBatchVecs = static_cast<int64_t>(NTHR) * U;
+  const int64_t nfull = nvec / kBatchVecs;
+  for (int64_t j = 0; j < nfull; ++j) {
+    const int64_t k0 = (j * WAVES + wave) * (U * 64) + lane;
+    u32x4 v[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) v[u] = __builtin_nontemporal_load(vin + k0 + u * 64);
+#pragma unroll
+    for (int u = 0; u < U; ++u) do_vec(k0 + u * 64, v[u]);
+  }
+  for (int64_t k = nfull * kBatchVecs + tid; k < nvec; k += NTHR) do_vec(k, __builtin_nontemporal_load(vin + k));
+
+  // scalars: [0, head) and [tail0, vocab); with mismatched phases that is the whole row
+  for (int64_t i = tid; i < head + (vocab - tail0); i += NTHR) {
+    const int64_t idx = (i < head) ? i : tail0 + (i - head);
+    float y = f(E::load1(rowp, idx));
+    if (idx == label) y += f.lab;
+    O::store1(outp, idx, y);
+  }
+}
+
+}  // namespace vrl

@@ -315,18 +315,20 @@ __device__ __forceinline__ float load_label_logit(const char* rowp, const int64_
 template <bool EXACT, bool WANT_Q>
 __device__ __forceinline__ void finalize_row(const Part& w, float xl, bool label_ok, const Scale<EXACT>& sc,
                                              int64_t row, float* out_logprob, float* out_entropy,
-                                             float* out_sum_pi_sq, int32_t* err_flag) {
-  float lp, H, sps;
+                                             float* out_sum_pi_sq, float* out_lse, int32_t* err_flag) {
+  float lp, H, sps, lse;
   if (w.m == neg_inf()) {
     // empty row or every logit -inf: logsumexp = -inf, x - (-inf) and softmax are NaN in torch
     lp = quiet_nan();
     H = quiet_nan();
     sps = quiet_nan();
+    lse = neg_inf();
   } else if (w.m == pos_inf()) {
     // a +inf logit: logsumexp = +inf
     lp = (sc.pre(xl) * sc.c == pos_inf()) ? quiet_nan() : neg_inf();
     H = quiet_nan();
     sps = quiet_nan();
+    lse = pos_inf();
   } else {
     const double S = static_cast<double>(w.s);
     const double l2s = log2(S);
@@ -334,6 +336,7 @@ __device__ __forceinline__ void finalize_row(const Part& w, float xl, bool label
     lp = static_cast<float>(kLn2d * (yl - l2s));
     H = static_cast<float>(kLn2d * (l2s - static_cast<double>(w.t) / S));
     sps = static_cast<float>(static_cast<double>(w.q) / (S * S));
+    lse = static_cast<float>(kLn2d * (static_cast<double>(w.m) + l2s));
   }
   if (out_logprob != nullptr) {
     if (!label_ok) {
@@ -343,6 +346,7 @@ __device__ __forceinline__ void finalize_row(const Part& w, float xl, bool label
     out_logprob[row] = lp;
   }
   if (out_entropy != nullptr) out_entropy[row] = H;
+  if (out_lse != nullptr) out_lse[row] = lse;
   if constexpr (WANT_Q) {
     if (out_sum_pi_sq != nullptr) out_sum_pi_sq[row] = sps;
   }
@@ -355,7 +359,7 @@ __global__ __launch_bounds__(WAVES * 64) void rowscore_kernel(
     const void* __restrict__ logits, int64_t vocab, int64_t row_stride,
     const int64_t* __restrict__ labels, const float* __restrict__ temperature,
     float* __restrict__ out_logprob, float* __restrict__ out_entropy,
-    float* __restrict__ out_sum_pi_sq, int32_t* err_flag) {
+    float* __restrict__ out_sum_pi_sq, float* __restrict__ out_lse, int32_t* err_flag) {
   const int64_t row = blockIdx.x;
   const char* rowp = static_cast<const char*>(logits) + row * row_stride * Elem<DT>::kBytes;
   const Scale<EXACT> sc = make_scale<EXACT>(temperature, row);
@@ -364,7 +368,7 @@ __global__ __launch_bounds__(WAVES * 64) void rowscore_kernel(
   if (out_logprob != nullptr && threadIdx.x == 0) xl = load_label_logit<DT>(rowp, labels, row, vocab, label_ok);
   const Part w = block_reduce_range<DT, WAVES, U, EXACT, NT, WANT_Q>(rowp, 0, vocab, sc);
   if (threadIdx.x == 0)
-    finalize_row<EXACT, WANT_Q>(w, xl, label_ok, sc, row, out_logprob, out_entropy, out_sum_pi_sq, err_flag);
+    finalize_row<EXACT, WANT_Q>(w, xl, label_ok, sc, row, out_logprob, out_entropy, out_sum_pi_sq, out_lse, err_flag);
 }
 
 // ---- few rows: several workgroups per row ------------------------------------
@@ -400,7 +404,7 @@ __global__ __launch_bounds__(64) void rowscore_merge_kernel(
     const void* __restrict__ logits, int64_t n_rows, int64_t vocab, int64_t row_stride,
     const int64_t* __restrict__ labels, const float* __restrict__ temperature, int n_splits,
     const float* __restrict__ partials, float* __restrict__ out_logprob, float* __restrict__ out_entropy,
-    float* __restrict__ out_sum_pi_sq, int32_t* err_flag) {
+    float* __restrict__ out_sum_pi_sq, float* __restrict__ out_lse, int32_t* err_flag) {
   const int64_t row = static_cast<int64_t>(blockIdx.x) * 64 + threadIdx.x;
   if (row >= n_rows) return;
   const char* rowp = static_cast<const char*>(logits) + row * row_stride * Elem<DT>::kBytes;
@@ -427,7 +431,7 @@ __global__ __launch_bounds__(64) void rowscore_merge_kernel(
     w.t += p.t;
     w.q += p.q;
   }
-  finalize_row<EXACT, WANT_Q>(w, xl, label_ok, sc, row, out_logprob, out_entropy, out_sum_pi_sq, err_flag);
+  finalize_row<EXACT, WANT_Q>(w, xl, label_ok, sc, row, out_logprob, out_entropy, out_sum_pi_sq, out_lse, err_flag);
 }
 
 }  // namespace vrl

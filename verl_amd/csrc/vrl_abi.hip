@@ -7,6 +7,7 @@
 #include <stdint.h>
 #include <string.h>
 
+#include "backward_kernels.h"
 #include "layout_kernels.h"
 #include "rowscore_kernels.h"
 #include "verify_kernels.h"
@@ -47,20 +48,25 @@ struct RowShape<VRL_BF16> {
 constexpr int kSplitWaves = 4;
 constexpr int kSplitUnroll = 2;
 constexpr int kMaxSplits = 64;
+// Shape of the backward workgroup (one per row): wavefronts, 128-bit loads/stores per lane and batch.
+constexpr int kBackwardWaves = 4;
+constexpr int kBackwardUnroll = 4;
 
 int check_rowscore(const void* logits, int dtype, int64_t n_rows, int64_t vocab, int64_t row_stride,
                    const int64_t* labels, const float* temperature, const float* out_logprob,
-                   const float* out_entropy, const float* out_sum_pi_sq, const int32_t* err_flag) {
+                   const float* out_entropy, const float* out_sum_pi_sq, const float* out_lse,
+                   const int32_t* err_flag) {
   if (dtype != VRL_F32 && dtype != VRL_BF16) return VRL_ERR_DTYPE;
   if (n_rows < 0 || vocab <= 0 || row_stride < vocab || n_rows > kMaxGrid) return VRL_ERR_SHAPE;
-  if (out_logprob == nullptr && out_entropy == nullptr && out_sum_pi_sq == nullptr) return VRL_ERR_ARG;
+  if (out_logprob == nullptr && out_entropy == nullptr && out_sum_pi_sq == nullptr && out_lse == nullptr)
+    return VRL_ERR_ARG;
   if (n_rows == 0) return VRL_OK;
   if (logits == nullptr) return VRL_ERR_NULL;
   if (out_logprob != nullptr && (labels == nullptr || err_flag == nullptr)) return VRL_ERR_NULL;
   const uintptr_t esize = (dtype == VRL_F32) ? 4 : 2;
   if (!aligned(logits, esize) || !aligned(labels, 8) || !aligned(temperature, 4) ||
       !aligned(out_logprob, 4) || !aligned(out_entropy, 4) || !aligned(out_sum_pi_sq, 4) ||
-      !aligned(err_flag, 4))
+      !aligned(out_lse, 4) || !aligned(err_flag, 4))
     return VRL_ERR_ALIGN;
   return VRL_OK;
 }
@@ -73,6 +79,7 @@ struct RowArgs {
   float* out_logprob;
   float* out_entropy;
   float* out_sum_pi_sq;
+  float* out_lse;
   int32_t* err_flag;
   int n_splits;     // 1: one workgroup per row
   float* partials;  // split path only
@@ -93,7 +100,7 @@ void launch_rows(const RowArgs& a) {
     vrl::rowscore_kernel<DT, W, U, EXACT, true, WANT_Q>
         <<<dim3(static_cast<unsigned>(a.n_rows)), dim3(W * 64), 0, a.stream>>>(
             a.logits, a.vocab, a.row_stride, a.labels, a.temperature, a.out_logprob, a.out_entropy,
-            a.out_sum_pi_sq, a.err_flag);
+            a.out_sum_pi_sq, a.out_lse, a.err_flag);
     return;
   }
   const int64_t slice = split_slice_elems(a.vocab, a.n_splits, DT);
@@ -103,7 +110,7 @@ void launch_rows(const RowArgs& a) {
   vrl::rowscore_merge_kernel<DT, EXACT, WANT_Q>
       <<<dim3(static_cast<unsigned>((a.n_rows + 63) / 64)), dim3(64), 0, a.stream>>>(
           a.logits, a.n_rows, a.vocab, a.row_stride, a.labels, a.temperature, a.n_splits, a.partials,
-          a.out_logprob, a.out_entropy, a.out_sum_pi_sq, a.err_flag);
+          a.out_logprob, a.out_entropy, a.out_sum_pi_sq, a.out_lse, a.err_flag);
 }
 
 template <int DT, bool EXACT>
@@ -163,12 +170,13 @@ extern "C" {
 
 int vrl_rowscore(const void* logits, int dtype, int64_t n_rows, int64_t vocab, int64_t row_stride,
                  const int64_t* labels, const float* temperature, float* out_logprob,
-                 float* out_entropy, float* out_sum_pi_sq, int32_t* err_flag, void* stream) {
+                 float* out_entropy, float* out_sum_pi_sq, float* out_lse, int32_t* err_flag,
+                 void* stream) {
   const int st = check_rowscore(logits, dtype, n_rows, vocab, row_stride, labels, temperature,
-                                out_logprob, out_entropy, out_sum_pi_sq, err_flag);
+                                out_logprob, out_entropy, out_sum_pi_sq, out_lse, err_flag);
   if (st != VRL_OK || n_rows == 0) return st;
   const RowArgs a{logits, n_rows, vocab, row_stride, labels, temperature, out_logprob, out_entropy,
-                  out_sum_pi_sq, err_flag, 1, nullptr, static_cast<hipStream_t>(stream)};
+                  out_sum_pi_sq, out_lse, err_flag, 1, nullptr, static_cast<hipStream_t>(stream)};
   launch_rows_any(dtype, a);
   return launch_status();
 }
@@ -190,10 +198,10 @@ int vrl_rowscore_split_plan(int dtype, int64_t n_rows, int64_t vocab) {
 
 int vrl_rowscore_split(const void* logits, int dtype, int64_t n_rows, int64_t vocab, int64_t row_stride,
                        const int64_t* labels, const float* temperature, float* out_logprob,
-                       float* out_entropy, float* out_sum_pi_sq, int32_t* err_flag, int n_splits,
-                       float* partials, void* stream) {
+                       float* out_entropy, float* out_sum_pi_sq, float* out_lse, int32_t* err_flag,
+                       int n_splits, float* partials, void* stream) {
   const int st = check_rowscore(logits, dtype, n_rows, vocab, row_stride, labels, temperature,
-                                out_logprob, out_entropy, out_sum_pi_sq, err_flag);
+                                out_logprob, out_entropy, out_sum_pi_sq, out_lse, err_flag);
   if (st != VRL_OK) return st;
   if (n_splits < 1 || n_splits > kMaxSplits) return VRL_ERR_ARG;
   if (n_rows * n_splits > kMaxGrid) return VRL_ERR_SHAPE;
@@ -201,8 +209,35 @@ int vrl_rowscore_split(const void* logits, int dtype, int64_t n_rows, int64_t vo
   if (n_splits > 1 && partials == nullptr) return VRL_ERR_NULL;
   if (!aligned(partials, 4)) return VRL_ERR_ALIGN;
   const RowArgs a{logits, n_rows, vocab, row_stride, labels, temperature, out_logprob, out_entropy,
-                  out_sum_pi_sq, err_flag, n_splits, partials, static_cast<hipStream_t>(stream)};
+                  out_sum_pi_sq, out_lse, err_flag, n_splits, partials, static_cast<hipStream_t>(stream)};
   launch_rows_any(dtype, a);
+  return launch_status();
+}
+
+int vrl_rowscore_backward(const void* logits, int dtype, int64_t n_rows, int64_t vocab, int64_t row_stride,
+                          const int64_t* labels, const float* temperature, const float* lse,
+                          const float* entropy, const float* g_logprob, const float* g_entropy,
+                          void* dlogits, int64_t d_row_stride, void* stream) {
+  if (dtype != VRL_F32 && dtype != VRL_BF16) return VRL_ERR_DTYPE;
+  if (n_rows < 0 || vocab <= 0 || row_stride < vocab || d_row_stride < vocab || n_rows > kMaxGrid)
+    return VRL_ERR_SHAPE;
+  if (g_logprob == nullptr && g_entropy == nullptr) return VRL_ERR_ARG;
+  if (n_rows == 0) return VRL_OK;
+  if (logits == nullptr || dlogits == nullptr || lse == nullptr) return VRL_ERR_NULL;
+  if (g_logprob != nullptr && labels == nullptr) return VRL_ERR_NULL;
+  if (g_entropy != nullptr && entropy == nullptr) return VRL_ERR_NULL;
+  const uintptr_t esize = (dtype == VRL_F32) ? 4 : 2;
+  if (!aligned(logits, esize) || !aligned(dlogits, esize) || !aligned(labels, 8) || !aligned(temperature, 4) ||
+      !aligned(lse, 4) || !aligned(entropy, 4) || !aligned(g_logprob, 4) || !aligned(g_entropy, 4))
+    return VRL_ERR_ALIGN;
+  const dim3 grid(static_cast<unsigned>(n_rows));
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  if (dtype == VRL_F32)
+    vrl::rowscore_backward_kernel<VRL_F32, kBackwardWaves, kBackwardUnroll><<<grid, dim3(kBackwardWaves * 64), 0, s>>>(
+        logits, vocab, row_stride, labels, temperature, lse, entropy, g_logprob, g_entropy, dlogits, d_row_stride);
+  else
+    vrl::rowscore_backward_kernel<VRL_BF16, kBackwardWaves, kBackwardUnroll><<<grid, dim3(kBackwardWaves * 64), 0, s>>>(
+        logits, vocab, row_stride, labels, temperature, lse, entropy, g_logprob, g_entropy, dlogits, d_row_stride);
   return launch_status();
 }
 
@@ -263,7 +298,7 @@ int vrl_truncate_draft(const int64_t* draft_ids, const uint8_t* mask, const int6
 
 int vrl_fused_score_verify(const void* logits, int dtype, int64_t n_rows, int64_t vocab,
                            int64_t row_stride, const int64_t* labels, const float* temperature,
-                           float* out_logprob, float* out_entropy, float* out_sum_pi_sq,
+                           float* out_logprob, float* out_entropy, float* out_sum_pi_sq, float* out_lse,
                            int32_t* err_flag, const float* logp_old, const float* log_u, const uint8_t* mask,
                            const int64_t* cu_seqlens, int64_t B, int64_t T, float thresh_offset,
                            float near_eps, uint8_t* accept, int32_t* first_reject,
@@ -272,14 +307,14 @@ int vrl_fused_score_verify(const void* logits, int dtype, int64_t n_rows, int64_
   // Check both halves before anything is enqueued.
   if (out_logprob == nullptr && n_rows > 0) return VRL_ERR_NULL;
   int st = check_rowscore(logits, dtype, n_rows, vocab, row_stride, labels, temperature, out_logprob,
-                          out_entropy, out_sum_pi_sq, err_flag);
+                          out_entropy, out_sum_pi_sq, out_lse, err_flag);
   if (st != VRL_OK) return st;
   st = check_verify(out_logprob, logp_old, log_u, mask, cu_seqlens, B, T, accept, first_reject,
                     prefix_len, near_count, draft_ids, out_ids, out_mask);
   if (st != VRL_OK) return st;
   if (cu_seqlens == nullptr && n_rows != B * T) return VRL_ERR_SHAPE;
   st = vrl_rowscore(logits, dtype, n_rows, vocab, row_stride, labels, temperature, out_logprob,
-                    out_entropy, out_sum_pi_sq, err_flag, stream);
+                    out_entropy, out_sum_pi_sq, out_lse, err_flag, stream);
   if (st != VRL_OK) return st;
   return vrl_spec_verify(out_logprob, logp_old, log_u, mask, cu_seqlens, B, T, thresh_offset, near_eps,
                          accept, first_reject, prefix_len, near_count, draft_ids, pad_id, out_ids,

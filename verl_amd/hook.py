@@ -10,9 +10,9 @@ verl/workers/engine/fsdp/transformer_impl.py:66 and siblings; the reference's
 own tests patch exactly that bound name,
 tests/workers/test_distillation_topk_symmetry_on_cpu.py:143-146).
 
-A replaced function sends GPU tensors of a supported dtype under no_grad to
-the HIP kernel. Anything else (CPU tensors on the driver, fp16/fp64, tensors
-that need a backward) is handed to the function it replaced, i.e. verl's own
+A replaced function sends GPU tensors of a supported dtype to the HIP kernels
+(forward, and backward when the logits need a gradient). Anything else (CPU
+tensors on the driver, fp16/fp64) is handed to the function it replaced, i.e. verl's own
 code, and counted in ``stats()``: this package adds no second implementation.
 """
 
@@ -49,7 +49,6 @@ def _eligible(logits) -> bool:
         and logits.dtype in (torch.float32, torch.bfloat16)
         and logits.dim() >= 1
         and logits.shape[-1] > 0
-        and not (torch.is_grad_enabled() and logits.requires_grad)
     )
 
 

@@ -239,6 +239,9 @@ def fused_score_verify(
     (packed); every per-token tensor has the logits' leading shape.
     """
     _check_logits(logits, "fused_score_verify")
+    if torch.is_grad_enabled() and logits.requires_grad:
+        raise NotImplementedError("fused_score_verify is a forward-only step (verification happens under no_grad); "
+                                  "use fused_logprob_entropy for the differentiable scores")
     dev = logits.device
     lead = tuple(logits.shape[:-1])
     V = logits.shape[-1]
@@ -265,7 +268,7 @@ def fused_score_verify(
         stream = torch.cuda.current_stream(dev).cuda_stream
         st = lib.vrl_fused_score_verify(
             x.data_ptr(), _DTYPE_CODES[x.dtype], n, V, x.stride(0) if n > 1 else V, lab.data_ptr(), _ptr(temp),
-            out_lp.data_ptr(), out_h.data_ptr(), None, flag.data_ptr(),
+            out_lp.data_ptr(), out_h.data_ptr(), None, None, flag.data_ptr(),
             lo.data_ptr(), lu.data_ptr(), _ptr(m8), _ptr(cu), B, T, off, float(near_eps),
             accept.data_ptr(), first.data_ptr(), prefix.data_ptr(), near.data_ptr(),
             _ptr(ids), int(pad_id), _ptr(out_ids), _ptr(out_mask), stream,

@@ -11,7 +11,10 @@ Differences from the reference that a caller can observe:
     returns the input dtype, :199-206; its flash-attn branch returns fp32);
   * a label outside [0, vocab) raises IndexError after the kernel ran
     (torch.gather device-asserts);
-  * inputs that require grad raise NotImplementedError (forward-only).
+  * the sum of squared probabilities is not differentiable here (the reference
+    computes it under no_grad for the optimal-baseline estimator only).
+Log-probs and entropy are differentiable with respect to the logits through one
+HIP backward kernel (vrl_rowscore_backward).
 """
 
 from __future__ import annotations
@@ -51,11 +54,12 @@ def _check_logits(logits: torch.Tensor, what: str) -> None:
         raise TypeError(f"{what}: logits dtype {logits.dtype} is not supported (float32 and bfloat16 are)")
     if logits.dim() < 1 or logits.shape[-1] == 0:
         raise ValueError(f"{what}: logits need a non-empty last (vocab) dimension, got shape {tuple(logits.shape)}")
-    if torch.is_grad_enabled() and logits.requires_grad:
-        raise NotImplementedError(
-            f"{what}: logits require grad, but this is the forward-only scoring path "
-            "(call it under torch.no_grad(), as the reference's compute_log_prob does)"
-        )
+
+
+def _is_view_safe(logits: torch.Tensor) -> bool:
+    """True when _rows_2d returns a view of ``logits`` (so writing a gradient over it is what the caller asked
+    for) and the tensor is not a leaf that autograd will want to read again."""
+    return logits.is_contiguous() and not logits.is_leaf
 
 
 def _rows_2d(logits: torch.Tensor) -> torch.Tensor:
@@ -85,6 +89,75 @@ def _temperature_rows(temperature, lead_shape, n_rows, device) -> Optional[torch
     return t.reshape(n_rows).contiguous()
 
 
+def _forward_2d(x, lab, temp, want_logprob, want_entropy, want_sum_pi_sq, want_lse, n_splits):
+    """Launch the forward kernels on (N, V) rows; returns (logprob, entropy, sum_pi_sq, lse, flag), None where not asked."""
+    n, V = x.shape
+    dev = x.device
+    f32 = dict(dtype=torch.float32, device=dev)
+    out_lp = torch.empty(n, **f32) if want_logprob else None
+    out_h = torch.empty(n, **f32) if want_entropy else None
+    out_q = torch.empty(n, **f32) if want_sum_pi_sq else None
+    out_lse = torch.empty(n, **f32) if want_lse else None
+    flag = torch.zeros(1, dtype=torch.int32, device=dev) if want_logprob else None
+    if n == 0:
+        return out_lp, out_h, out_q, out_lse, flag
+    lib = _lib.load()
+    dt = _DTYPE_CODES[x.dtype]
+    stride = x.stride(0) if n > 1 else V
+    splits = lib.vrl_rowscore_split_plan(dt, n, V) if n_splits is None else int(n_splits)
+    with torch.cuda.device(dev):
+        stream = torch.cuda.current_stream(dev).cuda_stream
+        if splits > 1:
+            partials = torch.empty(n * splits * 4, **f32)
+            st = lib.vrl_rowscore_split(
+                x.data_ptr(), dt, n, V, stride, _ptr(lab), _ptr(temp), _ptr(out_lp), _ptr(out_h), _ptr(out_q),
+                _ptr(out_lse), _ptr(flag), splits, partials.data_ptr(), stream,
+            )
+            _lib.check("vrl_rowscore_split", st)
+        else:
+            st = lib.vrl_rowscore(
+                x.data_ptr(), dt, n, V, stride, _ptr(lab), _ptr(temp), _ptr(out_lp), _ptr(out_h), _ptr(out_q),
+                _ptr(out_lse), _ptr(flag), stream,
+            )
+            _lib.check("vrl_rowscore", st)
+    return out_lp, out_h, out_q, out_lse, flag
+
+
+class _RowScoreFunction(torch.autograd.Function):
+    """Differentiable (log-prob, entropy) of the rows of ``x``; the gradient comes from vrl_rowscore_backward."""
+
+    @staticmethod
+    def forward(ctx, x, lab, temp, want_logprob, want_entropy, n_splits, inplace_backward):
+        ctx.set_materialize_grads(False)
+        lp, h, _, lse, flag = _forward_2d(x, lab, temp, want_logprob, True, False, True, n_splits)
+        ctx.save_for_backward(x, lab, temp, lse, h)
+        ctx.inplace = bool(inplace_backward)
+        return lp, (h if want_entropy else None), flag
+
+    @staticmethod
+    def backward(ctx, g_lp, g_h, _g_flag):
+        x, lab, temp, lse, h = ctx.saved_tensors
+        if g_lp is None and g_h is None:
+            return None, None, None, None, None, None, None
+        n, V = x.shape
+        dev = x.device
+        # In place: the gradient replaces the logits in their own storage, like the reference's
+        # flash-attn path does with inplace_backward=True (verl/utils/torch_functional.py:110-131).
+        dx = x if ctx.inplace else torch.empty((n, V), dtype=x.dtype, device=dev)
+        if n > 0:
+            gl = None if g_lp is None else g_lp.to(torch.float32).contiguous()
+            gh = None if g_h is None else g_h.to(torch.float32).contiguous()
+            lib = _lib.load()
+            with torch.cuda.device(dev):
+                st = lib.vrl_rowscore_backward(
+                    x.data_ptr(), _DTYPE_CODES[x.dtype], n, V, x.stride(0) if n > 1 else V, _ptr(lab), _ptr(temp),
+                    lse.data_ptr(), h.data_ptr(), _ptr(gl), _ptr(gh), dx.data_ptr(), dx.stride(0) if n > 1 else V,
+                    torch.cuda.current_stream(dev).cuda_stream,
+                )
+            _lib.check("vrl_rowscore_backward", st)
+        return dx, None, None, None, None, None, None
+
+
 def rowscore(
     logits: torch.Tensor,
     labels: Optional[torch.Tensor],
@@ -95,13 +168,16 @@ def rowscore(
     want_sum_pi_sq: bool = False,
     check_labels: bool = True,
     n_splits: Optional[int] = None,
+    inplace_backward: bool = False,
     what: str = "rowscore",
 ):
     """Launch the row kernel; returns (logprob | None, entropy | None) and, with ``want_sum_pi_sq``,
     a third entry, each fp32 of shape logits.shape[:-1].
 
     With few rows the work of one row is spread over ``n_splits`` workgroups (vrl_rowscore_split);
-    ``n_splits=None`` lets the library choose, 1 forces one workgroup per row.
+    ``n_splits=None`` lets the library choose, 1 forces one workgroup per row. When grad is enabled
+    and the logits require it, log-prob and entropy are differentiable with respect to the logits
+    (vrl_rowscore_backward); the sum of squared probabilities is not.
     """
     _check_logits(logits, what)
     if not (want_logprob or want_entropy or want_sum_pi_sq):
@@ -121,38 +197,23 @@ def rowscore(
         if labels.dtype.is_floating_point or labels.dtype == torch.bool:
             raise TypeError(f"{what}: labels must be an integer tensor, got {labels.dtype}")
         lab = labels.to(device=dev, dtype=torch.int64).reshape(n).contiguous()
-
     temp = _temperature_rows(temperature, lead, n, dev)
-    out_lp = torch.empty(n, dtype=torch.float32, device=dev) if want_logprob else None
-    out_h = torch.empty(n, dtype=torch.float32, device=dev) if want_entropy else None
-    out_q = torch.empty(n, dtype=torch.float32, device=dev) if want_sum_pi_sq else None
-    flag = torch.zeros(1, dtype=torch.int32, device=dev) if want_logprob else None
 
-    if n > 0:
-        lib = _lib.load()
-        dt = _DTYPE_CODES[x.dtype]
-        stride = x.stride(0) if n > 1 else V
-        splits = lib.vrl_rowscore_split_plan(dt, n, V) if n_splits is None else int(n_splits)
-        with torch.cuda.device(dev):
-            stream = torch.cuda.current_stream(dev).cuda_stream
-            if splits > 1:
-                partials = torch.empty(n * splits * 4, dtype=torch.float32, device=dev)
-                st = lib.vrl_rowscore_split(
-                    x.data_ptr(), dt, n, V, stride, _ptr(lab), _ptr(temp), _ptr(out_lp), _ptr(out_h), _ptr(out_q),
-                    _ptr(flag), splits, partials.data_ptr(), stream,
-                )
-                _lib.check("vrl_rowscore_split", st)
-            else:
-                st = lib.vrl_rowscore(
-                    x.data_ptr(), dt, n, V, stride, _ptr(lab), _ptr(temp), _ptr(out_lp), _ptr(out_h), _ptr(out_q),
-                    _ptr(flag), stream,
-                )
-                _lib.check("vrl_rowscore", st)
-        if want_logprob and check_labels and (int(flag.item()) & _lib.VRL_FLAG_LABEL_OOB):
-            raise IndexError(f"{what}: a label is outside [0, {V})")
+    needs_grad = torch.is_grad_enabled() and logits.requires_grad
+    out_q = None
+    if needs_grad and (want_logprob or want_entropy):
+        lp, h, flag = _RowScoreFunction.apply(x, lab, temp, want_logprob, want_entropy, n_splits, inplace_backward)
+        if want_sum_pi_sq:
+            with torch.no_grad():
+                out_q = _forward_2d(x, None, temp, False, False, True, False, n_splits)[2]
+    else:
+        with torch.no_grad():
+            lp, h, out_q, _, flag = _forward_2d(x, lab, temp, want_logprob, want_entropy, want_sum_pi_sq, False, n_splits)
+    if want_logprob and check_labels and n > 0 and (int(flag.item()) & _lib.VRL_FLAG_LABEL_OOB):
+        raise IndexError(f"{what}: a label is outside [0, {V})")
 
-    lp = out_lp.reshape(lead) if want_logprob else None
-    h = out_h.reshape(lead) if want_entropy else None
+    lp = lp.reshape(lead) if want_logprob else None
+    h = h.reshape(lead) if want_entropy else None
     if want_sum_pi_sq:
         return lp, h, out_q.reshape(lead)
     return lp, h
@@ -161,11 +222,13 @@ def rowscore(
 def logprobs_from_logits(logits: torch.Tensor, labels: torch.Tensor, inplace_backward: bool = True) -> torch.Tensor:
     """log softmax(logits)[labels], shape logits.shape[:-1], fp32.
 
-    Mirrors verl/utils/torch_functional.py:73-107. ``inplace_backward`` only
-    matters to the reference's flash-attn backward and is accepted and ignored.
+    Mirrors verl/utils/torch_functional.py:73-107. Differentiable with respect to the logits. With
+    ``inplace_backward`` (the reference's default, honoured by its flash-attn branch, :110-131) the
+    backward pass writes the gradient over the logits' own storage instead of allocating
+    another (N, V) tensor; as there, the logits must not be used again after backward.
     """
-    del inplace_backward
-    return rowscore(logits, labels, want_entropy=False, what="logprobs_from_logits")[0]
+    return rowscore(logits, labels, want_entropy=False, inplace_backward=inplace_backward and _is_view_safe(logits),
+                    what="logprobs_from_logits")[0]
 
 
 def logprobs_from_logits_v2(logits: torch.Tensor, labels: torch.Tensor) -> torch.Tensor:
