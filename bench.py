@@ -148,6 +148,71 @@ class Step:
         return e1, e2
 
 
+def bench_backward(args, dev):
+    """Throughput of vrl_rowscore_backward (gradient of log-prob and entropy with respect to the logits) on the
+    workload's rows: reads the logits once, writes the gradient once (2 * V * sizeof + per-row scalars)."""
+    w = synthetic.WORKLOADS[args.workload]
+    step = Step(w, dev, seed=1000 * int(args.workload[1]))
+    lse = torch.empty(step.n, dtype=torch.float32, device=dev)
+    st = step.lib.vrl_rowscore(step.logits.data_ptr(), step.dt, step.n, w.V, step.logits.stride(0), step.labels.data_ptr(),
+                               step._tp(), step.lp.data_ptr(), step.h.data_ptr(), None, lse.data_ptr(),
+                               step.flag.data_ptr(), step.stream)
+    _lib.check("vrl_rowscore", st)
+    g = torch.Generator(device=dev).manual_seed(99)
+    gl = torch.randn(step.n, generator=g, device=dev)
+    gh = torch.randn(step.n, generator=g, device=dev) * 0.01
+    dx = torch.empty_like(step.logits)
+
+    def run():
+        st = step.lib.vrl_rowscore_backward(step.logits.data_ptr(), step.dt, step.n, w.V, step.logits.stride(0),
+                                            step.labels.data_ptr(), step._tp(), lse.data_ptr(), step.h.data_ptr(),
+                                            gl.data_ptr(), gh.data_ptr(), dx.data_ptr(), dx.stride(0), step.stream)
+        _lib.check("vrl_rowscore_backward", st)
+
+    # guard: first rows against torch autograd in fp32
+    run()
+    rows = 256
+    xr = step.logits[:rows].float().requires_grad_(True)
+    z = xr if step.temp is None else xr / step.temp[:rows].clamp(min=1e-8).unsqueeze(-1)
+    lsm = torch.log_softmax(z, -1)
+    lpr = lsm.gather(-1, step.labels[:rows, None]).squeeze(-1)
+    hr = -(lsm.exp() * lsm).sum(-1)
+    ((lpr * gl[:rows]).sum() + (hr * gh[:rows]).sum()).backward()
+    err = (dx[:rows].float() - xr.grad).abs()
+    tol = xr.grad.abs() * (2.0 ** -7 if w.dtype == torch.bfloat16 else 0.0) + 2e-5
+    if not bool((err <= tol).all()):
+        raise SystemExit(f"bench: backward disagrees with torch autograd (max abs err {err.max().item()})")
+    for _ in range(args.warmup):
+        run()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        run()
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(args.steps)]
+    for a, b in evs:
+        a.record()
+        run()
+        b.record()
+    torch.cuda.synchronize()
+    avg_ms = sum(a.elapsed_time(b) for a, b in evs) / len(evs)
+    esize = 2 if w.dtype == torch.bfloat16 else 4
+    bytes_launch = step.n * (2 * w.V * esize + 8 + 4 + 4 + 4 + 4 + (4 if step.temp is not None else 0))
+    achieved = bytes_launch / (avg_ms * 1e-3) / 1e9
+    print(json.dumps({
+        "metric": "tokens/sec of the backward of the row op + achieved HBM GB/s", "value": step.n * args.steps / wall,
+        "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": wall * 1e3 / args.steps,
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16" if w.dtype == torch.bfloat16 else "f32", "data": "synthetic",
+        "config": {"workload": w.name, "layout": step.layout, "rows_per_step": step.n, "vocab": w.V,
+                   "step": "vrl_rowscore_backward through the C ABI (gradients of log-prob and entropy)"},
+        "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                     "frac": achieved / HBM_PEAK_GBPS, "traffic": None, "kernel": "rowscore_backward_kernel",
+                     "avg_kernel_ms": avg_ms, "algorithmic_bytes_per_launch": bytes_launch},
+    }), flush=True)
+
+
 class VerifyOnlyStep:
     """c5: 512 sequences with log-uniform lengths in [32, 16384], packed; only the verify kernel is timed
     (its logits would be 408 GB, scored in 8192-token micro-batches like c3)."""
@@ -271,6 +336,8 @@ def main():
     ap.add_argument("--workload", default="c2", choices=["c1", "c2", "c3", "c4", "c5"],
                     help="c5 times the verify kernel alone (its logits do not fit; they are scored like c3)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--backward", action="store_true",
+                    help="time vrl_rowscore_backward on the workload instead of the fused forward step")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run a plain device copy of known size (for scaling rocprofv3 byte counters)")
     args = ap.parse_args()
@@ -286,6 +353,9 @@ def main():
     torch.cuda.set_device(dev)
     if args.workload == "c5":
         bench_verify_only(args, dev)
+        return
+    if args.backward:
+        bench_backward(args, dev)
         return
     w = synthetic.WORKLOADS[args.workload]
     step = Step(w, dev, seed=1000 * int(args.workload[1]))
