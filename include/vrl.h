@@ -35,7 +35,7 @@ extern "C" {
 /* status codes */
 #define VRL_OK 0
 #define VRL_ERR_NULL (-1)      /* a required pointer is NULL */
-#define VRL_ERR_DTYPE (-2)     /* dtype is not one of VRL_F32 / VRL_BF16 */
+#define VRL_ERR_DTYPE (-2)     /* dtype is not one of VRL_F32 / VRL_BF16 / VRL_F16 */
 #define VRL_ERR_SHAPE (-3)     /* negative count, vocab <= 0, stride < vocab, too many rows */
 #define VRL_ERR_ALIGN (-4)     /* pointer not aligned to its element size */
 #define VRL_ERR_HIP (-5)       /* the HIP runtime refused the launch; see vrl_last_hip_error */
@@ -44,6 +44,7 @@ extern "C" {
 /* logits element types */
 #define VRL_F32 0
 #define VRL_BF16 1
+#define VRL_F16 2
 
 /* bits of *err_flag */
 #define VRL_FLAG_LABEL_OOB 1   /* some label was < 0 or >= vocab; that row's logprob is NaN */

@@ -51,6 +51,8 @@ def rowscore(logits: torch.Tensor, labels=None, temperature=None):
         buf, dt = x.numpy(), 0
     elif x.dtype == torch.bfloat16:
         buf, dt = x.view(torch.int16).numpy(), 1
+    elif x.dtype == torch.float16:
+        buf, dt = x.float().numpy(), 0  # every half is an exact float
     else:
         raise TypeError(x.dtype)
     n, V = x.shape

@@ -22,7 +22,7 @@ import torch
 
 from oracle import c_oracle, scoring
 
-TOL = {torch.float32: 1e-5, torch.bfloat16: 2e-3}
+TOL = {torch.float32: 1e-5, torch.bfloat16: 2e-3, torch.float16: 2e-3}
 TOL64 = 4e-6
 
 

@@ -64,7 +64,7 @@ def test_per_token_temperature_and_clamp(dev):
     assert lp.abs().max().item() <= 1e-5 and h.abs().max().item() <= 1e-5
 
 
-@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("V", [1, 2, 7, 8, 9, 63, 64, 65, 257, 1023, 1024, 1025, 4096, 8191, 32000, 50257])
 def test_vocab_sizes_and_ragged_tails(dev, dtype, V):
     g = torch.Generator(device=dev).manual_seed(V)
@@ -203,7 +203,17 @@ def test_rejects_cpu_and_unsupported_inputs(dev):
         spec_rl.fused_score_verify(x, torch.zeros(2, dtype=torch.long, device=dev), torch.zeros(2, device=dev), seed=0,
                                    cu_seqlens=torch.tensor([0, 2], device=dev))
     with pytest.raises(TypeError):
-        vf.entropy_from_logits(torch.randn(2, 10, device=dev).half())
+        vf.entropy_from_logits(torch.randn(2, 10, device=dev).double())
+
+
+def test_fp16_logits_full_vocab(dev):
+    g = torch.Generator(device=dev).manual_seed(16)
+    x = (torch.randn(64, 151936, generator=g, device=dev) * 3).half()
+    lab = torch.randint(0, 151936, (64,), generator=g, device=dev)
+    temp = torch.full((64,), 0.7, device=dev)
+    _check(x, lab)
+    _check(x, lab, temp)
+    _check(x[:, 5:150001], lab.clamp(max=149995))
 
 
 def test_rows_are_independent_and_deterministic(dev):

@@ -23,6 +23,7 @@ VRL_ERR_ARG = -6
 
 VRL_F32 = 0
 VRL_BF16 = 1
+VRL_F16 = 2
 
 VRL_FLAG_LABEL_OOB = 1
 VRL_FLAG_SLICE_RANGE = 2

@@ -62,6 +62,26 @@ struct ElemOut<1> {
   }
 };
 
+template <>
+struct ElemOut<2> {
+  typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
+  __device__ static __forceinline__ uint32_t pack2(float lo, float hi) {
+    const f32x2 v = {lo, hi};
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, f16x2));  // round to nearest even
+  }
+  __device__ static __forceinline__ u32x4 pack(const float* y) {
+    u32x4 v;
+    v.x = pack2(y[0], y[1]);
+    v.y = pack2(y[2], y[3]);
+    v.z = pack2(y[4], y[5]);
+    v.w = pack2(y[6], y[7]);
+    return v;
+  }
+  __device__ static __forceinline__ void store1(char* rowp, int64_t idx, float y) {
+    reinterpret_cast<_Float16*>(rowp)[idx] = static_cast<_Float16>(y);
+  }
+};
+
 struct RowGrad {
   float c;     // log2e / T
   float lse2;  // lse * log2e

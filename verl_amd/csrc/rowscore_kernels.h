@@ -96,6 +96,28 @@ struct Elem<1> {  // VRL_BF16: the upper half of an fp32
   }
 };
 
+template <>
+struct Elem<2> {  // VRL_F16: IEEE half
+  typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
+  typedef float f32x2v __attribute__((ext_vector_type(2)));
+  static constexpr int kBytes = 2;
+  static constexpr int kPerVec = 8;
+  __device__ static __forceinline__ void unpack2(uint32_t w, float* x) {
+    const f32x2v f = __builtin_convertvector(__builtin_bit_cast(f16x2, w), f32x2v);
+    x[0] = f.x;
+    x[1] = f.y;
+  }
+  __device__ static __forceinline__ void unpack(const u32x4& v, float* x) {
+    unpack2(v.x, x);
+    unpack2(v.y, x + 2);
+    unpack2(v.z, x + 4);
+    unpack2(v.w, x + 6);
+  }
+  __device__ static __forceinline__ float load1(const char* rowp, int64_t idx) {
+    return static_cast<float>(reinterpret_cast<const _Float16*>(rowp)[idx]);
+  }
+};
+
 // ---- temperature ---------------------------------------------------------
 // EXACT = false: y = x * c with c = log2e / T folded into one constant.
 // EXACT = true : q = RN(x / T) first (what `logits / temperature` gives per

@@ -27,6 +27,8 @@ int launch_status() {
 
 bool aligned(const void* p, uintptr_t a) { return (reinterpret_cast<uintptr_t>(p) & (a - 1)) == 0; }
 
+bool known_dtype(int dtype) { return dtype == VRL_F32 || dtype == VRL_BF16 || dtype == VRL_F16; }
+
 constexpr int64_t kMaxGrid = 0x7fffffffLL;
 
 // Workgroup shape of the row kernel (wavefronts per row, 128-bit loads per lane
@@ -44,6 +46,10 @@ template <>
 struct RowShape<VRL_BF16> {
   static constexpr int kWaves = 8, kUnroll = 2;
 };
+template <>
+struct RowShape<VRL_F16> {
+  static constexpr int kWaves = 8, kUnroll = 2;
+};
 // Shape of a workgroup that reduces one slice of a row (split path).
 constexpr int kSplitWaves = 4;
 constexpr int kSplitUnroll = 2;
@@ -58,7 +64,7 @@ int check_rowscore(const void* logits, int dtype, int64_t n_rows, int64_t vocab,
                    const int64_t* labels, const float* temperature, const float* out_logprob,
                    const float* out_entropy, const float* out_sum_pi_sq, const float* out_lse,
                    const int32_t* err_flag) {
-  if (dtype != VRL_F32 && dtype != VRL_BF16) return VRL_ERR_DTYPE;
+  if (!known_dtype(dtype)) return VRL_ERR_DTYPE;
   if (n_rows < 0 || vocab <= 0 || row_stride < vocab || n_rows > kMaxGrid) return VRL_ERR_SHAPE;
   if (out_logprob == nullptr && out_entropy == nullptr && out_sum_pi_sq == nullptr && out_lse == nullptr)
     return VRL_ERR_ARG;
@@ -130,8 +136,10 @@ void launch_rows_any(int dtype, const RowArgs& a) {
       launch_rows_q<VRL_F32, true>(a);
     else
       launch_rows_q<VRL_F32, false>(a);
-  } else {
+  } else if (dtype == VRL_BF16) {
     launch_rows_q<VRL_BF16, false>(a);
+  } else {
+    launch_rows_q<VRL_F16, false>(a);
   }
 }
 
@@ -184,7 +192,7 @@ int vrl_rowscore(const void* logits, int dtype, int64_t n_rows, int64_t vocab, i
 }
 
 int vrl_rowscore_split_plan(int dtype, int64_t n_rows, int64_t vocab) {
-  if ((dtype != VRL_F32 && dtype != VRL_BF16) || n_rows <= 0 || vocab <= 0) return 1;
+  if (!known_dtype(dtype) || n_rows <= 0 || vocab <= 0) return 1;
   // One workgroup per row fills the chip from about a thousand rows on.
   constexpr int64_t kTargetGroups = 2048;
   if (n_rows >= kTargetGroups / 2) return 1;
@@ -220,7 +228,7 @@ int vrl_rowscore_backward(const void* logits, int dtype, int64_t n_rows, int64_t
                           const int64_t* labels, const float* temperature, const float* lse,
                           const float* entropy, const float* g_logprob, const float* g_entropy,
                           void* dlogits, int64_t d_row_stride, void* stream) {
-  if (dtype != VRL_F32 && dtype != VRL_BF16) return VRL_ERR_DTYPE;
+  if (!known_dtype(dtype)) return VRL_ERR_DTYPE;
   if (n_rows < 0 || vocab <= 0 || row_stride < vocab || d_row_stride < vocab || n_rows > kMaxGrid)
     return VRL_ERR_SHAPE;
   if (g_logprob == nullptr && g_entropy == nullptr) return VRL_ERR_ARG;
@@ -237,8 +245,11 @@ int vrl_rowscore_backward(const void* logits, int dtype, int64_t n_rows, int64_t
   if (dtype == VRL_F32)
     vrl::rowscore_backward_kernel<VRL_F32, kBackwardWaves, kBackwardUnroll><<<grid, dim3(kBackwardWaves * 64), 0, s>>>(
         logits, vocab, row_stride, labels, temperature, lse, entropy, g_logprob, g_entropy, dlogits, d_row_stride);
-  else
+  else if (dtype == VRL_BF16)
     vrl::rowscore_backward_kernel<VRL_BF16, kBackwardWaves, kBackwardUnroll><<<grid, dim3(kBackwardWaves * 64), 0, s>>>(
+        logits, vocab, row_stride, labels, temperature, lse, entropy, g_logprob, g_entropy, dlogits, d_row_stride);
+  else
+    vrl::rowscore_backward_kernel<VRL_F16, kBackwardWaves, kBackwardUnroll><<<grid, dim3(kBackwardWaves * 64), 0, s>>>(
         logits, vocab, row_stride, labels, temperature, lse, entropy, g_logprob, g_entropy, dlogits, d_row_stride);
   return launch_status();
 }
@@ -327,7 +338,7 @@ const char* vrl_strerror(int status) {
   switch (status) {
     case VRL_OK: return "ok";
     case VRL_ERR_NULL: return "a required pointer is NULL";
-    case VRL_ERR_DTYPE: return "unsupported logits dtype (expected VRL_F32 or VRL_BF16)";
+    case VRL_ERR_DTYPE: return "unsupported logits dtype (expected VRL_F32, VRL_BF16 or VRL_F16)";
     case VRL_ERR_SHAPE: return "bad shape (negative count, vocab <= 0, row_stride < vocab, or too many rows)";
     case VRL_ERR_ALIGN: return "pointer is not aligned to its element size";
     case VRL_ERR_HIP: return "the HIP runtime refused the kernel launch";

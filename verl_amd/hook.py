@@ -12,7 +12,7 @@ tests/workers/test_distillation_topk_symmetry_on_cpu.py:143-146).
 
 A replaced function sends GPU tensors of a supported dtype to the HIP kernels
 (forward, and backward when the logits need a gradient). Anything else (CPU
-tensors on the driver, fp16/fp64) is handed to the function it replaced, i.e. verl's own
+tensors on the driver, fp64) is handed to the function it replaced, i.e. verl's own
 code, and counted in ``stats()``: this package adds no second implementation.
 """
 
@@ -46,7 +46,7 @@ def _eligible(logits) -> bool:
     return (
         isinstance(logits, torch.Tensor)
         and logits.is_cuda
-        and logits.dtype in (torch.float32, torch.bfloat16)
+        and logits.dtype in (torch.float32, torch.bfloat16, torch.float16)
         and logits.dim() >= 1
         and logits.shape[-1] > 0
     )

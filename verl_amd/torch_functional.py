@@ -35,7 +35,7 @@ __all__ = [
     "fused_logprob_entropy",
 ]
 
-_DTYPE_CODES = {torch.float32: _lib.VRL_F32, torch.bfloat16: _lib.VRL_BF16}
+_DTYPE_CODES = {torch.float32: _lib.VRL_F32, torch.bfloat16: _lib.VRL_BF16, torch.float16: _lib.VRL_F16}
 
 
 def _ptr(t: Optional[torch.Tensor]) -> Optional[int]:
@@ -51,7 +51,7 @@ def _check_logits(logits: torch.Tensor, what: str) -> None:
             "it has no CPU implementation"
         )
     if logits.dtype not in _DTYPE_CODES:
-        raise TypeError(f"{what}: logits dtype {logits.dtype} is not supported (float32 and bfloat16 are)")
+        raise TypeError(f"{what}: logits dtype {logits.dtype} is not supported (float32, bfloat16 and float16 are)")
     if logits.dim() < 1 or logits.shape[-1] == 0:
         raise ValueError(f"{what}: logits need a non-empty last (vocab) dimension, got shape {tuple(logits.shape)}")
 
