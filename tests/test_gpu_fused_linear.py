@@ -1,0 +1,94 @@
+"""LM head + scoring in token chunks (verl_amd.fused_linear) against torch on the same inputs.
+
+Tolerances are the reference's own for this comparison (tests/utils/test_linear_cross_entropy.py:211-224,
+261-269): forward atol = rtol = 1e-4 against the fp32 torch composition, gradients atol 1e-2 / rtol 1e-4,
+with inputs drawn like there (uniform(-0.5, 0.5), temperature 1.5).
+"""
+
+import pytest
+import torch
+
+from verl_amd.fused_linear import FusedLinearForPPO, fused_linear_for_ppo
+
+pytestmark = pytest.mark.gpu
+
+
+def _torch_reference(hidden, weight, labels, temperature):
+    """run_torch_entropy of the reference's test (fp32 GEMM, softmax/logsumexp/cross_entropy)."""
+    logits = torch.matmul(hidden.float(), weight.float().t()) / temperature
+    pd = torch.softmax(logits, dim=-1)
+    entropy = torch.logsumexp(logits, dim=-1) - torch.sum(pd * logits, dim=-1)
+    logprobs = -torch.nn.functional.cross_entropy(logits, labels, reduction="none")
+    return logprobs, entropy
+
+
+@pytest.mark.parametrize("T,D,V,chunk", [(300, 256, 32256, 128), (257, 128, 10007, 512), (64, 64, 151936, 17)])
+def test_fp32_forward_and_backward_match_torch(dev, T, D, V, chunk):
+    g = torch.Generator(device=dev).manual_seed(T + V)
+    hidden = torch.empty(T, D, device=dev).uniform_(-0.5, 0.5, generator=g).requires_grad_()
+    weight = torch.empty(V, D, device=dev).uniform_(-0.5, 0.5, generator=g).requires_grad_()
+    labels = torch.randint(0, V, (T,), generator=g, device=dev)
+    g_ent = torch.empty(T, device=dev).uniform_(-0.5, 0.5, generator=g)
+    g_lp = torch.empty(T, device=dev).uniform_(-1, 1, generator=g)
+    temperature = 1.5
+
+    ref_lp, ref_ent = _torch_reference(hidden, weight, labels, temperature)
+    d_ref_h, d_ref_w = torch.autograd.grad((ref_ent, ref_lp), (hidden, weight), (g_ent, g_lp))
+
+    lp, ent = fused_linear_for_ppo(hidden, weight, labels, temperature, chunk_size=chunk)
+    assert lp.dtype == torch.float32 and lp.shape == (T,) and ent.shape == (T,)
+    torch.testing.assert_close(ref_lp, lp, atol=1e-4, rtol=1e-4)
+    torch.testing.assert_close(ref_ent, ent, atol=1e-4, rtol=1e-4)
+    d_h, d_w = torch.autograd.grad((ent, lp), (hidden, weight), (g_ent, g_lp))
+    torch.testing.assert_close(d_ref_h, d_h, atol=1e-2, rtol=1e-4)
+    torch.testing.assert_close(d_ref_w, d_w, atol=1e-2, rtol=1e-4)
+    # much closer than the reference asks for
+    assert (d_ref_h - d_h).abs().max().item() <= 2e-4 and (d_ref_w - d_w).abs().max().item() <= 2e-4
+
+
+def test_bf16_module_3d_inputs(dev):
+    """bf16 like the engine runs it; 3-D hidden states as the reference's module accepts them."""
+    g = torch.Generator(device=dev).manual_seed(5)
+    B, S, D, V = 2, 150, 256, 32256
+    hidden = torch.empty(B, S, D, device=dev).uniform_(-0.5, 0.5, generator=g).bfloat16().requires_grad_()
+    weight = torch.empty(V, D, device=dev).uniform_(-0.5, 0.5, generator=g).bfloat16().requires_grad_()
+    labels = torch.randint(0, V, (B, S), generator=g, device=dev)
+    mod = FusedLinearForPPO(chunk_size=64)
+    lp, ent = mod(hidden, weight, labels, temperature=1.5)
+    assert lp.shape == (B, S) and ent.shape == (B, S)
+    # the kernels' share, exactly: fp32 math on the bf16 logits the library GEMM produced
+    logits = torch.matmul(hidden.detach().view(-1, D), weight.detach().t()).float() / 1.5
+    ref_lp = torch.log_softmax(logits, -1).gather(-1, labels.view(-1, 1)).squeeze(-1)
+    ref_ent = torch.logsumexp(logits, -1) - (torch.softmax(logits, -1) * logits).sum(-1)
+    assert (lp.view(-1) - ref_lp).abs().max().item() <= 2e-3 and (ent.view(-1) - ref_ent).abs().max().item() <= 2e-3
+    # against the all-fp32 reference the difference is the bf16 rounding of the logits (|logit| ~ 2.3 here)
+    f_lp, f_ent = _torch_reference(hidden.detach().view(-1, D), weight.detach(), labels.view(-1), 1.5)
+    assert (lp.view(-1) - f_lp).abs().max().item() <= 5e-2
+    g_lp = torch.empty(B, S, device=dev).uniform_(-1, 1, generator=g)
+    g_ent = torch.empty(B, S, device=dev).uniform_(-0.5, 0.5, generator=g)
+    d_h, d_w = torch.autograd.grad((ent, lp), (hidden, weight), (g_ent, g_lp))
+    hf = hidden.detach().float().requires_grad_()
+    wf = weight.detach().float().requires_grad_()
+    r_lp, r_ent = _torch_reference(hf.view(-1, D), wf, labels.view(-1), 1.5)
+    d_rh, d_rw = torch.autograd.grad((r_ent, r_lp), (hf, wf), (g_ent.view(-1), g_lp.view(-1)))
+    assert d_h.dtype == torch.bfloat16 and d_h.shape == hidden.shape and d_w.shape == weight.shape
+    torch.testing.assert_close(d_rh, d_h.float(), atol=2e-2, rtol=4e-2)   # the reference's bf16-kernel tolerance (:271-276)
+    torch.testing.assert_close(d_rw, d_w.float(), atol=2e-2, rtol=4e-2)
+
+
+def test_input_checks(dev):
+    h = torch.randn(4, 8, device=dev)
+    w = torch.randn(16, 8, device=dev)
+    ids = torch.zeros(4, dtype=torch.long, device=dev)
+    with pytest.raises(RuntimeError, match="no CPU implementation"):
+        fused_linear_for_ppo(h.cpu(), w.cpu(), ids.cpu())
+    with pytest.raises(TypeError):
+        fused_linear_for_ppo(h, w.bfloat16(), ids)
+    with pytest.raises(ValueError):
+        fused_linear_for_ppo(h, w, ids[:3])
+    with pytest.raises(ValueError):
+        fused_linear_for_ppo(h, w, ids, chunk_size=0)
+    with pytest.raises(IndexError):
+        fused_linear_for_ppo(h, w, torch.full((4,), 16, device=dev))
+    lp, ent = fused_linear_for_ppo(h[:0], w, ids[:0])
+    assert lp.shape == (0,) and ent.shape == (0,)

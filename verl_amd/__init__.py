@@ -11,6 +11,7 @@ Setting ``VERL_USE_EXTERNAL_MODULES=verl_amd.plugin`` makes verl import
 ``install()``.
 """
 
+from .fused_linear import FusedLinearForPPO, fused_linear_for_ppo
 from .hook import install, uninstall
 from .layout import response_slice, roll_labels
 from .spec_rl import (
@@ -36,6 +37,8 @@ __version__ = "0.1.0"
 __all__ = [
     "install",
     "uninstall",
+    "FusedLinearForPPO",
+    "fused_linear_for_ppo",
     "VerifyResult",
     "draw_log_uniforms",
     "fused_score_verify",

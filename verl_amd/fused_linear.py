@@ -1,0 +1,139 @@
+"""LM head + scoring without ever holding the full ``(tokens, vocab)`` logits.
+
+Same call as the reference's ``FusedLinearForPPO`` (verl/utils/experimental/torch_functional.py:211-231):
+``(hidden_states, vocab_weights, input_ids, temperature) -> (log_probs fp32, entropy)``, chunked over
+tokens. Per chunk the projection ``hidden @ W^T`` is one library GEMM (torch.matmul, i.e. hipBLASLt)
+into a reusable ``(chunk, vocab)`` buffer, and everything after it is the HIP row kernel: forward
+``vrl_rowscore`` (one pass over the chunk's logits), backward ``vrl_rowscore_backward`` writing the
+gradient over the recomputed logits in place, followed by the two GEMMs for ``d hidden`` and ``d W``.
+The reference does the post-GEMM part with ~10 torch ops per chunk (softmax, logsumexp, log_softmax,
+gather, scatter, ...; :27-79); peak extra memory here is one ``(chunk, vocab)`` buffer.
+"""
+
+from __future__ import annotations
+
+from typing import Optional
+
+import torch
+
+from . import _lib
+from .torch_functional import _DTYPE_CODES, _ptr
+
+__all__ = ["FusedLinearForPPO", "fused_linear_for_ppo"]
+
+
+def _score_chunk(lib, logits, labels, temp, lp, h, lse, flag, stream):
+    n, V = logits.shape
+    st = lib.vrl_rowscore(logits.data_ptr(), _DTYPE_CODES[logits.dtype], n, V, logits.stride(0) if n > 1 else V,
+                          labels.data_ptr(), _ptr(temp), lp.data_ptr(), h.data_ptr(), None, lse.data_ptr(),
+                          flag.data_ptr(), stream)
+    _lib.check("vrl_rowscore", st)
+
+
+class _FusedLinearForPPOFunction(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, hidden, weight, input_ids, temperature, chunk_size):
+        ctx.set_materialize_grads(False)
+        T, D = hidden.shape
+        V = weight.shape[0]
+        dev = hidden.device
+        f32 = dict(dtype=torch.float32, device=dev)
+        lp = torch.empty(T, **f32)
+        h = torch.empty(T, **f32)
+        lse = torch.empty(T, **f32)
+        flag = torch.zeros(1, dtype=torch.int32, device=dev)
+        temp = None if temperature == 1.0 else torch.full((min(chunk_size, max(T, 1)),), float(temperature), **f32)
+        lib = _lib.load()
+        buf = torch.empty((min(chunk_size, max(T, 1)), V), dtype=hidden.dtype, device=dev)
+        with torch.cuda.device(dev):
+            stream = torch.cuda.current_stream(dev).cuda_stream
+            for lo in range(0, T, chunk_size):
+                hi = min(lo + chunk_size, T)
+                logits = buf[: hi - lo]
+                torch.matmul(hidden[lo:hi], weight.t(), out=logits)
+                _score_chunk(lib, logits, input_ids[lo:hi], None if temp is None else temp[: hi - lo],
+                             lp[lo:hi], h[lo:hi], lse[lo:hi], flag, stream)
+        if T > 0 and (int(flag.item()) & _lib.VRL_FLAG_LABEL_OOB):
+            raise IndexError(f"fused_linear_for_ppo: an input id is outside [0, {V})")
+        ctx.save_for_backward(hidden, weight, input_ids, lse, h)
+        ctx.temperature = float(temperature)
+        ctx.chunk_size = int(chunk_size)
+        return lp, h.clone()
+
+    @staticmethod
+    def backward(ctx, g_lp: Optional[torch.Tensor], g_h: Optional[torch.Tensor]):
+        hidden, weight, input_ids, lse, h = ctx.saved_tensors
+        if g_lp is None and g_h is None:
+            return None, None, None, None, None
+        T, D = hidden.shape
+        V = weight.shape[0]
+        dev = hidden.device
+        chunk = ctx.chunk_size
+        f32 = dict(dtype=torch.float32, device=dev)
+        gl = None if g_lp is None else g_lp.to(torch.float32).contiguous()
+        gh = None if g_h is None else g_h.to(torch.float32).contiguous()
+        temp = None if ctx.temperature == 1.0 else torch.full((min(chunk, max(T, 1)),), ctx.temperature, **f32)
+        need_dh, need_dw = ctx.needs_input_grad[0], ctx.needs_input_grad[1]
+        d_hidden = torch.empty_like(hidden) if need_dh else None
+        d_weight = torch.zeros_like(weight) if need_dw else None
+        lib = _lib.load()
+        buf = torch.empty((min(chunk, max(T, 1)), V), dtype=hidden.dtype, device=dev)
+        dt = _DTYPE_CODES[hidden.dtype]
+        with torch.cuda.device(dev):
+            stream = torch.cuda.current_stream(dev).cuda_stream
+            for lo in range(0, T, chunk):
+                hi = min(lo + chunk, T)
+                n = hi - lo
+                logits = buf[:n]
+                torch.matmul(hidden[lo:hi], weight.t(), out=logits)
+                st = lib.vrl_rowscore_backward(
+                    logits.data_ptr(), dt, n, V, logits.stride(0) if n > 1 else V, input_ids[lo:hi].data_ptr(),
+                    None if temp is None else temp.data_ptr(), lse[lo:hi].data_ptr(), h[lo:hi].data_ptr(),
+                    None if gl is None else gl[lo:hi].data_ptr(), None if gh is None else gh[lo:hi].data_ptr(),
+                    logits.data_ptr(), logits.stride(0) if n > 1 else V, stream)   # gradient over the logits, in place
+                _lib.check("vrl_rowscore_backward", st)
+                if need_dh:
+                    torch.matmul(logits, weight, out=d_hidden[lo:hi])
+                if need_dw:
+                    d_weight.addmm_(logits.t(), hidden[lo:hi])
+        return d_hidden, d_weight, None, None, None
+
+
+def fused_linear_for_ppo(hidden_states: torch.Tensor, vocab_weights: torch.Tensor, input_ids: torch.Tensor,
+                         temperature: float = 1.0, chunk_size: int = 512):
+    """(log_probs fp32, entropy fp32) of ``softmax((hidden_states @ vocab_weights.T) / temperature)`` at ``input_ids``.
+
+    ``hidden_states`` is ``(tokens, hidden)`` or ``(batch, seq, hidden)`` with ``input_ids`` of the matching leading
+    shape; ``vocab_weights`` is ``(vocab, hidden)``; both bf16, fp16 or fp32 on the GPU. Differentiable with respect
+    to both.
+    """
+    if not hidden_states.is_cuda or not vocab_weights.is_cuda:
+        raise RuntimeError("fused_linear_for_ppo: tensors must be on the GPU; verl_amd has no CPU implementation")
+    if hidden_states.dtype != vocab_weights.dtype or hidden_states.dtype not in _DTYPE_CODES:
+        raise TypeError(f"fused_linear_for_ppo: hidden {hidden_states.dtype} / weights {vocab_weights.dtype} must share "
+                        "one of float32, bfloat16, float16")
+    if hidden_states.dim() not in (2, 3):
+        raise ValueError(f"fused_linear_for_ppo: hidden_states must be 2-D or 3-D, got shape {tuple(hidden_states.shape)}")
+    if tuple(input_ids.shape) != tuple(hidden_states.shape[:-1]):
+        raise ValueError(f"fused_linear_for_ppo: input_ids shape {tuple(input_ids.shape)} does not match "
+                         f"hidden_states {tuple(hidden_states.shape)}")
+    if vocab_weights.dim() != 2 or vocab_weights.shape[1] != hidden_states.shape[-1]:
+        raise ValueError("fused_linear_for_ppo: vocab_weights must be (vocab, hidden)")
+    if int(chunk_size) <= 0:
+        raise ValueError(f"chunk_size must be positive, got {chunk_size}")
+    lead = hidden_states.shape[:-1]
+    h2 = hidden_states.reshape(-1, hidden_states.shape[-1]).contiguous()
+    ids = input_ids.reshape(-1).to(torch.int64).contiguous()
+    lp, ent = _FusedLinearForPPOFunction.apply(h2, vocab_weights.contiguous(), ids, float(temperature), int(chunk_size))
+    return lp.reshape(lead), ent.reshape(lead)
+
+
+class FusedLinearForPPO(torch.nn.Module):
+    """Module form, constructed and called like verl's (verl/utils/experimental/torch_functional.py:211-231)."""
+
+    def __init__(self, chunk_size: int = 512):
+        super().__init__()
+        self.chunk_size = chunk_size
+
+    def forward(self, hidden_states, vocab_weights, input_ids, temperature: float = 1.0):
+        return fused_linear_for_ppo(hidden_states, vocab_weights, input_ids, temperature, self.chunk_size)
