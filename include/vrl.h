@@ -127,6 +127,31 @@ int vrl_response_slice(const float* values, const int64_t* cu_seqlens, const int
                        int64_t B, int64_t T_out, float* out, int32_t* err_flag, void* stream);
 
 /*
+ * vrl_rollout_corr — rollout correction on padded (B, T) log-probs in one launch:
+ *   lr = clamp(old - rollout, +-20);  k1 = -lr, k2 = lr^2/2, k3 = exp(lr) - 1 - lr
+ *   keep[b,t]    = every enabled criterion passes (token_k1/k2/k3 per token; seq_sum / seq_mean /
+ *                  seq_max of k1/k2/k3 per sequence; k1 criteria are two-sided [lo, hi], the others <= hi)
+ *   weights[b,t] = mask * exp(lr)  (is_mode 1)  or  mask * exp(clamp(sum_t lr, +-20))  (is_mode 2),
+ *                  then min(w, is_upper) (icepop 0) or zeroed outside [is_lower, is_upper] (icepop 1)
+ *   stats[b, :]  = vrl_rollout_corr_num_stats() per-sequence partial sums / extrema (layout: enum CorrStat in
+ *                  verl_amd/csrc/rollout_corr_kernels.h), enough to derive every metric of the step
+ *   seq_keep_bits[b] = bit i set when the sequence passes enabled sequence-level criterion i
+ * rs_bits: bit i enables criterion i in the order token_k1, token_k2, token_k3, seq_sum_k1..k3,
+ * seq_mean_k1..k3, seq_max_k2, seq_max_k3. rs_lo_host / rs_hi_host are HOST arrays of 11 floats holding the
+ * bounds as they are compared (natural log of the ratio bounds for k1 criteria). weights and keep may be NULL.
+ *
+ * Replaces the tensor work of verl/trainer/ppo/rollout_corr_helper.py:
+ *   compute_rollout_rejection_mask :197-413, compute_rollout_correction_weights :522-657,
+ *   compute_offpolicy_metrics :904-1010 (and the per-element parts of compute_rs_metrics :416-519 and
+ *   compute_is_metrics :660-783); the scalar metrics are finished on the host from `stats`.
+ */
+int vrl_rollout_corr(const float* old_log_prob, const float* rollout_log_prob, const uint8_t* mask, int64_t B,
+                     int64_t T, int is_mode, int icepop, float is_upper, float is_lower, float is_lower_metric,
+                     uint32_t rs_bits, const float* rs_lo_host, const float* rs_hi_host, float* weights,
+                     uint8_t* keep, float* stats, int32_t* seq_keep_bits, void* stream);
+int vrl_rollout_corr_num_stats(void);
+
+/*
  * vrl_spec_verify — SPEC-RL draft verification over B sequences.
  * For token i of sequence b:
  *   d = logp_new[i] - logp_old[i];  tau = log_u[i] + thresh_offset      (fp32, no contraction)

@@ -130,6 +130,28 @@ def test_split_and_slice_argument_errors(lib):
     assert g(None, None, None, 0, 4, None, None, None) == _lib.VRL_OK
 
 
+def test_rollout_corr_argument_errors(lib):
+    import ctypes
+
+    f = lib.vrl_rollout_corr
+    arr = (ctypes.c_float * 11)()
+    host = ctypes.cast(arr, ctypes.c_void_p)
+
+    def call(old=P, roll=P, B=2, T=8, is_mode=1, bits=1, lo=host, hi=host, w=P, keep=P, stats=P, sbits=P):
+        return f(old, roll, None, B, T, is_mode, 0, 2.0, 0.0, 0.5, bits, lo, hi, w, keep, stats, sbits, None)
+
+    assert call(B=-1) == _lib.VRL_ERR_SHAPE
+    assert call(is_mode=3) == _lib.VRL_ERR_ARG
+    assert call(bits=1 << 11) == _lib.VRL_ERR_ARG
+    assert call(lo=None) == _lib.VRL_ERR_NULL
+    assert call(stats=None) == _lib.VRL_ERR_NULL
+    assert call(sbits=None) == _lib.VRL_ERR_NULL
+    assert call(old=None) == _lib.VRL_ERR_NULL
+    assert call(roll=P + 2) == _lib.VRL_ERR_ALIGN
+    assert call(B=0, old=None, roll=None, stats=None, sbits=None) == _lib.VRL_OK
+    assert lib.vrl_rollout_corr_num_stats() == 40
+
+
 def test_verify_argument_errors(lib):
     f = lib.vrl_spec_verify
 

@@ -11,6 +11,7 @@ Setting ``VERL_USE_EXTERNAL_MODULES=verl_amd.plugin`` makes verl import
 ``install()``.
 """
 
+from . import rollout_corr
 from .fused_linear import FusedLinearForPPO, fused_linear_for_ppo
 from .hook import install, uninstall
 from .layout import response_slice, roll_labels

@@ -9,6 +9,7 @@
 
 #include "backward_kernels.h"
 #include "layout_kernels.h"
+#include "rollout_corr_kernels.h"
 #include "rowscore_kernels.h"
 #include "verify_kernels.h"
 
@@ -267,6 +268,37 @@ int vrl_rowscore_backward(const void* logits, int dtype, int64_t n_rows, int64_t
         logits, vocab, row_stride, labels, temperature, lse, entropy, g_logprob, g_entropy, dlogits, d_row_stride);
   return launch_status();
 }
+
+int vrl_rollout_corr(const float* old_log_prob, const float* rollout_log_prob, const uint8_t* mask, int64_t B,
+                     int64_t T, int is_mode, int icepop, float is_upper, float is_lower, float is_lower_metric,
+                     uint32_t rs_bits, const float* rs_lo_host, const float* rs_hi_host, float* weights,
+                     uint8_t* keep, float* stats, int32_t* seq_keep_bits, void* stream) {
+  if (B < 0 || T < 0 || B > kMaxGrid || T > kMaxGrid) return VRL_ERR_SHAPE;
+  if (is_mode < 0 || is_mode > 2 || (rs_bits >> vrl::kNumRsOptions) != 0) return VRL_ERR_ARG;
+  if (rs_bits != 0 && (rs_lo_host == nullptr || rs_hi_host == nullptr)) return VRL_ERR_NULL;
+  if (B == 0) return VRL_OK;
+  if (stats == nullptr || seq_keep_bits == nullptr) return VRL_ERR_NULL;
+  if (T > 0 && (old_log_prob == nullptr || rollout_log_prob == nullptr)) return VRL_ERR_NULL;
+  if (!aligned(old_log_prob, 4) || !aligned(rollout_log_prob, 4) || !aligned(weights, 4) || !aligned(stats, 4) ||
+      !aligned(seq_keep_bits, 4))
+    return VRL_ERR_ALIGN;
+  vrl::CorrCfg cfg;
+  cfg.is_mode = is_mode;
+  cfg.icepop = icepop ? 1 : 0;
+  cfg.is_upper = is_upper;
+  cfg.is_lower = is_lower;
+  cfg.is_lower_metric = is_lower_metric;
+  cfg.rs_bits = rs_bits;
+  for (int i = 0; i < vrl::kNumRsOptions; ++i) {
+    cfg.rs_lo[i] = (rs_bits != 0) ? rs_lo_host[i] : 0.f;
+    cfg.rs_hi[i] = (rs_bits != 0) ? rs_hi_host[i] : 0.f;
+  }
+  vrl::rollout_corr_kernel<4><<<dim3(static_cast<unsigned>(B)), dim3(256), 0, static_cast<hipStream_t>(stream)>>>(
+      old_log_prob, rollout_log_prob, mask, T, cfg, weights, keep, stats, seq_keep_bits);
+  return launch_status();
+}
+
+int vrl_rollout_corr_num_stats(void) { return vrl::kNumCorrStats; }
 
 int vrl_response_slice(const float* values, const int64_t* cu_seqlens, const int64_t* response_lens,
                        int64_t B, int64_t T_out, float* out, int32_t* err_flag, void* stream) {
