@@ -33,7 +33,7 @@ HBM_PEAK_GBPS = 8000.0
 # HBM bytes per row-kernel launch measured with rocprofv3 (--pmc FETCH_SIZE and --pmc WRITE_SIZE, one run each,
 # both scaled by what the same counter reads for a plain 1 GiB device copy: x1.999956 and x1.0). The workload
 # shapes are fixed, so the figure is a property of (kernel, shape); the counter summary is kept under profiles/.
-MEASURED_TRAFFIC_BYTES = {"c2": 19943708065, "c3": 2490920770, "c4": 67292648393}
+MEASURED_TRAFFIC_BYTES = {"c2": 19943644231, "c3": 2490946810, "c4": 67292547122}
 METRIC = "verified tokens/sec + achieved HBM GB/s (% of peak), vocab 152k bf16, 1 GPU"
 
 
