@@ -1,0 +1,151 @@
+"""The path end to end, the way verl's engine and driver would walk it on a packed micro-batch
+(verl/workers/engine/fsdp/transformer_impl.py:1149-1177, 1353-1418; verl/workers/utils/padding.py:97-141):
+roll the labels over the packed axis, score every token with its sample's temperature, slice the response
+positions into (B, T), verify the draft. Each stage is checked against the oracle's restatement of the same stage.
+Also: the installed shims route GPU tensors to the HIP path, and the entry points can be captured in a graph."""
+
+import sys
+import types
+
+import numpy as np
+import pytest
+import torch
+
+import verl_amd
+from verl_amd import _lib, hook, layout, spec_rl
+from verl_amd import torch_functional as vf
+from oracle import scoring, verify as overify
+
+pytestmark = pytest.mark.gpu
+
+
+def test_packed_micro_batch_end_to_end(dev):
+    g = torch.Generator().manual_seed(42)
+    B, V = 7, 20011
+    prompt = torch.randint(1, 40, (B,), generator=g)
+    resp = torch.randint(1, 90, (B,), generator=g)
+    seq = prompt + resp
+    cu = torch.zeros(B + 1, dtype=torch.int64)
+    cu[1:] = torch.cumsum(seq, 0)
+    nnz = int(cu[-1])
+    gd = torch.Generator(device=dev).manual_seed(43)
+    ids = torch.randint(0, V, (nnz,), generator=gd, device=dev)
+    logits = (torch.randn(nnz, V, generator=gd, device=dev) * 2.5).bfloat16()
+    temp_per_sample = torch.tensor([0.7, 1.0, 1.3, 0.9, 1.0, 0.6, 1.1], device=dev)
+    temp = torch.repeat_interleave(temp_per_sample, seq.to(dev))          # expand_as_nested(...).values()
+
+    labels = layout.roll_labels(ids)                                       # :1177
+    assert torch.equal(labels.cpu(), scoring.roll_labels(ids.cpu()))
+    lp, ent = vf.fused_logprob_entropy(logits, labels, temp)               # :1357-1399 in one pass
+    ref_lp, ref_ent = scoring.score_fp32(logits, labels, temp)
+    assert (lp - ref_lp).abs().max().item() <= 2e-3 and (ent - ref_ent).abs().max().item() <= 2e-3
+
+    T = int(resp.max())
+    lp_bt = layout.response_slice(lp, cu.to(dev), resp.to(dev), T)         # no_padding_2_padding
+    ent_bt = layout.response_slice(ent, cu.to(dev), resp.to(dev), T)
+    assert torch.equal(lp_bt.cpu(), scoring.response_slice(lp.cpu(), prompt.tolist(), resp.tolist(), T))
+    assert torch.equal(ent_bt.cpu(), scoring.response_slice(ent.cpu(), prompt.tolist(), resp.tolist(), T))
+    # position j of row b is the log-prob of response token j of sample b
+    b, j = 3, 5 % int(resp[3])
+    row = int(cu[b + 1]) - int(resp[b]) - 1 + j
+    assert lp_bt[b, j].item() == lp[row].item() and labels[row].item() == ids[row + 1].item()
+
+    mask = (torch.arange(T).unsqueeze(0) < resp.unsqueeze(1)).to(dev)
+    draft = torch.zeros(B, T, dtype=torch.int64, device=dev)
+    for bb in range(B):
+        e, r = int(cu[bb + 1]), int(resp[bb])
+        draft[bb, :r] = ids[e - r:e]
+    old = lp_bt + torch.randn(B, T, generator=gd, device=dev) * 0.3
+    res = spec_rl.spec_verify(lp_bt, old, mask, seed=7, lenience=float(np.exp(0.5)), draft_ids=draft, pad_id=0)
+    ref = overify.verify_loops(lp_bt, old, res.log_u, mask, res.thresh_offset, draft_ids=draft, pad_id=0)
+    assert np.array_equal(res.accept.cpu().numpy().astype(np.uint8), ref["accept"])
+    assert np.array_equal(res.first_reject.cpu().numpy(), ref["first_reject"])
+    assert np.array_equal(res.out_ids.cpu().numpy(), ref["out_ids"])
+    assert (res.prefix_len.cpu() <= resp).all()
+
+
+def test_installed_shims_send_gpu_tensors_to_the_hip_path(dev):
+    mods = {n: types.ModuleType(n) for n in ("verl", "verl.utils", "verl.utils.torch_functional")}
+    tf = mods["verl.utils.torch_functional"]
+    for name in hook.PATCHED_NAMES:
+        setattr(tf, name, getattr(scoring, name))        # the stand-in "verl" functions are the oracle's restatements
+    saved = {k: sys.modules.get(k) for k in mods}
+    sys.modules.update(mods)
+    try:
+        hook.install()
+        x = torch.randn(6, 999, device=dev)
+        lab = torch.randint(0, 999, (6,), device=dev)
+        lp = tf.logprobs_from_logits(x, lab)
+        h = tf.entropy_from_logits(x.bfloat16())
+        q = tf.calculate_sum_pi_squared_from_logits(x)
+        hc = tf.entropy_from_logits_with_chunking(x, chunk_size=4)
+        assert hook.stats() == {"hip_calls": 4, "passed_to_verl": 0}
+        assert (lp - scoring.logprobs_from_logits(x, lab)).abs().max().item() <= 1e-5
+        assert (h - scoring.entropy_from_logits(x.bfloat16().float())).abs().max().item() <= 2e-3
+        assert (q - scoring.calculate_sum_pi_squared_from_logits(x)).abs().max().item() <= 1e-6
+        assert torch.equal(hc, vf.entropy_from_logits(x))
+        tf.entropy_from_logits(x.cpu())                    # the driver's CPU tensors stay with verl's own function
+        tf.entropy_from_logits(x.double())
+        assert hook.stats() == {"hip_calls": 4, "passed_to_verl": 2}
+        xg = x.clone().requires_grad_(True)               # update_actor: gradient through the HIP backward
+        tf.logprobs_from_logits(xg * 1.0, lab, inplace_backward=True).sum().backward()
+        assert xg.grad is not None and hook.stats()["hip_calls"] == 5
+    finally:
+        hook.uninstall()
+        for k, v in saved.items():
+            if v is None:
+                sys.modules.pop(k, None)
+            else:
+                sys.modules[k] = v
+
+
+def test_entry_points_replay_from_a_graph(dev):
+    """The C ABI only enqueues kernels (no allocation, memset or synchronisation), so a caller may capture it.
+    Replay three times with new inputs written into the same buffers; every replay must equal the eager result."""
+    lib = _lib.load()
+    B, T, V = 4, 64, 30011
+    n = B * T
+    gd = torch.Generator(device=dev).manual_seed(5)
+    logits = torch.empty(n, V, dtype=torch.bfloat16, device=dev)
+    labels = torch.empty(n, dtype=torch.int64, device=dev)
+    old = torch.empty(n, device=dev); log_u = torch.empty(n, device=dev)
+    mask = torch.ones(n, dtype=torch.uint8, device=dev)
+    lp = torch.empty(n, device=dev); h = torch.empty(n, device=dev)
+    flag = torch.zeros(1, dtype=torch.int32, device=dev)
+    accept = torch.empty(n, dtype=torch.uint8, device=dev)
+    first = torch.empty(B, dtype=torch.int32, device=dev); prefix = torch.empty_like(first); near = torch.empty_like(first)
+    out_ids = torch.empty_like(labels); out_mask = torch.empty_like(mask)
+
+    def fill():
+        logits.copy_((torch.randn(n, V, generator=gd, device=dev) * 3).bfloat16())
+        labels.copy_(torch.randint(0, V, (n,), generator=gd, device=dev))
+        log_u.copy_(torch.log(torch.rand(n, generator=gd, device=dev)))
+        ref_lp, _ = vf.fused_logprob_entropy(logits, labels, n_splits=1)
+        old.copy_(ref_lp + torch.randn(n, generator=gd, device=dev) * 0.3)
+
+    def call(stream):
+        st = lib.vrl_fused_score_verify(
+            logits.data_ptr(), _lib.VRL_BF16, n, V, V, labels.data_ptr(), None, lp.data_ptr(), h.data_ptr(), None, None,
+            flag.data_ptr(), old.data_ptr(), log_u.data_ptr(), mask.data_ptr(), None, B, T, 0.0, 1e-6, accept.data_ptr(),
+            first.data_ptr(), prefix.data_ptr(), near.data_ptr(), labels.data_ptr(), 0, out_ids.data_ptr(),
+            out_mask.data_ptr(), stream)
+        assert st == 0
+
+    fill()
+    call(torch.cuda.current_stream(dev).cuda_stream)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        call(torch.cuda.current_stream(dev).cuda_stream)
+    for _ in range(3):
+        fill()
+        call(torch.cuda.current_stream(dev).cuda_stream)
+        torch.cuda.synchronize()
+        eager = [t.clone() for t in (lp, h, accept, first, prefix, near, out_ids, out_mask)]
+        for t in (lp, h, accept, first, prefix, near, out_ids, out_mask):
+            t.fill_(0) if t.dtype != torch.float32 else t.fill_(float("nan"))
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        for a, b in zip(eager, (lp, h, accept, first, prefix, near, out_ids, out_mask)):
+            assert torch.equal(a, b)
