@@ -206,3 +206,19 @@ def test_check_raises_with_text():
         _lib.check("vrl_rowscore", _lib.VRL_ERR_SHAPE)
     assert ei.value.status == _lib.VRL_ERR_SHAPE
     _lib.check("vrl_rowscore", _lib.VRL_OK)
+
+
+def test_header_is_plain_c(tmp_path):
+    """include/vrl.h must be usable from C (no C++ in the signatures): gcc -std=c99 compiles a user of it."""
+    import shutil
+    import subprocess
+
+    gcc = shutil.which("gcc")
+    if gcc is None:
+        pytest.skip("no gcc")
+    src = tmp_path / "user.c"
+    src.write_text('#include "vrl.h"\ntypedef int (*fn_t)(void);\nint main(void) { fn_t f = vrl_abi_version; (void)f; return VRL_OK; }\n')
+    inc = os.path.dirname(HEADER)
+    out = subprocess.run([gcc, "-std=c99", "-Wall", "-Wextra", "-Werror", "-pedantic", "-c", str(src), f"-I{inc}", "-o", str(tmp_path / "user.o")],
+                         stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    assert out.returncode == 0, out.stdout

@@ -1,0 +1,69 @@
+"""Seeded random shapes, strides, alignments, dtypes, temperatures and special values: the HIP row kernel (forward,
+both launch paths) against the fp64 C oracle and torch's NaN/inf pattern. 300 small cases, a few seconds."""
+
+import numpy as np
+import pytest
+import torch
+
+from verl_amd import torch_functional as vf
+from oracle import c_oracle, scoring
+
+pytestmark = pytest.mark.gpu
+
+DTYPES = [torch.float32, torch.bfloat16, torch.float16]
+
+
+def _case(rng, dev):
+    dtype = DTYPES[rng.integers(0, 3)]
+    n = int(rng.integers(1, 24))
+    V = int(rng.choice([rng.integers(1, 70), rng.integers(70, 3000), rng.integers(3000, 70000)]))
+    pad_l, pad_r = int(rng.integers(0, 9)), int(rng.integers(0, 9))
+    sigma = float(rng.choice([0.1, 1.0, 3.0, 8.0]))
+    shift = float(rng.choice([0.0, 0.0, -30.0, 50.0]))
+    g = torch.Generator(device=dev).manual_seed(int(rng.integers(0, 2**31)))
+    base = (torch.randn(n, pad_l + V + pad_r, generator=g, device=dev) * sigma + shift).to(dtype)
+    x = base[:, pad_l:pad_l + V]
+    lab = torch.randint(0, V, (n,), generator=g, device=dev)
+    temp = None
+    if rng.random() < 0.5:
+        temp = torch.rand(n, generator=g, device=dev) * 1.7 + 0.3
+    special = rng.random() < 0.25
+    if special and V > 3:
+        r = int(rng.integers(0, n))
+        cols = torch.randint(0, V, (max(1, V // 10),), generator=g, device=dev)
+        x[r, cols] = float("-inf")
+        lab[r] = int(((x[r] > float("-inf")).nonzero()[0]).item()) if bool((x[r] > float("-inf")).any()) else 0
+    splits = int(rng.choice([1, 1, 2, 3, 7]))
+    return x, lab, temp, splits, special
+
+
+def test_random_cases_against_fp64_oracle(dev):
+    rng = np.random.default_rng(20240607)
+    worst = 0.0
+    for i in range(300):
+        x, lab, temp, splits, special = _case(rng, dev)
+        lp, h, q = vf.fused_logprob_entropy(x, lab, temp, n_splits=splits, want_sum_pi_sq=True)
+        c_lp, c_h = c_oracle.rowscore(x.cpu().contiguous(), lab.cpu(), None if temp is None else temp.cpu())
+        got_lp, got_h = lp.cpu().double().numpy(), h.cpu().double().numpy()
+        assert np.array_equal(np.isnan(got_lp), np.isnan(c_lp)), i
+        assert np.array_equal(np.isnan(got_h), np.isnan(c_h)), i
+        fin = np.isfinite(c_lp)
+        # fp32 outputs: one ulp of the result plus the accumulation error. For 16-bit logits with a temperature
+        # the oracle (like the reference) rounds every quotient x/T to fp32 before reducing, the kernel does not
+        # (it folds 1/T into the exponent's multiplier); that rounding is half an fp32 ulp of the largest |x/T|.
+        slack = 0.0
+        if temp is not None and x.dtype != torch.float32:
+            xf = x.float()
+            zmax = float((xf[torch.isfinite(xf)].abs().max() / temp.min()).item())
+            slack = 2.4e-7 * zmax
+        tol_lp = 4e-6 + 2.4e-7 * np.abs(c_lp[fin]) + slack
+        assert np.all(np.abs(got_lp[fin] - c_lp[fin]) <= tol_lp), (i, np.abs(got_lp[fin] - c_lp[fin]).max())
+        finh = np.isfinite(c_h)
+        assert np.all(np.abs(got_h[finh] - c_h[finh]) <= 4e-6 + 2.4e-7 * np.abs(c_h[finh]) + slack), (i, np.abs(got_h[finh] - c_h[finh]).max())
+        worst = max(worst, float(np.abs(got_lp[fin] - c_lp[fin]).max(initial=0.0)), float(np.abs(got_h[finh] - c_h[finh]).max(initial=0.0)))
+        if not special:
+            z = x.float() if temp is None else scoring.apply_temperature(x.float(), temp)
+            ref_q = torch.softmax(z.double(), -1).pow(2).sum(-1)
+            assert ((q.double() - ref_q).abs() <= 1e-5 * ref_q + 1e-12).all(), i
+            assert bool((lp <= 1e-6).all()) and bool((h >= -1e-5).all())
+    print(f"worst absolute error over 300 cases: {worst:.2e}")
