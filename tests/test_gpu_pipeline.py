@@ -149,3 +149,39 @@ def test_entry_points_replay_from_a_graph(dev):
         torch.cuda.synchronize()
         for a, b in zip(eager, (lp, h, accept, first, prefix, near, out_ids, out_mask)):
             assert torch.equal(a, b)
+
+
+def test_two_threads_two_streams_are_independent(dev):
+    """The library keeps no state between calls: two host threads, each on its own stream with its own
+    buffers, get the same results as one thread alone."""
+    import threading
+
+    gd = torch.Generator(device=dev).manual_seed(77)
+    V = 50021
+    xs = [(torch.randn(300, V, generator=gd, device=dev) * 3).bfloat16() for _ in range(2)]
+    labs = [torch.randint(0, V, (300,), generator=gd, device=dev) for _ in range(2)]
+    expected = [vf.fused_logprob_entropy(x, l, 0.8) for x, l in zip(xs, labs)]
+    torch.cuda.synchronize()
+    results = [None, None]
+    errors = []
+
+    def work(i):
+        try:
+            s = torch.cuda.Stream(device=dev)
+            with torch.cuda.stream(s):
+                out = None
+                for _ in range(20):
+                    out = vf.fused_logprob_entropy(xs[i], labs[i], 0.8)
+                s.synchronize()
+            results[i] = out
+        except Exception as exc:  # surfaced below
+            errors.append(exc)
+
+    threads = [threading.Thread(target=work, args=(i,)) for i in range(2)]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    assert not errors, errors
+    for got, exp in zip(results, expected):
+        assert torch.equal(got[0], exp[0]) and torch.equal(got[1], exp[1])
