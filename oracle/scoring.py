@@ -153,3 +153,13 @@ def response_slice(values: torch.Tensor, prompt_lens, response_lens, max_respons
         piece = values[int(end) - r - 1 : int(end) - 1]
         rows.append(F.pad(piece, (*trailing, 0, max_response_len - r)))
     return torch.stack(rows, dim=0)
+
+
+def transpose_2d(x: torch.Tensor) -> torch.Tensor:
+    """Transposed contiguous copy, element bits untouched. The definition itself fixes the result
+    (out[c, r] = x[r, c]); numpy does the move, on the raw 16- or 32-bit patterns so that NaN payloads and
+    signed zeros cannot be normalised on the way."""
+    import numpy as np
+
+    words = x.contiguous().view(torch.int16 if x.element_size() == 2 else torch.int32).cpu().numpy()
+    return torch.from_numpy(np.ascontiguousarray(words.T)).view(x.dtype)

@@ -76,6 +76,28 @@ def test_bf16_module_3d_inputs(dev):
     torch.testing.assert_close(d_rw, d_w.float(), atol=2e-2, rtol=4e-2)
 
 
+def test_bf16_long_batch_uses_transposed_operands(dev):
+    """From 2048 tokens on the backward multiplies by a transposed copy of the weight (and always by a transposed
+    copy of the hidden chunk for 16-bit operands): same gradients as the products on the operands as stored."""
+    g = torch.Generator(device=dev).manual_seed(11)
+    T, D, V = 2304, 192, 20011
+    hidden = torch.empty(T, D, device=dev).uniform_(-0.5, 0.5, generator=g).bfloat16().requires_grad_()
+    weight = torch.empty(V, D, device=dev).uniform_(-0.5, 0.5, generator=g).bfloat16().requires_grad_()
+    labels = torch.randint(0, V, (T,), generator=g, device=dev)
+    g_lp = torch.empty(T, device=dev).uniform_(-1, 1, generator=g)
+    g_ent = torch.empty(T, device=dev).uniform_(-0.5, 0.5, generator=g)
+    lp, ent = fused_linear_for_ppo(hidden, weight, labels, 0.9, chunk_size=1000)
+    d_h, d_w = torch.autograd.grad((ent, lp), (hidden, weight), (g_ent, g_lp))
+    lp1, ent1 = fused_linear_for_ppo(hidden, weight, labels, 0.9)          # default chunk: one chunk here
+    assert torch.equal(lp, lp1) and torch.equal(ent, ent1)
+    hf = hidden.detach().float().requires_grad_()
+    wf = weight.detach().float().requires_grad_()
+    r_lp, r_ent = _torch_reference(hf, wf, labels, 0.9)
+    d_rh, d_rw = torch.autograd.grad((r_ent, r_lp), (hf, wf), (g_ent, g_lp))
+    torch.testing.assert_close(d_rh, d_h.float(), atol=2e-2, rtol=4e-2)
+    torch.testing.assert_close(d_rw, d_w.float(), atol=2e-2, rtol=4e-2)
+
+
 def test_input_checks(dev):
     h = torch.randn(4, 8, device=dev)
     w = torch.randn(16, 8, device=dev)

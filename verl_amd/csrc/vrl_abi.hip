@@ -11,6 +11,7 @@
 #include "layout_kernels.h"
 #include "rollout_corr_kernels.h"
 #include "rowscore_kernels.h"
+#include "transpose_kernels.h"
 #include "verify_kernels.h"
 
 namespace {
@@ -316,6 +317,38 @@ int vrl_response_slice(const float* values, const int64_t* cu_seqlens, const int
     return VRL_ERR_ALIGN;
   vrl::response_slice_kernel<<<dim3(static_cast<unsigned>(B)), dim3(256), 0, static_cast<hipStream_t>(stream)>>>(
       values, cu_seqlens, response_lens, T_out, out, err_flag);
+  return launch_status();
+}
+
+int vrl_transpose(const void* src, int elem_size, int64_t rows, int64_t cols, int64_t src_stride,
+                  void* dst, int64_t dst_stride, void* stream) {
+  if (elem_size != 2 && elem_size != 4) return VRL_ERR_DTYPE;
+  if (rows < 0 || cols < 0 || src_stride < cols || dst_stride < rows) return VRL_ERR_SHAPE;
+  if (rows == 0 || cols == 0) return VRL_OK;
+  if (src == nullptr || dst == nullptr) return VRL_ERR_NULL;
+  if (!aligned(src, elem_size) || !aligned(dst, elem_size)) return VRL_ERR_ALIGN;
+  {  // the two arrays must not share a byte
+    const char* s0 = static_cast<const char*>(src);
+    const char* s1 = s0 + ((rows - 1) * src_stride + cols) * elem_size;
+    const char* d0 = static_cast<const char*>(dst);
+    const char* d1 = d0 + ((cols - 1) * dst_stride + rows) * elem_size;
+    if (s0 < d1 && d0 < s1) return VRL_ERR_ARG;
+  }
+  const int tile = elem_size == 2 ? vrl::TransposeShape<2>::kTile : vrl::TransposeShape<4>::kTile;
+  const int64_t tiles_r = (rows + tile - 1) / tile;
+  const int64_t tiles_c = (cols + tile - 1) / tile;
+  if (tiles_r * tiles_c > kMaxGrid) return VRL_ERR_SHAPE;
+  const int vec_ok = aligned(src, 16) && aligned(dst, 16) && (src_stride * elem_size) % 16 == 0 &&
+                     (dst_stride * elem_size) % 16 == 0;
+  const dim3 grid(static_cast<unsigned>(tiles_r * tiles_c));
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  if (elem_size == 2) {
+    vrl::transpose_kernel<2><<<grid, dim3(256), 0, s>>>(static_cast<const char*>(src), rows, cols, src_stride,
+                                                        static_cast<char*>(dst), dst_stride, tiles_c, vec_ok);
+  } else {
+    vrl::transpose_kernel<4><<<grid, dim3(256), 0, s>>>(static_cast<const char*>(src), rows, cols, src_stride,
+                                                        static_cast<char*>(dst), dst_stride, tiles_c, vec_ok);
+  }
   return launch_status();
 }
 

@@ -2,7 +2,9 @@
 
 ``roll_labels`` restates the one-line label construction of the reference's engine
 (verl/workers/engine/fsdp/transformer_impl.py:1177); ``response_slice`` replaces the
-per-sequence Python loop of verl/workers/utils/padding.py:97-141 with one kernel launch.
+per-sequence Python loop of verl/workers/utils/padding.py:97-141 with one kernel launch;
+``transpose_2d`` is the bit-exact transposed copy the LM-head backward uses to give the library GEMM
+operands that are contiguous along the contraction axis.
 """
 
 from __future__ import annotations
@@ -13,7 +15,7 @@ import torch
 
 from . import _lib
 
-__all__ = ["roll_labels", "response_slice"]
+__all__ = ["roll_labels", "response_slice", "transpose_2d"]
 
 
 def roll_labels(input_ids_rmpad: torch.Tensor) -> torch.Tensor:
@@ -57,4 +59,31 @@ def response_slice(values: torch.Tensor, cu_seqlens: torch.Tensor, response_lens
     _lib.check("vrl_response_slice", st)
     if check and (int(flag.item()) & _lib.VRL_FLAG_SLICE_RANGE):
         raise ValueError("response_slice: a sequence has no prompt token, or a response length outside [0, max_response_len]")
+    return out
+
+
+def transpose_2d(x: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """Contiguous ``(cols, rows)`` copy of the 2-D tensor ``x`` (``rows, cols``; bf16, fp16 or fp32; any row
+    stride, unit column stride), bit for bit equal to ``x.t().contiguous()``. ``out`` may supply the result
+    buffer (same dtype, shape ``(cols, rows)``, unit column stride)."""
+    if not x.is_cuda:
+        raise RuntimeError(f"x is on {x.device}; verl_amd only runs on the GPU, it has no CPU implementation")
+    if x.dim() != 2:
+        raise ValueError(f"transpose_2d needs a 2-D tensor, got shape {tuple(x.shape)}")
+    if x.element_size() not in (2, 4) or x.is_complex():
+        raise TypeError(f"transpose_2d handles 2- and 4-byte element types, got {x.dtype}")
+    rows, cols = x.shape
+    if cols > 1 and x.stride(1) != 1 or (rows > 1 and x.stride(0) < cols):
+        x = x.contiguous()
+    if out is None:
+        out = torch.empty((cols, rows), dtype=x.dtype, device=x.device)
+    elif (out.dtype != x.dtype or tuple(out.shape) != (cols, rows) or out.device != x.device
+          or (rows > 1 and out.stride(1) != 1) or (cols > 1 and out.stride(0) < rows)):
+        raise ValueError("transpose_2d: out must be a (cols, rows) tensor of x's dtype and device with unit column stride")
+    lib = _lib.load()
+    with torch.cuda.device(x.device):
+        st = lib.vrl_transpose(x.data_ptr(), x.element_size(), rows, cols, x.stride(0) if rows > 1 else cols,
+                               out.data_ptr(), out.stride(0) if cols > 1 else rows,
+                               torch.cuda.current_stream(x.device).cuda_stream)
+    _lib.check("vrl_transpose", st)
     return out
