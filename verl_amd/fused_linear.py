@@ -41,7 +41,7 @@ def _score_chunk(lib, logits, labels, temp, lp, h, lse, flag, stream):
 
 class _FusedLinearForPPOFunction(torch.autograd.Function):
     @staticmethod
-    def forward(ctx, hidden, weight, input_ids, temperature, chunk_size):
+    def forward(ctx, hidden, weight, input_ids, temperature, chunk_size, keep_logits):
         ctx.set_materialize_grads(False)
         T, D = hidden.shape
         V = weight.shape[0]
@@ -53,12 +53,14 @@ class _FusedLinearForPPOFunction(torch.autograd.Function):
         flag = torch.zeros(1, dtype=torch.int32, device=dev)
         temp = None if temperature == 1.0 else torch.full((min(chunk_size, max(T, 1)),), float(temperature), **f32)
         lib = _lib.load()
-        buf = torch.empty((min(chunk_size, max(T, 1)), V), dtype=hidden.dtype, device=dev)
+        keep = bool(keep_logits) and T > 0 and (ctx.needs_input_grad[0] or ctx.needs_input_grad[1])
+        rows = T if keep else min(chunk_size, max(T, 1))
+        buf = torch.empty((rows, V), dtype=hidden.dtype, device=dev)
         with torch.cuda.device(dev):
             stream = torch.cuda.current_stream(dev).cuda_stream
             for lo in range(0, T, chunk_size):
                 hi = min(lo + chunk_size, T)
-                logits = buf[: hi - lo]
+                logits = buf[lo:hi] if keep else buf[: hi - lo]
                 torch.matmul(hidden[lo:hi], weight.t(), out=logits)
                 _score_chunk(lib, logits, input_ids[lo:hi], None if temp is None else temp[: hi - lo],
                              lp[lo:hi], h[lo:hi], lse[lo:hi], flag, stream)
@@ -67,13 +69,21 @@ class _FusedLinearForPPOFunction(torch.autograd.Function):
         ctx.save_for_backward(hidden, weight, input_ids, lse, h)
         ctx.temperature = float(temperature)
         ctx.chunk_size = int(chunk_size)
+        ctx.kept_logits = buf if keep else None
         return lp, h.clone()
 
     @staticmethod
     def backward(ctx, g_lp: Optional[torch.Tensor], g_h: Optional[torch.Tensor]):
         hidden, weight, input_ids, lse, h = ctx.saved_tensors
         if g_lp is None and g_h is None:
-            return None, None, None, None, None
+            return None, None, None, None, None, None
+        kept = ctx.kept_logits
+        if kept is not None:
+            ctx.kept_logits = None        # the gradient is written over them: they serve one backward
+        elif getattr(ctx, "kept_consumed", False):
+            raise RuntimeError("fused_linear_for_ppo(keep_logits=True): the kept logits were overwritten by the first "
+                               "backward; run the forward again, or use keep_logits=False")
+        ctx.kept_consumed = kept is not None
         T, D = hidden.shape
         V = weight.shape[0]
         dev = hidden.device
@@ -84,9 +94,9 @@ class _FusedLinearForPPOFunction(torch.autograd.Function):
         temp = None if ctx.temperature == 1.0 else torch.full((min(chunk, max(T, 1)),), ctx.temperature, **f32)
         need_dh, need_dw = ctx.needs_input_grad[0], ctx.needs_input_grad[1]
         d_hidden = torch.empty_like(hidden) if need_dh else None
-        d_weight = torch.zeros_like(weight) if need_dw else None
+        d_weight = (torch.empty_like(weight) if kept is not None else torch.zeros_like(weight)) if need_dw else None
         lib = _lib.load()
-        buf = torch.empty((min(chunk, max(T, 1)), V), dtype=hidden.dtype, device=dev)
+        buf = kept if kept is not None else torch.empty((min(chunk, max(T, 1)), V), dtype=hidden.dtype, device=dev)
         dt = _DTYPE_CODES[hidden.dtype]
         # For 16-bit operands the library GEMM is 25-35 % faster when both operands are contiguous along the
         # contraction axis (vocab for `d hidden`, tokens for `d W`); fp32 runs at the fp32 matrix peak either way.
@@ -97,29 +107,45 @@ class _FusedLinearForPPOFunction(torch.autograd.Function):
             for lo in range(0, T, chunk):
                 hi = min(lo + chunk, T)
                 n = hi - lo
-                logits = buf[:n]
-                torch.matmul(hidden[lo:hi], weight.t(), out=logits)
+                if kept is not None:
+                    logits = buf[lo:hi]
+                else:
+                    logits = buf[:n]
+                    torch.matmul(hidden[lo:hi], weight.t(), out=logits)
                 st = lib.vrl_rowscore_backward(
                     logits.data_ptr(), dt, n, V, logits.stride(0) if n > 1 else V, input_ids[lo:hi].data_ptr(),
                     None if temp is None else temp.data_ptr(), lse[lo:hi].data_ptr(), h[lo:hi].data_ptr(),
                     None if gl is None else gl[lo:hi].data_ptr(), None if gh is None else gh[lo:hi].data_ptr(),
                     logits.data_ptr(), logits.stride(0) if n > 1 else V, stream)   # gradient over the logits, in place
                 _lib.check("vrl_rowscore_backward", st)
+                if kept is not None:
+                    continue
                 if need_dh:
                     torch.matmul(logits, weight if weight_t is None else weight_t.t(), out=d_hidden[lo:hi])
                 if need_dw:
                     d_weight.addmm_(logits.t(), transpose_2d(hidden[lo:hi]).t() if half else hidden[lo:hi])
-        return d_hidden, d_weight, None, None, None
+            if kept is not None:
+                # the gradient over all tokens' logits is in `kept`: one product each, nothing to accumulate
+                if need_dh:
+                    torch.matmul(kept, weight if weight_t is None else weight_t.t(), out=d_hidden)
+                if need_dw:
+                    torch.matmul(kept.t(), transpose_2d(hidden).t() if half else hidden, out=d_weight)
+        return d_hidden, d_weight, None, None, None, None
 
 
 def fused_linear_for_ppo(hidden_states: torch.Tensor, vocab_weights: torch.Tensor, input_ids: torch.Tensor,
-                         temperature: float = 1.0, chunk_size: int = DEFAULT_CHUNK_TOKENS):
+                         temperature: float = 1.0, chunk_size: int = DEFAULT_CHUNK_TOKENS, keep_logits: bool = False):
     """(log_probs fp32, entropy fp32) of ``softmax((hidden_states @ vocab_weights.T) / temperature)`` at ``input_ids``.
 
     ``hidden_states`` is ``(tokens, hidden)`` or ``(batch, seq, hidden)`` with ``input_ids`` of the matching leading
     shape; ``vocab_weights`` is ``(vocab, hidden)``; both bf16, fp16 or fp32 on the GPU. Differentiable with respect
     to both. ``chunk_size`` tokens are projected at a time (one reusable ``(chunk_size, vocab)`` buffer); the result
-    does not depend on it, the default is sized for this GPU rather than the reference's 512.
+    depends on it only through the order in which the library sums a product of that height; the default is sized for
+    this GPU rather than the reference's 512.
+
+    ``keep_logits=True`` trades memory for time when gradients are needed: the forward keeps all
+    ``tokens x vocab`` logits (2.5 GB for 8192 x 152064 bf16), the backward writes their gradient over them instead of
+    projecting again and forms ``d hidden`` and ``d W`` with one product each. Such a graph can be differentiated once.
     """
     if not hidden_states.is_cuda or not vocab_weights.is_cuda:
         raise RuntimeError("fused_linear_for_ppo: tensors must be on the GPU; verl_amd has no CPU implementation")
@@ -138,16 +164,19 @@ def fused_linear_for_ppo(hidden_states: torch.Tensor, vocab_weights: torch.Tenso
     lead = hidden_states.shape[:-1]
     h2 = hidden_states.reshape(-1, hidden_states.shape[-1]).contiguous()
     ids = input_ids.reshape(-1).to(torch.int64).contiguous()
-    lp, ent = _FusedLinearForPPOFunction.apply(h2, vocab_weights.contiguous(), ids, float(temperature), int(chunk_size))
+    lp, ent = _FusedLinearForPPOFunction.apply(h2, vocab_weights.contiguous(), ids, float(temperature), int(chunk_size),
+                                               bool(keep_logits))
     return lp.reshape(lead), ent.reshape(lead)
 
 
 class FusedLinearForPPO(torch.nn.Module):
     """Module form, constructed and called like verl's (verl/utils/experimental/torch_functional.py:211-231)."""
 
-    def __init__(self, chunk_size: int = DEFAULT_CHUNK_TOKENS):
+    def __init__(self, chunk_size: int = DEFAULT_CHUNK_TOKENS, keep_logits: bool = False):
         super().__init__()
         self.chunk_size = chunk_size
+        self.keep_logits = keep_logits
 
     def forward(self, hidden_states, vocab_weights, input_ids, temperature: float = 1.0):
-        return fused_linear_for_ppo(hidden_states, vocab_weights, input_ids, temperature, self.chunk_size)
+        return fused_linear_for_ppo(hidden_states, vocab_weights, input_ids, temperature, self.chunk_size,
+                                    self.keep_logits)
