@@ -323,28 +323,37 @@ def bench_verify_only(args, dev):
     print(json.dumps(out), flush=True)
 
 
-def cpu_baseline(step: Step, budget_s: float = 20.0):
-    """The torch restatement of the reference composition on the host cores, on a slice of the same batch."""
+def cpu_baseline(step: Step, budget_s: float = 12.0, runs: int = 4):
+    """The torch restatement of the reference composition on the host cores, on a slice of the same batch.
+    A pilot on 1024 rows sizes the slice so that `runs` timed runs take about `budget_s` seconds together."""
     from oracle import scoring, verify as overify  # checker/baseline only
 
     w = step.w
-    rows = min(step.n, 1024)
-    x = step.logits[:rows].cpu()
-    lab = step.labels[:rows].cpu()
-    temp = None if step.temp is None else step.temp[:rows].cpu()
-    old = step.lp_old[:rows].cpu().view(1, rows)
-    lu = step.log_u[:rows].cpu().view(1, rows)
-    mk = step.mask8[:rows].cpu().view(1, rows)
 
-    def once():
-        t0 = time.perf_counter()
-        lp, h = scoring.score_reference(x, lab, temp)
-        overify.verify(lp.float().view(1, rows), old, lu, mk, step.off)
-        return time.perf_counter() - t0
+    def make(rows):
+        x = step.logits[:rows].cpu()
+        lab = step.labels[:rows].cpu()
+        temp = None if step.temp is None else step.temp[:rows].cpu()
+        old = step.lp_old[:rows].cpu().view(1, rows)
+        lu = step.log_u[:rows].cpu().view(1, rows)
+        mk = step.mask8[:rows].cpu().view(1, rows)
 
-    first = once()
-    reps = max(1, min(5, int(budget_s / max(first, 1e-3)) - 1))
-    times = [first] + [once() for _ in range(reps)]
+        def once():
+            t0 = time.perf_counter()
+            lp, h = scoring.score_reference(x, lab, temp)
+            overify.verify(lp.float().view(1, rows), old, lu, mk, step.off)
+            return time.perf_counter() - t0
+
+        return once
+
+    pilot_rows = min(step.n, 1024)
+    pilot = make(pilot_rows)
+    pilot()                                   # first touch: thread pool, allocator
+    per_row = pilot() / pilot_rows
+    rows = int(budget_s / runs / max(per_row, 1e-9))
+    rows = max(pilot_rows, min(step.n, 32768, rows // 1024 * 1024))
+    once = make(rows)
+    times = [once() for _ in range(runs)]
     best = statistics.median(times)
     return {
         "value": rows / best,
@@ -352,7 +361,8 @@ def cpu_baseline(step: Step, budget_s: float = 20.0):
         "cores": torch.get_num_threads(),
         "kind": "port",
         "sample": f"{rows} rows of the same batch (V={w.V}, {str(w.dtype).replace('torch.', '')}), "
-                  f"median of {len(times)} runs, torch {torch.__version__} on {os.cpu_count()} logical CPUs",
+                  f"median of {len(times)} runs ({sum(times):.1f} s of CPU work), torch {torch.__version__} on "
+                  f"{os.cpu_count()} logical CPUs",
     }
 
 
