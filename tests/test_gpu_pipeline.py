@@ -90,6 +90,12 @@ def test_installed_shims_send_gpu_tensors_to_the_hip_path(dev):
         xg = x.clone().requires_grad_(True)               # update_actor: gradient through the HIP backward
         tf.logprobs_from_logits(xg * 1.0, lab, inplace_backward=True).sum().backward()
         assert xg.grad is not None and hook.stats()["hip_calls"] == 5
+        # the engines wrap the entropy function in torch.compile (fsdp/transformer_impl.py:164-168 in the reference):
+        # the shim is run as it is, not traced
+        compiled = torch.compile(tf.entropy_from_logits, dynamic=True)
+        assert torch.equal(compiled(x), vf.entropy_from_logits(x))
+        assert torch.equal(compiled(x[:3]), vf.entropy_from_logits(x[:3]))
+        assert hook.stats()["hip_calls"] == 7
     finally:
         hook.uninstall()
         for k, v in saved.items():

@@ -119,6 +119,16 @@ def strerror(status: int) -> str:
     return load().vrl_strerror(status).decode()
 
 
+def stream_ptr(device) -> int:
+    """The raw ``hipStream_t`` of torch's current stream on ``device``, as the integer the ``void* stream`` arguments
+    take. Read from the runtime directly: the ``torch.cuda.Stream`` wrapper is replaced by a generic object without a
+    handle inside functions that torch.compile was told not to trace."""
+    import torch
+
+    index = device.index if getattr(device, "index", None) is not None else torch.cuda.current_device()
+    return int(torch._C._cuda_getCurrentRawStream(index))
+
+
 def check(func: str, status: int) -> None:
     """Raise VrlCallError for a negative status."""
     if status == VRL_OK:

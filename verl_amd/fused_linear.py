@@ -57,7 +57,7 @@ class _FusedLinearForPPOFunction(torch.autograd.Function):
         rows = T if keep else min(chunk_size, max(T, 1))
         buf = torch.empty((rows, V), dtype=hidden.dtype, device=dev)
         with torch.cuda.device(dev):
-            stream = torch.cuda.current_stream(dev).cuda_stream
+            stream = _lib.stream_ptr(dev)
             for lo in range(0, T, chunk_size):
                 hi = min(lo + chunk_size, T)
                 logits = buf[lo:hi] if keep else buf[: hi - lo]
@@ -103,7 +103,7 @@ class _FusedLinearForPPOFunction(torch.autograd.Function):
         half = hidden.element_size() == 2
         weight_t = transpose_2d(weight) if (half and need_dh and T >= _WEIGHT_TRANSPOSE_MIN_TOKENS) else None
         with torch.cuda.device(dev):
-            stream = torch.cuda.current_stream(dev).cuda_stream
+            stream = _lib.stream_ptr(dev)
             for lo in range(0, T, chunk):
                 hi = min(lo + chunk, T)
                 n = hi - lo

@@ -63,6 +63,10 @@ def _make_shim(name: str, original: Callable) -> Callable:
         _stats["passed_to_verl"] += 1
         return original(logits, *args, **kwargs)
 
+    # The engines wrap entropy_from_logits in torch.compile when use_torch_compile is set
+    # (verl/workers/engine/fsdp/transformer_impl.py:164-168). There is nothing to trace in a ctypes call into a
+    # finished kernel, so the tracer is told to run the shim as it is.
+    shim = torch.compiler.disable(shim)
     shim.__verl_amd_original__ = original
     return shim
 

@@ -55,7 +55,7 @@ def response_slice(values: torch.Tensor, cu_seqlens: torch.Tensor, response_lens
     lib = _lib.load()
     with torch.cuda.device(dev):
         st = lib.vrl_response_slice(v.data_ptr(), cu.data_ptr(), rl.data_ptr(), B, T, out.data_ptr(), flag.data_ptr(),
-                                    torch.cuda.current_stream(dev).cuda_stream)
+                                    _lib.stream_ptr(dev))
     _lib.check("vrl_response_slice", st)
     if check and (int(flag.item()) & _lib.VRL_FLAG_SLICE_RANGE):
         raise ValueError("response_slice: a sequence has no prompt token, or a response length outside [0, max_response_len]")
@@ -84,6 +84,6 @@ def transpose_2d(x: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.T
     with torch.cuda.device(x.device):
         st = lib.vrl_transpose(x.data_ptr(), x.element_size(), rows, cols, x.stride(0) if rows > 1 else cols,
                                out.data_ptr(), out.stride(0) if cols > 1 else rows,
-                               torch.cuda.current_stream(x.device).cuda_stream)
+                               _lib.stream_ptr(x.device))
     _lib.check("vrl_transpose", st)
     return out

@@ -171,7 +171,7 @@ def _launch(old, roll, mask8, *, is_mode=0, icepop=False, is_upper=1.0, is_lower
                                   _lib._c.cast(lo, _lib._c.c_void_p), _lib._c.cast(hi, _lib._c.c_void_p),
                                   None if res.weights is None else res.weights.data_ptr(),
                                   None if res.keep is None else res.keep.data_ptr(), stats.data_ptr(), bits.data_ptr(),
-                                  torch.cuda.current_stream(dev).cuda_stream)
+                                  _lib.stream_ptr(dev))
     _lib.check("vrl_rollout_corr", st)
     table = torch.cat([stats, bits.to(torch.float32).unsqueeze(1)], dim=1).cpu().numpy()  # the one copy to the host
     res.stats = table[:, :ns].astype(np.float64)

@@ -171,7 +171,7 @@ def spec_verify(
 
     lib = _lib.load()
     with torch.cuda.device(dev):
-        stream = torch.cuda.current_stream(dev).cuda_stream
+        stream = _lib.stream_ptr(dev)
         st = lib.vrl_spec_verify(
             ln.data_ptr(), lo.data_ptr(), lu.data_ptr(), _ptr(m8), _ptr(cu), B, T, off, float(near_eps),
             accept.data_ptr(), first.data_ptr(), prefix.data_ptr(), near.data_ptr(),
@@ -207,7 +207,7 @@ def truncate_draft(
     out_mask = torch.empty(shape, dtype=torch.uint8, device=dev)
     lib = _lib.load()
     with torch.cuda.device(dev):
-        stream = torch.cuda.current_stream(dev).cuda_stream
+        stream = _lib.stream_ptr(dev)
         st = lib.vrl_truncate_draft(ids.data_ptr(), _ptr(m8), _ptr(cu), B, T, fr.data_ptr(), int(pad_id),
                                     out_ids.data_ptr(), out_mask.data_ptr(), stream)
     _lib.check("vrl_truncate_draft", st)
@@ -265,7 +265,7 @@ def fused_score_verify(
 
     lib = _lib.load()
     with torch.cuda.device(dev):
-        stream = torch.cuda.current_stream(dev).cuda_stream
+        stream = _lib.stream_ptr(dev)
         st = lib.vrl_fused_score_verify(
             x.data_ptr(), _DTYPE_CODES[x.dtype], n, V, x.stride(0) if n > 1 else V, lab.data_ptr(), _ptr(temp),
             out_lp.data_ptr(), out_h.data_ptr(), None, None, flag.data_ptr(),

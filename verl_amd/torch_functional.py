@@ -106,7 +106,7 @@ def _forward_2d(x, lab, temp, want_logprob, want_entropy, want_sum_pi_sq, want_l
     stride = x.stride(0) if n > 1 else V
     splits = lib.vrl_rowscore_split_plan(dt, n, V) if n_splits is None else int(n_splits)
     with torch.cuda.device(dev):
-        stream = torch.cuda.current_stream(dev).cuda_stream
+        stream = _lib.stream_ptr(dev)
         if splits > 1:
             partials = torch.empty(n * splits * 4, **f32)
             st = lib.vrl_rowscore_split(
@@ -152,7 +152,7 @@ class _RowScoreFunction(torch.autograd.Function):
                 st = lib.vrl_rowscore_backward(
                     x.data_ptr(), _DTYPE_CODES[x.dtype], n, V, x.stride(0) if n > 1 else V, _ptr(lab), _ptr(temp),
                     lse.data_ptr(), h.data_ptr(), _ptr(gl), _ptr(gh), dx.data_ptr(), dx.stride(0) if n > 1 else V,
-                    torch.cuda.current_stream(dev).cuda_stream,
+                    _lib.stream_ptr(dev),
                 )
             _lib.check("vrl_rowscore_backward", st)
         return dx, None, None, None, None, None, None
