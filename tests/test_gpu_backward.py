@@ -133,3 +133,20 @@ def test_full_vocab_bf16_c3_shape_slice(dev):
     w1 = torch.randn(n, generator=g, device=dev)
     w2 = torch.randn(n, generator=g, device=dev)
     _compare(_ours(x, lab, temp, w1, w2), _reference_grad(x, lab, temp, w1, w2).bfloat16(), torch.bfloat16)
+
+
+@pytest.mark.parametrize("use_reentrant", [False, True])
+def test_entropy_under_activation_checkpointing(dev, use_reentrant):
+    """The engines may wrap the entropy function in torch.utils.checkpoint (entropy_checkpointing,
+    fsdp/transformer_impl.py:1371-1374 in the reference): the forward then runs twice, the gradient is the same."""
+    from torch.utils.checkpoint import checkpoint
+
+    g = torch.Generator(device=dev).manual_seed(21)
+    x = (torch.randn(40, 5003, generator=g, device=dev) * 2).requires_grad_(True)
+    w = torch.randn(40, generator=g, device=dev)
+    (vf.entropy_from_logits(x * 1.0) * w).sum().backward()
+    plain = x.grad.clone()
+    x.grad = None
+    h = checkpoint(vf.entropy_from_logits, x * 1.0, use_reentrant=use_reentrant)
+    (h * w).sum().backward()
+    assert torch.equal(x.grad, plain)
