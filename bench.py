@@ -2,6 +2,8 @@
 """Benchmark of the fused score + SPEC-RL verify path on one MI355X.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c2|c3|c4|c1|c5]
+    python bench.py --backward [--workload ...]          (the row op's backward kernel)
+    python bench.py --lm-head [--chunk N] [--keep-logits]  (LM head + scoring without the full logits)
 
 One step = one pass of vrl_fused_score_verify (row kernel + verify kernel, through
 the C ABI, outputs preallocated) over the whole synthetic batch, logits resident
@@ -323,6 +325,74 @@ def bench_verify_only(args, dev):
     print(json.dumps(out), flush=True)
 
 
+def bench_lm_head(args, dev):
+    """LM head + scoring without the full logits (verl_amd.fused_linear) at c3's micro-batch: 8192 tokens, hidden
+    3584 (Qwen2.5-7B), vocab 152064 bf16, temperature 1.5; forward and forward + backward. The step is bound by the
+    library GEMMs, so the roofline object is the bf16 matrix peak over the algorithmic flops (2*T*D*V forward,
+    4*T*D*V backward; the second projection of the backward is not algorithmic)."""
+    from verl_amd.fused_linear import fused_linear_for_ppo
+    from verl_amd.layout import transpose_2d
+
+    T, D, V = 8192, 3584, 152064
+    g = torch.Generator(device=dev).manual_seed(4000)
+    hidden = torch.empty(T, D, device=dev).uniform_(-0.5, 0.5, generator=g).bfloat16().requires_grad_()
+    weight = (torch.empty(V, D, device=dev).uniform_(-0.5, 0.5, generator=g) * 0.05).bfloat16().requires_grad_()
+    ids = torch.randint(0, V, (T,), generator=g, device=dev)
+    g_lp = torch.randn(T, generator=g, device=dev)
+    g_h = torch.randn(T, generator=g, device=dev) * 0.01
+    temperature, chunk, keep = 1.5, args.chunk, args.keep_logits
+
+    def fwd():
+        with torch.no_grad():
+            return fused_linear_for_ppo(hidden, weight, ids, temperature, chunk)
+
+    def fwd_bwd():
+        lp, h = fused_linear_for_ppo(hidden, weight, ids, temperature, chunk, keep)
+        return torch.autograd.grad((lp, h), (hidden, weight), (g_lp, g_h))
+
+    # guard: first tokens against torch in fp32 on the bf16 logits the same GEMM produces
+    lp, h = fwd()
+    z = torch.matmul(hidden[:256].detach(), weight.detach().t()).float() / temperature
+    e1 = (lp[:256] - torch.log_softmax(z, -1).gather(-1, ids[:256, None]).squeeze(-1)).abs().max().item()
+    e2 = (h[:256] - (torch.logsumexp(z, -1) - (torch.softmax(z, -1) * z).sum(-1))).abs().max().item()
+    if not (e1 <= 2e-3 and e2 <= 2e-3):
+        raise SystemExit(f"bench: LM-head scores disagree with torch (logprob {e1}, entropy {e2})")
+
+    def timed(fn):
+        spin_up(fn, 300.0)
+        for _ in range(args.warmup):
+            fn()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            fn()
+        torch.cuda.synchronize()
+        return (time.perf_counter() - t0) / args.steps
+
+    t_f = timed(fwd)
+    t_fb = timed(fwd_bwd)
+    wt = torch.empty(D, V, dtype=weight.dtype, device=dev)
+    t_tr = timed(lambda: transpose_2d(weight.detach(), wt))
+    flops_f, flops_fb = 2.0 * T * D * V, 6.0 * T * D * V
+    print(json.dumps({
+        "metric": "tokens/sec of LM head + scoring, forward + backward, never holding more than one chunk of logits",
+        "value": T / t_fb, "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": t_fb * 1e3, "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16",
+        "data": "synthetic",
+        "config": {"workload": "lm_head_8192x3584_v152064_bf16", "chunk_tokens": chunk, "keep_logits": keep,
+                   "temperature": temperature,
+                   "step": "verl_amd.fused_linear_for_ppo forward + torch.autograd.grad for hidden and weight"},
+        "forward_ms": t_f * 1e3,
+        "forward_tokens_per_s": T / t_f,
+        "roofline": {"bound": "mfma", "achieved": flops_fb / t_fb / 1e12, "peak": 2500.0, "unit": "TFLOP/s",
+                     "frac": flops_fb / t_fb / 1e12 / 2500.0, "traffic": None,
+                     "kernel": "hipBLASLt bf16 GEMMs (library) + rowscore_kernel + rowscore_backward_kernel",
+                     "forward_tflops": flops_f / t_f / 1e12},
+        "weight_transpose": {"ms": t_tr * 1e3, "gbps": 2.0 * V * D * 2 / t_tr / 1e9, "kernel": "transpose_kernel<2>"},
+        "parity_guard": {"rows": 256, "max_abs_err_logprob": e1, "max_abs_err_entropy": e2},
+    }), flush=True)
+
+
 def cpu_baseline(step: Step, budget_s: float = 12.0, runs: int = 4):
     """The torch restatement of the reference composition on the host cores, on a slice of the same batch.
     A pilot on 1024 rows sizes the slice so that `runs` timed runs take about `budget_s` seconds together."""
@@ -376,6 +446,10 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--backward", action="store_true",
                     help="time vrl_rowscore_backward on the workload instead of the fused forward step")
+    ap.add_argument("--lm-head", action="store_true",
+                    help="time the LM head + scoring step (verl_amd.fused_linear) instead of the fused forward step")
+    ap.add_argument("--chunk", type=int, default=4096, help="--lm-head: tokens projected at a time")
+    ap.add_argument("--keep-logits", action="store_true", help="--lm-head: keep the logits for the backward")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run a plain device copy of known size (for scaling rocprofv3 byte counters)")
     args = ap.parse_args()
@@ -389,6 +463,9 @@ def main():
 
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
+    if args.lm_head:
+        bench_lm_head(args, dev)
+        return
     if args.workload == "c5":
         bench_verify_only(args, dev)
         return
