@@ -131,6 +131,24 @@ def test_split_and_slice_argument_errors(lib):
     assert g(None, None, None, 0, 4, None, None, None) == _lib.VRL_OK
 
 
+def test_transpose_argument_errors(lib):
+    t = lib.vrl_transpose
+    Q = P + (1 << 20)                      # a second, disjoint address
+    assert t(P, 1, 4, 4, 4, Q, 4, None) == _lib.VRL_ERR_DTYPE
+    assert t(P, 8, 4, 4, 4, Q, 4, None) == _lib.VRL_ERR_DTYPE
+    assert t(P, 2, -1, 4, 4, Q, 4, None) == _lib.VRL_ERR_SHAPE
+    assert t(P, 2, 4, 4, 3, Q, 4, None) == _lib.VRL_ERR_SHAPE      # source pitch below the column count
+    assert t(P, 2, 4, 4, 4, Q, 3, None) == _lib.VRL_ERR_SHAPE      # destination pitch below the row count
+    assert t(None, 2, 4, 4, 4, Q, 4, None) == _lib.VRL_ERR_NULL
+    assert t(P, 2, 4, 4, 4, None, 4, None) == _lib.VRL_ERR_NULL
+    assert t(P + 1, 2, 4, 4, 4, Q, 4, None) == _lib.VRL_ERR_ALIGN
+    assert t(P, 4, 4, 4, 4, Q + 2, 4, None) == _lib.VRL_ERR_ALIGN
+    assert t(P, 4, 4, 4, 4, P, 4, None) == _lib.VRL_ERR_ARG        # in place
+    assert t(P, 4, 4, 4, 4, P + 60, 4, None) == _lib.VRL_ERR_ARG   # last source word = first destination word
+    assert t(None, 2, 0, 4, 4, None, 4, None) == _lib.VRL_OK       # nothing to move
+    assert t(None, 4, 4, 0, 0, None, 4, None) == _lib.VRL_OK
+
+
 def test_rollout_corr_argument_errors(lib):
     import ctypes
 
