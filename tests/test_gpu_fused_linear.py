@@ -8,7 +8,7 @@ with inputs drawn like there (uniform(-0.5, 0.5), temperature 1.5).
 import pytest
 import torch
 
-from verl_amd.fused_linear import FusedLinearForPPO, fused_linear_for_ppo
+from verl_amd.fused_linear import linear_cross_entropy, FusedLinearForPPO, fused_linear_for_ppo
 
 pytestmark = pytest.mark.gpu
 
@@ -128,6 +128,40 @@ def test_keep_logits_same_results_one_backward(dev, dtype):
     mod = FusedLinearForPPO(chunk_size=512, keep_logits=True)
     lp3, ent3 = mod(hidden, weight, labels, 1.3)
     assert torch.equal(lp3, lp0)
+
+
+def test_linear_cross_entropy_call_and_reductions(dev):
+    """The call of the reference's Triton-backed function (verl/utils/kernel/linear_cross_entropy.py:38-119): 3-D
+    hidden states, flattened fp32 outputs, reduction on the log-probs only; checked the way the reference checks its
+    kernel against torch (tests/utils/test_linear_cross_entropy.py:211-224)."""
+    g = torch.Generator(device=dev).manual_seed(9)
+    B, S, D, V = 2, 70, 128, 4099
+    hidden = torch.empty(B, S, D, device=dev).uniform_(-0.5, 0.5, generator=g).requires_grad_()
+    weight = torch.empty(V, D, device=dev).uniform_(-0.5, 0.5, generator=g).requires_grad_()
+    labels = torch.randint(0, V, (B, S), generator=g, device=dev)
+    ref_lp, ref_ent = _torch_reference(hidden.detach().view(-1, D), weight.detach(), labels.view(-1), 1.5)
+    lp, ent = linear_cross_entropy(hidden, weight, labels, 1.5, "none")
+    assert lp.shape == (B * S,) and ent.shape == (B * S,) and lp.dtype == torch.float32
+    torch.testing.assert_close(lp, ref_lp, atol=1e-4, rtol=1e-4)
+    torch.testing.assert_close(ent, ref_ent, atol=1e-4, rtol=1e-4)
+    for red, want in (("sum", ref_lp.sum()), ("mean", ref_lp.mean()), ("MEAN", ref_lp.mean())):
+        lp_r, ent_r = linear_cross_entropy(hidden, weight, labels, 1.5, red)
+        assert lp_r.shape == () and ent_r.shape == (B * S,)
+        torch.testing.assert_close(lp_r, want, atol=1e-3, rtol=1e-4)
+    lp_m, ent_m = linear_cross_entropy(hidden, weight, labels, 1.5, "mean")
+    (lp_m + ent_m.sum()).backward()
+    hf = hidden.detach().clone().requires_grad_()
+    wf = weight.detach().clone().requires_grad_()
+    r_lp, r_ent = _torch_reference(hf.view(-1, D), wf, labels.view(-1), 1.5)
+    (r_lp.mean() + r_ent.sum()).backward()
+    torch.testing.assert_close(hidden.grad, hf.grad, atol=1e-4, rtol=1e-4)
+    torch.testing.assert_close(weight.grad, wf.grad, atol=1e-4, rtol=1e-4)
+    with pytest.raises(ValueError, match="Invalid reduction"):
+        linear_cross_entropy(hidden, weight, labels, 1.5, "max")
+    with pytest.raises(TypeError):
+        linear_cross_entropy(hidden, weight, labels, 1)
+    with pytest.raises(NotImplementedError):
+        linear_cross_entropy(hidden, weight, labels, 1.5, "none", dist_process_group=object())
 
 
 def test_input_checks(dev):

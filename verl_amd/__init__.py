@@ -12,9 +12,9 @@ Setting ``VERL_USE_EXTERNAL_MODULES=verl_amd.plugin`` makes verl import
 """
 
 from . import rollout_corr
-from .fused_linear import FusedLinearForPPO, fused_linear_for_ppo
+from .fused_linear import FusedLinearForPPO, fused_linear_for_ppo, linear_cross_entropy
 from .hook import install, uninstall
-from .layout import response_slice, roll_labels
+from .layout import response_slice, roll_labels, transpose_2d
 from .spec_rl import (
     VerifyResult,
     draw_log_uniforms,
@@ -40,6 +40,7 @@ __all__ = [
     "uninstall",
     "FusedLinearForPPO",
     "fused_linear_for_ppo",
+    "linear_cross_entropy",
     "VerifyResult",
     "draw_log_uniforms",
     "fused_score_verify",
@@ -48,6 +49,7 @@ __all__ = [
     "truncate_draft",
     "response_slice",
     "roll_labels",
+    "transpose_2d",
     "calculate_sum_pi_squared_from_logits",
     "entropy_from_logits",
     "entropy_from_logits_with_chunking",

@@ -20,7 +20,7 @@ from . import _lib
 from .layout import transpose_2d
 from .torch_functional import _DTYPE_CODES, _ptr
 
-__all__ = ["FusedLinearForPPO", "fused_linear_for_ppo", "DEFAULT_CHUNK_TOKENS"]
+__all__ = ["FusedLinearForPPO", "fused_linear_for_ppo", "linear_cross_entropy", "DEFAULT_CHUNK_TOKENS"]
 
 # The reference's default is 512 tokens per chunk. On a 288 GB part a (4096, 152064) bf16 buffer is 1.2 GB, the
 # projection reaches 1.4 PFLOP/s instead of 0.86 at 512, and the weight gradient is accumulated 8x less often.
@@ -167,6 +167,30 @@ def fused_linear_for_ppo(hidden_states: torch.Tensor, vocab_weights: torch.Tenso
     lp, ent = _FusedLinearForPPOFunction.apply(h2, vocab_weights.contiguous(), ids, float(temperature), int(chunk_size),
                                                bool(keep_logits))
     return lp.reshape(lead), ent.reshape(lead)
+
+
+def linear_cross_entropy(hidden: torch.Tensor, weight: torch.Tensor, labels: torch.Tensor, temperature: float = 1.0,
+                         reduction: str = "none", dist_process_group=None):
+    """Same call as the reference's Triton-backed ``linear_cross_entropy``
+    (verl/utils/kernel/linear_cross_entropy.py:38-119): ``hidden`` ``(..., hidden_size)``, ``weight``
+    ``(vocab, hidden_size)``, ``labels`` ``(...)`` -> ``(logprobs, entropy)``, both fp32 over the flattened tokens.
+    ``reduction`` ("none", "sum", "mean") applies to the log-probs only, as there (verl/utils/kernel/kernels.py:431-438);
+    the entropy stays per token. Served by ``fused_linear_for_ppo``. A vocabulary sharded over a process group is not
+    part of this one-GPU build and raises."""
+    if dist_process_group is not None:
+        raise NotImplementedError("linear_cross_entropy: a vocabulary sharded over a process group is not supported")
+    if not isinstance(temperature, float):
+        raise TypeError(f"temperature must be a float, but got {type(temperature)}")
+    red = str(reduction).lower()
+    if red not in ("none", "sum", "mean"):
+        raise ValueError(f"Invalid reduction: {reduction}")
+    h2 = hidden.reshape(-1, hidden.shape[-1])
+    lp, ent = fused_linear_for_ppo(h2, weight, labels.reshape(-1), temperature)
+    if red == "sum":
+        lp = lp.sum()
+    elif red == "mean":
+        lp = lp.mean()
+    return lp, ent
 
 
 class FusedLinearForPPO(torch.nn.Module):
