@@ -443,6 +443,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--workload", default="c2", choices=["c1", "c2", "c3", "c4", "c5"],
                     help="c5 times the verify kernel alone (its logits do not fit; they are scored like c3)")
+    ap.add_argument("--vocab", type=int, default=0, help="run the workload's recipe at another vocabulary size")
+    ap.add_argument("--seqs", type=int, default=0, help="... with another number of sequences")
+    ap.add_argument("--dtype", choices=["bf16", "f32"], default=None, help="... with another logits element type")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--backward", action="store_true",
                     help="time vrl_rowscore_backward on the workload instead of the fused forward step")
@@ -473,6 +476,16 @@ def main():
         bench_backward(args, dev)
         return
     w = synthetic.WORKLOADS[args.workload]
+    if args.vocab or args.seqs or args.dtype:
+        # the workload's recipe at another vocabulary / batch / element type (e.g. 32000, 128256, 129280, 262144)
+        kw = {"name": w.name + "_resized"}
+        if args.vocab:
+            kw["V"] = args.vocab
+        if args.seqs:
+            kw["B"] = args.seqs
+        if args.dtype:
+            kw["dtype"] = {"bf16": torch.bfloat16, "f32": torch.float32}[args.dtype]
+        w = w.scaled(**kw)
     step = Step(w, dev, seed=1000 * int(args.workload[1]))
     err_lp, err_h = step.check_against_torch()
 
@@ -545,7 +558,7 @@ def main():
             "peak": HBM_PEAK_GBPS,
             "unit": "GB/s",
             "frac": achieved / HBM_PEAK_GBPS,
-            "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload),
+            "traffic": None if (args.vocab or args.seqs or args.dtype) else MEASURED_TRAFFIC_BYTES.get(args.workload),
             "kernel": "rowscore_kernel",
             "avg_kernel_ms": avg_kern_ms,
             "algorithmic_bytes_per_launch": bytes_score,
