@@ -191,6 +191,18 @@ def test_label_out_of_range_raises(dev):
     assert torch.isnan(lp[2]) and torch.isfinite(lp[[0, 1, 3]]).all()
 
 
+def test_label_check_can_be_switched_off_for_the_reference_named_functions(dev, monkeypatch):
+    """The check costs one host synchronisation per call; with the module switch off the call returns without
+    reading anything back and the bad row is NaN."""
+    x = torch.randn(4, 50, device=dev)
+    lab = torch.tensor([0, 1, 50, 3], device=dev)
+    monkeypatch.setattr(vf, "LABEL_CHECK", False)
+    lp = vf.logprobs_from_logits(x, lab)
+    assert torch.isnan(lp[2]) and torch.isfinite(lp[[0, 1, 3]]).all()
+    with pytest.raises(IndexError):
+        vf.fused_logprob_entropy(x, lab, check_labels=True)      # an explicit request still checks
+
+
 def test_rejects_cpu_and_unsupported_inputs(dev):
     with pytest.raises(RuntimeError, match="no CPU implementation"):
         vf.logprobs_from_logits(torch.randn(2, 10), torch.zeros(2, dtype=torch.long))

@@ -25,6 +25,7 @@ import numpy as np
 import torch
 
 from . import _lib
+from . import torch_functional as _tf
 from .torch_functional import _DTYPE_CODES, _check_logits, _ptr, _rows_2d, _temperature_rows
 
 __all__ = ["VerifyResult", "draw_log_uniforms", "thresh_offset_from_lenience", "spec_verify", "truncate_draft", "fused_score_verify"]
@@ -231,7 +232,7 @@ def fused_score_verify(
     cu_seqlens: Optional[torch.Tensor] = None,
     draft_ids: Optional[torch.Tensor] = None,
     pad_id: int = 0,
-    check_labels: bool = True,
+    check_labels: Optional[bool] = None,
 ):
     """Score ``logits`` and verify the draft in one call: (log-probs, entropy, VerifyResult).
 
@@ -274,6 +275,8 @@ def fused_score_verify(
             _ptr(ids), int(pad_id), _ptr(out_ids), _ptr(out_mask), stream,
         )
     _lib.check("vrl_fused_score_verify", st)
+    if check_labels is None:
+        check_labels = _tf.LABEL_CHECK
     if check_labels and (int(flag.item()) & _lib.VRL_FLAG_LABEL_OOB):
         raise IndexError(f"fused_score_verify: a label is outside [0, {V})")
     res = VerifyResult(

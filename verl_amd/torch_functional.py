@@ -19,6 +19,7 @@ HIP backward kernel (vrl_rowscore_backward).
 
 from __future__ import annotations
 
+import os
 from typing import Optional, Union
 
 import torch
@@ -34,6 +35,11 @@ __all__ = [
     "calculate_sum_pi_squared_from_logits",
     "fused_logprob_entropy",
 ]
+
+# Raising IndexError for a label outside [0, vocab) means reading the kernel's error flag back, i.e. one host
+# synchronisation per call. Callers that must not synchronise (graph capture, deep launch queues) switch it off here
+# or with VERL_AMD_LABEL_CHECK=0; such a row's log-prob is NaN either way.
+LABEL_CHECK = os.environ.get("VERL_AMD_LABEL_CHECK", "1") not in ("0", "false", "False")
 
 _DTYPE_CODES = {torch.float32: _lib.VRL_F32, torch.bfloat16: _lib.VRL_BF16, torch.float16: _lib.VRL_F16}
 
@@ -166,7 +172,7 @@ def rowscore(
     want_logprob: bool = True,
     want_entropy: bool = True,
     want_sum_pi_sq: bool = False,
-    check_labels: bool = True,
+    check_labels: Optional[bool] = None,
     n_splits: Optional[int] = None,
     inplace_backward: bool = False,
     what: str = "rowscore",
@@ -177,9 +183,12 @@ def rowscore(
     With few rows the work of one row is spread over ``n_splits`` workgroups (vrl_rowscore_split);
     ``n_splits=None`` lets the library choose, 1 forces one workgroup per row. When grad is enabled
     and the logits require it, log-prob and entropy are differentiable with respect to the logits
-    (vrl_rowscore_backward); the sum of squared probabilities is not.
+    (vrl_rowscore_backward); the sum of squared probabilities is not. ``check_labels`` (default: the module's
+    ``LABEL_CHECK``) reads the kernel's error flag back and raises IndexError for a label outside the vocabulary.
     """
     _check_logits(logits, what)
+    if check_labels is None:
+        check_labels = LABEL_CHECK
     if not (want_logprob or want_entropy or want_sum_pi_sq):
         raise ValueError(f"{what}: nothing to compute")
     lead = logits.shape[:-1]
@@ -274,7 +283,7 @@ def fused_logprob_entropy(
     labels: torch.Tensor,
     temperature: Union[None, float, torch.Tensor] = None,
     *,
-    check_labels: bool = True,
+    check_labels: Optional[bool] = None,
     want_sum_pi_sq: bool = False,
     n_splits: Optional[int] = None,
 ):
