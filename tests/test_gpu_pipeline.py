@@ -105,6 +105,49 @@ def test_installed_shims_send_gpu_tensors_to_the_hip_path(dev):
                 sys.modules[k] = v
 
 
+def test_installed_fused_linear_entry_points_serve_gpu_tensors(dev):
+    from verl_amd.fused_linear import fused_linear_for_ppo
+
+    class RefModule(torch.nn.Module):
+        def __init__(self, chunk_size=512):
+            super().__init__()
+
+        def forward(self, hidden_states, vocab_weights, input_ids, temperature=1.0):
+            raise AssertionError("GPU tensors must not reach the stand-in reference module")
+
+    def ref_lce(*a, **k):
+        raise AssertionError("GPU tensors must not reach the stand-in reference function")
+
+    names = ("verl", "verl.utils", "verl.utils.torch_functional", "verl.utils.experimental",
+             "verl.utils.experimental.torch_functional", "verl.utils.kernel", "verl.utils.kernel.linear_cross_entropy")
+    mods = {n: types.ModuleType(n) for n in names}
+    mods["verl.utils.experimental.torch_functional"].FusedLinearForPPO = RefModule
+    mods["verl.utils.kernel.linear_cross_entropy"].linear_cross_entropy = ref_lce
+    saved = {k: sys.modules.get(k) for k in mods}
+    sys.modules.update(mods)
+    try:
+        hook.install()
+        g = torch.Generator(device=dev).manual_seed(2)
+        h = torch.empty(2, 30, 64, device=dev).uniform_(-0.5, 0.5, generator=g).bfloat16()
+        w = torch.empty(1000, 64, device=dev).uniform_(-0.5, 0.5, generator=g).bfloat16()
+        ids = torch.randint(0, 1000, (2, 30), generator=g, device=dev)
+        want = fused_linear_for_ppo(h, w, ids, 1.2)
+        mod = mods["verl.utils.experimental.torch_functional"].FusedLinearForPPO()
+        got = mod.forward(hidden_states=h, vocab_weights=w, input_ids=ids, temperature=1.2)   # dense_common.py:122-128
+        assert torch.equal(got[0], want[0]) and torch.equal(got[1], want[1])
+        lce = mods["verl.utils.kernel.linear_cross_entropy"].linear_cross_entropy
+        lp, ent = lce(h, w, ids, 1.2, "none")                                                   # dense_common.py:189-195
+        assert torch.equal(lp, want[0].reshape(-1)) and torch.equal(ent, want[1].reshape(-1))
+        assert hook.stats() == {"hip_calls": 2, "passed_to_verl": 0}
+    finally:
+        hook.uninstall()
+        for k, v in saved.items():
+            if v is None:
+                sys.modules.pop(k, None)
+            else:
+                sys.modules[k] = v
+
+
 def test_entry_points_replay_from_a_graph(dev):
     """The C ABI only enqueues kernels (no allocation, memset or synchronisation), so a caller may capture it.
     Replay three times with new inputs written into the same buffers; every replay must equal the eager result."""

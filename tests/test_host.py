@@ -119,6 +119,45 @@ def test_install_patches_module_and_bound_names(fake_verl):
     assert inst.stats() == {"hip_calls": 0, "passed_to_verl": 0}
 
 
+def test_install_patches_the_fused_linear_entry_points_when_present(fake_verl):
+    mods, _ = fake_verl
+
+    class RefModule:
+        def __init__(self, chunk_size=512):
+            self.chunk_size = chunk_size
+
+        def forward(self, hidden_states, vocab_weights, input_ids, temperature=1.0):
+            return ("verl", "FusedLinearForPPO", self.chunk_size)
+
+    def ref_lce(hidden, weight, labels, temperature=1.0, reduction="none", dist_process_group=None):
+        return ("verl", "linear_cross_entropy", reduction)
+
+    extra = {n: types.ModuleType(n) for n in ("verl.utils.experimental", "verl.utils.experimental.torch_functional",
+                                                "verl.utils.kernel", "verl.utils.kernel.linear_cross_entropy")}
+    extra["verl.utils.experimental.torch_functional"].FusedLinearForPPO = RefModule
+    extra["verl.utils.kernel.linear_cross_entropy"].linear_cross_entropy = ref_lce
+    sys.modules.update(extra)
+    try:
+        replaced = inst.install()
+        assert "verl.utils.experimental.torch_functional.FusedLinearForPPO" in replaced
+        assert "verl.utils.kernel.linear_cross_entropy.linear_cross_entropy" in replaced
+        cls = extra["verl.utils.experimental.torch_functional"].FusedLinearForPPO
+        assert cls is not RefModule and cls.__verl_amd_original__ is RefModule
+        h, w, ids = torch.randn(3, 8), torch.randn(16, 8), torch.zeros(3, dtype=torch.long)
+        # CPU tensors: the reference's own module and function serve the call, constructed as the caller asked
+        assert cls().forward(hidden_states=h, vocab_weights=w, input_ids=ids, temperature=1.0) == ("verl", "FusedLinearForPPO", 512)
+        assert cls(64).forward(h, w, ids) == ("verl", "FusedLinearForPPO", 64)
+        lce = extra["verl.utils.kernel.linear_cross_entropy"].linear_cross_entropy
+        assert lce(h, w, ids, 1.0, "mean") == ("verl", "linear_cross_entropy", "mean")
+        assert inst.stats()["passed_to_verl"] == 3
+        inst.uninstall()
+        assert extra["verl.utils.experimental.torch_functional"].FusedLinearForPPO is RefModule
+        assert extra["verl.utils.kernel.linear_cross_entropy"].linear_cross_entropy is ref_lce
+    finally:
+        for n in extra:
+            sys.modules.pop(n, None)
+
+
 def test_plugin_module_installs_on_import(fake_verl):
     mods, _ = fake_verl
     tf = mods["verl.utils.torch_functional"]

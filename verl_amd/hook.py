@@ -10,6 +10,11 @@ verl/workers/engine/fsdp/transformer_impl.py:66 and siblings; the reference's
 own tests patch exactly that bound name,
 tests/workers/test_distillation_topk_symmetry_on_cpu.py:143-146).
 
+Also replaced, when the modules import (they are opt-in paths of the reference, use_fused_kernels):
+    verl.utils.experimental.torch_functional.FusedLinearForPPO :211-231
+    verl.utils.kernel.linear_cross_entropy.linear_cross_entropy :119
+which the model forwards look up at call time (verl/models/transformers/dense_common.py:89,157).
+
 A replaced function sends GPU tensors of a supported dtype to the HIP kernels
 (forward, and backward when the logits need a gradient). Anything else (CPU
 tensors on the driver, fp64) is handed to the function it replaced, i.e. verl's own
@@ -25,6 +30,7 @@ from typing import Callable, Dict, List, Tuple
 
 import torch
 
+from . import fused_linear as _fl
 from . import torch_functional as _amd
 
 TARGET_MODULE = "verl.utils.torch_functional"
@@ -71,6 +77,52 @@ def _make_shim(name: str, original: Callable) -> Callable:
     return shim
 
 
+def _eligible_pair(hidden, weight) -> bool:
+    return (_eligible(hidden) and isinstance(weight, torch.Tensor) and weight.is_cuda and weight.dtype == hidden.dtype
+            and weight.dim() == 2)
+
+
+def _make_fused_linear_class(original_cls):
+    class FusedLinearForPPO(_fl.FusedLinearForPPO):
+        """verl_amd's module with the reference's class as the fallback for inputs the kernels do not take."""
+
+        def __init__(self, chunk_size=None):
+            super().__init__(_fl.DEFAULT_CHUNK_TOKENS if chunk_size is None else chunk_size)
+            self._verl_module = original_cls() if chunk_size is None else original_cls(chunk_size)
+
+        def forward(self, hidden_states, vocab_weights, input_ids, temperature=1.0):
+            if _eligible_pair(hidden_states, vocab_weights):
+                _stats["hip_calls"] += 1
+                return super().forward(hidden_states, vocab_weights, input_ids, temperature)
+            _stats["passed_to_verl"] += 1
+            return self._verl_module.forward(hidden_states, vocab_weights, input_ids, temperature)
+
+    FusedLinearForPPO.__verl_amd_original__ = original_cls
+    return FusedLinearForPPO
+
+
+def _make_linear_cross_entropy(original):
+    @functools.wraps(original)
+    def linear_cross_entropy(hidden, weight, labels, temperature=1.0, reduction="none", dist_process_group=None):
+        if dist_process_group is None and _eligible_pair(hidden, weight):
+            _stats["hip_calls"] += 1
+            return _fl.linear_cross_entropy(hidden, weight, labels, temperature, reduction)
+        _stats["passed_to_verl"] += 1
+        return original(hidden, weight, labels, temperature, reduction, dist_process_group)
+
+    linear_cross_entropy = torch.compiler.disable(linear_cross_entropy)
+    linear_cross_entropy.__verl_amd_original__ = original
+    return linear_cross_entropy
+
+
+# (module below the package root, attribute, shim factory)
+_OPTIONAL_TARGETS = (
+    ("utils.experimental.torch_functional", "FusedLinearForPPO", _make_fused_linear_class),
+    ("utils.kernel.linear_cross_entropy", "linear_cross_entropy", _make_linear_cross_entropy),
+)
+_optional_patched: List[Tuple[object, str, object]] = []
+
+
 def stats() -> dict:
     """Calls served by the HIP kernel vs handed back to verl since install()."""
     return dict(_stats)
@@ -105,6 +157,17 @@ def install(target_module: str = TARGET_MODULE) -> List[str]:
                 _rebound.append((other, name, _originals[name]))
                 replaced.append(f"{mod_name}.{name}")
     _installed_in.append(mod)
+    for sub, name, factory in _OPTIONAL_TARGETS:
+        try:
+            other = importlib.import_module(root + sub)
+        except ImportError:
+            continue
+        original = getattr(other, name, None)
+        if original is None:
+            continue
+        setattr(other, name, factory(original))
+        _optional_patched.append((other, name, original))
+        replaced.append(f"{root}{sub}.{name}")
     return replaced
 
 
@@ -121,5 +184,8 @@ def uninstall() -> None:
             setattr(mod, name, original)
     _installed_in.clear()
     _originals.clear()
+    for other, name, original in _optional_patched:
+        setattr(other, name, original)
+    _optional_patched.clear()
     _stats["hip_calls"] = 0
     _stats["passed_to_verl"] = 0
