@@ -127,6 +127,19 @@ int vrl_response_slice(const float* values, const int64_t* cu_seqlens, const int
                        int64_t B, int64_t T_out, float* out, int32_t* err_flag, void* stream);
 
 /*
+ * vrl_response_pack — packed per-token values (total_nnz,) -> packed response values (sum of response_lens,):
+ *   out[out_offsets[b] + j] = values[cu_seqlens[b+1] - response_lens[b] - 1 + j],  j < response_lens[b]
+ * out_offsets is the caller's exclusive prefix sum of response_lens (B+1 entries, last = out_total).
+ * A sequence without a prompt token, a negative length, or a window that is not exactly
+ * [out_offsets[b], out_offsets[b+1]) inside the output sets VRL_FLAG_SLICE_RANGE and writes nothing for it.
+ *
+ * Replaces verl/workers/utils/padding.py:194-210 (response_from_nested) for fp32 per-token vectors.
+ */
+int vrl_response_pack(const float* values, const int64_t* cu_seqlens, const int64_t* response_lens,
+                      const int64_t* out_offsets, int64_t B, int64_t out_total, float* out, int32_t* err_flag,
+                      void* stream);
+
+/*
  * vrl_transpose — out-of-place transposition of a 2-D array of 2-byte (bf16, fp16) or
  * 4-byte (fp32) elements, bit for bit:
  *   dst[c * dst_stride + r] = src[r * src_stride + c],   r < rows, c < cols

@@ -155,6 +155,17 @@ def response_slice(values: torch.Tensor, prompt_lens, response_lens, max_respons
     return torch.stack(rows, dim=0)
 
 
+def response_from_nested(values: torch.Tensor, seq_offsets, response_lens):
+    """Packed model output -> packed response part: for each sequence values[end - resp_len - 1 : end - 1], joined.
+    Returns (values, offsets) as the jagged tensor of verl/workers/utils/padding.py:194-210 holds them;
+    ``seq_offsets`` are that function's ``tensor.offsets()`` (B+1 entries)."""
+    response_lens = [int(r) for r in response_lens]
+    ends = [int(e) for e in seq_offsets][1:]
+    pieces = [values[end - r - 1 : end - 1] for r, end in zip(response_lens, ends, strict=True)]
+    offsets = np.concatenate([[0], np.cumsum(response_lens)]).astype(np.int64)
+    return (torch.cat(pieces) if pieces else values[:0]), torch.from_numpy(offsets)
+
+
 def transpose_2d(x: torch.Tensor) -> torch.Tensor:
     """Transposed contiguous copy, element bits untouched. The definition itself fixes the result
     (out[c, r] = x[r, c]); numpy does the move, on the raw 16- or 32-bit patterns so that NaN payloads and

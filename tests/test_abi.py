@@ -131,6 +131,18 @@ def test_split_and_slice_argument_errors(lib):
     assert g(None, None, None, 0, 4, None, None, None) == _lib.VRL_OK
 
 
+def test_response_pack_argument_errors(lib):
+    g = lib.vrl_response_pack
+    assert g(P, P, P, P, -1, 4, P, P, None) == _lib.VRL_ERR_SHAPE
+    assert g(P, P, P, P, 2, -1, P, P, None) == _lib.VRL_ERR_SHAPE
+    assert g(None, P, P, P, 2, 4, P, P, None) == _lib.VRL_ERR_NULL
+    assert g(P, P, P, None, 2, 4, P, P, None) == _lib.VRL_ERR_NULL
+    assert g(P, P, P, P, 2, 4, None, P, None) == _lib.VRL_ERR_NULL
+    assert g(P, P, P, P, 2, 4, P, None, None) == _lib.VRL_ERR_NULL
+    assert g(P, P, P, P + 4, 2, 4, P, P, None) == _lib.VRL_ERR_ALIGN
+    assert g(None, None, None, None, 0, 0, None, None, None) == _lib.VRL_OK
+
+
 def test_transpose_argument_errors(lib):
     t = lib.vrl_transpose
     Q = P + (1 << 20)                      # a second, disjoint address

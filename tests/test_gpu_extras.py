@@ -134,3 +134,31 @@ def test_response_slice_random_and_errors(dev):
     out = layout.response_slice(vals.to(dev), cu.to(dev), resp.to(dev), int(resp.max()) - 1, check=False)
     assert torch.all(out[resp.argmax()] == 0)
     assert layout.response_slice(vals[:0].to(dev), cu[:1].to(dev), resp[:0].to(dev), 4).shape == (0, 4)
+
+
+def test_response_from_packed_matches_oracle_and_flags_bad_sequences(dev):
+    g = torch.Generator().manual_seed(14)
+    B = 53
+    prompt = torch.randint(1, 40, (B,), generator=g)
+    resp = torch.randint(0, 700, (B,), generator=g)
+    resp[7] = 0
+    cu = torch.zeros(B + 1, dtype=torch.int64)
+    cu[1:] = torch.cumsum(prompt + resp, 0)
+    vals = torch.randn(int(cu[-1]), generator=g)
+    got, got_cu = layout.response_from_packed(vals.to(dev), cu.to(dev), resp.to(dev))
+    ref, ref_cu = scoring.response_from_nested(vals, cu.tolist(), resp.tolist())
+    assert torch.equal(got.cpu(), ref) and torch.equal(got_cu.cpu(), ref_cu)
+    # the reference fixture's windows: full[2:4] and full[6:7]
+    full = torch.arange(8, dtype=torch.float32, device=dev)
+    v, o = layout.response_from_packed(full, torch.tensor([0, 5, 8], device=dev), torch.tensor([2, 1], device=dev))
+    assert v.tolist() == [2.0, 3.0, 6.0] and o.tolist() == [0, 2, 3]
+    with pytest.raises(ValueError):   # a sequence without a prompt token
+        layout.response_from_packed(vals.to(dev), cu.to(dev), (prompt + resp).to(dev))
+    bad = resp.clone()
+    bad[3] = -2
+    with pytest.raises(ValueError):
+        layout.response_from_packed(vals.to(dev), cu.to(dev), bad.to(dev))
+    out, out_cu = layout.response_from_packed(vals[:0].to(dev), cu[:1].to(dev), resp[:0].to(dev))
+    assert out.shape == (0,) and out_cu.tolist() == [0]
+    with pytest.raises(RuntimeError, match="no CPU implementation"):
+        layout.response_from_packed(vals, cu, resp)

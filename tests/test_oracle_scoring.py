@@ -252,6 +252,26 @@ def test_response_slice_reference_fixture():
         scoring.response_slice(full, prompt_lens=[3, 2], response_lens=[2, 2])
 
 
+def test_response_from_nested_is_the_padded_slice_without_its_padding():
+    """verl/workers/utils/padding.py:194-210 takes the same window per sequence as no_padding_2_padding (:135-138)
+    and joins the pieces instead of padding them: on the reference's fixture the pieces are full[2:4] and full[6:7]."""
+    full = torch.arange(8, dtype=torch.float32) * 1.5
+    vals, offs = scoring.response_from_nested(full, [0, 5, 8], [2, 1])
+    assert torch.equal(vals, torch.cat([full[2:4], full[6:7]])) and offs.tolist() == [0, 2, 3]
+    g = torch.Generator().manual_seed(8)
+    prompt = torch.randint(1, 9, (20,), generator=g)
+    resp = torch.randint(0, 30, (20,), generator=g)
+    cu = [0] + torch.cumsum(prompt + resp, 0).tolist()
+    x = torch.randn(cu[-1], generator=g)
+    vals, offs = scoring.response_from_nested(x, cu, resp.tolist())
+    padded = scoring.response_slice(x, prompt.tolist(), resp.tolist())
+    for b in range(20):
+        r = int(resp[b])
+        assert torch.equal(vals[offs[b]:offs[b + 1]], padded[b, :r]) and int(offs[b + 1] - offs[b]) == r
+    with pytest.raises(ValueError):
+        scoring.response_from_nested(x, cu, resp.tolist()[:-1])     # strict zip, like the reference's
+
+
 def test_roll_is_global_not_per_shard():
     """tests/models/test_fused_kernels_ulysses_sp_on_cpu.py:69-90: roll then slice differs from slice then roll
     exactly at shard boundaries."""

@@ -25,4 +25,25 @@ __global__ __launch_bounds__(256) void response_slice_kernel(
   for (int64_t j = threadIdx.x; j < T_out; j += 256) dst[j] = (ok && j < r) ? values[first + j] : 0.f;
 }
 
+// Packed in, packed out: the response positions of sequence b, shifted like above, go to
+// out[out_offsets[b] .. out_offsets[b] + r). grid.x = B, block = 256.
+__global__ __launch_bounds__(256) void response_pack_kernel(
+    const float* __restrict__ values, const int64_t* __restrict__ cu_seqlens,
+    const int64_t* __restrict__ response_lens, const int64_t* __restrict__ out_offsets, int64_t out_total,
+    float* __restrict__ out, int32_t* err_flag) {
+  const int64_t b = blockIdx.x;
+  const int64_t begin = cu_seqlens[b];
+  const int64_t end = cu_seqlens[b + 1];
+  const int64_t r = response_lens[b];
+  const int64_t first = end - r - 1;
+  const int64_t o = out_offsets[b];
+  // the output window must be the caller's prefix sum of the response lengths and lie inside the output
+  const bool ok = (r >= 0) && (first >= begin) && (o >= 0) && (o + r <= out_total) && (out_offsets[b + 1] - o == r);
+  if (!ok) {
+    if (threadIdx.x == 0) atomicOr(err_flag, 2);
+    return;  // no barrier follows
+  }
+  for (int64_t j = threadIdx.x; j < r; j += 256) out[o + j] = values[first + j];
+}
+
 }  // namespace vrl

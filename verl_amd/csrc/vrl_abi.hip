@@ -320,6 +320,22 @@ int vrl_response_slice(const float* values, const int64_t* cu_seqlens, const int
   return launch_status();
 }
 
+int vrl_response_pack(const float* values, const int64_t* cu_seqlens, const int64_t* response_lens,
+                      const int64_t* out_offsets, int64_t B, int64_t out_total, float* out, int32_t* err_flag,
+                      void* stream) {
+  if (B < 0 || out_total < 0 || B > kMaxGrid) return VRL_ERR_SHAPE;
+  if (B == 0) return VRL_OK;
+  if (values == nullptr || cu_seqlens == nullptr || response_lens == nullptr || out_offsets == nullptr ||
+      err_flag == nullptr || (out == nullptr && out_total > 0))
+    return VRL_ERR_NULL;
+  if (!aligned(values, 4) || !aligned(cu_seqlens, 8) || !aligned(response_lens, 8) || !aligned(out_offsets, 8) ||
+      !aligned(out, 4) || !aligned(err_flag, 4))
+    return VRL_ERR_ALIGN;
+  vrl::response_pack_kernel<<<dim3(static_cast<unsigned>(B)), dim3(256), 0, static_cast<hipStream_t>(stream)>>>(
+      values, cu_seqlens, response_lens, out_offsets, out_total, out, err_flag);
+  return launch_status();
+}
+
 int vrl_transpose(const void* src, int elem_size, int64_t rows, int64_t cols, int64_t src_stride,
                   void* dst, int64_t dst_stride, void* stream) {
   if (elem_size != 2 && elem_size != 4) return VRL_ERR_DTYPE;

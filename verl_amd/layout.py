@@ -15,7 +15,7 @@ import torch
 
 from . import _lib
 
-__all__ = ["roll_labels", "response_slice", "transpose_2d"]
+__all__ = ["roll_labels", "response_slice", "response_from_packed", "transpose_2d"]
 
 
 def roll_labels(input_ids_rmpad: torch.Tensor) -> torch.Tensor:
@@ -60,6 +60,39 @@ def response_slice(values: torch.Tensor, cu_seqlens: torch.Tensor, response_lens
     if check and (int(flag.item()) & _lib.VRL_FLAG_SLICE_RANGE):
         raise ValueError("response_slice: a sequence has no prompt token, or a response length outside [0, max_response_len]")
     return out
+
+
+def response_from_packed(values: torch.Tensor, cu_seqlens: torch.Tensor, response_lens: torch.Tensor,
+                         check: bool = True):
+    """Packed per-token fp32 ``values`` (total_nnz,) -> (packed response values ``(sum(response_lens),)``, their
+    ``cu_seqlens`` ``(B+1,)`` int64): sequence b contributes ``values[end_b - r_b - 1 : end_b - 1]``. The packed
+    counterpart of ``response_slice``; the reference does it with a Python loop and ``as_nested_tensor``
+    (verl/workers/utils/padding.py:194-210), to whose ``(values, offsets)`` pair the two results correspond."""
+    if not values.is_cuda:
+        raise RuntimeError(f"values is on {values.device}; verl_amd only runs on the GPU, it has no CPU implementation")
+    if values.dim() != 1:
+        raise ValueError(f"values must be 1-D (total_nnz,), got shape {tuple(values.shape)}")
+    dev = values.device
+    v = values.to(torch.float32).contiguous()
+    cu = cu_seqlens.to(device=dev, dtype=torch.int64).contiguous()
+    rl = response_lens.to(device=dev, dtype=torch.int64).contiguous()
+    B = rl.numel()
+    if cu.numel() != B + 1:
+        raise ValueError(f"cu_seqlens must have B+1 = {B + 1} entries, got {cu.numel()}")
+    out_cu = torch.zeros(B + 1, dtype=torch.int64, device=dev)
+    if B > 0:
+        out_cu[1:] = torch.cumsum(rl.clamp(min=0), 0)
+    total = int(out_cu[-1].item()) if B > 0 else 0
+    out = torch.empty(total, dtype=torch.float32, device=dev)
+    flag = torch.zeros(1, dtype=torch.int32, device=dev)
+    lib = _lib.load()
+    with torch.cuda.device(dev):
+        st = lib.vrl_response_pack(v.data_ptr(), cu.data_ptr(), rl.data_ptr(), out_cu.data_ptr(), B, total,
+                                   out.data_ptr() if total > 0 else None, flag.data_ptr(), _lib.stream_ptr(dev))
+    _lib.check("vrl_response_pack", st)
+    if check and (int(flag.item()) & _lib.VRL_FLAG_SLICE_RANGE):
+        raise ValueError("response_from_packed: a sequence has no prompt token, or a negative response length")
+    return out, out_cu
 
 
 def transpose_2d(x: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:
