@@ -150,3 +150,29 @@ def test_entropy_under_activation_checkpointing(dev, use_reentrant):
     h = checkpoint(vf.entropy_from_logits, x * 1.0, use_reentrant=use_reentrant)
     (h * w).sum().backward()
     assert torch.equal(x.grad, plain)
+
+
+def test_fp32_peaked_rows_at_low_temperature_stay_as_close_to_fp64_as_torch(dev):
+    """|z| ~ 100 (logits up to 35 at temperature 0.36): the exponent must not pick up roundings of size ulp(|z|) that
+    torch's own fp32 autograd does not have. Compared with the fp64 gradient of the same composition."""
+    g = torch.Generator(device=dev).manual_seed(31)
+    n, V = 6, 58902
+    x = torch.randn(n, V, generator=g, device=dev) * 8.0
+    x[torch.arange(n), torch.randint(0, V, (n,), generator=g, device=dev)] = 35.0
+    lab = torch.randint(0, V, (n,), generator=g, device=dev)
+    temp = torch.tensor([0.36, 0.5, 0.7, 1.0, 1.8, 0.36], device=dev)
+    g1 = torch.randn(n, generator=g, device=dev)
+    g2 = torch.randn(n, generator=g, device=dev) * 0.3
+
+    def grad(xx, fn, cast):
+        xx = xx.requires_grad_(True)
+        lp, h = fn(xx)
+        ((lp * g1.to(cast)).sum() + (h * g2.to(cast)).sum()).backward()
+        return xx.grad
+
+    g64 = grad(x.double(), lambda t: scoring.score_reference(t, lab, temp.double()), torch.float64)
+    g32 = grad(x.clone(), lambda t: scoring.score_reference(t, lab, temp), torch.float32)
+    ours = grad(x.clone(), lambda t: vf.fused_logprob_entropy(t, lab, temp), torch.float32)
+    e_torch = (g32.double() - g64).abs().max().item()
+    e_ours = (ours.double() - g64).abs().max().item()
+    assert e_ours <= 2.0 * e_torch + 2e-6, (e_ours, e_torch)

@@ -67,3 +67,30 @@ def test_random_cases_against_fp64_oracle(dev):
             assert ((q.double() - ref_q).abs() <= 1e-5 * ref_q + 1e-12).all(), i
             assert bool((lp <= 1e-6).all()) and bool((h >= -1e-5).all())
     print(f"worst absolute error over 300 cases: {worst:.2e}")
+
+
+def test_random_cases_backward_against_torch_autograd(dev):
+    """Gradients of (log-prob, entropy) for the same random cases against torch's autograd of the fp32 composition:
+    absolute 4e-6 x the gradient scale for fp32 logits, plus one rounding step of the output type for 16-bit logits."""
+    rng = np.random.default_rng(777)
+    worst = 0.0
+    for i in range(400):
+        x, lab, temp, splits, special = _case(rng, dev)
+        if special:
+            continue
+        g = torch.Generator(device=dev).manual_seed(i)
+        g1 = torch.randn(x.shape[0], generator=g, device=dev)
+        g2 = torch.randn(x.shape[0], generator=g, device=dev) * 0.3
+        xr = x.detach().float().requires_grad_(True)
+        lpr, hr = scoring.score_reference(xr, lab, temp)
+        ((lpr * g1).sum() + (hr * g2).sum()).backward()
+        xo = x.detach().clone().requires_grad_(True)
+        lp, h = vf.fused_logprob_entropy(xo, lab, temp, n_splits=splits)
+        ((lp * g1).sum() + (h * g2).sum()).backward()
+        scale = float((g1.abs() + g2.abs() * 30).max()) / (1.0 if temp is None else float(temp.min()))
+        rel = {torch.float32: 0.0, torch.bfloat16: 2.0 ** -7, torch.float16: 2.0 ** -10}[x.dtype]
+        err = (xo.grad.float() - xr.grad).abs()
+        tol = xr.grad.abs() * rel + 4e-6 * scale + (6e-8 if x.dtype == torch.float16 else 1e-7)
+        assert bool((err <= tol).all()), (i, x.dtype, tuple(x.shape), float((err - tol).max()))
+        worst = max(worst, float(err.max()))
+    print(f"worst absolute gradient difference: {worst:.2e}")

@@ -8,6 +8,10 @@
 // verl/utils/experimental/torch_functional.py:66-79. In the log2 domain:
 //   u = fma(x, c, -lse*log2e);  p = v_exp_f32(u);  dx = p * fma(u, a, b)  (+ g_l/T at the label)
 // with a = -g_h*ln2/T and b = -(g_l + g_h*H)/T constant over the row.
+// For fp32 logits the exponent is formed the way torch forms it instead, so that its only rounding of size
+// ulp(|z|) is the one torch has too: z = RN(x / T) (exact division, as in the forward kernel), d = z - lse
+// (= log p), p = v_exp_f32(d * log2e), dx = p * fma(d, a', b) with a' = -g_h / T. With peaked rows at low
+// temperature (|z| ~ 100) the folded form above is ~5x further from the fp64 gradient than torch's fp32 autograd.
 // lse and H come from the forward pass. The gradient has the logits' dtype and
 // may be written over the logits themselves (every element is read and then
 // written by the same lane).
@@ -15,6 +19,8 @@
 
 #include <hip/hip_runtime.h>
 #include <stdint.h>
+
+#include <type_traits>
 
 #include "rowscore_kernels.h"
 
@@ -97,8 +103,22 @@ struct RowGrad {
   }
 };
 
-// grid.x = n_rows, block = WAVES*64.
-template <int DT, int WAVES, int U>
+// The fp32 form: the quotient and log p are formed like torch forms them.
+struct RowGradExact {
+  Scale<true> sc;  // T, RN(1/T)
+  float lse;
+  float a;    // -g_h / T
+  float b;    // -(g_l + g_h * H) / T
+  float lab;  // g_l / T, added at the label
+  __device__ __forceinline__ float operator()(float x) const {
+    const float d = sc.pre(x) - lse;  // log p
+    const float p = hw_exp2(d * kLog2e);
+    return (p == 0.f) ? 0.f : p * __builtin_fmaf(d, a, b);
+  }
+};
+
+// grid.x = n_rows, block = WAVES*64. EXACT selects RowGradExact (fp32 logits).
+template <int DT, int WAVES, int U, bool EXACT = (DT == 0)>
 __global__ __launch_bounds__(WAVES * 64) void rowscore_backward_kernel(
     const void* logits, int64_t vocab, int64_t row_stride, const int64_t* __restrict__ labels,
     const float* __restrict__ temperature, const float* __restrict__ lse, const float* __restrict__ entropy,
@@ -124,10 +144,18 @@ __global__ __launch_bounds__(WAVES * 64) void rowscore_backward_kernel(
   const float gl = (g_logprob != nullptr) ? g_logprob[row] : 0.f;
   const float gh = (g_entropy != nullptr) ? g_entropy[row] : 0.f;
   const float H = (g_entropy != nullptr) ? entropy[row] : 0.f;
-  RowGrad f;
-  f.c = kLog2e * rT;
-  f.lse2 = lse[row] * kLog2e;
-  f.a = -(gh * kLn2f) * rT;
+  typename std::conditional<EXACT, RowGradExact, RowGrad>::type f;
+  if constexpr (EXACT) {
+    f.sc.c = kLog2e;
+    f.sc.T = T;
+    f.sc.r = rT;
+    f.lse = lse[row];
+    f.a = -gh * rT;
+  } else {
+    f.c = kLog2e * rT;
+    f.lse2 = lse[row] * kLog2e;
+    f.a = -(gh * kLn2f) * rT;
+  }
   f.b = -(gl + gh * H) * rT;
   f.lab = gl * rT;
   // a label outside [0, vocab) was reported by the forward pass; here it simply matches nothing
