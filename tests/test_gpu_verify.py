@@ -143,6 +143,16 @@ def test_empty_shapes(dev):
     z = torch.empty(3, 0, device=dev)
     res = sv.spec_verify(z, z, None, log_u=z)
     assert res.first_reject.tolist() == [0, 0, 0] and res.prefix_len.tolist() == [0, 0, 0]
+    # packed layout whose sequences are all empty: no token tensor has storage
+    e = torch.empty(0, device=dev)
+    cu = torch.zeros(4, dtype=torch.int64, device=dev)
+    res = sv.spec_verify(e, e, None, log_u=e, cu_seqlens=cu, draft_ids=torch.empty(0, dtype=torch.long, device=dev))
+    assert res.first_reject.tolist() == [0, 0, 0] and res.near_count.tolist() == [0, 0, 0] and res.out_ids.shape == (0,)
+    ids, mask = sv.truncate_draft(torch.empty(0, dtype=torch.long, device=dev), None, res.first_reject, cu_seqlens=cu)
+    assert ids.shape == (0,) and mask.shape == (0,)
+    lp, h, res = sv.fused_score_verify(torch.empty(0, 100, device=dev), torch.empty(0, dtype=torch.long, device=dev), e,
+                                       log_u=e, cu_seqlens=cu)
+    assert lp.shape == (0,) and res.prefix_len.tolist() == [0, 0, 0]
 
 
 def test_c5_imbalance_verify_only_full_size(dev):

@@ -170,6 +170,14 @@ def spec_verify(
     off = thresh_offset_from_lenience(lenience, lenience_mode) if thresh_offset is None else float(np.float32(thresh_offset))
     accept, first, prefix, near, ids, out_ids, out_mask = _verify_buffers(shape, B, dev, draft_ids, draft_ids is not None)
 
+    if ln.numel() == 0:
+        # no token at all (B empty sequences): nothing to launch, every sequence's results are zero
+        for t in (first, prefix, near):
+            t.zero_()
+        return VerifyResult(
+            accept=accept.view(torch.bool), first_reject=first, prefix_len=prefix, near_count=near, log_u=lu,
+            thresh_offset=off, out_ids=out_ids, out_mask=None if out_mask is None else out_mask.view(torch.bool),
+        )
     lib = _lib.load()
     with torch.cuda.device(dev):
         stream = _lib.stream_ptr(dev)
@@ -206,6 +214,8 @@ def truncate_draft(
     fr = first_reject.to(device=dev, dtype=torch.int32).contiguous()
     out_ids = torch.empty_like(ids)
     out_mask = torch.empty(shape, dtype=torch.uint8, device=dev)
+    if ids.numel() == 0:
+        return out_ids, out_mask.view(torch.bool)
     lib = _lib.load()
     with torch.cuda.device(dev):
         stream = _lib.stream_ptr(dev)
@@ -264,6 +274,14 @@ def fused_score_verify(
     flag = torch.zeros(1, dtype=torch.int32, device=dev)
     accept, first, prefix, near, ids, out_ids, out_mask = _verify_buffers(lead, B, dev, draft_ids, draft_ids is not None)
 
+    if n == 0:
+        for t in (first, prefix, near):
+            t.zero_()
+        res = VerifyResult(
+            accept=accept.view(torch.bool), first_reject=first, prefix_len=prefix, near_count=near, log_u=lu,
+            thresh_offset=off, out_ids=out_ids, out_mask=None if out_mask is None else out_mask.view(torch.bool),
+        )
+        return out_lp.reshape(lead), out_h.reshape(lead), res
     lib = _lib.load()
     with torch.cuda.device(dev):
         stream = _lib.stream_ptr(dev)
