@@ -114,6 +114,11 @@ def test_install_patches_module_and_bound_names(fake_verl):
     assert tf.entropy_from_logits_with_chunking(x, chunk_size=3) == ("verl", "entropy_from_logits_with_chunking")
     assert inst.stats() == {"hip_calls": 0, "passed_to_verl": 4}
 
+    class Wrapped(torch.Tensor):        # stands for DTensor and other tensor subclasses
+        pass
+
+    assert not inst._eligible(torch.randn(2, 5).as_subclass(Wrapped))
+
     inst.uninstall()
     assert tf.logprobs_from_logits is orig and eng.logprobs_from_logits is orig
     assert inst.stats() == {"hip_calls": 0, "passed_to_verl": 0}

@@ -49,8 +49,10 @@ _stats = {"hip_calls": 0, "passed_to_verl": 0}
 
 
 def _eligible(logits) -> bool:
+    # plain tensors only: a DTensor, a nested or a fake tensor has no single device buffer to hand to a kernel
     return (
-        isinstance(logits, torch.Tensor)
+        type(logits) in (torch.Tensor, torch.nn.Parameter)
+        and not logits.is_nested
         and logits.is_cuda
         and logits.dtype in (torch.float32, torch.bfloat16, torch.float16)
         and logits.dim() >= 1
