@@ -261,3 +261,45 @@ def test_full_size_c2_against_torch_fp32_on_device(dev):
     assert torch.all(lp <= 0)
     # N(0,3) logits: logsumexp ~ log V + 4.5 = 16.4; 70 % of labels are boosted by 8: mean ~ 0.7*(-8.4) + 0.3*(-16.4)
     assert -12.0 < lp.mean().item() < -9.5
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_response_slice_of_longer_logits_is_scored_without_a_copy(dev, dtype, monkeypatch):
+    """logits[:, -R-1:-1] of a (B, S, V) tensor (verl/utils/torch_functional.py:615 feeds exactly that): same numbers
+    as the contiguous copy, with gradients landing in the right rows of the full tensor."""
+    g = torch.Generator(device=dev).manual_seed(17)
+    B, S, R, V = 3, 40, 13, 3001
+    full = (torch.randn(B, S, V, generator=g, device=dev) * 2).to(dtype)
+    lab = torch.randint(0, V, (B, R), generator=g, device=dev)
+    temp = torch.rand(B, R, generator=g, device=dev) + 0.5
+    view = full[:, -R - 1:-1]
+    assert not view.is_contiguous() and vf._is_batch_of_row_slices(view)
+    copies = []
+    real_contiguous = torch.Tensor.contiguous
+    monkeypatch.setattr(torch.Tensor, "contiguous", lambda t, *a, **k: (copies.append(t.numel()), real_contiguous(t, *a, **k))[1])
+    lp, h, q = vf.fused_logprob_entropy(view, lab, temp, want_sum_pi_sq=True)
+    assert max(copies, default=0) < V          # nothing of the logits' size was copied
+    monkeypatch.undo()
+    ref = vf.fused_logprob_entropy(view.contiguous(), lab, temp, want_sum_pi_sq=True)
+    # A row's summation tree depends on where its 16-byte vectors start and on how many workgroups share it, and
+    # both differ between the slice and its copy: same numbers to fp32 rounding, not bit for bit.
+    assert lp.shape == (B, R) and (lp - ref[0]).abs().max().item() <= 4e-6 and (h - ref[1]).abs().max().item() <= 4e-6
+    assert ((q - ref[2]).abs() <= 4e-6 * ref[2].abs() + 1e-12).all()
+    from _parity import assert_scores_match
+    assert_scores_match(lp.reshape(-1), h.reshape(-1), view.reshape(-1, V), lab.reshape(-1), temp.reshape(-1), cpu_torch=False)
+    assert (vf.entropy_from_logits(view) - vf.entropy_from_logits(view.contiguous())).abs().max().item() <= 4e-6
+    assert (vf.logprobs_from_logits(view, lab) - vf.logprobs_from_logits(view.contiguous(), lab)).abs().max().item() <= 4e-6
+    # gradient through the slice
+    leaf = full.clone().requires_grad_(True)
+    w = torch.randn(B, R, generator=g, device=dev)
+    (vf.logprobs_from_logits(leaf[:, -R - 1:-1], lab) * w).sum().backward()
+    leaf2 = full.clone().requires_grad_(True)
+    (vf.logprobs_from_logits(leaf2[:, -R - 1:-1].contiguous(), lab) * w).sum().backward()
+    tol = 1e-6 if dtype == torch.float32 else 2.0 ** -7
+    assert (leaf.grad.float() - leaf2.grad.float()).abs().max().item() <= tol and bool((leaf.grad[:, :S - R - 1] == 0).all())
+    with pytest.raises(ValueError):
+        vf.logprobs_from_logits(view, lab[:, :-1])
+    with pytest.raises(IndexError):
+        bad = lab.clone()
+        bad[1, 2] = V
+        vf.logprobs_from_logits(view, bad)

@@ -68,6 +68,19 @@ def _is_view_safe(logits: torch.Tensor) -> bool:
     return logits.is_contiguous() and not logits.is_leaf
 
 
+_MAX_ROW_SLICE_BATCH = 256
+
+
+def _is_batch_of_row_slices(logits: torch.Tensor) -> bool:
+    """A 3-D (B, R, V) tensor with unit vocab stride and rows V or more apart whose batch stride does not let it be
+    viewed as (B*R, V): a slice along the sequence axis of a longer tensor."""
+    if logits.dim() != 3 or logits.shape[0] < 2 or logits.shape[0] > _MAX_ROW_SLICE_BATCH or logits.shape[1] == 0:
+        return False
+    B, Rr, V = logits.shape
+    sb, sr, sv = logits.stride()
+    return sv == 1 and sr >= V and sb != Rr * sr
+
+
 def _rows_2d(logits: torch.Tensor) -> torch.Tensor:
     """(..., V) -> (N, V) with unit stride along V; a view whenever torch allows one."""
     V = logits.shape[-1]
@@ -191,6 +204,23 @@ def rowscore(
         check_labels = LABEL_CHECK
     if not (want_logprob or want_entropy or want_sum_pi_sq):
         raise ValueError(f"{what}: nothing to compute")
+    if _is_batch_of_row_slices(logits):
+        # (B, R, V) cut out of a longer (B, S, V) tensor, e.g. logits[:, -R-1:-1] in
+        # verl/utils/torch_functional.py:615: flattening would copy B*R*V elements; each logits[b] is a 2-D block
+        # the kernel reads in place (its rows are V apart), so it is scored per b instead.
+        if want_logprob and (labels is None or tuple(labels.shape) != tuple(logits.shape[:-1])):
+            raise ValueError(f"{what}: labels shape {None if labels is None else tuple(labels.shape)} does not match "
+                             f"logits leading shape {tuple(logits.shape[:-1])}")
+        per_b_temperature = isinstance(temperature, torch.Tensor) and temperature.numel() != 1
+        if per_b_temperature and temperature.numel() != logits.shape[0] * logits.shape[1]:
+            raise ValueError(f"temperature has {temperature.numel()} entries, expected one per token "
+                             f"({logits.shape[0] * logits.shape[1]}) for logits leading shape {tuple(logits.shape[:-1])}")
+        t3 = temperature.reshape(logits.shape[:-1]) if per_b_temperature else None
+        parts = [rowscore(logits[b], None if labels is None else labels[b], t3[b] if per_b_temperature else temperature,
+                          want_logprob=want_logprob, want_entropy=want_entropy, want_sum_pi_sq=want_sum_pi_sq,
+                          check_labels=check_labels, n_splits=n_splits, inplace_backward=False, what=what)
+                 for b in range(logits.shape[0])]
+        return tuple(None if parts[0][k] is None else torch.stack([p[k] for p in parts]) for k in range(len(parts[0])))
     lead = logits.shape[:-1]
     V = logits.shape[-1]
     x = _rows_2d(logits)
