@@ -110,3 +110,38 @@ def test_c4_whole_workload_resident(dev):
     assert np.array_equal(res.accept.cpu().numpy().astype(np.uint8), ref["accept"])
     assert np.array_equal(res.first_reject.cpu().numpy(), ref["first_reject"])
     assert np.array_equal(res.near_count.cpu().numpy(), ref["near_count"])
+
+
+@pytest.mark.parametrize("dtype,V", [(torch.float32, (1 << 29) + 100003), (torch.bfloat16, (1 << 30) + 100003)])
+def test_one_row_longer_than_two_gibibytes(dev, dtype, V):
+    """Offsets inside a row beyond 2^31 bytes (64-bit indexing in the kernels), forward and backward, against the
+    closed form for a row of zeros with three raised entries, two of them past the 2 GiB mark."""
+    import math
+    from verl_amd import torch_functional as vf
+
+    x = torch.zeros(2, V, dtype=dtype, device=dev)
+    hot = {V - 1: 5.0, V - 70001: 3.0, 7: 4.0}
+    for k, v in hot.items():
+        x[:, k] = v
+    assert (V - 70001) * x.element_size() > 2**31
+    S = (V - 3) + sum(math.exp(v) for v in hot.values())
+    lse = math.log(S)
+    H = lse - sum(v * math.exp(v) for v in hot.values()) / S
+    lab = torch.tensor([V - 1, V - 70001], device=dev)
+    for splits in (None, 1):
+        lp, h = vf.fused_logprob_entropy(x, lab, n_splits=splits)
+        assert abs(lp[0].item() - (5.0 - lse)) <= 4e-6 and abs(lp[1].item() - (3.0 - lse)) <= 4e-6
+        # half a billion fp32 additions per sum, result ~20 (one fp32 step there is 1.9e-6): a few steps
+        assert abs(h[0].item() - H) <= 1e-5 and abs(h[1].item() - H) <= 1e-5
+    # backward, in place over the row: d lp[r] / d x = onehot(label) - p
+    xg = x[:1].clone().requires_grad_(True)
+    vf.logprobs_from_logits((xg * 1.0), lab[:1], inplace_backward=True).sum().backward()
+    g = xg.grad[0]
+    # p = exp(x - lse) with lse ~ 20 rounded to fp32: a relative 4e-6 on every probability; one rounding step of the
+    # output type for bf16
+    tol = 4e-6 if dtype == torch.float32 else 2.0 ** -8
+    assert abs(g[V - 1].item() - (1.0 - math.exp(5.0) / S)) <= tol
+    assert abs(g[V - 70001].item() + math.exp(3.0) / S) <= tol * math.exp(3.0) / S + 1e-12
+    assert abs(g[7].item() + math.exp(4.0) / S) <= tol * math.exp(4.0) / S + 1e-12
+    assert abs(g[V // 2].item() + 1.0 / S) <= tol / S + 1e-15
+    assert abs(g.double().sum().item()) <= 1e-3   # the gradient of a log-prob sums to zero over the row
