@@ -145,3 +145,46 @@ def test_one_row_longer_than_two_gibibytes(dev, dtype, V):
     assert abs(g[7].item() + math.exp(4.0) / S) <= tol * math.exp(4.0) / S + 1e-12
     assert abs(g[V // 2].item() + 1.0 / S) <= tol / S + 1e-15
     assert abs(g.double().sum().item()) <= 1e-3   # the gradient of a log-prob sums to zero over the row
+
+
+def test_very_long_sequences_verify(dev):
+    """Two padded sequences of five million tokens: positions beyond any 16-bit or LDS-sized assumption; first
+    rejections placed by hand near the end and in the middle, the rest accepts by construction (d = 0.5 >= log u)."""
+    T = 5_000_011
+    ln = torch.zeros(2, T, device=dev)
+    lo = torch.full((2, T), -0.5, device=dev)
+    g = torch.Generator(device=dev).manual_seed(1)
+    log_u = torch.log(torch.rand(2, T, generator=g, device=dev))          # <= 0 < 0.5
+    mask = torch.ones(2, T, dtype=torch.uint8, device=dev)
+    mask[1, T - 1000:] = 0
+    lo[0, T - 3] = 10.0                                                    # d = -10: rejected whatever u is (log u > -10 here)
+    lo[1, 2_345_678] = 10.0
+    log_u[0, T - 3] = -1.0
+    log_u[1, 2_345_678] = -1.0
+    ids = torch.arange(2 * T, device=dev).view(2, T)
+    res = sv.spec_verify(ln, lo, mask, log_u=log_u, thresh_offset=0.0, draft_ids=ids, pad_id=-1)
+    assert res.first_reject.tolist() == [T - 3, 2_345_678] and res.prefix_len.tolist() == [T - 3, 2_345_678]
+    assert int(res.accept[0].sum()) == T - 1 and int(res.accept[1].sum()) == T - 1000 - 1
+    assert bool((res.out_ids[0, :T - 3] == ids[0, :T - 3]).all()) and bool((res.out_ids[0, T - 3:] == -1).all())
+    assert int(res.out_mask[1].sum()) == 2_345_678
+
+
+def test_transpose_beyond_four_gibibytes(dev):
+    """70000 x 16384 fp32 = 4.6 GB: byte offsets past 2^32 on both sides. Transposing twice gives the array back,
+    and sampled entries sit where the definition puts them."""
+    from verl_amd import layout
+
+    rows, cols = 70000, 16384
+    x = torch.arange(rows * cols, device=dev, dtype=torch.int32).view(rows, cols)   # every entry names its own place
+    y = layout.transpose_2d(x)
+    assert y.shape == (cols, rows)
+    r = torch.tensor([0, 1, 127, 128, 65535, 65536, 69999], device=dev)
+    c = torch.tensor([0, 5, 64, 8191, 16383], device=dev)
+    assert torch.equal(y[c][:, r], x[r][:, c].t())
+    assert int(y[cols - 1, rows - 1]) == int(x[rows - 1, cols - 1])
+    del x
+    back = layout.transpose_2d(y)
+    expect_first = torch.arange(cols, device=dev, dtype=torch.int32)
+    assert torch.equal(back[0], expect_first) and torch.equal(back[rows - 1], expect_first + (rows - 1) * cols)
+    # a checksum over everything: sum of all entries mod 2^61 equals the closed form of sum(0 .. n-1) in wrapped int32
+    assert int(back.view(-1)[::4097].to(torch.int64).sum()) == int(torch.arange(0, rows * cols, 4097, dtype=torch.int64).to(torch.int32).to(torch.int64).sum())
