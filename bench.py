@@ -369,8 +369,18 @@ def bench_lm_head(args, dev):
         torch.cuda.synchronize()
         return (time.perf_counter() - t0) / args.steps
 
+    from verl_amd.fused_linear import lm_head_score_mfma
+
+    def fwd_mfma():
+        return lm_head_score_mfma(hidden.detach(), weight.detach(), ids, temperature)
+
+    lp_m, h_m = fwd_mfma()
+    e3 = (lp_m[:256] - torch.log_softmax(z, -1).gather(-1, ids[:256, None]).squeeze(-1)).abs().max().item()
+    if not e3 <= 3e-2:   # z holds bf16-rounded logits, the kernel keeps them in fp32
+        raise SystemExit(f"bench: matrix-core LM-head scores disagree with torch ({e3})")
     t_f = timed(fwd)
     t_fb = timed(fwd_bwd)
+    t_m = timed(fwd_mfma)
     wt = torch.empty(D, V, dtype=weight.dtype, device=dev)
     t_tr = timed(lambda: transpose_2d(weight.detach(), wt))
     flops_f, flops_fb = 2.0 * T * D * V, 6.0 * T * D * V
@@ -388,6 +398,9 @@ def bench_lm_head(args, dev):
                      "frac": flops_fb / t_fb / 1e12 / 2500.0, "traffic": None,
                      "kernel": "hipBLASLt bf16 GEMMs (library) + rowscore_kernel + rowscore_backward_kernel",
                      "forward_tflops": flops_f / t_f / 1e12},
+        "single_kernel_forward": {"ms": t_m * 1e3, "tflops": flops_f / t_m / 1e12, "frac_of_mfma_peak": flops_f / t_m / 1e12 / 2500.0,
+                                  "kernel": "lmhead_partial_kernel<bf16> + lmhead_finish_kernel (vrl_lmhead_score)",
+                                  "note": "hand-written MFMA kernel, logits never written; slower than the library GEMM path above"},
         "weight_transpose": {"ms": t_tr * 1e3, "gbps": 2.0 * V * D * 2 / t_tr / 1e9, "kernel": "transpose_kernel<2>"},
         "parity_guard": {"rows": 256, "max_abs_err_logprob": e1, "max_abs_err_entropy": e2},
     }), flush=True)

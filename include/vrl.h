@@ -156,6 +156,29 @@ int vrl_transpose(const void* src, int elem_size, int64_t rows, int64_t cols, in
                   void* dst, int64_t dst_stride, void* stream);
 
 /*
+ * vrl_lmhead_score — LM head and scoring in one pass on the matrix cores, without logits in memory:
+ *   z[t, v] = (sum_k hidden[t, k] * weight[v, k]) / max(temperature[t], 1e-8)
+ *   logprob[t] = z[t, label[t]] - logsumexp(z[t, :]),  entropy[t] = logsumexp - sum(softmax * z),  lse[t] = logsumexp
+ * hidden (n_tokens, hidden_size) and weight (vocab, hidden_size) are bf16 or fp16 (dtype as for vrl_rowscore),
+ * row-major with row pitches h_stride / w_stride in elements; products are accumulated in fp32 (the logits are
+ * NOT rounded to the operand type on the way, unlike a GEMM that writes them out). Forward only.
+ * `partials` is caller-owned scratch of n_tokens * n_splits * 4 floats; vrl_lmhead_plan gives n_splits.
+ * Requirements checked on the host: n_tokens >= 256, vocab >= 256, hidden_size a multiple of 64, pitches multiples
+ * of 8 elements, 16-byte aligned operands, each operand below 4 GiB, 1 <= n_splits <= 64. out_logprob (with labels
+ * and err_flag), out_entropy, out_lse: any may be NULL, not all.
+ *
+ * Replaces the reference's fused linear + cross-entropy forward:
+ *   verl/utils/kernel/linear_cross_entropy.py:38-85 (LinearCrossEntropy.forward)
+ *   verl/utils/kernel/kernels.py:183-451 (efficient_entropy_kernel_general_mainloop + epilogue, Triton)
+ */
+int vrl_lmhead_score(const void* hidden, const void* weight, int dtype, int64_t n_tokens, int64_t vocab,
+                     int64_t hidden_size, int64_t h_stride, int64_t w_stride, const int64_t* labels,
+                     const float* temperature, int n_splits, float* partials, float* out_logprob,
+                     float* out_entropy, float* out_lse, int32_t* err_flag, void* stream);
+/* Vocabulary splits per 256-token block that fill the part (about one workgroup per CU) for this shape. */
+int vrl_lmhead_plan(int64_t n_tokens, int64_t vocab);
+
+/*
  * vrl_rollout_corr — rollout correction on padded (B, T) log-probs in one launch:
  *   lr = clamp(old - rollout, +-20);  k1 = -lr, k2 = lr^2/2, k3 = exp(lr) - 1 - lr
  *   keep[b,t]    = every enabled criterion passes (token_k1/k2/k3 per token; seq_sum / seq_mean /

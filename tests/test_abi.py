@@ -143,6 +143,28 @@ def test_response_pack_argument_errors(lib):
     assert g(None, None, None, None, 0, 0, None, None, None) == _lib.VRL_OK
 
 
+def test_lmhead_argument_errors(lib):
+    f = lib.vrl_lmhead_score
+    ok = dict(h=P, w=P, dt=_lib.VRL_BF16, T=512, V=1024, K=128, hs=128, ws=128, lab=P, temp=None, S=2, part=P, lp=P, ent=P,
+              lse=None, flag=P)
+
+    def call(**kw):
+        a = {**ok, **kw}
+        return f(a["h"], a["w"], a["dt"], a["T"], a["V"], a["K"], a["hs"], a["ws"], a["lab"], a["temp"], a["S"], a["part"],
+                 a["lp"], a["ent"], a["lse"], a["flag"], None)
+
+    assert call(dt=_lib.VRL_F32) == _lib.VRL_ERR_DTYPE
+    assert call(T=255) == _lib.VRL_ERR_SHAPE and call(V=100) == _lib.VRL_ERR_SHAPE
+    assert call(K=96) == _lib.VRL_ERR_SHAPE and call(hs=64) == _lib.VRL_ERR_SHAPE and call(ws=132) == _lib.VRL_ERR_SHAPE
+    assert call(S=0) == _lib.VRL_ERR_SHAPE and call(S=65) == _lib.VRL_ERR_SHAPE
+    assert call(V=1 << 25, K=64, hs=64, ws=64) == _lib.VRL_ERR_SHAPE          # weight of 4 GiB: 32-bit offsets
+    assert call(lp=None, ent=None) == _lib.VRL_ERR_ARG
+    assert call(h=None) == _lib.VRL_ERR_NULL and call(part=None) == _lib.VRL_ERR_NULL
+    assert call(lab=None) == _lib.VRL_ERR_NULL and call(flag=None) == _lib.VRL_ERR_NULL
+    assert call(h=P + 8) == _lib.VRL_ERR_ALIGN and call(w=P + 2) == _lib.VRL_ERR_ALIGN
+    assert lib.vrl_lmhead_plan(8192, 152064) == 8 and lib.vrl_lmhead_plan(0, 5) == 1
+
+
 def test_transpose_argument_errors(lib):
     t = lib.vrl_transpose
     Q = P + (1 << 20)                      # a second, disjoint address

@@ -12,7 +12,7 @@ Setting ``VERL_USE_EXTERNAL_MODULES=verl_amd.plugin`` makes verl import
 """
 
 from . import rollout_corr
-from .fused_linear import FusedLinearForPPO, fused_linear_for_ppo, linear_cross_entropy
+from .fused_linear import FusedLinearForPPO, fused_linear_for_ppo, linear_cross_entropy, lm_head_score_mfma
 from .hook import install, uninstall
 from .layout import response_slice, roll_labels, transpose_2d
 from .spec_rl import (
@@ -41,6 +41,7 @@ __all__ = [
     "FusedLinearForPPO",
     "fused_linear_for_ppo",
     "linear_cross_entropy",
+    "lm_head_score_mfma",
     "VerifyResult",
     "draw_log_uniforms",
     "fused_score_verify",

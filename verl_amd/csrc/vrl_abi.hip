@@ -9,6 +9,7 @@
 
 #include "backward_kernels.h"
 #include "layout_kernels.h"
+#include "lmhead_kernels.h"
 #include "rollout_corr_kernels.h"
 #include "rowscore_kernels.h"
 #include "transpose_kernels.h"
@@ -190,6 +191,28 @@ int verify_waves(const int64_t* cu_seqlens, int64_t B, int64_t T) {
   return B <= 4096 ? 16 : 4;
 }
 
+template <int DT>
+int launch_lmhead(const void* hidden, const void* weight, int64_t T, int64_t V, int64_t K, int64_t h_stride,
+                         int64_t w_stride, const int64_t* labels, const float* temperature, int n_splits,
+                         float* partials, float* out_logprob, float* out_entropy, float* out_lse,
+                         int32_t* err_flag, hipStream_t s) {
+  const int64_t tblocks = (T + vrl::kLmTokens - 1) / vrl::kLmTokens;
+  const int64_t vtiles = (V + vrl::kLmVocab - 1) / vrl::kLmVocab;
+  const int tiles_per_split = static_cast<int>((vtiles + n_splits - 1) / n_splits);
+  // 8 token blocks x 4 splits per XCD when the grid divides that way (see the kernel's mapping)
+  const int xcd_map = (tblocks % 8 == 0 && n_splits % 4 == 0 && ((tblocks / 8) * (n_splits / 4)) % 8 == 0) ? 1 : 0;
+  if (hipFuncSetAttribute(reinterpret_cast<const void*>(vrl::lmhead_partial_kernel<DT>),
+                          hipFuncAttributeMaxDynamicSharedMemorySize, vrl::kLmLdsBytes) != hipSuccess)
+    return launch_status();
+  vrl::lmhead_partial_kernel<DT><<<dim3(static_cast<unsigned>(tblocks * n_splits)), dim3(256), vrl::kLmLdsBytes, s>>>(
+      static_cast<const uint16_t*>(weight), static_cast<const uint16_t*>(hidden), V, T, K, w_stride, h_stride,
+      temperature, n_splits, tiles_per_split, xcd_map, partials);
+  vrl::lmhead_finish_kernel<DT><<<dim3(static_cast<unsigned>((T + 3) / 4)), dim3(256), 0, s>>>(
+      static_cast<const char*>(weight), static_cast<const char*>(hidden), V, T, K, w_stride, h_stride, labels,
+      temperature, n_splits, partials, out_logprob, out_entropy, out_lse, err_flag);
+  return launch_status();
+}
+
 }  // namespace
 
 extern "C" {
@@ -334,6 +357,46 @@ int vrl_response_pack(const float* values, const int64_t* cu_seqlens, const int6
   vrl::response_pack_kernel<<<dim3(static_cast<unsigned>(B)), dim3(256), 0, static_cast<hipStream_t>(stream)>>>(
       values, cu_seqlens, response_lens, out_offsets, out_total, out, err_flag);
   return launch_status();
+}
+
+int vrl_lmhead_plan(int64_t n_tokens, int64_t vocab) {
+  if (n_tokens <= 0 || vocab <= 0) return 1;
+  const int64_t tblocks = (n_tokens + vrl::kLmTokens - 1) / vrl::kLmTokens;
+  const int64_t vtiles = (vocab + vrl::kLmVocab - 1) / vrl::kLmVocab;
+  int64_t s = (256 + tblocks - 1) / tblocks;  // one workgroup per CU
+  s = ((s + 3) / 4) * 4;                       // groups of 4 splits share an XCD with 8 token blocks
+  if (s > vrl::kLmMaxSplits) s = vrl::kLmMaxSplits;
+  if (s > vtiles) s = vtiles;
+  if (s < 1) s = 1;
+  return static_cast<int>(s);
+}
+
+int vrl_lmhead_score(const void* hidden, const void* weight, int dtype, int64_t n_tokens, int64_t vocab,
+                     int64_t hidden_size, int64_t h_stride, int64_t w_stride, const int64_t* labels,
+                     const float* temperature, int n_splits, float* partials, float* out_logprob,
+                     float* out_entropy, float* out_lse, int32_t* err_flag, void* stream) {
+  if (dtype != VRL_BF16 && dtype != VRL_F16) return VRL_ERR_DTYPE;
+  if (n_tokens < vrl::kLmTokens || vocab < vrl::kLmVocab || hidden_size <= 0 || hidden_size % vrl::kLmK != 0 ||
+      h_stride < hidden_size || w_stride < hidden_size || h_stride % 8 != 0 || w_stride % 8 != 0 ||
+      n_splits < 1 || n_splits > vrl::kLmMaxSplits)
+    return VRL_ERR_SHAPE;
+  // 32-bit byte offsets inside each operand; grid size
+  if (vocab * w_stride * 2 >= (1LL << 32) || n_tokens * h_stride * 2 >= (1LL << 32)) return VRL_ERR_SHAPE;
+  if (((n_tokens + vrl::kLmTokens - 1) / vrl::kLmTokens) * n_splits > kMaxGrid || (n_tokens + 3) / 4 > kMaxGrid)
+    return VRL_ERR_SHAPE;
+  if (out_logprob == nullptr && out_entropy == nullptr && out_lse == nullptr) return VRL_ERR_ARG;
+  if (hidden == nullptr || weight == nullptr || partials == nullptr) return VRL_ERR_NULL;
+  if (out_logprob != nullptr && (labels == nullptr || err_flag == nullptr)) return VRL_ERR_NULL;
+  if (!aligned(hidden, 16) || !aligned(weight, 16) || !aligned(labels, 8) || !aligned(temperature, 4) ||
+      !aligned(partials, 4) || !aligned(out_logprob, 4) || !aligned(out_entropy, 4) || !aligned(out_lse, 4) ||
+      !aligned(err_flag, 4))
+    return VRL_ERR_ALIGN;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  if (dtype == VRL_BF16)
+    return launch_lmhead<VRL_BF16>(hidden, weight, n_tokens, vocab, hidden_size, h_stride, w_stride, labels, temperature,
+                                   n_splits, partials, out_logprob, out_entropy, out_lse, err_flag, s);
+  return launch_lmhead<VRL_F16>(hidden, weight, n_tokens, vocab, hidden_size, h_stride, w_stride, labels, temperature,
+                                n_splits, partials, out_logprob, out_entropy, out_lse, err_flag, s);
 }
 
 int vrl_transpose(const void* src, int elem_size, int64_t rows, int64_t cols, int64_t src_stride,

@@ -20,7 +20,8 @@ from . import _lib
 from .layout import transpose_2d
 from .torch_functional import _DTYPE_CODES, _ptr
 
-__all__ = ["FusedLinearForPPO", "fused_linear_for_ppo", "linear_cross_entropy", "DEFAULT_CHUNK_TOKENS"]
+__all__ = ["FusedLinearForPPO", "fused_linear_for_ppo", "linear_cross_entropy", "lm_head_score_mfma",
+           "DEFAULT_CHUNK_TOKENS"]
 
 # The reference's default is 512 tokens per chunk. On a 288 GB part a (4096, 152064) bf16 buffer is 1.2 GB, the
 # projection reaches 1.4 PFLOP/s instead of 0.86 at 512, and the weight gradient is accumulated 8x less often.
@@ -166,6 +167,66 @@ def fused_linear_for_ppo(hidden_states: torch.Tensor, vocab_weights: torch.Tenso
     ids = input_ids.reshape(-1).to(torch.int64).contiguous()
     lp, ent = _FusedLinearForPPOFunction.apply(h2, vocab_weights.contiguous(), ids, float(temperature), int(chunk_size),
                                                bool(keep_logits))
+    return lp.reshape(lead), ent.reshape(lead)
+
+
+def lm_head_score_mfma(hidden_states: torch.Tensor, vocab_weights: torch.Tensor, input_ids: torch.Tensor,
+                       temperature=1.0, n_splits: Optional[int] = None):
+    """Forward-only (log_probs, entropy), fp32, from one hand-written matrix-core kernel that never writes logits
+    (``vrl_lmhead_score``): the counterpart of the reference's Triton ``efficient_entropy_forward``
+    (verl/utils/kernel/kernels.py:531-756). bf16 or fp16 operands, at least 256 tokens and 256 vocabulary entries,
+    hidden size a multiple of 64. ``temperature`` is a float or one value per token. The logits are kept in fp32
+    (a GEMM that writes them rounds them to the operand type first), so results are slightly closer to the
+    all-fp32 value than ``fused_linear_for_ppo``'s. On MI355X it is slower than the library GEMM + row kernel that
+    ``fused_linear_for_ppo`` uses (9.3 ms against 6.4 ms at 8192 x 3584 -> 152064); it needs no logits buffer at all.
+    """
+    if not hidden_states.is_cuda or not vocab_weights.is_cuda:
+        raise RuntimeError("lm_head_score_mfma: tensors must be on the GPU; verl_amd has no CPU implementation")
+    if hidden_states.dtype != vocab_weights.dtype or hidden_states.dtype not in (torch.bfloat16, torch.float16):
+        raise TypeError(f"lm_head_score_mfma: hidden {hidden_states.dtype} / weights {vocab_weights.dtype} must both be "
+                        "bfloat16 or both float16")
+    if torch.is_grad_enabled() and (hidden_states.requires_grad or vocab_weights.requires_grad):
+        raise NotImplementedError("lm_head_score_mfma is forward-only; use fused_linear_for_ppo when gradients are needed")
+    if hidden_states.dim() not in (2, 3) or vocab_weights.dim() != 2 or vocab_weights.shape[1] != hidden_states.shape[-1]:
+        raise ValueError("lm_head_score_mfma: hidden_states must be (tokens, hidden) or (batch, seq, hidden) and "
+                         "vocab_weights (vocab, hidden)")
+    if tuple(input_ids.shape) != tuple(hidden_states.shape[:-1]):
+        raise ValueError(f"lm_head_score_mfma: input_ids shape {tuple(input_ids.shape)} does not match hidden_states "
+                         f"{tuple(hidden_states.shape)}")
+    lead = hidden_states.shape[:-1]
+    h = hidden_states.detach().reshape(-1, hidden_states.shape[-1]).contiguous()
+    w = vocab_weights.detach().contiguous()
+    T, K = h.shape
+    V = w.shape[0]
+    if T < 256 or V < 256 or K % 64 != 0:
+        raise ValueError(f"lm_head_score_mfma needs >= 256 tokens, >= 256 vocabulary entries and a hidden size that is "
+                         f"a multiple of 64; got {T}, {V}, {K}")
+    dev = h.device
+    ids = input_ids.reshape(-1).to(device=dev, dtype=torch.int64).contiguous()
+    temp = None
+    if isinstance(temperature, torch.Tensor):
+        temp = temperature.to(device=dev, dtype=torch.float32).reshape(-1)
+        temp = temp.expand(T).contiguous() if temp.numel() == 1 else temp.contiguous()
+        if temp.numel() != T:
+            raise ValueError(f"temperature has {temp.numel()} entries, expected one per token ({T})")
+    elif float(temperature) != 1.0:
+        temp = torch.full((T,), float(temperature), dtype=torch.float32, device=dev)
+    lib = _lib.load()
+    splits = lib.vrl_lmhead_plan(T, V) if n_splits is None else int(n_splits)
+    f32 = dict(dtype=torch.float32, device=dev)
+    partials = torch.empty(T * splits * 4, **f32)
+    lp = torch.empty(T, **f32)
+    ent = torch.empty(T, **f32)
+    flag = torch.zeros(1, dtype=torch.int32, device=dev)
+    with torch.cuda.device(dev):
+        st = lib.vrl_lmhead_score(h.data_ptr(), w.data_ptr(), _DTYPE_CODES[h.dtype], T, V, K, h.stride(0), w.stride(0),
+                                  ids.data_ptr(), _ptr(temp), splits, partials.data_ptr(), lp.data_ptr(), ent.data_ptr(),
+                                  None, flag.data_ptr(), _lib.stream_ptr(dev))
+    _lib.check("vrl_lmhead_score", st)
+    from . import torch_functional as _tf
+
+    if _tf.LABEL_CHECK and (int(flag.item()) & _lib.VRL_FLAG_LABEL_OOB):
+        raise IndexError(f"lm_head_score_mfma: an input id is outside [0, {V})")
     return lp.reshape(lead), ent.reshape(lead)
 
 
