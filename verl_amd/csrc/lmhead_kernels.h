@@ -53,11 +53,10 @@ struct LmFrag<2> {
   }
 };
 
-// One wave instruction moves 8 tile rows x 128 bytes into LDS (lane l -> byte l*16 of the 1 KiB block).
-// Lane l serves row r = l>>3, physical slot p = l&7, which holds logical 16-byte chunk p ^ r of that row
-// (the swizzle that makes the 128-bit fragment reads conflict-free).
-// tile: uniform pointer to (first row of the tile, k step); lane_off: this lane's (r * stride + chunk * 8) * 2;
-// row_block_bytes: 8 rows in bytes (uniform).
+// One wave instruction moves 8 tile rows x 128 bytes into LDS (lane l lands at byte l*16 of the 1 KiB block):
+// lane l serves row r = l>>3 of the block and physical 16-byte slot p = l&7, and fetches the logical chunk that the
+// swizzle assigns to that slot (two lane offsets: blocks of 8 rows alternate in the swizzle's row bits).
+// tile: uniform pointer to (first row of the tile, k step); row_block_bytes: 8 rows in bytes (uniform).
 __device__ __forceinline__ void load_tile(const char* __restrict__ tile, uint32_t lane_off_even, uint32_t lane_off_odd,
                                           int64_t row_block_bytes, char* lds_tile, int wave) {
 #pragma unroll
@@ -97,7 +96,6 @@ __global__ __launch_bounds__(256, 1) void lmhead_partial_kernel(
       const int x = (int)(id & 7);
       const int64_t local = id >> 3;            // 0 .. tblocks*n_splits/8
       const int64_t tgroups = tblocks / 8;      // groups of 8 token blocks
-      const int sgroups = n_splits / 4;         // groups of 4 splits
       // super index over (tgroup, sgroup) pairs: 8 consecutive ones run at a time (one per XCD)
       const int64_t super = (local / 32) * 8 + x;
       const int64_t within = local % 32;
@@ -105,7 +103,6 @@ __global__ __launch_bounds__(256, 1) void lmhead_partial_kernel(
       const int sg = (int)(super / tgroups);
       tb = tg * 8 + (within & 7);
       split = sg * 4 + (int)(within >> 3);
-      (void)sgroups;
     } else {
       split = (int)(id % n_splits);
       tb = id / n_splits;
