@@ -79,14 +79,14 @@ def test_installed_shims_send_gpu_tensors_to_the_hip_path(dev):
         h = tf.entropy_from_logits(x.bfloat16())
         q = tf.calculate_sum_pi_squared_from_logits(x)
         hc = tf.entropy_from_logits_with_chunking(x, chunk_size=4)
-        assert hook.stats() == {"hip_calls": 4, "passed_to_verl": 0}
+        assert hook.stats() == {"hip_calls": 4, "passed_to_verl": 0, "memo_hits": 0}
         assert (lp - scoring.logprobs_from_logits(x, lab)).abs().max().item() <= 1e-5
         assert (h - scoring.entropy_from_logits(x.bfloat16().float())).abs().max().item() <= 2e-3
         assert (q - scoring.calculate_sum_pi_squared_from_logits(x)).abs().max().item() <= 1e-6
         assert torch.equal(hc, vf.entropy_from_logits(x))
         tf.entropy_from_logits(x.cpu())                    # the driver's CPU tensors stay with verl's own function
         tf.entropy_from_logits(x.double())
-        assert hook.stats() == {"hip_calls": 4, "passed_to_verl": 2}
+        assert hook.stats() == {"hip_calls": 4, "passed_to_verl": 2, "memo_hits": 0}
         xg = x.clone().requires_grad_(True)               # update_actor: gradient through the HIP backward
         tf.logprobs_from_logits(xg * 1.0, lab, inplace_backward=True).sum().backward()
         assert xg.grad is not None and hook.stats()["hip_calls"] == 5
@@ -96,6 +96,77 @@ def test_installed_shims_send_gpu_tensors_to_the_hip_path(dev):
         assert torch.equal(compiled(x), vf.entropy_from_logits(x))
         assert torch.equal(compiled(x[:3]), vf.entropy_from_logits(x[:3]))
         assert hook.stats()["hip_calls"] == 7
+    finally:
+        hook.uninstall()
+        for k, v in saved.items():
+            if v is None:
+                sys.modules.pop(k, None)
+            else:
+                sys.modules[k] = v
+
+
+def test_one_pass_serves_entropy_and_logprobs_of_the_same_tensor(dev, monkeypatch):
+    """compute_log_prob asks for the entropy and the label log-probs of one logits tensor in two calls
+    (fsdp/transformer_impl.py:1364-1376, :1395-1399 in the reference): the second call must not read the logits
+    again, and nothing stale may ever be served."""
+    mods = {n: types.ModuleType(n) for n in ("verl", "verl.utils", "verl.utils.torch_functional")}
+    tf = mods["verl.utils.torch_functional"]
+    for name in hook.PATCHED_NAMES:
+        setattr(tf, name, getattr(scoring, name))
+    saved = {k: sys.modules.get(k) for k in mods}
+    sys.modules.update(mods)
+    try:
+        hook.install()
+        g = torch.Generator(device=dev).manual_seed(8)
+        V = 5003
+        x = (torch.randn(300, V, generator=g, device=dev) * 3).bfloat16()
+        lab = torch.randint(0, V, (300,), generator=g, device=dev)
+        want_h, want_lp = vf.entropy_from_logits(x), vf.logprobs_from_logits(x, lab)
+        launches = []
+        real = vf._forward_2d
+        monkeypatch.setattr(vf, "_forward_2d", lambda *a, **k: (launches.append(1), real(*a, **k))[1])
+        with torch.no_grad():
+            h = tf.entropy_from_logits(x)                      # the engine's order: entropy, then log-probs
+            lp = tf.logprobs_from_logits(x, lab)
+        assert len(launches) == 1 and hook.stats()["memo_hits"] == 1
+        assert torch.equal(h, want_h) and (lp - want_lp).abs().max().item() <= 2e-6
+        with torch.no_grad():                                   # the other order: log-probs first, entropy is then a lookup
+            y = x.clone()
+            lp2 = tf.logprobs_from_logits(y, lab)
+            h2 = tf.entropy_from_logits_with_chunking(y, chunk_size=128)
+        assert len(launches) == 2 and hook.stats()["memo_hits"] == 2
+        assert torch.equal(lp2, want_lp) and torch.equal(h2, want_h)
+        # an in-place write (also through a view) invalidates what was kept
+        with torch.no_grad():
+            y[5:7].mul_(0.5)
+            h3 = tf.entropy_from_logits(y)
+        assert len(launches) == 3 and not torch.equal(h3[5:7], want_h[5:7])
+        n0 = len(launches)
+        assert torch.equal(h3, vf.entropy_from_logits(y)) and len(launches) == n0 + 1
+        # another tensor object, even at the same address with the same contents, is never served from the old one
+        with torch.no_grad():
+            del y
+            z = x.clone()
+            tf.logprobs_from_logits(z, lab)
+        assert len(launches) == n0 + 2
+        # a label outside the vocabulary raises on the gather route too
+        with torch.no_grad(), pytest.raises(IndexError):
+            bad = lab.clone()
+            bad[0] = V
+            tf.logprobs_from_logits(z, bad)
+        # with gradients the ordinary differentiable route is taken
+        before = hook.stats()["memo_hits"]
+        zg = z.float().requires_grad_(True)
+        tf.entropy_from_logits(zg).sum().backward()
+        tf.logprobs_from_logits(zg, lab).sum().backward()
+        assert hook.stats()["memo_hits"] == before and zg.grad is not None
+        # and it can be switched off
+        monkeypatch.setattr(hook, "MEMO", False)
+        n0 = len(launches)
+        with torch.no_grad():
+            tf.entropy_from_logits(x)
+            tf.logprobs_from_logits(x, lab)
+        assert len(launches) == n0 + 2
     finally:
         hook.uninstall()
         for k, v in saved.items():
@@ -138,7 +209,7 @@ def test_installed_fused_linear_entry_points_serve_gpu_tensors(dev):
         lce = mods["verl.utils.kernel.linear_cross_entropy"].linear_cross_entropy
         lp, ent = lce(h, w, ids, 1.2, "none")                                                   # dense_common.py:189-195
         assert torch.equal(lp, want[0].reshape(-1)) and torch.equal(ent, want[1].reshape(-1))
-        assert hook.stats() == {"hip_calls": 2, "passed_to_verl": 0}
+        assert hook.stats() == {"hip_calls": 2, "passed_to_verl": 0, "memo_hits": 0}
     finally:
         hook.uninstall()
         for k, v in saved.items():

@@ -25,11 +25,14 @@ from __future__ import annotations
 
 import functools
 import importlib
+import os
 import sys
+import weakref
 from typing import Callable, Dict, List, Tuple
 
 import torch
 
+from . import _lib
 from . import fused_linear as _fl
 from . import torch_functional as _amd
 
@@ -43,9 +46,89 @@ PATCHED_NAMES = (
     "calculate_sum_pi_squared_from_logits",
 )
 
+# One pass serves two calls. verl's engines ask for the entropy and for the label log-probs of the SAME logits tensor
+# in two separate calls (verl/workers/engine/fsdp/transformer_impl.py:1364-1376 and :1395-1399). Without gradients
+# the first of the two (whichever it is) runs the row kernel once and keeps entropy and logsumexp per row; the second
+# is then a gather (log-prob = logit[label] - logsumexp) or a lookup, not another pass over the logits.
+# What is kept is tied to the tensor OBJECT (weak reference), its version counter (any in-place write bumps it, also
+# through views), its address, shape, strides, dtype and the stream: a new tensor that happens to reuse the address
+# is a different object and never matches. VERL_AMD_MEMO=0 switches it off.
+MEMO = os.environ.get("VERL_AMD_MEMO", "1") not in ("0", "false", "False")
+
+
+class _RowMemo:
+    __slots__ = ("ref", "version", "ptr", "shape", "stride", "dtype", "stream", "entropy", "lse")
+
+    def matches(self, logits, stream) -> bool:
+        return (self.ref is not None and self.ref() is logits and self.version == logits._version
+                and self.ptr == logits.data_ptr() and self.shape == tuple(logits.shape)
+                and self.stride == tuple(logits.stride()) and self.dtype == logits.dtype and self.stream == stream)
+
+
+_memo = _RowMemo()
+_memo.ref = None
+
+
+def _memo_store(logits, stream, entropy, lse) -> None:
+    _memo.ref = weakref.ref(logits)
+    _memo.version = logits._version
+    _memo.ptr = logits.data_ptr()
+    _memo.shape = tuple(logits.shape)
+    _memo.stride = tuple(logits.stride())
+    _memo.dtype = logits.dtype
+    _memo.stream = stream
+    _memo.entropy = entropy
+    _memo.lse = lse
+
+
+def _memo_clear() -> None:
+    _memo.ref = None
+    _memo.entropy = None
+    _memo.lse = None
+
+
+_LOGPROB_NAMES = ("logprobs_from_logits", "logprobs_from_logits_v2", "logprobs_from_logits_naive")
+_ENTROPY_NAMES = ("entropy_from_logits", "entropy_from_logits_with_chunking")
+
+
+def _memo_serve(name, logits, args, kwargs):
+    """The result of ``name(logits, ...)`` from one shared pass, or None when the ordinary route must be taken."""
+    if not MEMO or torch.is_grad_enabled() and logits.requires_grad:
+        return None
+    stream = _lib.stream_ptr(logits.device)
+    hit = _memo.matches(logits, stream)
+    if name in _ENTROPY_NAMES:
+        if hit:
+            _stats["memo_hits"] += 1
+            return _memo.entropy
+        got = _amd._score_once(logits, None)
+        if got is None:
+            return None
+        _memo_store(logits, stream, got[1], got[2])
+        return got[1]
+    if name in _LOGPROB_NAMES:
+        labels = args[0] if args else kwargs.get("labels")
+        if not isinstance(labels, torch.Tensor) or tuple(labels.shape) != tuple(logits.shape[:-1]):
+            return None
+        if hit:
+            V = logits.shape[-1]
+            lab = labels.to(device=logits.device, dtype=torch.int64)
+            if _amd.LABEL_CHECK and bool(((lab < 0) | (lab >= V)).any()):
+                raise IndexError(f"{name}: a label is outside [0, {V})")
+            picked = torch.gather(logits, -1, lab.clamp(0, V - 1).unsqueeze(-1)).squeeze(-1)
+            _stats["memo_hits"] += 1
+            return picked.float() - _memo.lse
+        got = _amd._score_once(logits, labels)
+        if got is None:
+            return None
+        _memo_store(logits, stream, got[1], got[2])
+        return got[0]
+    return None
+
+
 _originals: Dict[str, Callable] = {}
 _rebound: List[Tuple[object, str, Callable]] = []
-_stats = {"hip_calls": 0, "passed_to_verl": 0}
+_stats = {"hip_calls": 0, "passed_to_verl": 0, "memo_hits": 0}
 
 
 def _eligible(logits) -> bool:
@@ -63,18 +146,27 @@ def _eligible(logits) -> bool:
 def _make_shim(name: str, original: Callable) -> Callable:
     ours = getattr(_amd, name)
 
-    @functools.wraps(original)
-    def shim(logits, *args, **kwargs):
+    def serve(logits, *args, **kwargs):
         if _eligible(logits):
             _stats["hip_calls"] += 1
+            served = _memo_serve(name, logits, args, kwargs)
+            if served is not None:
+                return served
             return ours(logits, *args, **kwargs)
         _stats["passed_to_verl"] += 1
         return original(logits, *args, **kwargs)
 
     # The engines wrap entropy_from_logits in torch.compile when use_torch_compile is set
     # (verl/workers/engine/fsdp/transformer_impl.py:164-168). There is nothing to trace in a ctypes call into a
-    # finished kernel, so the tracer is told to run the shim as it is.
-    shim = torch.compiler.disable(shim)
+    # finished kernel. torch.compile unwraps a function that is itself marked torch.compiler.disable and traces
+    # it anyway, so the mark goes on an inner function and the patched name is a plain wrapper around it: the
+    # tracer sees one call it must not enter and runs it as it is.
+    serve_untraced = torch.compiler.disable(serve)
+
+    @functools.wraps(original)
+    def shim(logits, *args, **kwargs):
+        return serve_untraced(logits, *args, **kwargs)
+
     shim.__verl_amd_original__ = original
     return shim
 
@@ -104,15 +196,19 @@ def _make_fused_linear_class(original_cls):
 
 
 def _make_linear_cross_entropy(original):
-    @functools.wraps(original)
-    def linear_cross_entropy(hidden, weight, labels, temperature=1.0, reduction="none", dist_process_group=None):
+    def serve(hidden, weight, labels, temperature=1.0, reduction="none", dist_process_group=None):
         if dist_process_group is None and _eligible_pair(hidden, weight):
             _stats["hip_calls"] += 1
             return _fl.linear_cross_entropy(hidden, weight, labels, temperature, reduction)
         _stats["passed_to_verl"] += 1
         return original(hidden, weight, labels, temperature, reduction, dist_process_group)
 
-    linear_cross_entropy = torch.compiler.disable(linear_cross_entropy)
+    serve_untraced = torch.compiler.disable(serve)   # see _make_shim
+
+    @functools.wraps(original)
+    def linear_cross_entropy(hidden, weight, labels, temperature=1.0, reduction="none", dist_process_group=None):
+        return serve_untraced(hidden, weight, labels, temperature, reduction, dist_process_group)
+
     linear_cross_entropy.__verl_amd_original__ = original
     return linear_cross_entropy
 
@@ -191,3 +287,5 @@ def uninstall() -> None:
     _optional_patched.clear()
     _stats["hip_calls"] = 0
     _stats["passed_to_verl"] = 0
+    _stats["memo_hits"] = 0
+    _memo_clear()

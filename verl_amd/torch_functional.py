@@ -258,6 +258,28 @@ def rowscore(
     return lp, h
 
 
+def _score_once(logits: torch.Tensor, labels: Optional[torch.Tensor]):
+    """No-grad helper for callers that keep per-row results of one pass around: (logprob | None, entropy, lse), each
+    fp32 of shape logits.shape[:-1]; None when the logits are not a plain row-major block (the caller then takes the
+    ordinary route)."""
+    if _is_batch_of_row_slices(logits):
+        return None
+    lead = logits.shape[:-1]
+    x = _rows_2d(logits)
+    if x.data_ptr() != logits.data_ptr() or x.shape[0] == 0:
+        return None
+    lab = None
+    if labels is not None:
+        if tuple(labels.shape) != tuple(lead) or labels.dtype.is_floating_point or labels.dtype == torch.bool:
+            return None
+        lab = labels.to(device=x.device, dtype=torch.int64).reshape(-1).contiguous()
+    with torch.no_grad():
+        lp, h, _, lse, flag = _forward_2d(x, lab, None, lab is not None, True, False, True, None)
+    if lab is not None and LABEL_CHECK and (int(flag.item()) & _lib.VRL_FLAG_LABEL_OOB):
+        raise IndexError(f"a label is outside [0, {logits.shape[-1]})")
+    return (None if lp is None else lp.reshape(lead)), h.reshape(lead), lse.reshape(lead)
+
+
 def logprobs_from_logits(logits: torch.Tensor, labels: torch.Tensor, inplace_backward: bool = True) -> torch.Tensor:
     """log softmax(logits)[labels], shape logits.shape[:-1], fp32.
 
