@@ -160,6 +160,13 @@ def test_one_pass_serves_entropy_and_logprobs_of_the_same_tensor(dev, monkeypatc
         tf.entropy_from_logits(zg).sum().backward()
         tf.logprobs_from_logits(zg, lab).sum().backward()
         assert hook.stats()["memo_hits"] == before and zg.grad is not None
+        # inference-mode tensors carry no version counter: served by the ordinary route
+        with torch.inference_mode():
+            xi = x.clone()
+            n0 = len(launches)
+            hi = tf.entropy_from_logits(xi)
+            tf.logprobs_from_logits(xi, lab)
+        assert len(launches) == n0 + 2 and torch.equal(hi, want_h)
         # and it can be switched off
         monkeypatch.setattr(hook, "MEMO", False)
         n0 = len(launches)

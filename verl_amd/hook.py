@@ -93,8 +93,8 @@ _ENTROPY_NAMES = ("entropy_from_logits", "entropy_from_logits_with_chunking")
 
 def _memo_serve(name, logits, args, kwargs):
     """The result of ``name(logits, ...)`` from one shared pass, or None when the ordinary route must be taken."""
-    if not MEMO or torch.is_grad_enabled() and logits.requires_grad:
-        return None
+    if not MEMO or (torch.is_grad_enabled() and logits.requires_grad) or logits.is_inference():
+        return None   # (inference-mode tensors have no version counter to check against)
     stream = _lib.stream_ptr(logits.device)
     hit = _memo.matches(logits, stream)
     if name in _ENTROPY_NAMES:
