@@ -28,7 +28,7 @@ import importlib
 import os
 import sys
 import weakref
-from typing import Callable, Dict, List, Tuple
+from typing import Callable, Dict, List, Optional, Tuple
 
 import torch
 
@@ -57,34 +57,39 @@ MEMO = os.environ.get("VERL_AMD_MEMO", "1") not in ("0", "false", "False")
 
 
 class _RowMemo:
+    """What one pass over a logits tensor left behind. Built completely before it is published and never changed
+    afterwards, so a reader in another thread sees either the whole of it or the one before."""
+
     __slots__ = ("ref", "version", "ptr", "shape", "stride", "dtype", "stream", "entropy", "lse")
 
+    def __init__(self, logits, stream, entropy, lse):
+        self.ref = weakref.ref(logits)
+        self.version = logits._version
+        self.ptr = logits.data_ptr()
+        self.shape = tuple(logits.shape)
+        self.stride = tuple(logits.stride())
+        self.dtype = logits.dtype
+        self.stream = stream
+        self.entropy = entropy
+        self.lse = lse
+
     def matches(self, logits, stream) -> bool:
-        return (self.ref is not None and self.ref() is logits and self.version == logits._version
-                and self.ptr == logits.data_ptr() and self.shape == tuple(logits.shape)
-                and self.stride == tuple(logits.stride()) and self.dtype == logits.dtype and self.stream == stream)
+        return (self.ref() is logits and self.version == logits._version and self.ptr == logits.data_ptr()
+                and self.shape == tuple(logits.shape) and self.stride == tuple(logits.stride())
+                and self.dtype == logits.dtype and self.stream == stream)
 
 
-_memo = _RowMemo()
-_memo.ref = None
+_memo: Optional[_RowMemo] = None
 
 
 def _memo_store(logits, stream, entropy, lse) -> None:
-    _memo.ref = weakref.ref(logits)
-    _memo.version = logits._version
-    _memo.ptr = logits.data_ptr()
-    _memo.shape = tuple(logits.shape)
-    _memo.stride = tuple(logits.stride())
-    _memo.dtype = logits.dtype
-    _memo.stream = stream
-    _memo.entropy = entropy
-    _memo.lse = lse
+    global _memo
+    _memo = _RowMemo(logits, stream, entropy, lse)   # one reference assignment
 
 
 def _memo_clear() -> None:
-    _memo.ref = None
-    _memo.entropy = None
-    _memo.lse = None
+    global _memo
+    _memo = None
 
 
 _LOGPROB_NAMES = ("logprobs_from_logits", "logprobs_from_logits_v2", "logprobs_from_logits_naive")
@@ -96,11 +101,12 @@ def _memo_serve(name, logits, args, kwargs):
     if not MEMO or (torch.is_grad_enabled() and logits.requires_grad) or logits.is_inference():
         return None   # (inference-mode tensors have no version counter to check against)
     stream = _lib.stream_ptr(logits.device)
-    hit = _memo.matches(logits, stream)
+    memo = _memo   # one read: the object it names cannot change under us
+    hit = memo is not None and memo.matches(logits, stream)
     if name in _ENTROPY_NAMES:
         if hit:
             _stats["memo_hits"] += 1
-            return _memo.entropy
+            return memo.entropy
         got = _amd._score_once(logits, None)
         if got is None:
             return None
@@ -117,7 +123,7 @@ def _memo_serve(name, logits, args, kwargs):
                 raise IndexError(f"{name}: a label is outside [0, {V})")
             picked = torch.gather(logits, -1, lab.clamp(0, V - 1).unsqueeze(-1)).squeeze(-1)
             _stats["memo_hits"] += 1
-            return picked.float() - _memo.lse
+            return picked.float() - memo.lse
         got = _amd._score_once(logits, labels)
         if got is None:
             return None
