@@ -136,6 +136,9 @@ def test_one_pass_serves_entropy_and_logprobs_of_the_same_tensor(dev, monkeypatc
             h2 = tf.entropy_from_logits_with_chunking(y, chunk_size=128)
         assert len(launches) == 2 and hook.stats()["memo_hits"] == 2
         assert torch.equal(lp2, want_lp) and torch.equal(h2, want_h)
+        with torch.no_grad():                                   # what a caller does to its result stays its own business
+            h2.zero_()
+            assert torch.equal(tf.entropy_from_logits(y), want_h)
         # an in-place write (also through a view) invalidates what was kept
         with torch.no_grad():
             y[5:7].mul_(0.5)

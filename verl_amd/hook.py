@@ -70,7 +70,7 @@ class _RowMemo:
         self.stride = tuple(logits.stride())
         self.dtype = logits.dtype
         self.stream = stream
-        self.entropy = entropy
+        self.entropy = entropy.clone()   # private: the caller may write into the tensor it was given
         self.lse = lse
 
     def matches(self, logits, stream) -> bool:
@@ -106,7 +106,7 @@ def _memo_serve(name, logits, args, kwargs):
     if name in _ENTROPY_NAMES:
         if hit:
             _stats["memo_hits"] += 1
-            return memo.entropy
+            return memo.entropy.clone()
         got = _amd._score_once(logits, None)
         if got is None:
             return None
