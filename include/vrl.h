@@ -40,6 +40,7 @@ extern "C" {
 #define VRL_ERR_ALIGN (-4)     /* pointer not aligned to its element size */
 #define VRL_ERR_HIP (-5)       /* the HIP runtime refused the launch; see vrl_last_hip_error */
 #define VRL_ERR_ARG (-6)       /* inconsistent optional arguments */
+#define VRL_ERR_SCRATCH (-7)   /* the request does not fit the library's static scratch (vrl_rowscore_split_static) */
 
 /* logits element types */
 #define VRL_F32 0
@@ -92,6 +93,24 @@ int vrl_rowscore_split(const void* logits, int dtype, int64_t n_rows, int64_t vo
                        float* out_entropy, float* out_sum_pi_sq, float* out_lse, int32_t* err_flag,
                        int n_splits, float* partials, void* stream);
 int vrl_rowscore_split_plan(int dtype, int64_t n_rows, int64_t vocab);
+
+/*
+ * vrl_rowscore_split_static — vrl_rowscore_split for callers that cannot allocate: code under HIP graph
+ * capture, tight serving loops, harnesses that forbid hipMalloc. It has no counterpart in the reference.
+ * Same arguments and results (bit for bit) as vrl_rowscore_split minus `partials`: the partial results live in
+ * a static device array inside the library of VRL_STATIC_PARTIALS_MAX (row, slice) entries of 16 bytes
+ * (128 KiB on every GPU the library runs on, held until the process ends). n_rows * n_splits beyond that
+ * returns VRL_ERR_SCRATCH and launches nothing (n_splits == 1 needs no scratch and takes any n_rows).
+ * The call allocates and frees nothing. Every call on one GPU shares that GPU's array: calls that overlap in
+ * time on one GPU (two streams, two threads) race and must be serialised by the caller; calls on different
+ * GPUs are independent. The first call on a device looks the array's address up (hipGetSymbolAddress), so
+ * make one call outside any graph capture first.
+ */
+#define VRL_STATIC_PARTIALS_MAX 8192
+int vrl_rowscore_split_static(const void* logits, int dtype, int64_t n_rows, int64_t vocab, int64_t row_stride,
+                              const int64_t* labels, const float* temperature, float* out_logprob,
+                              float* out_entropy, float* out_sum_pi_sq, float* out_lse, int32_t* err_flag,
+                              int n_splits, void* stream);
 
 /*
  * vrl_rowscore_backward — gradient of the row op with respect to the logits,

@@ -46,7 +46,8 @@ def test_library_exports_every_declared_symbol(lib):
 
 def test_status_codes_match_header_and_have_text(lib):
     text = open(HEADER).read()
-    for name in ("VRL_OK", "VRL_ERR_NULL", "VRL_ERR_DTYPE", "VRL_ERR_SHAPE", "VRL_ERR_ALIGN", "VRL_ERR_HIP", "VRL_ERR_ARG"):
+    for name in ("VRL_OK", "VRL_ERR_NULL", "VRL_ERR_DTYPE", "VRL_ERR_SHAPE", "VRL_ERR_ALIGN", "VRL_ERR_HIP", "VRL_ERR_ARG",
+                 "VRL_ERR_SCRATCH"):
         m = re.search(rf"#define {name} \(?(-?\d+)\)?", text)
         assert int(m.group(1)) == getattr(_lib, name), name
         assert lib.vrl_strerror(getattr(_lib, name)).decode() not in ("", "unknown vrl status")
@@ -99,6 +100,21 @@ def test_split_and_slice_argument_errors(lib):
     assert call(partials=P + 2) == _lib.VRL_ERR_ALIGN
     assert call(dtype=9) == _lib.VRL_ERR_DTYPE
     assert call(n=0, partials=None) == _lib.VRL_OK
+
+    g = lib.vrl_rowscore_split_static
+
+    def call_static(n=4, splits=4, lp=P, dtype=_lib.VRL_BF16):
+        return g(P, dtype, n, 100000, 100000, P, None, lp, P, None, None, P, splits, None)
+
+    assert call_static(splits=0) == _lib.VRL_ERR_ARG
+    assert call_static(splits=65) == _lib.VRL_ERR_ARG
+    assert call_static(dtype=9) == _lib.VRL_ERR_DTYPE
+    assert call_static(lp=P + 2) == _lib.VRL_ERR_ALIGN
+    assert call_static(n=0) == _lib.VRL_OK
+    assert call_static(n=129, splits=64) == _lib.VRL_ERR_SCRATCH      # 8256 partials > VRL_STATIC_PARTIALS_MAX
+    assert call_static(n=8193, splits=2) == _lib.VRL_ERR_SCRATCH
+    m = re.search(r"#define VRL_STATIC_PARTIALS_MAX (\d+)", open(HEADER).read())
+    assert int(m.group(1)) == _lib.STATIC_PARTIALS_MAX
     plan = lib.vrl_rowscore_split_plan
     assert plan(_lib.VRL_BF16, 8192, 151936) == 1          # enough rows: one workgroup per row
     assert plan(_lib.VRL_BF16, 2048, 151936) == 1

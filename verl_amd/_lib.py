@@ -20,6 +20,8 @@ VRL_ERR_SHAPE = -3
 VRL_ERR_ALIGN = -4
 VRL_ERR_HIP = -5
 VRL_ERR_ARG = -6
+VRL_ERR_SCRATCH = -7
+STATIC_PARTIALS_MAX = 8192
 
 VRL_F32 = 0
 VRL_BF16 = 1
@@ -40,6 +42,7 @@ _F32 = _c.c_float
 SIGNATURES = {
     "vrl_rowscore": (_INT, [_P, _INT, _I64, _I64, _I64, _P, _P, _P, _P, _P, _P, _P, _P]),
     "vrl_rowscore_split": (_INT, [_P, _INT, _I64, _I64, _I64, _P, _P, _P, _P, _P, _P, _P, _INT, _P, _P]),
+    "vrl_rowscore_split_static": (_INT, [_P, _INT, _I64, _I64, _I64, _P, _P, _P, _P, _P, _P, _P, _INT, _P]),
     "vrl_rowscore_backward": (_INT, [_P, _INT, _I64, _I64, _I64, _P, _P, _P, _P, _P, _P, _P, _I64, _P]),
     "vrl_rowscore_split_plan": (_INT, [_INT, _I64, _I64]),
     "vrl_response_slice": (_INT, [_P, _P, _P, _I64, _I64, _P, _P, _P]),

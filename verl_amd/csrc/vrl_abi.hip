@@ -7,6 +7,8 @@
 #include <stdint.h>
 #include <string.h>
 
+#include <atomic>
+
 #include "backward_kernels.h"
 #include "layout_kernels.h"
 #include "lmhead_kernels.h"
@@ -33,6 +35,15 @@ bool aligned(const void* p, uintptr_t a) { return (reinterpret_cast<uintptr_t>(p
 bool known_dtype(int dtype) { return dtype == VRL_F32 || dtype == VRL_BF16 || dtype == VRL_F16; }
 
 constexpr int64_t kMaxGrid = 0x7fffffffLL;
+
+// Device-resident scratch of vrl_rowscore_split_static: VRL_STATIC_PARTIALS_MAX (row, slice) partials of 4 floats.
+// Each GPU the library runs on holds its own copy of this array at its own address until the process ends. On the
+// host the name `scratch` is only a handle for hipGetSymbolAddress, never a device address: kernels and copies get
+// the per-device pointer that static_scratch() looks up once per device.
+static __device__ __align__(256) float scratch[VRL_STATIC_PARTIALS_MAX * 4];
+
+constexpr int kMaxDevices = 64;
+std::atomic<float*> g_scratch_ptr[kMaxDevices];
 
 // Workgroup shape of the row kernel (wavefronts per row, 128-bit loads per lane
 // and batch), chosen by measurement on MI355X at 8192 x 151936 and 32768 x 152064.
@@ -110,6 +121,26 @@ int64_t split_slice_elems(int64_t vocab, int n_splits, int dtype) {
 // 8-wavefront shape is ahead (6.99 against 6.85).
 constexpr int64_t kWideRowsBelow = 16384;
 constexpr int64_t kWideVocabFrom = 16384;  // shorter rows would leave most of 1024 lanes without a vector
+
+// Address of `scratch` on the current device (looked up on the first call per device; two threads racing through the
+// first call store the same value).
+int static_scratch(float** out) {
+  int dev = -1;
+  if (hipGetDevice(&dev) != hipSuccess) return launch_status();
+  if (dev < 0 || dev >= kMaxDevices) return VRL_ERR_SHAPE;
+  float* p = g_scratch_ptr[dev].load(std::memory_order_acquire);
+  if (p == nullptr) {
+    void* sym = nullptr;
+    if (hipGetSymbolAddress(&sym, HIP_SYMBOL(scratch)) != hipSuccess || sym == nullptr) {
+      const int st = launch_status();
+      return st != VRL_OK ? st : VRL_ERR_HIP;
+    }
+    p = static_cast<float*>(sym);
+    g_scratch_ptr[dev].store(p, std::memory_order_release);
+  }
+  *out = p;
+  return VRL_OK;
+}
 
 template <int DT, int W, int U, bool EXACT, bool WANT_Q>
 void launch_row_kernel(const RowArgs& a) {
@@ -261,6 +292,30 @@ int vrl_rowscore_split(const void* logits, int dtype, int64_t n_rows, int64_t vo
   if (n_rows == 0) return VRL_OK;
   if (n_splits > 1 && partials == nullptr) return VRL_ERR_NULL;
   if (!aligned(partials, 4)) return VRL_ERR_ALIGN;
+  const RowArgs a{logits, n_rows, vocab, row_stride, labels, temperature, out_logprob, out_entropy,
+                  out_sum_pi_sq, out_lse, err_flag, n_splits, partials, static_cast<hipStream_t>(stream)};
+  launch_rows_any(dtype, a);
+  return launch_status();
+}
+
+int vrl_rowscore_split_static(const void* logits, int dtype, int64_t n_rows, int64_t vocab, int64_t row_stride,
+                              const int64_t* labels, const float* temperature, float* out_logprob,
+                              float* out_entropy, float* out_sum_pi_sq, float* out_lse, int32_t* err_flag,
+                              int n_splits, void* stream) {
+  const int st = check_rowscore(logits, dtype, n_rows, vocab, row_stride, labels, temperature,
+                                out_logprob, out_entropy, out_sum_pi_sq, out_lse, err_flag);
+  if (st != VRL_OK) return st;
+  if (n_splits < 1 || n_splits > kMaxSplits) return VRL_ERR_ARG;
+  if (n_rows * n_splits > kMaxGrid) return VRL_ERR_SHAPE;
+  if (n_splits > 1 && n_rows * n_splits > VRL_STATIC_PARTIALS_MAX) return VRL_ERR_SCRATCH;
+  if (n_rows == 0) return VRL_OK;
+  float* partials = nullptr;
+  if (n_splits > 1) {
+    const int ss = static_scratch(&partials);
+    if (ss != VRL_OK) return ss;
+  }
+  // Every (row, slice) partial the merge kernel reads is written by the split kernel of the same call first, so
+  // nothing in the array has to start at zero.
   const RowArgs a{logits, n_rows, vocab, row_stride, labels, temperature, out_logprob, out_entropy,
                   out_sum_pi_sq, out_lse, err_flag, n_splits, partials, static_cast<hipStream_t>(stream)};
   launch_rows_any(dtype, a);
@@ -505,6 +560,8 @@ const char* vrl_strerror(int status) {
     case VRL_ERR_ALIGN: return "pointer is not aligned to its element size";
     case VRL_ERR_HIP: return "the HIP runtime refused the kernel launch";
     case VRL_ERR_ARG: return "inconsistent optional arguments";
+    case VRL_ERR_SCRATCH:
+      return "n_rows * n_splits exceeds VRL_STATIC_PARTIALS_MAX, the size of the library's static scratch";
     default: return "unknown vrl status";
   }
 }
