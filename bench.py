@@ -266,14 +266,16 @@ class VerifyOnlyStep:
         self.near = torch.empty(self.B, dtype=torch.int32, device=dev)
         self.out_ids = torch.empty_like(self.ids)
         self.out_mask = torch.empty(self.n, dtype=torch.uint8, device=dev)
+        self.flag = torch.zeros(1, dtype=torch.int32, device=dev)
         self.lib = _lib.load()
         self.stream = torch.cuda.current_stream(dev).cuda_stream
 
     def verify(self):
         st = self.lib.vrl_spec_verify(
             self.lp.data_ptr(), self.lp_old.data_ptr(), self.log_u.data_ptr(), None, self.cu.data_ptr(), self.B, 0,
-            self.off, 1e-6, self.accept.data_ptr(), self.first.data_ptr(), self.prefix.data_ptr(),
-            self.near.data_ptr(), self.ids.data_ptr(), 0, self.out_ids.data_ptr(), self.out_mask.data_ptr(), self.stream)
+            self.n, self.off, 1e-6, self.accept.data_ptr(), self.first.data_ptr(), self.prefix.data_ptr(),
+            self.near.data_ptr(), self.ids.data_ptr(), 0, self.out_ids.data_ptr(), self.out_mask.data_ptr(),
+            self.flag.data_ptr(), self.stream)
         _lib.check("vrl_spec_verify", st)
 
 

@@ -19,7 +19,13 @@
  *     for verify logp/mask/accept) are indexed by the same r.
  *   - Sequence space: sequence b owns rows [cu_seqlens[b], cu_seqlens[b+1])
  *     when cu_seqlens != NULL (packed layout, B+1 int64 entries), else rows
- *     [b*T, (b+1)*T) (padded (B, T) layout).
+ *     [b*T, (b+1)*T) (padded (B, T) layout). `n_tokens` is the length of every
+ *     per-token array: B*T for the padded layout (checked on the host). The
+ *     packed offsets live on the device, so the kernels hold them to n_tokens:
+ *     a span is cut to [0, n_tokens] before anything is indexed with it, and
+ *     offsets that are not a partition of [0, n_tokens] set VRL_FLAG_SEQ_RANGE
+ *     in *err_flag (the reference asserts the same, verl/workers/utils/padding.py:129-130).
+ *     No access ever leaves the arrays, whatever cu_seqlens holds.
  */
 #ifndef VRL_H_
 #define VRL_H_
@@ -30,7 +36,7 @@
 extern "C" {
 #endif
 
-#define VRL_ABI_VERSION 1
+#define VRL_ABI_VERSION 2
 
 /* status codes */
 #define VRL_OK 0
@@ -50,6 +56,8 @@ extern "C" {
 /* bits of *err_flag */
 #define VRL_FLAG_LABEL_OOB 1   /* some label was < 0 or >= vocab; that row's logprob is NaN */
 #define VRL_FLAG_SLICE_RANGE 2 /* vrl_response_slice: a sequence had no prompt token or a bad response length */
+#define VRL_FLAG_SEQ_RANGE 4   /* packed layout: cu_seqlens is not a partition of [0, n_tokens] (first entry != 0,
+                                  last != n_tokens, decreasing, or out of range) */
 
 /*
  * vrl_rowscore — one HBM pass over (n_rows, vocab) logits producing, per row,
@@ -77,6 +85,19 @@ int vrl_rowscore(const void* logits, int dtype, int64_t n_rows, int64_t vocab, i
                  const int64_t* labels, const float* temperature, float* out_logprob,
                  float* out_entropy, float* out_sum_pi_sq, float* out_lse, int32_t* err_flag,
                  void* stream);
+
+/*
+ * vrl_label_logprob — log-probs of the labels from a logsumexp that an earlier pass over the same rows left behind:
+ *   logprob[r] = z[label[r]] - lse[r],   z as in vrl_rowscore
+ * One element load per row instead of a pass over the row: what a caller runs when it asked vrl_rowscore for the
+ * entropy (and out_lse) first and needs the label log-probs of the same logits afterwards, which is the order of the
+ * reference's engine (verl/workers/engine/fsdp/transformer_impl.py:1364-1376 entropy, :1395-1399 log-probs). The
+ * result is within one rounding of lse (fp32) of what vrl_rowscore writes to out_logprob. A label outside [0, vocab)
+ * gives NaN and VRL_FLAG_LABEL_OOB. Replaces the gather of verl/utils/torch_functional.py:194-198.
+ */
+int vrl_label_logprob(const void* logits, int dtype, int64_t n_rows, int64_t vocab, int64_t row_stride,
+                      const int64_t* labels, const float* temperature, const float* lse, float* out_logprob,
+                      int32_t* err_flag, void* stream);
 
 /*
  * vrl_rowscore_split — the same results for FEW rows: n_splits workgroups share
@@ -135,28 +156,30 @@ int vrl_rowscore_backward(const void* logits, int dtype, int64_t n_rows, int64_t
  * vrl_response_slice — packed per-token values (total_nnz,) -> padded (B, T_out)
  * response block: out[b, j] = values[cu_seqlens[b+1] - response_lens[b] - 1 + j]
  * for j < response_lens[b], else 0 (the model output at a position scores the
- * NEXT token, hence the shift by one). Sets VRL_FLAG_SLICE_RANGE and writes a
- * zero row when a sequence has no prompt token, or response_lens[b] is outside
- * [0, T_out].
+ * NEXT token, hence the shift by one). `values` has n_tokens entries. Sets
+ * VRL_FLAG_SLICE_RANGE and writes a zero row when a sequence has no prompt token,
+ * or response_lens[b] is outside [0, T_out]; VRL_FLAG_SEQ_RANGE and a zero row when
+ * the sequence's offsets do not fit n_tokens (see "Sequence space" above).
  *
  * Replaces verl/workers/utils/padding.py:97-141 (no_padding_2_padding) for fp32
  * per-token vectors; fixture: tests/models/test_fsdp_no_padding_on_gpu.py:180-201.
  */
 int vrl_response_slice(const float* values, const int64_t* cu_seqlens, const int64_t* response_lens,
-                       int64_t B, int64_t T_out, float* out, int32_t* err_flag, void* stream);
+                       int64_t B, int64_t n_tokens, int64_t T_out, float* out, int32_t* err_flag, void* stream);
 
 /*
  * vrl_response_pack — packed per-token values (total_nnz,) -> packed response values (sum of response_lens,):
  *   out[out_offsets[b] + j] = values[cu_seqlens[b+1] - response_lens[b] - 1 + j],  j < response_lens[b]
  * out_offsets is the caller's exclusive prefix sum of response_lens (B+1 entries, last = out_total).
  * A sequence without a prompt token, a negative length, or a window that is not exactly
- * [out_offsets[b], out_offsets[b+1]) inside the output sets VRL_FLAG_SLICE_RANGE and writes nothing for it.
+ * [out_offsets[b], out_offsets[b+1]) inside the output sets VRL_FLAG_SLICE_RANGE and writes nothing for it;
+ * offsets that do not fit the n_tokens entries of `values` set VRL_FLAG_SEQ_RANGE and write nothing for it.
  *
  * Replaces verl/workers/utils/padding.py:194-210 (response_from_nested) for fp32 per-token vectors.
  */
 int vrl_response_pack(const float* values, const int64_t* cu_seqlens, const int64_t* response_lens,
-                      const int64_t* out_offsets, int64_t B, int64_t out_total, float* out, int32_t* err_flag,
-                      void* stream);
+                      const int64_t* out_offsets, int64_t B, int64_t n_tokens, int64_t out_total, float* out,
+                      int32_t* err_flag, void* stream);
 
 /*
  * vrl_transpose — out-of-place transposition of a 2-D array of 2-byte (bf16, fp16) or
@@ -235,6 +258,8 @@ int vrl_rollout_corr_num_stats(void);
  *   near_count[b]   = number of valid tokens with |d - tau| < near_eps
  * Optional truncated draft (all three or none): for positions >= first_reject
  *   out_ids = pad_id, out_mask = 0; below it they copy draft_ids / mask.
+ * err_flag is required for the packed layout (VRL_FLAG_SEQ_RANGE; tokens that no
+ * in-range span covers are not written) and may be NULL for the padded one.
  *
  * No function in the reference computes this (its recipe/ submodule is not
  * vendored: .gitmodules:1-3). Layout, mask and sign conventions follow
@@ -243,10 +268,10 @@ int vrl_rollout_corr_num_stats(void);
  * which is where a caller would slot it in (ray_trainer.py:1647-1660).
  */
 int vrl_spec_verify(const float* logp_new, const float* logp_old, const float* log_u,
-                    const uint8_t* mask, const int64_t* cu_seqlens, int64_t B, int64_t T,
+                    const uint8_t* mask, const int64_t* cu_seqlens, int64_t B, int64_t T, int64_t n_tokens,
                     float thresh_offset, float near_eps, uint8_t* accept, int32_t* first_reject,
                     int32_t* prefix_len, int32_t* near_count, const int64_t* draft_ids,
-                    int64_t pad_id, int64_t* out_ids, uint8_t* out_mask, void* stream);
+                    int64_t pad_id, int64_t* out_ids, uint8_t* out_mask, int32_t* err_flag, void* stream);
 
 /*
  * vrl_truncate_draft — apply an already known first_reject[b] to a draft:
@@ -255,16 +280,16 @@ int vrl_spec_verify(const float* logp_new, const float* logp_old, const float* l
  * reference step is the mask rewrite at verl/trainer/ppo/rollout_corr_helper.py:1061.
  */
 int vrl_truncate_draft(const int64_t* draft_ids, const uint8_t* mask, const int64_t* cu_seqlens,
-                       int64_t B, int64_t T, const int32_t* first_reject, int64_t pad_id,
-                       int64_t* out_ids, uint8_t* out_mask, void* stream);
+                       int64_t B, int64_t T, int64_t n_tokens, const int32_t* first_reject, int64_t pad_id,
+                       int64_t* out_ids, uint8_t* out_mask, int32_t* err_flag, void* stream);
 
 /*
  * vrl_fused_score_verify — scoring and verification of the same batch in one
  * call: the results of vrl_rowscore, and of vrl_spec_verify fed with the
  * log-probs just computed (logp_new = out_logprob, which is therefore required).
- * Row space and sequence space are as above: n_rows must equal cu_seqlens[B]
- * (packed) or B*T (padded); the host checks only the padded case, cu_seqlens
- * lives on the device.
+ * Row space and sequence space are as above with n_tokens = n_rows: the host
+ * checks n_rows == B*T (padded); the verify kernel holds the packed offsets to
+ * n_rows and reports VRL_FLAG_SEQ_RANGE through the same err_flag.
  *
  * Two launches on `stream`: the row kernel, then the verify kernel. (Doing the
  * verification inside the row kernel, by the last workgroup of each sequence,

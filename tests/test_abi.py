@@ -139,24 +139,43 @@ def test_split_and_slice_argument_errors(lib):
     assert back(dx=P + 1) == _lib.VRL_ERR_ALIGN
     assert back(n=0, x=None, dx=None, lse=None) == _lib.VRL_OK
 
-    g = lib.vrl_response_slice
-    assert g(P, P, P, -1, 4, P, P, None) == _lib.VRL_ERR_SHAPE
-    assert g(None, P, P, 2, 4, P, P, None) == _lib.VRL_ERR_NULL
-    assert g(P, P, P, 2, 4, P, None, None) == _lib.VRL_ERR_NULL
-    assert g(P, P + 4, P, 2, 4, P, P, None) == _lib.VRL_ERR_ALIGN
-    assert g(None, None, None, 0, 4, None, None, None) == _lib.VRL_OK
+    g = lib.vrl_response_slice     # (values, cu, response_lens, B, n_tokens, T_out, out, err_flag, stream)
+    assert g(P, P, P, -1, 9, 4, P, P, None) == _lib.VRL_ERR_SHAPE
+    assert g(P, P, P, 2, -1, 4, P, P, None) == _lib.VRL_ERR_SHAPE
+    assert g(None, P, P, 2, 9, 4, P, P, None) == _lib.VRL_ERR_NULL
+    assert g(P, P, P, 2, 9, 4, P, None, None) == _lib.VRL_ERR_NULL
+    assert g(P, P + 4, P, 2, 9, 4, P, P, None) == _lib.VRL_ERR_ALIGN
+    assert g(None, None, None, 0, 0, 4, None, None, None) == _lib.VRL_OK
+
+
+def test_label_logprob_argument_errors_and_flag_values(lib):
+    f = lib.vrl_label_logprob     # (logits, dtype, n_rows, vocab, row_stride, labels, temperature, lse, out, err_flag, stream)
+    assert f(P, 9, 4, 100, 100, P, None, P, P, P, None) == _lib.VRL_ERR_DTYPE
+    assert f(P, _lib.VRL_BF16, -1, 100, 100, P, None, P, P, P, None) == _lib.VRL_ERR_SHAPE
+    assert f(P, _lib.VRL_BF16, 4, 100, 99, P, None, P, P, P, None) == _lib.VRL_ERR_SHAPE
+    for missing in (0, 5, 7, 8, 9):
+        args = [P, _lib.VRL_BF16, 4, 100, 100, P, None, P, P, P, None]
+        args[missing] = None
+        assert f(*args) == _lib.VRL_ERR_NULL, missing
+    assert f(P, _lib.VRL_F32, 4, 100, 100, P, None, P + 2, P, P, None) == _lib.VRL_ERR_ALIGN
+    assert f(None, _lib.VRL_F32, 0, 100, 100, None, None, None, None, None, None) == _lib.VRL_OK
+    text = open(HEADER).read()
+    for name in ("VRL_FLAG_LABEL_OOB", "VRL_FLAG_SLICE_RANGE", "VRL_FLAG_SEQ_RANGE"):
+        m = re.search(rf"#define {name} (\d+)", text)
+        assert int(m.group(1)) == getattr(_lib, name), name
 
 
 def test_response_pack_argument_errors(lib):
-    g = lib.vrl_response_pack
-    assert g(P, P, P, P, -1, 4, P, P, None) == _lib.VRL_ERR_SHAPE
-    assert g(P, P, P, P, 2, -1, P, P, None) == _lib.VRL_ERR_SHAPE
-    assert g(None, P, P, P, 2, 4, P, P, None) == _lib.VRL_ERR_NULL
-    assert g(P, P, P, None, 2, 4, P, P, None) == _lib.VRL_ERR_NULL
-    assert g(P, P, P, P, 2, 4, None, P, None) == _lib.VRL_ERR_NULL
-    assert g(P, P, P, P, 2, 4, P, None, None) == _lib.VRL_ERR_NULL
-    assert g(P, P, P, P + 4, 2, 4, P, P, None) == _lib.VRL_ERR_ALIGN
-    assert g(None, None, None, None, 0, 0, None, None, None) == _lib.VRL_OK
+    g = lib.vrl_response_pack      # (values, cu, response_lens, out_offsets, B, n_tokens, out_total, out, err_flag, stream)
+    assert g(P, P, P, P, -1, 9, 4, P, P, None) == _lib.VRL_ERR_SHAPE
+    assert g(P, P, P, P, 2, 9, -1, P, P, None) == _lib.VRL_ERR_SHAPE
+    assert g(P, P, P, P, 2, -9, 4, P, P, None) == _lib.VRL_ERR_SHAPE
+    assert g(None, P, P, P, 2, 9, 4, P, P, None) == _lib.VRL_ERR_NULL
+    assert g(P, P, P, None, 2, 9, 4, P, P, None) == _lib.VRL_ERR_NULL
+    assert g(P, P, P, P, 2, 9, 4, None, P, None) == _lib.VRL_ERR_NULL
+    assert g(P, P, P, P, 2, 9, 4, P, None, None) == _lib.VRL_ERR_NULL
+    assert g(P, P, P, P + 4, 2, 9, 4, P, P, None) == _lib.VRL_ERR_ALIGN
+    assert g(None, None, None, None, 0, 0, 0, None, None, None) == _lib.VRL_OK
 
 
 def test_lmhead_argument_errors(lib):
@@ -224,8 +243,14 @@ def test_rollout_corr_argument_errors(lib):
 def test_verify_argument_errors(lib):
     f = lib.vrl_spec_verify
 
-    def call(ln=P, lo=P, lu=P, mask=None, cu=None, B=2, T=8, accept=P, first=P, prefix=P, near=P, ids=None, out_ids=None, out_mask=None):
-        return f(ln, lo, lu, mask, cu, B, T, 0.0, 1e-6, accept, first, prefix, near, ids, 0, out_ids, out_mask, None)
+    def call(ln=P, lo=P, lu=P, mask=None, cu=None, B=2, T=8, n=16, accept=P, first=P, prefix=P, near=P, ids=None,
+             out_ids=None, out_mask=None, flag=None):
+        return f(ln, lo, lu, mask, cu, B, T, n, 0.0, 1e-6, accept, first, prefix, near, ids, 0, out_ids, out_mask, flag, None)
+
+    assert call(n=15) == _lib.VRL_ERR_SHAPE                       # padded: the arrays hold exactly B*T tokens
+    assert call(n=-1) == _lib.VRL_ERR_SHAPE
+    assert call(cu=P, n=100) == _lib.VRL_ERR_NULL                 # packed: the offsets are checked on the device, which
+    assert call(cu=P, n=100, flag=P + 2) == _lib.VRL_ERR_ALIGN    # needs somewhere to report to
 
     assert call(B=-1) == _lib.VRL_ERR_SHAPE
     assert call(T=-1) == _lib.VRL_ERR_SHAPE
@@ -236,17 +261,19 @@ def test_verify_argument_errors(lib):
     assert call(ids=P) == _lib.VRL_ERR_ARG                      # draft without outputs
     assert call(ids=P, out_ids=P) == _lib.VRL_ERR_ARG
     assert call(lo=P + 2) == _lib.VRL_ERR_ALIGN
-    assert call(cu=P + 4) == _lib.VRL_ERR_ALIGN
-    assert call(B=0, ln=None, lo=None, lu=None, accept=None, first=None, prefix=None, near=None) == _lib.VRL_OK
+    assert call(cu=P + 4, flag=P) == _lib.VRL_ERR_ALIGN
+    assert call(B=0, n=0, ln=None, lo=None, lu=None, accept=None, first=None, prefix=None, near=None) == _lib.VRL_OK
 
 
 def test_truncate_and_fused_argument_errors(lib):
-    t = lib.vrl_truncate_draft
-    assert t(P, None, None, -1, 4, P, 0, P, P, None) == _lib.VRL_ERR_SHAPE
-    assert t(None, None, None, 2, 4, P, 0, P, P, None) == _lib.VRL_ERR_NULL
-    assert t(P, None, None, 2, 4, None, 0, P, P, None) == _lib.VRL_ERR_NULL
-    assert t(P + 4, None, None, 2, 4, P, 0, P, P, None) == _lib.VRL_ERR_ALIGN
-    assert t(None, None, None, 0, 4, None, 0, None, None, None) == _lib.VRL_OK
+    t = lib.vrl_truncate_draft     # (ids, mask, cu, B, T, n_tokens, first_reject, pad_id, out_ids, out_mask, err_flag, stream)
+    assert t(P, None, None, -1, 4, 8, P, 0, P, P, None, None) == _lib.VRL_ERR_SHAPE
+    assert t(P, None, None, 2, 4, 7, P, 0, P, P, None, None) == _lib.VRL_ERR_SHAPE      # padded: n_tokens == B*T
+    assert t(P, None, P, 2, 0, 7, P, 0, P, P, None, None) == _lib.VRL_ERR_NULL          # packed needs err_flag
+    assert t(None, None, None, 2, 4, 8, P, 0, P, P, None, None) == _lib.VRL_ERR_NULL
+    assert t(P, None, None, 2, 4, 8, None, 0, P, P, None, None) == _lib.VRL_ERR_NULL
+    assert t(P + 4, None, None, 2, 4, 8, P, 0, P, P, None, None) == _lib.VRL_ERR_ALIGN
+    assert t(None, None, None, 0, 4, 0, None, 0, None, None, None, None) == _lib.VRL_OK
 
     f = lib.vrl_fused_score_verify
 

@@ -178,5 +178,13 @@ def test_input_checks(dev):
         fused_linear_for_ppo(h, w, ids, chunk_size=0)
     with pytest.raises(IndexError):
         fused_linear_for_ppo(h, w, torch.full((4,), 16, device=dev))
+    # the kernels read the ids through a raw device pointer: ids that live on the host are moved, never dereferenced
+    got = fused_linear_for_ppo(h, w, ids.cpu())
+    want = fused_linear_for_ppo(h, w, ids)
+    assert torch.equal(got[0], want[0]) and torch.equal(got[1], want[1])
+    with pytest.raises(TypeError):
+        fused_linear_for_ppo(h, w, ids.float())
+    with pytest.raises(TypeError):
+        fused_linear_for_ppo(h, w, ids.bool())
     lp, ent = fused_linear_for_ppo(h[:0], w, ids[:0])
     assert lp.shape == (0,) and ent.shape == (0,)

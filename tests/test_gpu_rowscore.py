@@ -191,16 +191,35 @@ def test_label_out_of_range_raises(dev):
     assert torch.isnan(lp[2]) and torch.isfinite(lp[[0, 1, 3]]).all()
 
 
-def test_label_check_can_be_switched_off_for_the_reference_named_functions(dev, monkeypatch):
-    """The check costs one host synchronisation per call; with the module switch off the call returns without
-    reading anything back and the bad row is NaN."""
+def test_label_check_modes(dev):
+    """Reading the error flag back costs one host synchronisation per call ("sync", the default of direct calls).
+    "off" never looks and the bad row is NaN; "deferred" looks later, without waiting for the GPU inside a call."""
+    from verl_amd import errors
+
     x = torch.randn(4, 50, device=dev)
     lab = torch.tensor([0, 1, 50, 3], device=dev)
-    monkeypatch.setattr(vf, "LABEL_CHECK", False)
-    lp = vf.logprobs_from_logits(x, lab)
-    assert torch.isnan(lp[2]) and torch.isfinite(lp[[0, 1, 3]]).all()
+    with errors.using("off"):
+        lp = vf.logprobs_from_logits(x, lab)
+        assert torch.isnan(lp[2]) and torch.isfinite(lp[[0, 1, 3]]).all()
+        with pytest.raises(IndexError):
+            vf.fused_logprob_entropy(x, lab, check_labels=True)      # an explicit request still checks
+    with errors.using("deferred"):
+        lp = vf.logprobs_from_logits(x, lab)                         # returns at once, the row is NaN
+        assert errors.pending() == 1
+        with pytest.raises(IndexError):
+            errors.check_errors()
+        assert errors.pending() == 0
+        lp = vf.logprobs_from_logits(x, lab)
+        torch.cuda.synchronize()
+        with pytest.raises(IndexError):                              # the next call notices what the last one left
+            vf.entropy_from_logits(x)
+        vf.entropy_from_logits(x)
+        errors.check_errors()
+    lp, _ = vf.fused_logprob_entropy(x, lab, check_labels="deferred")
     with pytest.raises(IndexError):
-        vf.fused_logprob_entropy(x, lab, check_labels=True)      # an explicit request still checks
+        errors.check_errors()
+    with pytest.raises(ValueError):
+        vf.fused_logprob_entropy(x, lab, check_labels="later")
 
 
 def test_rejects_cpu_and_unsupported_inputs(dev):

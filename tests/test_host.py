@@ -112,7 +112,7 @@ def test_install_patches_module_and_bound_names(fake_verl):
     assert eng.logprobs_from_logits(x, torch.zeros(2, dtype=torch.long), inplace_backward=False) == ("verl", "logprobs_from_logits")
     assert tf.entropy_from_logits(x.double()) == ("verl", "entropy_from_logits")
     assert tf.entropy_from_logits_with_chunking(x, chunk_size=3) == ("verl", "entropy_from_logits_with_chunking")
-    assert inst.stats() == {"hip_calls": 0, "passed_to_verl": 4, "memo_hits": 0}
+    assert {k: inst.stats()[k] for k in ("hip_calls", "passed_to_verl", "memo_hits")} == {"hip_calls": 0, "passed_to_verl": 4, "memo_hits": 0}
 
     class Wrapped(torch.Tensor):        # stands for DTensor and other tensor subclasses
         pass
@@ -121,7 +121,7 @@ def test_install_patches_module_and_bound_names(fake_verl):
 
     inst.uninstall()
     assert tf.logprobs_from_logits is orig and eng.logprobs_from_logits is orig
-    assert inst.stats() == {"hip_calls": 0, "passed_to_verl": 0, "memo_hits": 0}
+    assert {k: inst.stats()[k] for k in ("hip_calls", "passed_to_verl", "memo_hits")} == {"hip_calls": 0, "passed_to_verl": 0, "memo_hits": 0}
 
 
 def test_install_patches_the_fused_linear_entry_points_when_present(fake_verl):

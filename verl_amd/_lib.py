@@ -11,7 +11,8 @@ import os
 import threading
 
 LIB_NAME = "libvrl_hip.so"
-LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), LIB_NAME)
+# VERL_AMD_LIB names another build of the same library (the host-sanitised one the ABI tests run against).
+LIB_PATH = os.environ.get("VERL_AMD_LIB") or os.path.join(os.path.dirname(os.path.abspath(__file__)), LIB_NAME)
 
 VRL_OK = 0
 VRL_ERR_NULL = -1
@@ -29,8 +30,9 @@ VRL_F16 = 2
 
 VRL_FLAG_LABEL_OOB = 1
 VRL_FLAG_SLICE_RANGE = 2
+VRL_FLAG_SEQ_RANGE = 4
 
-ABI_VERSION = 1
+ABI_VERSION = 2
 
 _c = ctypes
 _P = _c.c_void_p
@@ -41,12 +43,13 @@ _F32 = _c.c_float
 # name -> (restype, argtypes); mirrors include/vrl.h one to one.
 SIGNATURES = {
     "vrl_rowscore": (_INT, [_P, _INT, _I64, _I64, _I64, _P, _P, _P, _P, _P, _P, _P, _P]),
+    "vrl_label_logprob": (_INT, [_P, _INT, _I64, _I64, _I64, _P, _P, _P, _P, _P, _P]),
     "vrl_rowscore_split": (_INT, [_P, _INT, _I64, _I64, _I64, _P, _P, _P, _P, _P, _P, _P, _INT, _P, _P]),
     "vrl_rowscore_split_static": (_INT, [_P, _INT, _I64, _I64, _I64, _P, _P, _P, _P, _P, _P, _P, _INT, _P]),
     "vrl_rowscore_backward": (_INT, [_P, _INT, _I64, _I64, _I64, _P, _P, _P, _P, _P, _P, _P, _I64, _P]),
     "vrl_rowscore_split_plan": (_INT, [_INT, _I64, _I64]),
-    "vrl_response_slice": (_INT, [_P, _P, _P, _I64, _I64, _P, _P, _P]),
-    "vrl_response_pack": (_INT, [_P, _P, _P, _P, _I64, _I64, _P, _P, _P]),
+    "vrl_response_slice": (_INT, [_P, _P, _P, _I64, _I64, _I64, _P, _P, _P]),
+    "vrl_response_pack": (_INT, [_P, _P, _P, _P, _I64, _I64, _I64, _P, _P, _P]),
     "vrl_lmhead_score": (_INT, [_P, _P, _INT, _I64, _I64, _I64, _I64, _I64, _P, _P, _INT, _P, _P, _P, _P, _P, _P]),
     "vrl_lmhead_plan": (_INT, [_I64, _I64]),
     "vrl_transpose": (_INT, [_P, _INT, _I64, _I64, _I64, _P, _I64, _P]),
@@ -57,9 +60,9 @@ SIGNATURES = {
     "vrl_rollout_corr_num_stats": (_INT, []),
     "vrl_spec_verify": (
         _INT,
-        [_P, _P, _P, _P, _P, _I64, _I64, _F32, _F32, _P, _P, _P, _P, _P, _I64, _P, _P, _P],
+        [_P, _P, _P, _P, _P, _I64, _I64, _I64, _F32, _F32, _P, _P, _P, _P, _P, _I64, _P, _P, _P, _P],
     ),
-    "vrl_truncate_draft": (_INT, [_P, _P, _P, _I64, _I64, _P, _I64, _P, _P, _P]),
+    "vrl_truncate_draft": (_INT, [_P, _P, _P, _I64, _I64, _I64, _P, _I64, _P, _P, _P, _P]),
     "vrl_fused_score_verify": (
         _INT,
         [_P, _INT, _I64, _I64, _I64, _P, _P, _P, _P, _P, _P, _P]

@@ -42,11 +42,40 @@ def hipcc_path() -> str:
     raise RuntimeError("hipcc not found (looked at $HIPCC, PATH and /opt/rocm/bin/hipcc)")
 
 
-def build(verbose: bool = True) -> str:
-    """Compile every HIP source into ``verl_amd/libvrl_hip.so`` and return its path."""
-    cmd = [hipcc_path(), *HIPCC_FLAGS, f"-I{INCLUDE_DIR}", f"-I{CSRC_DIR}"]
+# Host pass only (the argument checks and launchers of the C ABI) under AddressSanitizer and UBSan; the device
+# code is compiled as usual. Each -fsanitize= sits directly behind -Xarch_host.
+HOST_SANITIZE_FLAGS = [
+    "-Xarch_host", "-fsanitize=address",
+    "-Xarch_host", "-fsanitize=undefined",
+    "-Xarch_host", "-fno-omit-frame-pointer",
+    "-g",
+]
+
+
+def asan_runtime() -> str:
+    """The shared AddressSanitizer runtime of hipcc's clang: a sanitised shared library needs it preloaded into the
+    process that loads it (``LD_PRELOAD``)."""
+    clang = os.path.join(os.path.dirname(os.path.realpath(hipcc_path())), "..", "lib", "llvm", "bin", "clang")
+    if not os.path.exists(clang):
+        clang = "/opt/rocm/lib/llvm/bin/clang"
+    out = subprocess.run([clang, "--print-file-name=libclang_rt.asan-x86_64.so"], stdout=subprocess.PIPE, text=True)
+    path = out.stdout.strip()
+    if out.returncode != 0 or not os.path.isabs(path) or not os.path.exists(path):
+        raise RuntimeError("AddressSanitizer runtime of hipcc's clang not found")
+    return path
+
+
+def build(verbose: bool = True, sanitize_host: bool = False, out_path: str | None = None) -> str:
+    """Compile every HIP source into ``verl_amd/libvrl_hip.so`` (or ``out_path``) and return its path. With
+    ``sanitize_host`` the host side is instrumented with ASan + UBSan (for tests of the ABI's argument handling;
+    load it through ``VERL_AMD_LIB`` with ``asan_runtime()`` preloaded)."""
+    lib_path = out_path or LIB_PATH
+    flags = list(HIPCC_FLAGS)
+    if sanitize_host:
+        flags = [("-O1" if f == "-O3" else f) for f in flags] + HOST_SANITIZE_FLAGS
+    cmd = [hipcc_path(), *flags, f"-I{INCLUDE_DIR}", f"-I{CSRC_DIR}"]
     cmd += [os.path.join(CSRC_DIR, s) for s in SOURCES]
-    tmp = LIB_PATH + ".tmp"
+    tmp = lib_path + ".tmp"
     cmd += ["-o", tmp]
     if verbose:
         print("[verl_amd.build]", " ".join(cmd), flush=True)
@@ -57,8 +86,8 @@ def build(verbose: bool = True) -> str:
         raise RuntimeError(f"hipcc failed ({proc.returncode}):\n{out}")
     if verbose and out.strip():
         print(out, flush=True)
-    os.replace(tmp, LIB_PATH)
-    return LIB_PATH
+    os.replace(tmp, lib_path)
+    return lib_path
 
 
 if __name__ == "__main__":

@@ -456,4 +456,29 @@ __global__ __launch_bounds__(64) void rowscore_merge_kernel(
   finalize_row<EXACT, WANT_Q>(w, xl, label_ok, sc, row, out_logprob, out_entropy, out_sum_pi_sq, out_lse, err_flag);
 }
 
+// ---- label log-prob from a known logsumexp ------------------------------------
+// grid.x = ceil(n_rows / 256), block = 256: one lane per row, no barrier. logprob = z[label] - lse with the same
+// scaling of the label logit as finalize_row (double, one rounding at the end); lse = -inf / +inf / NaN propagate by
+// plain arithmetic to what torch's `x.gather(label) - logsumexp(x)` gives.
+template <int DT, bool EXACT>
+__global__ __launch_bounds__(256) void label_logprob_kernel(
+    const void* __restrict__ logits, int64_t n_rows, int64_t vocab, int64_t row_stride,
+    const int64_t* __restrict__ labels, const float* __restrict__ temperature, const float* __restrict__ lse,
+    float* __restrict__ out_logprob, int32_t* err_flag) {
+  const int64_t row = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x;
+  if (row >= n_rows) return;
+  const char* rowp = static_cast<const char*>(logits) + row * row_stride * Elem<DT>::kBytes;
+  const Scale<EXACT> sc = make_scale<EXACT>(temperature, row);
+  bool label_ok = true;
+  const float xl = load_label_logit<DT>(rowp, labels, row, vocab, label_ok);
+  float lp = quiet_nan();
+  if (label_ok) {
+    const double z = kLn2d * (static_cast<double>(sc.pre(xl)) * static_cast<double>(sc.c));
+    lp = static_cast<float>(z - static_cast<double>(lse[row]));
+  } else {
+    atomicOr(err_flag, 1);
+  }
+  out_logprob[row] = lp;
+}
+
 }  // namespace vrl

@@ -21,12 +21,25 @@ struct SeqSpan {
   int64_t len;
 };
 
-__device__ __forceinline__ SeqSpan seq_span(const int64_t* cu_seqlens, int64_t b, int64_t T) {
+constexpr int kFlagSeqRange = 4;  // VRL_FLAG_SEQ_RANGE
+
+// Rows [start, start + len) of sequence b (workgroup b of a grid of B). Packed offsets come from device memory the
+// host cannot see, so they are held to the arrays' size here: a span is cut to [0, n_tokens] (an inverted one to
+// nothing), and offsets that are not a partition of [0, n_tokens] (first != 0, last != n_tokens, decreasing, out of
+// range) set VRL_FLAG_SEQ_RANGE. Nothing outside the per-token arrays is ever touched.
+__device__ __forceinline__ SeqSpan seq_span(const int64_t* cu_seqlens, int64_t b, int64_t T, int64_t n_tokens,
+                                            int32_t* err_flag) {
   SeqSpan s;
   if (cu_seqlens != nullptr) {
-    s.start = cu_seqlens[b];
-    s.len = cu_seqlens[b + 1] - s.start;
-    if (s.len < 0) s.len = 0;
+    int64_t lo = cu_seqlens[b];
+    int64_t hi = cu_seqlens[b + 1];
+    const bool bad = (lo < 0) || (hi > n_tokens) || (hi < lo) || (b == 0 && lo != 0) ||
+                     (b + 1 == static_cast<int64_t>(gridDim.x) && hi != n_tokens);
+    if (bad && threadIdx.x == 0 && err_flag != nullptr) atomicOr(err_flag, kFlagSeqRange);
+    lo = lo < 0 ? 0 : (lo > n_tokens ? n_tokens : lo);
+    hi = hi < lo ? lo : (hi > n_tokens ? n_tokens : hi);
+    s.start = lo;
+    s.len = hi - lo;
   } else {
     s.start = b * T;
     s.len = T;
@@ -63,6 +76,8 @@ struct VerifyArgs {
   const int64_t* cu_seqlens;
   int64_t B;
   int64_t T;
+  int64_t n_tokens;   // length of every per-token array
+  int32_t* err_flag;  // VRL_FLAG_SEQ_RANGE lands here (packed layout)
   float thresh_offset;
   float near_eps;
   uint8_t* accept;
@@ -82,7 +97,7 @@ __device__ __forceinline__ void verify_sequence(const VerifyArgs& v, int64_t b) 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = tid >> 6;
-  const SeqSpan sp = seq_span(v.cu_seqlens, b, v.T);
+  const SeqSpan sp = seq_span(v.cu_seqlens, b, v.T, v.n_tokens, v.err_flag);
 
   // wave-uniform running results
   int first = kNoReject;  // earliest rejected position seen by this wavefront
@@ -183,10 +198,10 @@ __global__ __launch_bounds__(WAVES * 64) void spec_verify_kernel(const VerifyArg
 template <int WAVES>
 __global__ __launch_bounds__(WAVES * 64) void truncate_draft_kernel(
     const int64_t* __restrict__ draft_ids, const uint8_t* __restrict__ mask,
-    const int64_t* __restrict__ cu_seqlens, int64_t T, const int32_t* __restrict__ first_reject,
-    int64_t pad_id, int64_t* __restrict__ out_ids, uint8_t* __restrict__ out_mask) {
+    const int64_t* __restrict__ cu_seqlens, int64_t T, int64_t n_tokens, const int32_t* __restrict__ first_reject,
+    int64_t pad_id, int64_t* __restrict__ out_ids, uint8_t* __restrict__ out_mask, int32_t* err_flag) {
   const int64_t b = blockIdx.x;
-  const SeqSpan sp = seq_span(cu_seqlens, b, T);
+  const SeqSpan sp = seq_span(cu_seqlens, b, T, n_tokens, err_flag);
   truncate_span<WAVES>(sp, first_reject[b], draft_ids, mask, pad_id, out_ids, out_mask);
 }
 

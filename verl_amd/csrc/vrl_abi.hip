@@ -191,19 +191,34 @@ void launch_rows_any(int dtype, const RowArgs& a) {
   }
 }
 
+// Size rules of the sequence space: padded (B, T) arrays hold exactly B*T tokens; packed arrays hold n_tokens and
+// the device-side offsets are checked against it by the kernels, which need somewhere to report to.
+int check_layout(const int64_t* cu_seqlens, int64_t B, int64_t T, int64_t n_tokens, const int32_t* err_flag) {
+  if (B < 0 || T < 0 || n_tokens < 0 || B > kMaxGrid || T > kMaxGrid) return VRL_ERR_SHAPE;
+  if (cu_seqlens == nullptr) {
+    if (n_tokens != B * T) return VRL_ERR_SHAPE;
+  } else if (B > 0 && err_flag == nullptr) {
+    return VRL_ERR_NULL;
+  }
+  if (!aligned(cu_seqlens, 8) || !aligned(err_flag, 4)) return VRL_ERR_ALIGN;
+  return VRL_OK;
+}
+
 int check_verify(const float* logp_new, const float* logp_old, const float* log_u, const uint8_t* mask,
-                 const int64_t* cu_seqlens, int64_t B, int64_t T, const uint8_t* accept,
-                 const int32_t* first_reject, const int32_t* prefix_len, const int32_t* near_count,
-                 const int64_t* draft_ids, const int64_t* out_ids, const uint8_t* out_mask) {
+                 const int64_t* cu_seqlens, int64_t B, int64_t T, int64_t n_tokens, const int32_t* err_flag,
+                 const uint8_t* accept, const int32_t* first_reject, const int32_t* prefix_len,
+                 const int32_t* near_count, const int64_t* draft_ids, const int64_t* out_ids,
+                 const uint8_t* out_mask) {
   (void)mask;
-  if (B < 0 || T < 0 || B > kMaxGrid || T > kMaxGrid) return VRL_ERR_SHAPE;
+  const int ls = check_layout(cu_seqlens, B, T, n_tokens, err_flag);
+  if (ls != VRL_OK) return ls;
   const bool any_trunc = (draft_ids != nullptr) || (out_ids != nullptr) || (out_mask != nullptr);
   const bool all_trunc = (draft_ids != nullptr) && (out_ids != nullptr) && (out_mask != nullptr);
   if (any_trunc && !all_trunc) return VRL_ERR_ARG;
   if (B == 0) return VRL_OK;
   if (first_reject == nullptr || prefix_len == nullptr || near_count == nullptr) return VRL_ERR_NULL;
-  // A padded layout with T == 0 has no tokens: the kernel only writes the per-sequence zeros.
-  const bool has_tokens = (cu_seqlens != nullptr) || (T > 0);
+  // Without tokens the kernel only writes the per-sequence zeros.
+  const bool has_tokens = n_tokens > 0;
   if (has_tokens && (logp_new == nullptr || logp_old == nullptr || log_u == nullptr || accept == nullptr))
     return VRL_ERR_NULL;
   if (!aligned(logp_new, 4) || !aligned(logp_old, 4) || !aligned(log_u, 4) || !aligned(cu_seqlens, 8) ||
@@ -232,9 +247,18 @@ int launch_lmhead(const void* hidden, const void* weight, int64_t T, int64_t V, 
   const int tiles_per_split = static_cast<int>((vtiles + n_splits - 1) / n_splits);
   // 8 token blocks x 4 splits per XCD when the grid divides that way (see the kernel's mapping)
   const int xcd_map = (tblocks % 8 == 0 && n_splits % 4 == 0 && ((tblocks / 8) * (n_splits / 4)) % 8 == 0) ? 1 : 0;
-  if (hipFuncSetAttribute(reinterpret_cast<const void*>(vrl::lmhead_partial_kernel<DT>),
-                          hipFuncAttributeMaxDynamicSharedMemorySize, vrl::kLmLdsBytes) != hipSuccess)
-    return launch_status();
+  {  // the kernel's LDS request is above the default limit: raise it once per device, not per launch
+    static std::atomic<bool> raised[kMaxDevices];
+    int dev = -1;
+    if (hipGetDevice(&dev) != hipSuccess) return launch_status();
+    if (dev < 0 || dev >= kMaxDevices) return VRL_ERR_SHAPE;
+    if (!raised[dev].load(std::memory_order_acquire)) {
+      if (hipFuncSetAttribute(reinterpret_cast<const void*>(vrl::lmhead_partial_kernel<DT>),
+                              hipFuncAttributeMaxDynamicSharedMemorySize, vrl::kLmLdsBytes) != hipSuccess)
+        return launch_status();
+      raised[dev].store(true, std::memory_order_release);
+    }
+  }
   vrl::lmhead_partial_kernel<DT><<<dim3(static_cast<unsigned>(tblocks * n_splits)), dim3(256), vrl::kLmLdsBytes, s>>>(
       static_cast<const uint16_t*>(weight), static_cast<const uint16_t*>(hidden), V, T, K, w_stride, h_stride,
       temperature, n_splits, tiles_per_split, xcd_map, partials);
@@ -258,6 +282,37 @@ int vrl_rowscore(const void* logits, int dtype, int64_t n_rows, int64_t vocab, i
   const RowArgs a{logits, n_rows, vocab, row_stride, labels, temperature, out_logprob, out_entropy,
                   out_sum_pi_sq, out_lse, err_flag, 1, nullptr, static_cast<hipStream_t>(stream)};
   launch_rows_any(dtype, a);
+  return launch_status();
+}
+
+int vrl_label_logprob(const void* logits, int dtype, int64_t n_rows, int64_t vocab, int64_t row_stride,
+                      const int64_t* labels, const float* temperature, const float* lse, float* out_logprob,
+                      int32_t* err_flag, void* stream) {
+  if (!known_dtype(dtype)) return VRL_ERR_DTYPE;
+  if (n_rows < 0 || vocab <= 0 || row_stride < vocab || (n_rows + 255) / 256 > kMaxGrid) return VRL_ERR_SHAPE;
+  if (n_rows == 0) return VRL_OK;
+  if (logits == nullptr || labels == nullptr || lse == nullptr || out_logprob == nullptr || err_flag == nullptr)
+    return VRL_ERR_NULL;
+  const uintptr_t esize = (dtype == VRL_F32) ? 4 : 2;
+  if (!aligned(logits, esize) || !aligned(labels, 8) || !aligned(temperature, 4) || !aligned(lse, 4) ||
+      !aligned(out_logprob, 4) || !aligned(err_flag, 4))
+    return VRL_ERR_ALIGN;
+  const dim3 grid(static_cast<unsigned>((n_rows + 255) / 256));
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  if (dtype == VRL_F32) {
+    if (temperature != nullptr)
+      vrl::label_logprob_kernel<VRL_F32, true><<<grid, dim3(256), 0, s>>>(logits, n_rows, vocab, row_stride, labels,
+                                                                          temperature, lse, out_logprob, err_flag);
+    else
+      vrl::label_logprob_kernel<VRL_F32, false><<<grid, dim3(256), 0, s>>>(logits, n_rows, vocab, row_stride, labels,
+                                                                           temperature, lse, out_logprob, err_flag);
+  } else if (dtype == VRL_BF16) {
+    vrl::label_logprob_kernel<VRL_BF16, false><<<grid, dim3(256), 0, s>>>(logits, n_rows, vocab, row_stride, labels,
+                                                                          temperature, lse, out_logprob, err_flag);
+  } else {
+    vrl::label_logprob_kernel<VRL_F16, false><<<grid, dim3(256), 0, s>>>(logits, n_rows, vocab, row_stride, labels,
+                                                                         temperature, lse, out_logprob, err_flag);
+  }
   return launch_status();
 }
 
@@ -384,33 +439,33 @@ int vrl_rollout_corr(const float* old_log_prob, const float* rollout_log_prob, c
 int vrl_rollout_corr_num_stats(void) { return vrl::kNumCorrStats; }
 
 int vrl_response_slice(const float* values, const int64_t* cu_seqlens, const int64_t* response_lens,
-                       int64_t B, int64_t T_out, float* out, int32_t* err_flag, void* stream) {
-  if (B < 0 || T_out < 0 || B > kMaxGrid) return VRL_ERR_SHAPE;
+                       int64_t B, int64_t n_tokens, int64_t T_out, float* out, int32_t* err_flag, void* stream) {
+  if (B < 0 || T_out < 0 || n_tokens < 0 || B > kMaxGrid) return VRL_ERR_SHAPE;
   if (B == 0 || T_out == 0) return VRL_OK;
-  if (values == nullptr || cu_seqlens == nullptr || response_lens == nullptr || out == nullptr ||
+  if ((values == nullptr && n_tokens > 0) || cu_seqlens == nullptr || response_lens == nullptr || out == nullptr ||
       err_flag == nullptr)
     return VRL_ERR_NULL;
   if (!aligned(values, 4) || !aligned(cu_seqlens, 8) || !aligned(response_lens, 8) || !aligned(out, 4) ||
       !aligned(err_flag, 4))
     return VRL_ERR_ALIGN;
   vrl::response_slice_kernel<<<dim3(static_cast<unsigned>(B)), dim3(256), 0, static_cast<hipStream_t>(stream)>>>(
-      values, cu_seqlens, response_lens, T_out, out, err_flag);
+      values, cu_seqlens, response_lens, n_tokens, T_out, out, err_flag);
   return launch_status();
 }
 
 int vrl_response_pack(const float* values, const int64_t* cu_seqlens, const int64_t* response_lens,
-                      const int64_t* out_offsets, int64_t B, int64_t out_total, float* out, int32_t* err_flag,
-                      void* stream) {
-  if (B < 0 || out_total < 0 || B > kMaxGrid) return VRL_ERR_SHAPE;
+                      const int64_t* out_offsets, int64_t B, int64_t n_tokens, int64_t out_total, float* out,
+                      int32_t* err_flag, void* stream) {
+  if (B < 0 || out_total < 0 || n_tokens < 0 || B > kMaxGrid) return VRL_ERR_SHAPE;
   if (B == 0) return VRL_OK;
-  if (values == nullptr || cu_seqlens == nullptr || response_lens == nullptr || out_offsets == nullptr ||
+  if ((values == nullptr && n_tokens > 0) || cu_seqlens == nullptr || response_lens == nullptr || out_offsets == nullptr ||
       err_flag == nullptr || (out == nullptr && out_total > 0))
     return VRL_ERR_NULL;
   if (!aligned(values, 4) || !aligned(cu_seqlens, 8) || !aligned(response_lens, 8) || !aligned(out_offsets, 8) ||
       !aligned(out, 4) || !aligned(err_flag, 4))
     return VRL_ERR_ALIGN;
   vrl::response_pack_kernel<<<dim3(static_cast<unsigned>(B)), dim3(256), 0, static_cast<hipStream_t>(stream)>>>(
-      values, cu_seqlens, response_lens, out_offsets, out_total, out, err_flag);
+      values, cu_seqlens, response_lens, out_offsets, n_tokens, out_total, out, err_flag);
   return launch_status();
 }
 
@@ -487,15 +542,16 @@ int vrl_transpose(const void* src, int elem_size, int64_t rows, int64_t cols, in
 }
 
 int vrl_spec_verify(const float* logp_new, const float* logp_old, const float* log_u,
-                    const uint8_t* mask, const int64_t* cu_seqlens, int64_t B, int64_t T,
+                    const uint8_t* mask, const int64_t* cu_seqlens, int64_t B, int64_t T, int64_t n_tokens,
                     float thresh_offset, float near_eps, uint8_t* accept, int32_t* first_reject,
                     int32_t* prefix_len, int32_t* near_count, const int64_t* draft_ids,
-                    int64_t pad_id, int64_t* out_ids, uint8_t* out_mask, void* stream) {
-  const int st = check_verify(logp_new, logp_old, log_u, mask, cu_seqlens, B, T, accept, first_reject,
-                              prefix_len, near_count, draft_ids, out_ids, out_mask);
+                    int64_t pad_id, int64_t* out_ids, uint8_t* out_mask, int32_t* err_flag, void* stream) {
+  const int st = check_verify(logp_new, logp_old, log_u, mask, cu_seqlens, B, T, n_tokens, err_flag, accept,
+                              first_reject, prefix_len, near_count, draft_ids, out_ids, out_mask);
   if (st != VRL_OK || B == 0) return st;
-  const vrl::VerifyArgs v{logp_new, logp_old, log_u, mask, cu_seqlens, B, T, thresh_offset, near_eps,
-                          accept, first_reject, prefix_len, near_count, draft_ids, pad_id, out_ids, out_mask};
+  const vrl::VerifyArgs v{logp_new, logp_old, log_u, mask, cu_seqlens, B, T, n_tokens, err_flag, thresh_offset,
+                          near_eps, accept, first_reject, prefix_len, near_count, draft_ids, pad_id, out_ids,
+                          out_mask};
   const dim3 grid(static_cast<unsigned>(B));
   hipStream_t s = static_cast<hipStream_t>(stream);
   switch (verify_waves(cu_seqlens, B, T)) {
@@ -507,21 +563,20 @@ int vrl_spec_verify(const float* logp_new, const float* logp_old, const float* l
 }
 
 int vrl_truncate_draft(const int64_t* draft_ids, const uint8_t* mask, const int64_t* cu_seqlens,
-                       int64_t B, int64_t T, const int32_t* first_reject, int64_t pad_id,
-                       int64_t* out_ids, uint8_t* out_mask, void* stream) {
-  if (B < 0 || T < 0 || B > kMaxGrid || T > kMaxGrid) return VRL_ERR_SHAPE;
-  if (B == 0 || (cu_seqlens == nullptr && T == 0)) return VRL_OK;
+                       int64_t B, int64_t T, int64_t n_tokens, const int32_t* first_reject, int64_t pad_id,
+                       int64_t* out_ids, uint8_t* out_mask, int32_t* err_flag, void* stream) {
+  const int ls = check_layout(cu_seqlens, B, T, n_tokens, err_flag);
+  if (ls != VRL_OK) return ls;
+  if (B == 0 || n_tokens == 0) return VRL_OK;
   if (draft_ids == nullptr || first_reject == nullptr || out_ids == nullptr || out_mask == nullptr)
     return VRL_ERR_NULL;
-  if (!aligned(draft_ids, 8) || !aligned(out_ids, 8) || !aligned(cu_seqlens, 8) ||
-      !aligned(first_reject, 4))
-    return VRL_ERR_ALIGN;
+  if (!aligned(draft_ids, 8) || !aligned(out_ids, 8) || !aligned(first_reject, 4)) return VRL_ERR_ALIGN;
   const dim3 grid(static_cast<unsigned>(B));
   hipStream_t s = static_cast<hipStream_t>(stream);
   switch (verify_waves(cu_seqlens, B, T)) {
-    case 1: vrl::truncate_draft_kernel<1><<<grid, dim3(64), 0, s>>>(draft_ids, mask, cu_seqlens, T, first_reject, pad_id, out_ids, out_mask); break;
-    case 4: vrl::truncate_draft_kernel<4><<<grid, dim3(256), 0, s>>>(draft_ids, mask, cu_seqlens, T, first_reject, pad_id, out_ids, out_mask); break;
-    default: vrl::truncate_draft_kernel<16><<<grid, dim3(1024), 0, s>>>(draft_ids, mask, cu_seqlens, T, first_reject, pad_id, out_ids, out_mask); break;
+    case 1: vrl::truncate_draft_kernel<1><<<grid, dim3(64), 0, s>>>(draft_ids, mask, cu_seqlens, T, n_tokens, first_reject, pad_id, out_ids, out_mask, err_flag); break;
+    case 4: vrl::truncate_draft_kernel<4><<<grid, dim3(256), 0, s>>>(draft_ids, mask, cu_seqlens, T, n_tokens, first_reject, pad_id, out_ids, out_mask, err_flag); break;
+    default: vrl::truncate_draft_kernel<16><<<grid, dim3(1024), 0, s>>>(draft_ids, mask, cu_seqlens, T, n_tokens, first_reject, pad_id, out_ids, out_mask, err_flag); break;
   }
   return launch_status();
 }
@@ -539,16 +594,16 @@ int vrl_fused_score_verify(const void* logits, int dtype, int64_t n_rows, int64_
   int st = check_rowscore(logits, dtype, n_rows, vocab, row_stride, labels, temperature, out_logprob,
                           out_entropy, out_sum_pi_sq, out_lse, err_flag);
   if (st != VRL_OK) return st;
-  st = check_verify(out_logprob, logp_old, log_u, mask, cu_seqlens, B, T, accept, first_reject,
+  // the row space is the token space: n_rows is what the packed offsets are held to
+  st = check_verify(out_logprob, logp_old, log_u, mask, cu_seqlens, B, T, n_rows, err_flag, accept, first_reject,
                     prefix_len, near_count, draft_ids, out_ids, out_mask);
   if (st != VRL_OK) return st;
-  if (cu_seqlens == nullptr && n_rows != B * T) return VRL_ERR_SHAPE;
   st = vrl_rowscore(logits, dtype, n_rows, vocab, row_stride, labels, temperature, out_logprob,
                     out_entropy, out_sum_pi_sq, out_lse, err_flag, stream);
   if (st != VRL_OK) return st;
-  return vrl_spec_verify(out_logprob, logp_old, log_u, mask, cu_seqlens, B, T, thresh_offset, near_eps,
+  return vrl_spec_verify(out_logprob, logp_old, log_u, mask, cu_seqlens, B, T, n_rows, thresh_offset, near_eps,
                          accept, first_reject, prefix_len, near_count, draft_ids, pad_id, out_ids,
-                         out_mask, stream);
+                         out_mask, err_flag, stream);
 }
 
 const char* vrl_strerror(int status) {

@@ -17,6 +17,7 @@ from typing import Optional
 import torch
 
 from . import _lib
+from . import errors as _errors
 from .layout import transpose_2d
 from .torch_functional import _DTYPE_CODES, _ptr
 
@@ -65,8 +66,8 @@ class _FusedLinearForPPOFunction(torch.autograd.Function):
                 torch.matmul(hidden[lo:hi], weight.t(), out=logits)
                 _score_chunk(lib, logits, input_ids[lo:hi], None if temp is None else temp[: hi - lo],
                              lp[lo:hi], h[lo:hi], lse[lo:hi], flag, stream)
-        if T > 0 and (int(flag.item()) & _lib.VRL_FLAG_LABEL_OOB):
-            raise IndexError(f"fused_linear_for_ppo: an input id is outside [0, {V})")
+        if T > 0:
+            _errors.report(flag, {_lib.VRL_FLAG_LABEL_OOB: (IndexError, f"fused_linear_for_ppo: an input id is outside [0, {V})")})
         ctx.save_for_backward(hidden, weight, input_ids, lse, h)
         ctx.temperature = float(temperature)
         ctx.chunk_size = int(chunk_size)
@@ -162,9 +163,13 @@ def fused_linear_for_ppo(hidden_states: torch.Tensor, vocab_weights: torch.Tenso
         raise ValueError("fused_linear_for_ppo: vocab_weights must be (vocab, hidden)")
     if int(chunk_size) <= 0:
         raise ValueError(f"chunk_size must be positive, got {chunk_size}")
+    if input_ids.dtype.is_floating_point or input_ids.dtype == torch.bool:
+        raise TypeError(f"fused_linear_for_ppo: input_ids must be an integer tensor, got {input_ids.dtype}")
+    _errors.poll()
     lead = hidden_states.shape[:-1]
     h2 = hidden_states.reshape(-1, hidden_states.shape[-1]).contiguous()
-    ids = input_ids.reshape(-1).to(torch.int64).contiguous()
+    # the kernels read the ids through a raw device pointer: they must live next to the hidden states
+    ids = input_ids.reshape(-1).to(device=h2.device, dtype=torch.int64).contiguous()
     lp, ent = _FusedLinearForPPOFunction.apply(h2, vocab_weights.contiguous(), ids, float(temperature), int(chunk_size),
                                                bool(keep_logits))
     return lp.reshape(lead), ent.reshape(lead)
@@ -223,10 +228,7 @@ def lm_head_score_mfma(hidden_states: torch.Tensor, vocab_weights: torch.Tensor,
                                   ids.data_ptr(), _ptr(temp), splits, partials.data_ptr(), lp.data_ptr(), ent.data_ptr(),
                                   None, flag.data_ptr(), _lib.stream_ptr(dev))
     _lib.check("vrl_lmhead_score", st)
-    from . import torch_functional as _tf
-
-    if _tf.LABEL_CHECK and (int(flag.item()) & _lib.VRL_FLAG_LABEL_OOB):
-        raise IndexError(f"lm_head_score_mfma: an input id is outside [0, {V})")
+    _errors.report(flag, {_lib.VRL_FLAG_LABEL_OOB: (IndexError, f"lm_head_score_mfma: an input id is outside [0, {V})")})
     return lp.reshape(lead), ent.reshape(lead)
 
 

@@ -27,14 +27,22 @@ import functools
 import importlib
 import os
 import sys
+import threading
 import weakref
 from typing import Callable, Dict, List, Optional, Tuple
 
 import torch
 
 from . import _lib
+from . import errors as _errors
 from . import fused_linear as _fl
 from . import torch_functional as _amd
+
+# Device-side errors (a label outside the vocabulary) of the installed functions are looked at without ever waiting for
+# the GPU, like the asynchronous device assert of the torch.gather they replace (verl/utils/torch_functional.py:69):
+# at a later shim call once the kernel has finished, or in check_errors(). VERL_AMD_CHECK=sync|off overrides.
+SHIM_CHECK_MODE = _errors.ENV_MODE or "deferred"
+check_errors = _errors.check_errors
 
 TARGET_MODULE = "verl.utils.torch_functional"
 PATCHED_NAMES = (
@@ -47,22 +55,28 @@ PATCHED_NAMES = (
 )
 
 # One pass serves two calls. verl's engines ask for the entropy and for the label log-probs of the SAME logits tensor
-# in two separate calls (verl/workers/engine/fsdp/transformer_impl.py:1364-1376 and :1395-1399). Without gradients
-# the first of the two (whichever it is) runs the row kernel once and keeps entropy and logsumexp per row; the second
-# is then a gather (log-prob = logit[label] - logsumexp) or a lookup, not another pass over the logits.
-# What is kept is tied to the tensor OBJECT (weak reference), its version counter (any in-place write bumps it, also
-# through views), its address, shape, strides, dtype and the stream: a new tensor that happens to reuse the address
-# is a different object and never matches. VERL_AMD_MEMO=0 switches it off.
+# in two separate calls (verl/workers/engine/fsdp/transformer_impl.py:1364-1376 and :1395-1399). The first of the two
+# runs the row kernel once and leaves what the other needs: after an entropy call the per-row logsumexp (the log-prob
+# call is then one element load per row, vrl_label_logprob), after a log-prob call the per-row entropy. With
+# gradients the pair also shares ONE backward pass over the logits (see _EntropyLseFunction in torch_functional).
+#
+# What is left behind is tied to the tensor OBJECT (weak reference), its version counter (any in-place write through
+# torch bumps it, also through views), its address, shape, strides, dtype, the stream and whether gradients are being
+# recorded. It is single-use and short-lived: only the NEXT shim call can take it, only a call of the other kind
+# (log-prob after entropy, entropy after log-prob), and it is dropped whatever that next call is. A write that torch's
+# version counter does not see (``logits.data`` ops, a raw-pointer kernel such as the in-place backward, replay of a
+# captured graph into a static buffer) between the two calls of a pair is NOT detected. Nothing is shared while the
+# stream is being captured. VERL_AMD_MEMO=0 switches the sharing off.
 MEMO = os.environ.get("VERL_AMD_MEMO", "1") not in ("0", "false", "False")
 
 
 class _RowMemo:
-    """What one pass over a logits tensor left behind. Built completely before it is published and never changed
-    afterwards, so a reader in another thread sees either the whole of it or the one before."""
+    """What one pass over a logits tensor left for the other call of the pair."""
 
-    __slots__ = ("ref", "version", "ptr", "shape", "stride", "dtype", "stream", "entropy", "lse")
+    __slots__ = ("ref", "version", "ptr", "shape", "stride", "dtype", "stream", "needs_grad", "kind", "entropy", "lse",
+                 "pair")
 
-    def __init__(self, logits, stream, entropy, lse):
+    def __init__(self, logits, stream, needs_grad, kind, entropy=None, lse=None, pair=None):
         self.ref = weakref.ref(logits)
         self.version = logits._version
         self.ptr = logits.data_ptr()
@@ -70,66 +84,109 @@ class _RowMemo:
         self.stride = tuple(logits.stride())
         self.dtype = logits.dtype
         self.stream = stream
-        self.entropy = entropy.clone()   # private: the caller may write into the tensor it was given
+        self.needs_grad = needs_grad
+        self.kind = kind          # "entropy": left by an entropy call (holds lse); "logprob": by a log-prob call (holds entropy)
+        self.entropy = entropy
         self.lse = lse
+        self.pair = pair          # grad mode, kind "entropy": the dict the two autograd nodes share
 
-    def matches(self, logits, stream) -> bool:
+    def matches(self, logits, stream, needs_grad) -> bool:
         return (self.ref() is logits and self.version == logits._version and self.ptr == logits.data_ptr()
                 and self.shape == tuple(logits.shape) and self.stride == tuple(logits.stride())
-                and self.dtype == logits.dtype and self.stream == stream)
+                and self.dtype == logits.dtype and self.stream == stream and self.needs_grad == needs_grad)
 
 
-_memo: Optional[_RowMemo] = None
+_memo_local = threading.local()   # per thread: a pair of calls is made by one thread
 
 
-def _memo_store(logits, stream, entropy, lse) -> None:
-    global _memo
-    _memo = _RowMemo(logits, stream, entropy, lse)   # one reference assignment
+def _memo_take() -> Optional[_RowMemo]:
+    memo = getattr(_memo_local, "memo", None)
+    _memo_local.memo = None
+    return memo
+
+
+def _memo_store(memo: _RowMemo) -> None:
+    _memo_local.memo = memo
 
 
 def _memo_clear() -> None:
-    global _memo
-    _memo = None
+    _memo_local.memo = None
 
 
 _LOGPROB_NAMES = ("logprobs_from_logits", "logprobs_from_logits_v2", "logprobs_from_logits_naive")
 _ENTROPY_NAMES = ("entropy_from_logits", "entropy_from_logits_with_chunking")
 
 
+def _plain_rows(logits):
+    """(N, V) view of ``logits`` when it is one plain row-major block, else None."""
+    if _amd._is_batch_of_row_slices(logits):
+        return None
+    x = _amd._rows_2d(logits)
+    if x.data_ptr() != logits.data_ptr() or x.shape[0] == 0:
+        return None
+    return x
+
+
 def _memo_serve(name, logits, args, kwargs):
-    """The result of ``name(logits, ...)`` from one shared pass, or None when the ordinary route must be taken."""
-    if not MEMO or (torch.is_grad_enabled() and logits.requires_grad) or logits.is_inference():
+    """The result of ``name(logits, ...)`` from a pass shared with the other call of the pair, or None when the
+    ordinary route must be taken. Whatever happens, a record left by the call before is gone afterwards."""
+    memo = _memo_take()
+    if not MEMO or logits.is_inference() or torch.cuda.is_current_stream_capturing():
         return None   # (inference-mode tensors have no version counter to check against)
+    if name not in _ENTROPY_NAMES and name not in _LOGPROB_NAMES:
+        return None
+    x = _plain_rows(logits)
+    if x is None:
+        return None
+    lead = logits.shape[:-1]
+    needs_grad = torch.is_grad_enabled() and logits.requires_grad
     stream = _lib.stream_ptr(logits.device)
-    memo = _memo   # one read: the object it names cannot change under us
-    hit = memo is not None and memo.matches(logits, stream)
+    hit = memo is not None and memo.matches(logits, stream, needs_grad)
+
     if name in _ENTROPY_NAMES:
-        if hit:
+        if name == "entropy_from_logits_with_chunking":
+            chunk = args[0] if args else kwargs.get("chunk_size", 2048)
+            if int(chunk) <= 0:
+                return None   # the ordinary route raises
+        if hit and memo.kind == "logprob":
             _stats["memo_hits"] += 1
-            return memo.entropy.clone()
-        got = _amd._score_once(logits, None)
-        if got is None:
-            return None
-        _memo_store(logits, stream, got[1], got[2])
-        return got[1]
-    if name in _LOGPROB_NAMES:
-        labels = args[0] if args else kwargs.get("labels")
-        if not isinstance(labels, torch.Tensor) or tuple(labels.shape) != tuple(logits.shape[:-1]):
-            return None
-        if hit:
-            V = logits.shape[-1]
-            lab = labels.to(device=logits.device, dtype=torch.int64)
-            if _amd.LABEL_CHECK and bool(((lab < 0) | (lab >= V)).any()):
-                raise IndexError(f"{name}: a label is outside [0, {V})")
-            picked = torch.gather(logits, -1, lab.clamp(0, V - 1).unsqueeze(-1)).squeeze(-1)
-            _stats["memo_hits"] += 1
-            return picked.float() - memo.lse
-        got = _amd._score_once(logits, labels)
-        if got is None:
-            return None
-        _memo_store(logits, stream, got[1], got[2])
-        return got[0]
-    return None
+            return memo.entropy
+        if needs_grad:
+            pair = {}
+            h, lse = _amd._EntropyLseFunction.apply(x, None, None, pair)
+            _memo_store(_RowMemo(logits, stream, True, "entropy", lse=lse, pair=pair))
+        else:
+            with torch.no_grad():
+                _, h, _, lse, _ = _amd._forward_2d(x, None, None, False, True, False, True, None)
+            _memo_store(_RowMemo(logits, stream, False, "entropy", lse=lse))
+        return h.reshape(lead)
+
+    labels = args[0] if args else kwargs.get("labels")
+    if (not isinstance(labels, torch.Tensor) or tuple(labels.shape) != tuple(lead) or labels.dtype.is_floating_point
+            or labels.dtype == torch.bool):
+        return None
+    lab = labels.to(device=x.device, dtype=torch.int64).reshape(-1).contiguous()
+    inplace = False
+    if name == "logprobs_from_logits":
+        inplace = bool(args[1] if len(args) > 1 else kwargs.get("inplace_backward", True)) and _amd._is_view_safe(logits)
+    messages = _amd._label_messages(name, logits.shape[-1])
+    if hit and memo.kind == "entropy":
+        _stats["memo_hits"] += 1
+        if needs_grad:
+            lp, flag = _amd._LabelLogprobFunction.apply(x, lab, None, memo.lse, memo.pair, inplace, None)
+        else:
+            with torch.no_grad():
+                lp, flag = _amd._label_logprob(x, lab, None, memo.lse)
+        _errors.report(flag, messages)
+        return lp.reshape(lead)
+    if needs_grad:
+        lp, h, flag = _amd._RowScoreFunction.apply(x, lab, None, True, True, None, inplace, None)
+    else:
+        with torch.no_grad():
+            lp, h, _, _, flag = _amd._forward_2d(x, lab, None, True, True, False, False, None)
+    _memo_store(_RowMemo(logits, stream, needs_grad, "logprob", entropy=h.reshape(lead)))
+    _errors.report(flag, messages)
+    return lp.reshape(lead)
 
 
 _originals: Dict[str, Callable] = {}
@@ -155,10 +212,13 @@ def _make_shim(name: str, original: Callable) -> Callable:
     def serve(logits, *args, **kwargs):
         if _eligible(logits):
             _stats["hip_calls"] += 1
-            served = _memo_serve(name, logits, args, kwargs)
-            if served is not None:
-                return served
-            return ours(logits, *args, **kwargs)
+            with _errors.using(SHIM_CHECK_MODE):
+                _errors.poll()
+                served = _memo_serve(name, logits, args, kwargs)
+                if served is not None:
+                    return served
+                return ours(logits, *args, **kwargs)
+        _memo_clear()
         _stats["passed_to_verl"] += 1
         return original(logits, *args, **kwargs)
 
@@ -193,7 +253,8 @@ def _make_fused_linear_class(original_cls):
         def forward(self, hidden_states, vocab_weights, input_ids, temperature=1.0):
             if _eligible_pair(hidden_states, vocab_weights):
                 _stats["hip_calls"] += 1
-                return super().forward(hidden_states, vocab_weights, input_ids, temperature)
+                with _errors.using(SHIM_CHECK_MODE):
+                    return super().forward(hidden_states, vocab_weights, input_ids, temperature)
             _stats["passed_to_verl"] += 1
             return self._verl_module.forward(hidden_states, vocab_weights, input_ids, temperature)
 
@@ -205,7 +266,8 @@ def _make_linear_cross_entropy(original):
     def serve(hidden, weight, labels, temperature=1.0, reduction="none", dist_process_group=None):
         if dist_process_group is None and _eligible_pair(hidden, weight):
             _stats["hip_calls"] += 1
-            return _fl.linear_cross_entropy(hidden, weight, labels, temperature, reduction)
+            with _errors.using(SHIM_CHECK_MODE):
+                return _fl.linear_cross_entropy(hidden, weight, labels, temperature, reduction)
         _stats["passed_to_verl"] += 1
         return original(hidden, weight, labels, temperature, reduction, dist_process_group)
 
@@ -228,8 +290,9 @@ _optional_patched: List[Tuple[object, str, object]] = []
 
 
 def stats() -> dict:
-    """Calls served by the HIP kernel vs handed back to verl since install()."""
-    return dict(_stats)
+    """Calls served by the HIP kernels vs handed back to verl since install(), second calls of a pair served from the
+    first one's pass, and the passes over logits launched so far (forward, backward, label gathers)."""
+    return {**_stats, **_amd.counters}
 
 
 def install(target_module: str = TARGET_MODULE) -> List[str]:

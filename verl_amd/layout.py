@@ -14,6 +14,7 @@ from typing import Optional
 import torch
 
 from . import _lib
+from . import errors as _errors
 
 __all__ = ["roll_labels", "response_slice", "response_from_packed", "transpose_2d"]
 
@@ -28,14 +29,26 @@ def roll_labels(input_ids_rmpad: torch.Tensor) -> torch.Tensor:
     return torch.roll(input_ids_rmpad, shifts=-1, dims=-1)
 
 
+def _slice_messages(what: str, n_tokens: int) -> dict:
+    return {
+        _lib.VRL_FLAG_SEQ_RANGE: (ValueError, f"{what}: cu_seqlens is not a partition of the {n_tokens} values "
+                                  "(it must start at 0, never decrease and end at the number of values)"),
+        _lib.VRL_FLAG_SLICE_RANGE: (ValueError, f"{what}: a sequence has no prompt token, or a response length "
+                                    "outside its bounds"),
+    }
+
+
 def response_slice(values: torch.Tensor, cu_seqlens: torch.Tensor, response_lens: torch.Tensor,
-                   max_response_len: Optional[int] = None, check: bool = True) -> torch.Tensor:
+                   max_response_len: Optional[int] = None, check=None) -> torch.Tensor:
     """Packed per-token fp32 ``values`` (total_nnz,) -> ``(B, max_response_len)`` block of response positions.
 
     Row b holds ``values[end_b - r_b - 1 : end_b - 1]`` (model output is shifted left by one token) padded
     with zeros, where ``end_b = cu_seqlens[b+1]`` and ``r_b = response_lens[b]``. Like the reference it
-    requires every sequence to have a prompt token; with ``check`` a violation raises ValueError.
+    requires every sequence to have a prompt token and ``cu_seqlens`` to partition ``values``
+    (verl/workers/utils/padding.py:129-130); a violation writes a zero row and raises ValueError, when and how is
+    ``check``'s business (verl_amd.errors: None = the mode in force, True = now, False = never, "deferred").
     """
+    _errors.poll()
     if not values.is_cuda:
         raise RuntimeError(f"values is on {values.device}; verl_amd only runs on the GPU, it has no CPU implementation")
     if values.dim() != 1:
@@ -54,16 +67,16 @@ def response_slice(values: torch.Tensor, cu_seqlens: torch.Tensor, response_lens
     flag = torch.zeros(1, dtype=torch.int32, device=dev)
     lib = _lib.load()
     with torch.cuda.device(dev):
-        st = lib.vrl_response_slice(v.data_ptr(), cu.data_ptr(), rl.data_ptr(), B, T, out.data_ptr(), flag.data_ptr(),
-                                    _lib.stream_ptr(dev))
+        st = lib.vrl_response_slice(v.data_ptr() if v.numel() else None, cu.data_ptr(), rl.data_ptr(), B, v.numel(), T,
+                                    out.data_ptr(), flag.data_ptr(), _lib.stream_ptr(dev))
     _lib.check("vrl_response_slice", st)
-    if check and (int(flag.item()) & _lib.VRL_FLAG_SLICE_RANGE):
-        raise ValueError("response_slice: a sequence has no prompt token, or a response length outside [0, max_response_len]")
+    if B > 0 and T > 0:
+        _errors.report(flag, _slice_messages("response_slice", v.numel()), check)
     return out
 
 
 def response_from_packed(values: torch.Tensor, cu_seqlens: torch.Tensor, response_lens: torch.Tensor,
-                         check: bool = True):
+                         check=None):
     """Packed per-token fp32 ``values`` (total_nnz,) -> (packed response values ``(sum(response_lens),)``, their
     ``cu_seqlens`` ``(B+1,)`` int64): sequence b contributes ``values[end_b - r_b - 1 : end_b - 1]``. The packed
     counterpart of ``response_slice``; the reference does it with a Python loop and ``as_nested_tensor``
@@ -87,11 +100,12 @@ def response_from_packed(values: torch.Tensor, cu_seqlens: torch.Tensor, respons
     flag = torch.zeros(1, dtype=torch.int32, device=dev)
     lib = _lib.load()
     with torch.cuda.device(dev):
-        st = lib.vrl_response_pack(v.data_ptr(), cu.data_ptr(), rl.data_ptr(), out_cu.data_ptr(), B, total,
-                                   out.data_ptr() if total > 0 else None, flag.data_ptr(), _lib.stream_ptr(dev))
+        st = lib.vrl_response_pack(v.data_ptr() if v.numel() else None, cu.data_ptr(), rl.data_ptr(), out_cu.data_ptr(),
+                                   B, v.numel(), total, out.data_ptr() if total > 0 else None, flag.data_ptr(),
+                                   _lib.stream_ptr(dev))
     _lib.check("vrl_response_pack", st)
-    if check and (int(flag.item()) & _lib.VRL_FLAG_SLICE_RANGE):
-        raise ValueError("response_from_packed: a sequence has no prompt token, or a negative response length")
+    if B > 0:
+        _errors.report(flag, _slice_messages("response_from_packed", v.numel()), check)
     return out, out_cu
 
 

@@ -25,7 +25,7 @@ import numpy as np
 import torch
 
 from . import _lib
-from . import torch_functional as _tf
+from . import errors as _errors
 from .torch_functional import _DTYPE_CODES, _check_logits, _ptr, _rows_2d, _temperature_rows
 
 __all__ = ["VerifyResult", "draw_log_uniforms", "thresh_offset_from_lenience", "spec_verify", "truncate_draft", "fused_score_verify"]
@@ -110,8 +110,21 @@ def _layout(shape, cu_seqlens: Optional[torch.Tensor], device):
     return int(cu.numel() - 1), 0, cu
 
 
-def _verify_buffers(shape, B, device, draft_ids, want_truncated):
-    accept = torch.empty(tuple(shape), dtype=torch.uint8, device=device)
+def _seq_messages(what: str, n_tokens: int, vocab: Optional[int] = None) -> dict:
+    """What the kernels' error bits mean for ``what``. The packed offsets live on the device: the kernels hold them
+    to the arrays' length (nothing outside is touched) and report through the flag, like the reference's assert at
+    verl/workers/utils/padding.py:129-130."""
+    msgs = {}
+    if vocab is not None:
+        msgs[_lib.VRL_FLAG_LABEL_OOB] = (IndexError, f"{what}: a label is outside [0, {vocab})")
+    msgs[_lib.VRL_FLAG_SEQ_RANGE] = (ValueError, f"{what}: cu_seqlens is not a partition of the {n_tokens} tokens "
+                                     "(it must start at 0, never decrease and end at the number of tokens)")
+    return msgs
+
+
+def _verify_buffers(shape, B, device, draft_ids, want_truncated, packed=False, pad_id=0):
+    # packed: tokens that no in-range span covers are not written by the kernel, so they start as "not accepted"
+    accept = (torch.zeros if packed else torch.empty)(tuple(shape), dtype=torch.uint8, device=device)
     first = torch.empty(B, dtype=torch.int32, device=device)
     prefix = torch.empty(B, dtype=torch.int32, device=device)
     near = torch.empty(B, dtype=torch.int32, device=device)
@@ -120,8 +133,8 @@ def _verify_buffers(shape, B, device, draft_ids, want_truncated):
         if tuple(draft_ids.shape) != tuple(shape):
             raise ValueError(f"draft_ids shape {tuple(draft_ids.shape)} does not match {tuple(shape)}")
         ids = draft_ids.to(device=device, dtype=torch.int64).contiguous()
-        out_ids = torch.empty_like(ids)
-        out_mask = torch.empty(tuple(shape), dtype=torch.uint8, device=device)
+        out_ids = torch.full_like(ids, int(pad_id)) if packed else torch.empty_like(ids)
+        out_mask = (torch.zeros if packed else torch.empty)(tuple(shape), dtype=torch.uint8, device=device)
     return accept, first, prefix, near, ids, out_ids, out_mask
 
 
@@ -151,13 +164,16 @@ def spec_verify(
     cu_seqlens: Optional[torch.Tensor] = None,
     draft_ids: Optional[torch.Tensor] = None,
     pad_id: int = 0,
+    check=None,
 ) -> VerifyResult:
     """Verify a draft against new log-probs; see the module docstring for the rule.
 
     Layouts: padded ``(B, T)`` tensors, or packed 1-D token tensors with
-    ``cu_seqlens`` (``B+1`` row offsets). With ``draft_ids`` the truncated draft
-    and mask come back too.
+    ``cu_seqlens`` (``B+1`` row offsets that partition the tokens; anything else raises
+    ValueError, when and how is ``check``'s business as in verl_amd.errors). With
+    ``draft_ids`` the truncated draft and mask come back too.
     """
+    _errors.poll()
     if not logp_new.is_cuda:
         raise RuntimeError(f"logp_new is on {logp_new.device}; verl_amd only runs on the GPU, it has no CPU implementation")
     dev = logp_new.device
@@ -168,7 +184,9 @@ def spec_verify(
     lu = _resolve_log_u(log_u, uniforms, seed, shape, dev)
     m8 = _mask_u8(response_mask, shape, dev)
     off = thresh_offset_from_lenience(lenience, lenience_mode) if thresh_offset is None else float(np.float32(thresh_offset))
-    accept, first, prefix, near, ids, out_ids, out_mask = _verify_buffers(shape, B, dev, draft_ids, draft_ids is not None)
+    accept, first, prefix, near, ids, out_ids, out_mask = _verify_buffers(shape, B, dev, draft_ids,
+                                                                         draft_ids is not None, cu is not None, pad_id)
+    flag = torch.zeros(1, dtype=torch.int32, device=dev) if cu is not None else None
 
     if ln.numel() == 0:
         # no token at all (B empty sequences): nothing to launch, every sequence's results are zero
@@ -182,11 +200,13 @@ def spec_verify(
     with torch.cuda.device(dev):
         stream = _lib.stream_ptr(dev)
         st = lib.vrl_spec_verify(
-            ln.data_ptr(), lo.data_ptr(), lu.data_ptr(), _ptr(m8), _ptr(cu), B, T, off, float(near_eps),
+            ln.data_ptr(), lo.data_ptr(), lu.data_ptr(), _ptr(m8), _ptr(cu), B, T, ln.numel(), off, float(near_eps),
             accept.data_ptr(), first.data_ptr(), prefix.data_ptr(), near.data_ptr(),
-            _ptr(ids), int(pad_id), _ptr(out_ids), _ptr(out_mask), stream,
+            _ptr(ids), int(pad_id), _ptr(out_ids), _ptr(out_mask), _ptr(flag), stream,
         )
     _lib.check("vrl_spec_verify", st)
+    if flag is not None and B > 0:
+        _errors.report(flag, _seq_messages("spec_verify", ln.numel()), check)
     return VerifyResult(
         accept=accept.view(torch.bool), first_reject=first, prefix_len=prefix, near_count=near, log_u=lu,
         thresh_offset=off, out_ids=out_ids, out_mask=None if out_mask is None else out_mask.view(torch.bool),
@@ -200,8 +220,10 @@ def truncate_draft(
     *,
     pad_id: int = 0,
     cu_seqlens: Optional[torch.Tensor] = None,
+    check=None,
 ):
     """(ids, mask) with every position >= first_reject[b] set to pad_id / False."""
+    _errors.poll()
     if not draft_ids.is_cuda:
         raise RuntimeError(f"draft_ids is on {draft_ids.device}; verl_amd only runs on the GPU, it has no CPU implementation")
     dev = draft_ids.device
@@ -212,16 +234,20 @@ def truncate_draft(
     ids = draft_ids.to(dtype=torch.int64).contiguous()
     m8 = _mask_u8(response_mask, shape, dev)
     fr = first_reject.to(device=dev, dtype=torch.int32).contiguous()
-    out_ids = torch.empty_like(ids)
-    out_mask = torch.empty(shape, dtype=torch.uint8, device=dev)
+    packed = cu is not None
+    out_ids = torch.full_like(ids, int(pad_id)) if packed else torch.empty_like(ids)
+    out_mask = (torch.zeros if packed else torch.empty)(shape, dtype=torch.uint8, device=dev)
     if ids.numel() == 0:
         return out_ids, out_mask.view(torch.bool)
+    flag = torch.zeros(1, dtype=torch.int32, device=dev) if packed else None
     lib = _lib.load()
     with torch.cuda.device(dev):
         stream = _lib.stream_ptr(dev)
-        st = lib.vrl_truncate_draft(ids.data_ptr(), _ptr(m8), _ptr(cu), B, T, fr.data_ptr(), int(pad_id),
-                                    out_ids.data_ptr(), out_mask.data_ptr(), stream)
+        st = lib.vrl_truncate_draft(ids.data_ptr(), _ptr(m8), _ptr(cu), B, T, ids.numel(), fr.data_ptr(), int(pad_id),
+                                    out_ids.data_ptr(), out_mask.data_ptr(), _ptr(flag), stream)
     _lib.check("vrl_truncate_draft", st)
+    if packed and B > 0:
+        _errors.report(flag, _seq_messages("truncate_draft", ids.numel()), check)
     return out_ids, out_mask.view(torch.bool)
 
 
@@ -242,14 +268,16 @@ def fused_score_verify(
     cu_seqlens: Optional[torch.Tensor] = None,
     draft_ids: Optional[torch.Tensor] = None,
     pad_id: int = 0,
-    check_labels: Optional[bool] = None,
+    check_labels=None,
 ):
     """Score ``logits`` and verify the draft in one call: (log-probs, entropy, VerifyResult).
 
     ``logits`` is ``(B, T, V)`` (padded) or ``(N, V)`` with ``cu_seqlens``
-    (packed); every per-token tensor has the logits' leading shape.
+    (packed); every per-token tensor has the logits' leading shape. ``check_labels`` governs both device-side
+    checks, labels inside the vocabulary (IndexError) and packed offsets that partition the rows (ValueError).
     """
     _check_logits(logits, "fused_score_verify")
+    _errors.poll()
     if torch.is_grad_enabled() and logits.requires_grad:
         raise NotImplementedError("fused_score_verify is a forward-only step (verification happens under no_grad); "
                                   "use fused_logprob_entropy for the differentiable scores")
@@ -272,7 +300,8 @@ def fused_score_verify(
     out_lp = torch.empty(n, dtype=torch.float32, device=dev)
     out_h = torch.empty(n, dtype=torch.float32, device=dev)
     flag = torch.zeros(1, dtype=torch.int32, device=dev)
-    accept, first, prefix, near, ids, out_ids, out_mask = _verify_buffers(lead, B, dev, draft_ids, draft_ids is not None)
+    accept, first, prefix, near, ids, out_ids, out_mask = _verify_buffers(lead, B, dev, draft_ids,
+                                                                         draft_ids is not None, cu is not None, pad_id)
 
     if n == 0:
         for t in (first, prefix, near):
@@ -293,10 +322,7 @@ def fused_score_verify(
             _ptr(ids), int(pad_id), _ptr(out_ids), _ptr(out_mask), stream,
         )
     _lib.check("vrl_fused_score_verify", st)
-    if check_labels is None:
-        check_labels = _tf.LABEL_CHECK
-    if check_labels and (int(flag.item()) & _lib.VRL_FLAG_LABEL_OOB):
-        raise IndexError(f"fused_score_verify: a label is outside [0, {V})")
+    _errors.report(flag, _seq_messages("fused_score_verify", n, V), check_labels)
     res = VerifyResult(
         accept=accept.view(torch.bool), first_reject=first, prefix_len=prefix, near_count=near, log_u=lu,
         thresh_offset=off, out_ids=out_ids, out_mask=None if out_mask is None else out_mask.view(torch.bool),

@@ -19,12 +19,12 @@ HIP backward kernel (vrl_rowscore_backward).
 
 from __future__ import annotations
 
-import os
 from typing import Optional, Union
 
 import torch
 
 from . import _lib
+from . import errors as _errors
 
 __all__ = [
     "logprobs_from_logits",
@@ -36,10 +36,11 @@ __all__ = [
     "fused_logprob_entropy",
 ]
 
-# Raising IndexError for a label outside [0, vocab) means reading the kernel's error flag back, i.e. one host
-# synchronisation per call. Callers that must not synchronise (graph capture, deep launch queues) switch it off here
-# or with VERL_AMD_LABEL_CHECK=0; such a row's log-prob is NaN either way.
-LABEL_CHECK = os.environ.get("VERL_AMD_LABEL_CHECK", "1") not in ("0", "false", "False")
+# A label outside [0, vocab) makes that row's log-prob NaN and sets a bit in the kernel's error flag. How the flag
+# turns into an IndexError is verl_amd.errors' business: "sync" reads it back at once (one host synchronisation per
+# call, the default for direct calls), "deferred" looks at it later without ever waiting for the GPU (what the
+# installed shims use), "off" never looks. ``check_labels`` arguments take None (the mode in force), True ("sync"),
+# False ("off") or a mode name.
 
 _DTYPE_CODES = {torch.float32: _lib.VRL_F32, torch.bfloat16: _lib.VRL_BF16, torch.float16: _lib.VRL_F16}
 
@@ -108,8 +109,13 @@ def _temperature_rows(temperature, lead_shape, n_rows, device) -> Optional[torch
     return t.reshape(n_rows).contiguous()
 
 
-def _forward_2d(x, lab, temp, want_logprob, want_entropy, want_sum_pi_sq, want_lse, n_splits):
-    """Launch the forward kernels on (N, V) rows; returns (logprob, entropy, sum_pi_sq, lse, flag), None where not asked."""
+def _label_messages(what: str, vocab: int) -> dict:
+    return {_lib.VRL_FLAG_LABEL_OOB: (IndexError, f"{what}: a label is outside [0, {vocab})")}
+
+
+def _forward_2d(x, lab, temp, want_logprob, want_entropy, want_sum_pi_sq, want_lse, n_splits, flag=None):
+    """Launch the forward kernels on (N, V) rows; returns (logprob, entropy, sum_pi_sq, lse, flag), None where not
+    asked. ``flag`` may bring the int32 error flag to OR into (several launches then share one)."""
     n, V = x.shape
     dev = x.device
     f32 = dict(dtype=torch.float32, device=dev)
@@ -117,7 +123,8 @@ def _forward_2d(x, lab, temp, want_logprob, want_entropy, want_sum_pi_sq, want_l
     out_h = torch.empty(n, **f32) if want_entropy else None
     out_q = torch.empty(n, **f32) if want_sum_pi_sq else None
     out_lse = torch.empty(n, **f32) if want_lse else None
-    flag = torch.zeros(1, dtype=torch.int32, device=dev) if want_logprob else None
+    if flag is None and want_logprob:
+        flag = torch.zeros(1, dtype=torch.int32, device=dev)
     if n == 0:
         return out_lp, out_h, out_q, out_lse, flag
     lib = _lib.load()
@@ -139,42 +146,130 @@ def _forward_2d(x, lab, temp, want_logprob, want_entropy, want_sum_pi_sq, want_l
                 _ptr(out_lse), _ptr(flag), stream,
             )
             _lib.check("vrl_rowscore", st)
+    counters["forward_passes"] += 1
     return out_lp, out_h, out_q, out_lse, flag
+
+
+# Kernel passes over (N, V) logits launched from this module since import (what a caller can count to see how many
+# times its logits were streamed): forward row kernels, backward row kernels, per-row label gathers.
+counters = {"forward_passes": 0, "backward_passes": 0, "label_gathers": 0}
+
+
+def _backward_2d(x, lab, temp, lse, h, g_lp, g_h, inplace):
+    """dlogits of (N, V) rows from vrl_rowscore_backward, one pass; over x's own storage when ``inplace``."""
+    n, V = x.shape
+    dev = x.device
+    # In place: the gradient replaces the logits in their own storage, like the reference's
+    # flash-attn path does with inplace_backward=True (verl/utils/torch_functional.py:110-131).
+    dx = x if inplace else torch.empty((n, V), dtype=x.dtype, device=dev)
+    if n > 0:
+        gl = None if g_lp is None else g_lp.to(torch.float32).contiguous()
+        gh = None if g_h is None else g_h.to(torch.float32).contiguous()
+        lib = _lib.load()
+        with torch.cuda.device(dev):
+            st = lib.vrl_rowscore_backward(
+                x.data_ptr(), _DTYPE_CODES[x.dtype], n, V, x.stride(0) if n > 1 else V, _ptr(lab), _ptr(temp),
+                lse.data_ptr(), h.data_ptr(), _ptr(gl), _ptr(gh), dx.data_ptr(), dx.stride(0) if n > 1 else V,
+                _lib.stream_ptr(dev),
+            )
+        _lib.check("vrl_rowscore_backward", st)
+        counters["backward_passes"] += 1
+    return dx
+
+
+def _label_logprob(x, lab, temp, lse, flag=None):
+    """(logprob, flag) of (N, V) rows from a logsumexp an earlier pass left behind (vrl_label_logprob)."""
+    n, V = x.shape
+    dev = x.device
+    out = torch.empty(n, dtype=torch.float32, device=dev)
+    if flag is None:
+        flag = torch.zeros(1, dtype=torch.int32, device=dev)
+    if n > 0:
+        lib = _lib.load()
+        with torch.cuda.device(dev):
+            st = lib.vrl_label_logprob(x.data_ptr(), _DTYPE_CODES[x.dtype], n, V, x.stride(0) if n > 1 else V,
+                                       lab.data_ptr(), _ptr(temp), lse.data_ptr(), out.data_ptr(), flag.data_ptr(),
+                                       _lib.stream_ptr(dev))
+        _lib.check("vrl_label_logprob", st)
+        counters["label_gathers"] += 1
+    return out, flag
+
+
+class _EntropyLseFunction(torch.autograd.Function):
+    """(entropy, logsumexp) of the rows of ``x`` from one pass, for a caller that asks for the entropy first and for the
+    label log-probs of the same logits afterwards (the order of verl/workers/engine/fsdp/transformer_impl.py:1364-1399).
+    The log-probs then come from ``_LabelLogprobFunction``, which consumes this node's logsumexp; autograd therefore
+    runs that node's backward first, it leaves the log-probs' incoming gradient and the labels in ``pair``, and this
+    node's backward makes ONE pass over the logits with both gradients instead of two passes and an accumulation."""
+
+    @staticmethod
+    def forward(ctx, x, temp, n_splits, pair):
+        ctx.set_materialize_grads(False)
+        _, h, _, lse, _ = _forward_2d(x, None, temp, False, True, False, True, n_splits)
+        ctx.save_for_backward(x, temp, lse, h)
+        ctx.pair = pair
+        return h, lse
+
+    @staticmethod
+    def backward(ctx, g_h, g_lse):
+        x, temp, lse, h = ctx.saved_tensors
+        g_lp, lab = ctx.pair.get("g_lp"), ctx.pair.get("labels")
+        if g_lse is not None and g_lp is None:
+            raise RuntimeError("verl_amd: the shared logsumexp received a gradient that did not come from the label "
+                               "log-probs; it is an internal tensor and must not be used elsewhere")
+        if g_lp is None and g_h is None:
+            return None, None, None, None
+        inplace = bool(ctx.pair.get("inplace", False))
+        ctx.pair.pop("g_lp", None)
+        return _backward_2d(x, lab, temp, lse, h, g_lp, g_h, inplace), None, None, None
+
+
+class _LabelLogprobFunction(torch.autograd.Function):
+    """logprob = z[label] - lse with ``lse`` from ``_EntropyLseFunction``. Its backward hands the incoming gradient to
+    that node (through ``pair`` and, so that the node runs at all, as the gradient of lse) and returns no dense
+    gradient for the logits itself."""
+
+    @staticmethod
+    def forward(ctx, x, lab, temp, lse, pair, inplace, flag):
+        ctx.set_materialize_grads(False)
+        lp, flag = _label_logprob(x, lab, temp, lse, flag)
+        ctx.save_for_backward(lab)
+        ctx.pair = pair
+        ctx.inplace = bool(inplace)
+        ctx.mark_non_differentiable(flag)
+        return lp, flag
+
+    @staticmethod
+    def backward(ctx, g_lp, _g_flag):
+        if g_lp is None:
+            return None, None, None, None, None, None, None
+        (lab,) = ctx.saved_tensors
+        ctx.pair["g_lp"] = g_lp
+        ctx.pair["labels"] = lab
+        ctx.pair["inplace"] = ctx.inplace
+        return None, None, None, -g_lp, None, None, None
 
 
 class _RowScoreFunction(torch.autograd.Function):
     """Differentiable (log-prob, entropy) of the rows of ``x``; the gradient comes from vrl_rowscore_backward."""
 
     @staticmethod
-    def forward(ctx, x, lab, temp, want_logprob, want_entropy, n_splits, inplace_backward):
+    def forward(ctx, x, lab, temp, want_logprob, want_entropy, n_splits, inplace_backward, flag):
         ctx.set_materialize_grads(False)
-        lp, h, _, lse, flag = _forward_2d(x, lab, temp, want_logprob, True, False, True, n_splits)
+        lp, h, _, lse, flag = _forward_2d(x, lab, temp, want_logprob, True, False, True, n_splits, flag)
         ctx.save_for_backward(x, lab, temp, lse, h)
         ctx.inplace = bool(inplace_backward)
+        if flag is not None:
+            ctx.mark_non_differentiable(flag)
         return lp, (h if want_entropy else None), flag
 
     @staticmethod
     def backward(ctx, g_lp, g_h, _g_flag):
         x, lab, temp, lse, h = ctx.saved_tensors
         if g_lp is None and g_h is None:
-            return None, None, None, None, None, None, None
-        n, V = x.shape
-        dev = x.device
-        # In place: the gradient replaces the logits in their own storage, like the reference's
-        # flash-attn path does with inplace_backward=True (verl/utils/torch_functional.py:110-131).
-        dx = x if ctx.inplace else torch.empty((n, V), dtype=x.dtype, device=dev)
-        if n > 0:
-            gl = None if g_lp is None else g_lp.to(torch.float32).contiguous()
-            gh = None if g_h is None else g_h.to(torch.float32).contiguous()
-            lib = _lib.load()
-            with torch.cuda.device(dev):
-                st = lib.vrl_rowscore_backward(
-                    x.data_ptr(), _DTYPE_CODES[x.dtype], n, V, x.stride(0) if n > 1 else V, _ptr(lab), _ptr(temp),
-                    lse.data_ptr(), h.data_ptr(), _ptr(gl), _ptr(gh), dx.data_ptr(), dx.stride(0) if n > 1 else V,
-                    _lib.stream_ptr(dev),
-                )
-            _lib.check("vrl_rowscore_backward", st)
-        return dx, None, None, None, None, None, None
+            return None, None, None, None, None, None, None, None
+        dx = _backward_2d(x, lab if g_lp is not None else None, temp, lse, h, g_lp, g_h, ctx.inplace)
+        return dx, None, None, None, None, None, None, None
 
 
 def rowscore(
@@ -185,10 +280,11 @@ def rowscore(
     want_logprob: bool = True,
     want_entropy: bool = True,
     want_sum_pi_sq: bool = False,
-    check_labels: Optional[bool] = None,
+    check_labels=None,
     n_splits: Optional[int] = None,
     inplace_backward: bool = False,
     what: str = "rowscore",
+    _flag: Optional[torch.Tensor] = None,
 ):
     """Launch the row kernel; returns (logprob | None, entropy | None) and, with ``want_sum_pi_sq``,
     a third entry, each fp32 of shape logits.shape[:-1].
@@ -196,12 +292,14 @@ def rowscore(
     With few rows the work of one row is spread over ``n_splits`` workgroups (vrl_rowscore_split);
     ``n_splits=None`` lets the library choose, 1 forces one workgroup per row. When grad is enabled
     and the logits require it, log-prob and entropy are differentiable with respect to the logits
-    (vrl_rowscore_backward); the sum of squared probabilities is not. ``check_labels`` (default: the module's
-    ``LABEL_CHECK``) reads the kernel's error flag back and raises IndexError for a label outside the vocabulary.
+    (vrl_rowscore_backward); the sum of squared probabilities is not. ``check_labels`` says how a label outside
+    the vocabulary becomes an IndexError (verl_amd.errors: None = the mode in force, True = read the flag back now,
+    False = never, "deferred" = later and without waiting for the GPU). ``_flag`` (internal) brings a shared error
+    flag; whoever passes it reports it.
     """
     _check_logits(logits, what)
-    if check_labels is None:
-        check_labels = LABEL_CHECK
+    if _flag is None:
+        _errors.poll()
     if not (want_logprob or want_entropy or want_sum_pi_sq):
         raise ValueError(f"{what}: nothing to compute")
     if _is_batch_of_row_slices(logits):
@@ -216,10 +314,16 @@ def rowscore(
             raise ValueError(f"temperature has {temperature.numel()} entries, expected one per token "
                              f"({logits.shape[0] * logits.shape[1]}) for logits leading shape {tuple(logits.shape[:-1])}")
         t3 = temperature.reshape(logits.shape[:-1]) if per_b_temperature else None
+        # one error flag for the whole loop, looked at once
+        shared = _flag
+        if shared is None and want_logprob:
+            shared = torch.zeros(1, dtype=torch.int32, device=logits.device)
         parts = [rowscore(logits[b], None if labels is None else labels[b], t3[b] if per_b_temperature else temperature,
                           want_logprob=want_logprob, want_entropy=want_entropy, want_sum_pi_sq=want_sum_pi_sq,
-                          check_labels=check_labels, n_splits=n_splits, inplace_backward=False, what=what)
+                          n_splits=n_splits, inplace_backward=False, what=what, _flag=shared)
                  for b in range(logits.shape[0])]
+        if want_logprob and _flag is None:
+            _errors.report(shared, _label_messages(what, logits.shape[-1]), check_labels)
         return tuple(None if parts[0][k] is None else torch.stack([p[k] for p in parts]) for k in range(len(parts[0])))
     lead = logits.shape[:-1]
     V = logits.shape[-1]
@@ -241,43 +345,23 @@ def rowscore(
     needs_grad = torch.is_grad_enabled() and logits.requires_grad
     out_q = None
     if needs_grad and (want_logprob or want_entropy):
-        lp, h, flag = _RowScoreFunction.apply(x, lab, temp, want_logprob, want_entropy, n_splits, inplace_backward)
+        lp, h, flag = _RowScoreFunction.apply(x, lab, temp, want_logprob, want_entropy, n_splits, inplace_backward,
+                                              _flag)
         if want_sum_pi_sq:
             with torch.no_grad():
                 out_q = _forward_2d(x, None, temp, False, False, True, False, n_splits)[2]
     else:
         with torch.no_grad():
-            lp, h, out_q, _, flag = _forward_2d(x, lab, temp, want_logprob, want_entropy, want_sum_pi_sq, False, n_splits)
-    if want_logprob and check_labels and n > 0 and (int(flag.item()) & _lib.VRL_FLAG_LABEL_OOB):
-        raise IndexError(f"{what}: a label is outside [0, {V})")
+            lp, h, out_q, _, flag = _forward_2d(x, lab, temp, want_logprob, want_entropy, want_sum_pi_sq, False,
+                                                n_splits, _flag)
+    if want_logprob and n > 0 and _flag is None:
+        _errors.report(flag, _label_messages(what, V), check_labels)
 
     lp = lp.reshape(lead) if want_logprob else None
     h = h.reshape(lead) if want_entropy else None
     if want_sum_pi_sq:
         return lp, h, out_q.reshape(lead)
     return lp, h
-
-
-def _score_once(logits: torch.Tensor, labels: Optional[torch.Tensor]):
-    """No-grad helper for callers that keep per-row results of one pass around: (logprob | None, entropy, lse), each
-    fp32 of shape logits.shape[:-1]; None when the logits are not a plain row-major block (the caller then takes the
-    ordinary route)."""
-    if _is_batch_of_row_slices(logits):
-        return None
-    lead = logits.shape[:-1]
-    x = _rows_2d(logits)
-    if x.data_ptr() != logits.data_ptr() or x.shape[0] == 0:
-        return None
-    lab = None
-    if labels is not None:
-        if tuple(labels.shape) != tuple(lead) or labels.dtype.is_floating_point or labels.dtype == torch.bool:
-            return None
-        lab = labels.to(device=x.device, dtype=torch.int64).reshape(-1).contiguous()
-    with torch.no_grad():
-        lp, h, _, lse, flag = _forward_2d(x, lab, None, lab is not None, True, False, True, None)
-    if lab is not None and LABEL_CHECK and (int(flag.item()) & _lib.VRL_FLAG_LABEL_OOB):
-        raise IndexError(f"a label is outside [0, {logits.shape[-1]})")
-    return (None if lp is None else lp.reshape(lead)), h.reshape(lead), lse.reshape(lead)
 
 
 def logprobs_from_logits(logits: torch.Tensor, labels: torch.Tensor, inplace_backward: bool = True) -> torch.Tensor:
@@ -335,7 +419,7 @@ def fused_logprob_entropy(
     labels: torch.Tensor,
     temperature: Union[None, float, torch.Tensor] = None,
     *,
-    check_labels: Optional[bool] = None,
+    check_labels=None,
     want_sum_pi_sq: bool = False,
     n_splits: Optional[int] = None,
 ):
