@@ -153,6 +153,32 @@ int vrl_rowscore_backward(const void* logits, int dtype, int64_t n_rows, int64_t
                           void* dlogits, int64_t d_row_stride, void* stream);
 
 /*
+ * vrl_score_responses — ONE launch from packed logits (n_rows, vocab) to the padded (B, T_out) response blocks:
+ *   label[r]           = labels[r], or input_ids[(r + 1) mod n_rows] when input_ids is given instead
+ *                        (the roll of verl/workers/engine/fsdp/transformer_impl.py:1177; exactly one of the two,
+ *                        or neither when only the entropy is asked for)
+ *   logprob / entropy  as vrl_rowscore
+ *   resp_logprob[b, j] = logprob[cu_seqlens[b+1] - response_lens[b] - 1 + j]  for j < response_lens[b], else 0
+ *   resp_entropy[b, j] likewise            (the left shift by one of verl/workers/utils/padding.py:135-138)
+ * resp_logprob / resp_entropy: at least one. out_logprob / out_entropy (n_rows, per token) are optional extras of the
+ * block of the same kind; when neither is given, rows outside every response window are not read at all (a prompt
+ * token's logits cost no memory traffic).
+ * Device-side checks, reported through *err_flag: a label outside [0, vocab) (VRL_FLAG_LABEL_OOB, that entry NaN);
+ * a sequence without a prompt token or with response_lens[b] outside [0, T_out] (VRL_FLAG_SLICE_RANGE, its row all
+ * zero); cu_seqlens not a partition of [0, n_rows] (VRL_FLAG_SEQ_RANGE, the offending sequences' rows all zero).
+ * No content of cu_seqlens or response_lens can make the kernel touch memory outside the arrays.
+ *
+ * Replaces, as one kernel, the sequence
+ *   verl/workers/engine/fsdp/transformer_impl.py:1177 (labels = roll(input_ids, -1)), :1357 (temperature),
+ *   :1364-1399 (entropy, log-probs), :1401-1418 + verl/workers/utils/padding.py:97-141 (no_padding_2_padding).
+ */
+int vrl_score_responses(const void* logits, int dtype, int64_t n_rows, int64_t vocab, int64_t row_stride,
+                        const int64_t* labels, const int64_t* input_ids, const float* temperature,
+                        const int64_t* cu_seqlens, const int64_t* response_lens, int64_t B, int64_t T_out,
+                        float* out_logprob, float* out_entropy, float* resp_logprob, float* resp_entropy,
+                        int32_t* err_flag, void* stream);
+
+/*
  * vrl_response_slice — packed per-token values (total_nnz,) -> padded (B, T_out)
  * response block: out[b, j] = values[cu_seqlens[b+1] - response_lens[b] - 1 + j]
  * for j < response_lens[b], else 0 (the model output at a position scores the

@@ -165,6 +165,36 @@ def test_label_logprob_argument_errors_and_flag_values(lib):
         assert int(m.group(1)) == getattr(_lib, name), name
 
 
+def test_score_responses_argument_errors(lib):
+    f = lib.vrl_score_responses
+    ok = dict(x=P, dt=_lib.VRL_BF16, n=8, V=100, stride=100, lab=None, ids=P, temp=None, cu=P, rl=P, B=2, T=4, tlp=None,
+              th=None, rlp=P, rh=P, flag=P)
+
+    def call(**kw):
+        a = {**ok, **kw}
+        return f(a["x"], a["dt"], a["n"], a["V"], a["stride"], a["lab"], a["ids"], a["temp"], a["cu"], a["rl"], a["B"],
+                 a["T"], a["tlp"], a["th"], a["rlp"], a["rh"], a["flag"], None)
+
+    assert call(dt=4) == _lib.VRL_ERR_DTYPE
+    assert call(n=-1) == _lib.VRL_ERR_SHAPE
+    assert call(stride=50) == _lib.VRL_ERR_SHAPE
+    assert call(T=-1) == _lib.VRL_ERR_SHAPE
+    assert call(n=2**31 - 1) == _lib.VRL_ERR_SHAPE                 # rows + sequences must fit one grid
+    assert call(B=0) == _lib.VRL_ERR_SHAPE                         # rows that belong to no sequence
+    assert call(rlp=None, rh=None) == _lib.VRL_ERR_ARG
+    assert call(lab=P) == _lib.VRL_ERR_ARG                         # labels and input_ids together
+    assert call(tlp=P, rlp=None) == _lib.VRL_ERR_ARG               # a per-token vector without its block
+    assert call(th=P, rh=None) == _lib.VRL_ERR_ARG
+    assert call(cu=None) == _lib.VRL_ERR_NULL
+    assert call(rl=None) == _lib.VRL_ERR_NULL
+    assert call(flag=None) == _lib.VRL_ERR_NULL
+    assert call(x=None) == _lib.VRL_ERR_NULL
+    assert call(ids=None) == _lib.VRL_ERR_NULL                     # log-probs asked for, no source of labels
+    assert call(cu=P + 4) == _lib.VRL_ERR_ALIGN
+    assert call(rh=P + 2) == _lib.VRL_ERR_ALIGN
+    assert call(n=0, B=0, x=None, cu=None, rl=None, flag=None) == _lib.VRL_OK
+
+
 def test_response_pack_argument_errors(lib):
     g = lib.vrl_response_pack      # (values, cu, response_lens, out_offsets, B, n_tokens, out_total, out, err_flag, stream)
     assert g(P, P, P, P, -1, 9, 4, P, P, None) == _lib.VRL_ERR_SHAPE

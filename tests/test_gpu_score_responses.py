@@ -1,0 +1,218 @@
+"""vrl_score_responses: one launch from packed logits to the padded (B, T) response blocks — the label roll
+(verl/workers/engine/fsdp/transformer_impl.py:1177), temperature, entropy and log-probs (:1357-1399) and
+no_padding_2_padding (verl/workers/utils/padding.py:97-141) in the row kernel itself.
+
+Checked against the reference-held fixture, against the oracle's restatement of the same sequence of steps, and bit for
+bit against this library's separate entry points (vrl_rowscore followed by vrl_response_slice)."""
+
+import numpy as np
+import pytest
+import torch
+
+import verl_amd
+from verl_amd import _lib, errors, layout
+from verl_amd import torch_functional as vf
+from oracle import scoring
+from _parity import assert_scores_match
+
+pytestmark = pytest.mark.gpu
+
+
+def _batch(dev, seed, B, V, dtype, max_prompt=40, max_resp=90, scale=2.5):
+    g = torch.Generator().manual_seed(seed)
+    prompt = torch.randint(1, max_prompt, (B,), generator=g)
+    resp = torch.randint(0, max_resp, (B,), generator=g)
+    cu = torch.zeros(B + 1, dtype=torch.int64)
+    cu[1:] = torch.cumsum(prompt + resp, 0)
+    n = int(cu[-1])
+    gd = torch.Generator(device=dev).manual_seed(seed + 1)
+    ids = torch.randint(0, V, (n,), generator=gd, device=dev)
+    logits = (torch.randn(n, V, generator=gd, device=dev) * scale).to(dtype)
+    return prompt, resp, cu, ids, logits
+
+
+def test_reference_fixture_through_the_single_launch(dev):
+    """tests/models/test_fsdp_no_padding_on_gpu.py:180-201 in the reference: seed 0, vocab 32, sequences of 5 and 3
+    tokens with 2 and 1 response tokens -> rows [2:4] and [6:7] of the packed log-probs, zero-padded to (2, 2)."""
+    torch.manual_seed(0)
+    logits = torch.randn(2, 5, 32)
+    flat = torch.cat([logits[0, :5], logits[1, :3]], dim=0).to(dev)
+    ids = torch.tensor([11, 12, 13, 14, 15, 21, 22, 23], device=dev)
+    cu = torch.tensor([0, 5, 8], device=dev)
+    resp = torch.tensor([2, 1], device=dev)
+    r_lp, r_h = verl_amd.score_responses(flat, cu, resp, 2, input_ids=ids)
+    full = scoring.logprobs_from_logits(flat.cpu(), scoring.roll_labels(ids.cpu()))
+    full_h = scoring.entropy_from_logits(flat.cpu())
+    expected = torch.stack([full[2:4], torch.nn.functional.pad(full[6:7], (0, 1))])
+    expected_h = torch.stack([full_h[2:4], torch.nn.functional.pad(full_h[6:7], (0, 1))])
+    assert r_lp.shape == (2, 2) and (r_lp.cpu() - expected).abs().max().item() <= 1e-5
+    assert (r_h.cpu() - expected_h).abs().max().item() <= 1e-5
+    assert r_lp[1, 1].item() == 0.0 and r_h[1, 1].item() == 0.0
+    # ready-made labels instead of the ids give the same block
+    r2, _ = verl_amd.score_responses(flat, cu, resp, 2, labels=layout.roll_labels(ids))
+    assert torch.equal(r2, r_lp)
+
+
+@pytest.mark.parametrize("dtype,tol", [(torch.float32, 1e-5), (torch.bfloat16, 2e-3)])
+@pytest.mark.parametrize("with_temperature", [False, True])
+def test_random_packed_batches_against_oracle_and_separate_entry_points(dev, dtype, tol, with_temperature):
+    B, V = 23, 4099
+    prompt, resp, cu, ids, logits = _batch(dev, 77, B, V, dtype)
+    n = logits.shape[0]
+    temp = None
+    if with_temperature:
+        per_seq = 0.5 + torch.rand(B, generator=torch.Generator().manual_seed(3))
+        temp = torch.repeat_interleave(per_seq, prompt + resp).to(dev)
+    for T in (int(resp.max()), int(resp.max()) + 37):
+        r_lp, r_h, t_lp, t_h = verl_amd.score_responses(logits, cu.to(dev), resp.to(dev), T, input_ids=ids,
+                                                        temperature=temp, per_token=True)
+        # bit for bit what the separate launches give
+        lp, h = vf.fused_logprob_entropy(logits, layout.roll_labels(ids), temp)
+        assert torch.equal(t_lp, lp) and torch.equal(t_h, h)
+        assert torch.equal(r_lp, layout.response_slice(lp, cu.to(dev), resp.to(dev), T))
+        assert torch.equal(r_h, layout.response_slice(h, cu.to(dev), resp.to(dev), T))
+        # without the per-token vectors only the response rows are scored: same blocks
+        s_lp, s_h = verl_amd.score_responses(logits, cu.to(dev), resp.to(dev), T, input_ids=ids, temperature=temp)
+        assert torch.equal(s_lp, r_lp) and torch.equal(s_h, r_h)
+        only_h = verl_amd.score_responses(logits, cu.to(dev), resp.to(dev), T, temperature=temp, want_logprob=False)
+        assert only_h[0] is None and torch.equal(only_h[1], r_h)
+        only_lp = verl_amd.score_responses(logits, cu.to(dev), resp.to(dev), T, input_ids=ids, temperature=temp,
+                                           want_entropy=False)
+        assert only_lp[1] is None and torch.equal(only_lp[0], r_lp)
+        # the oracle's restatement of the reference's steps: per token with the shared parity rule (the fp64 value
+        # within 4e-6; torch's fp32 composition within the bar widened by torch's own distance from the fp64 value) ...
+        assert_scores_match(t_lp, t_h, logits, layout.roll_labels(ids), temp)
+        # ... and the slicing exactly, on the fp64 values
+        ref_lp, ref_h = scoring.score_fp64(logits.cpu(), scoring.roll_labels(ids.cpu()), None if temp is None else temp.cpu())
+        want_lp = scoring.response_slice(ref_lp.float(), prompt.tolist(), resp.tolist(), T)
+        want_h = scoring.response_slice(ref_h.float(), prompt.tolist(), resp.tolist(), T)
+        assert (r_lp.cpu() - want_lp).abs().max().item() <= 4e-6
+        assert (r_h.cpu() - want_h).abs().max().item() <= 4e-6
+        assert torch.equal(r_lp.cpu() == 0, want_lp == 0)
+
+
+def test_prompt_rows_do_not_matter_without_per_token_outputs(dev):
+    """Only rows inside a response window are scored when no per-token vector is asked for: whatever the prompt rows
+    hold (here NaN), the blocks are the same."""
+    B, V = 9, 3001
+    prompt, resp, cu, ids, logits = _batch(dev, 5, B, V, torch.bfloat16)
+    T = int(resp.max())
+    want = verl_amd.score_responses(logits, cu.to(dev), resp.to(dev), T, input_ids=ids)
+    poisoned = logits.clone()
+    for b in range(B):
+        end, r = int(cu[b + 1]), int(resp[b])
+        poisoned[int(cu[b]):end - r - 1] = float("nan")
+        poisoned[end - 1] = float("nan")
+    got = verl_amd.score_responses(poisoned, cu.to(dev), resp.to(dev), T, input_ids=ids)
+    assert torch.equal(got[0], want[0]) and torch.equal(got[1], want[1])
+
+
+def test_device_side_checks(dev):
+    B, V = 6, 1000
+    prompt, resp, cu, ids, logits = _batch(dev, 9, B, V, torch.float32)
+    resp = torch.clamp(resp, min=1)
+    cu = torch.zeros(B + 1, dtype=torch.int64)
+    cu[1:] = torch.cumsum(prompt + resp, 0)
+    n = int(cu[-1])
+    gd = torch.Generator(device=dev).manual_seed(10)
+    ids = torch.randint(0, V, (n,), generator=gd, device=dev)
+    logits = torch.randn(n, V, generator=gd, device=dev)
+    T = int(resp.max())
+    cud, rd = cu.to(dev), resp.to(dev)
+    good = verl_amd.score_responses(logits, cud, rd, T, input_ids=ids)
+    # a sequence whose "response" swallows its prompt: ValueError, and its row is zero when nobody looks
+    bad_r = resp.clone()
+    bad_r[2] = prompt[2] + resp[2]
+    with pytest.raises(ValueError, match="prompt token"):
+        verl_amd.score_responses(logits, cud, bad_r.to(dev), int(bad_r.max()), input_ids=ids)
+    out = verl_amd.score_responses(logits, cud, bad_r.to(dev), int(bad_r.max()), input_ids=ids, check=False)
+    assert torch.all(out[0][2] == 0) and torch.equal(out[0][3, :T], good[0][3])
+    # a response longer than the block
+    with pytest.raises(ValueError, match="response length"):
+        verl_amd.score_responses(logits, cud, rd, T - 1, input_ids=ids)
+    # offsets that do not partition the rows
+    for bad in ([0] + (cu[1:-1]).tolist() + [n + 5], [1] + cu[1:].tolist(), cu.flip(0).tolist()):
+        with pytest.raises(ValueError, match="partition"):
+            verl_amd.score_responses(logits, torch.tensor(bad, device=dev), rd, T, input_ids=ids)
+    # a label outside the vocabulary lands in the block as NaN and raises IndexError
+    bad_ids = ids.clone()
+    first_resp_row = int(cu[1]) - int(resp[0]) - 1
+    bad_ids[first_resp_row + 1] = V
+    with pytest.raises(IndexError):
+        verl_amd.score_responses(logits, cud, rd, T, input_ids=bad_ids)
+    with errors.using("deferred"):
+        out = verl_amd.score_responses(logits, cud, rd, T, input_ids=bad_ids)
+        with pytest.raises(IndexError):
+            errors.check_errors()
+    assert torch.isnan(out[0][0, 0]) and torch.equal(out[0][1:], good[0][1:])
+    # argument errors found on the host
+    with pytest.raises(ValueError):
+        verl_amd.score_responses(logits, cud, rd, T)                                   # no labels for the log-probs
+    with pytest.raises(ValueError):
+        verl_amd.score_responses(logits, cud, rd, T, input_ids=ids, labels=ids)
+    with pytest.raises(ValueError):
+        verl_amd.score_responses(logits, cud[:-1], rd, T, input_ids=ids)
+    with pytest.raises(ValueError):
+        verl_amd.score_responses(logits.view(1, n, V), cud, rd, T, input_ids=ids)
+    with pytest.raises(NotImplementedError):
+        verl_amd.score_responses(logits.clone().requires_grad_(True), cud, rd, T, input_ids=ids)
+    empty = verl_amd.score_responses(logits[:0], cud[:1], rd[:0], 4, input_ids=ids[:0])
+    assert empty[0].shape == (0, 4)
+
+
+def test_bad_offsets_leave_the_guard_regions_alone(dev):
+    from _guards import BAD_OFFSETS, Arena
+
+    lib = _lib.load()
+    N, V, B, T = 100, 512, 3, 16
+    g = torch.Generator().manual_seed(8)
+    for case, offsets in sorted(BAD_OFFSETS.items()):
+        ar = Arena(dev)
+        logits = ar.make(N * V, torch.bfloat16, (torch.randn(N * V, generator=g) * 2).bfloat16())
+        ids = ar.make(N, torch.int64, torch.randint(0, V, (N,), generator=g))
+        cu = ar.make(B + 1, torch.int64, torch.tensor(offsets, dtype=torch.int64))
+        rl = ar.make(B, torch.int64, torch.tensor([4, 7, 9], dtype=torch.int64))
+        t_lp = ar.make(N, torch.float32)
+        t_h = ar.make(N, torch.float32)
+        r_lp = ar.make(B * T, torch.float32)
+        r_h = ar.make(B * T, torch.float32)
+        flag = ar.make(1, torch.int32, torch.zeros(1, dtype=torch.int32))
+        print(f"[score_responses] cu_seqlens={offsets} over {N} rows", flush=True)
+        for per_token in (True, False):
+            flag.zero_()
+            with torch.cuda.device(dev):
+                st = lib.vrl_score_responses(logits.data_ptr(), _lib.VRL_BF16, N, V, V, None, ids.data_ptr(), None,
+                                             cu.data_ptr(), rl.data_ptr(), B, T, t_lp.data_ptr() if per_token else None,
+                                             t_h.data_ptr() if per_token else None, r_lp.data_ptr(), r_h.data_ptr(),
+                                             flag.data_ptr(), _lib.stream_ptr(dev))
+            assert st == _lib.VRL_OK
+            torch.cuda.synchronize(dev)
+            assert int(flag.item()) & _lib.VRL_FLAG_SEQ_RANGE, case
+            assert ar.guards_intact(), case
+            assert torch.isfinite(r_lp).all() and torch.isfinite(r_h).all(), case   # every block element was written
+
+
+def test_c3_micro_batch_full_size(dev):
+    """One 8192-token packed micro-batch at vocabulary 151936 bf16 (the GRPO workload's shape): the single launch
+    equals the separate launches bit for bit."""
+    V, n = 151936, 8192
+    lens = [2048, 1700, 1500, 1200, 1000, 744]
+    assert sum(lens) == n
+    resp = torch.tensor([1500, 1000, 1499, 600, 999, 700])
+    cu = torch.zeros(len(lens) + 1, dtype=torch.int64)
+    cu[1:] = torch.cumsum(torch.tensor(lens), 0)
+    gd = torch.Generator(device=dev).manual_seed(33)
+    logits = torch.empty(n, V, dtype=torch.bfloat16, device=dev)
+    for i in range(0, n, 1024):
+        logits[i:i + 1024] = (torch.randn(1024, V, generator=gd, device=dev) * 3).bfloat16()
+    ids = torch.randint(0, V, (n,), generator=gd, device=dev)
+    T = 2048
+    r_lp, r_h = verl_amd.score_responses(logits, cu.to(dev), resp.to(dev), T, input_ids=ids, temperature=0.9)
+    lp, h = vf.fused_logprob_entropy(logits, layout.roll_labels(ids), 0.9)
+    assert torch.equal(r_lp, layout.response_slice(lp, cu.to(dev), resp.to(dev), T))
+    assert torch.equal(r_h, layout.response_slice(h, cu.to(dev), resp.to(dev), T))
+    rows = torch.arange(0, n, 997)
+    ref_lp, ref_h = scoring.score_fp32(logits[rows.to(dev)].cpu(), layout.roll_labels(ids)[rows.to(dev)].cpu(),
+                                       torch.full((rows.numel(),), 0.9))
+    assert (lp[rows.to(dev)].cpu() - ref_lp).abs().max().item() <= 2e-3
+    assert (h[rows.to(dev)].cpu() - ref_h).abs().max().item() <= 2e-3

@@ -31,7 +31,9 @@ from .torch_functional import (
     logprobs_from_logits,
     logprobs_from_logits_naive,
     logprobs_from_logits_v2,
+    score_responses,
 )
+from .errors import check_errors
 
 __version__ = "0.1.0"
 
@@ -58,4 +60,6 @@ __all__ = [
     "logprobs_from_logits",
     "logprobs_from_logits_naive",
     "logprobs_from_logits_v2",
+    "score_responses",
+    "check_errors",
 ]

@@ -334,44 +334,53 @@ __device__ __forceinline__ float load_label_logit(const char* rowp, const int64_
 // One thread turns the row's (M, S, T, Q) into the outputs. The last step is
 // done in double: it runs once per row and keeps the result's error at the
 // level of the fp32 accumulation.
-template <bool EXACT, bool WANT_Q>
-__device__ __forceinline__ void finalize_row(const Part& w, float xl, bool label_ok, const Scale<EXACT>& sc,
-                                             int64_t row, float* out_logprob, float* out_entropy,
-                                             float* out_sum_pi_sq, float* out_lse, int32_t* err_flag) {
+struct RowResult {
   float lp, H, sps, lse;
+};
+
+template <bool EXACT>
+__device__ __forceinline__ RowResult row_result(const Part& w, float xl, const Scale<EXACT>& sc) {
+  RowResult r;
   if (w.m == neg_inf()) {
     // empty row or every logit -inf: logsumexp = -inf, x - (-inf) and softmax are NaN in torch
-    lp = quiet_nan();
-    H = quiet_nan();
-    sps = quiet_nan();
-    lse = neg_inf();
+    r.lp = quiet_nan();
+    r.H = quiet_nan();
+    r.sps = quiet_nan();
+    r.lse = neg_inf();
   } else if (w.m == pos_inf()) {
     // a +inf logit: logsumexp = +inf
-    lp = (sc.pre(xl) * sc.c == pos_inf()) ? quiet_nan() : neg_inf();
-    H = quiet_nan();
-    sps = quiet_nan();
-    lse = pos_inf();
+    r.lp = (sc.pre(xl) * sc.c == pos_inf()) ? quiet_nan() : neg_inf();
+    r.H = quiet_nan();
+    r.sps = quiet_nan();
+    r.lse = pos_inf();
   } else {
     const double S = static_cast<double>(w.s);
     const double l2s = log2(S);
     const double yl = static_cast<double>(sc.pre(xl)) * static_cast<double>(sc.c) - static_cast<double>(w.m);
-    lp = static_cast<float>(kLn2d * (yl - l2s));
-    H = static_cast<float>(kLn2d * (l2s - static_cast<double>(w.t) / S));
-    sps = static_cast<float>(static_cast<double>(w.q) / (S * S));
-    lse = static_cast<float>(kLn2d * (static_cast<double>(w.m) + l2s));
+    r.lp = static_cast<float>(kLn2d * (yl - l2s));
+    r.H = static_cast<float>(kLn2d * (l2s - static_cast<double>(w.t) / S));
+    r.sps = static_cast<float>(static_cast<double>(w.q) / (S * S));
+    r.lse = static_cast<float>(kLn2d * (static_cast<double>(w.m) + l2s));
   }
+  return r;
+}
+
+template <bool EXACT, bool WANT_Q>
+__device__ __forceinline__ RowResult finalize_row(const Part& w, float xl, bool label_ok, const Scale<EXACT>& sc,
+                                                  int64_t row, float* out_logprob, float* out_entropy,
+                                                  float* out_sum_pi_sq, float* out_lse, int32_t* err_flag) {
+  RowResult r = row_result<EXACT>(w, xl, sc);
+  if (!label_ok) r.lp = quiet_nan();
   if (out_logprob != nullptr) {
-    if (!label_ok) {
-      lp = quiet_nan();
-      atomicOr(err_flag, 1);
-    }
-    out_logprob[row] = lp;
+    if (!label_ok) atomicOr(err_flag, 1);
+    out_logprob[row] = r.lp;
   }
-  if (out_entropy != nullptr) out_entropy[row] = H;
-  if (out_lse != nullptr) out_lse[row] = lse;
+  if (out_entropy != nullptr) out_entropy[row] = r.H;
+  if (out_lse != nullptr) out_lse[row] = r.lse;
   if constexpr (WANT_Q) {
-    if (out_sum_pi_sq != nullptr) out_sum_pi_sq[row] = sps;
+    if (out_sum_pi_sq != nullptr) out_sum_pi_sq[row] = r.sps;
   }
+  return r;
 }
 
 // ---- one workgroup per row ---------------------------------------------------
@@ -391,6 +400,117 @@ __global__ __launch_bounds__(WAVES * 64) void rowscore_kernel(
   const Part w = block_reduce_range<DT, WAVES, U, EXACT, NT, WANT_Q>(rowp, 0, vocab, sc);
   if (threadIdx.x == 0)
     finalize_row<EXACT, WANT_Q>(w, xl, label_ok, sc, row, out_logprob, out_entropy, out_sum_pi_sq, out_lse, err_flag);
+}
+
+// ---- packed logits -> padded (B, T_out) response blocks in one launch -----------
+// grid.x = n_rows + B, block = WAVES*64.
+//   Workgroup r < n_rows scores row r like rowscore_kernel, with the label taken from `labels[r]` or, when
+//   `input_ids` is given instead, from the packed ids rolled by one: input_ids[(r + 1) mod n_rows]
+//   (verl/workers/engine/fsdp/transformer_impl.py:1177). It finds its sequence b by bisection over cu_seqlens
+//   (uniform loads) and, when r lies in that sequence's response window [end - resp - 1, end - 1), also writes its
+//   results to column r - (end - resp - 1) of row b of the padded blocks (verl/workers/utils/padding.py:135-138).
+//   With no per-token output asked for, a row outside every window is not read at all.
+//   Workgroup n_rows + b validates sequence b (offsets inside [0, n_rows] and ordered: VRL_FLAG_SEQ_RANGE; a prompt
+//   token before the response and 0 <= resp <= T_out: VRL_FLAG_SLICE_RANGE) and writes the zeros of row b: columns
+//   [resp, T_out) of a valid sequence, the whole row of an invalid one, whose rows then write nothing to the blocks.
+// Whatever cu_seqlens and response_lens hold, writes stay inside the arrays: block writes go to row b < B, column
+// j in [0, T_out). No thread meets a barrier that another one skips: a workgroup leaves as a whole or not at all.
+struct ResponseWindow {
+  int64_t first;  // first row of the window
+  int64_t resp;   // its length
+  bool ok;
+};
+
+__device__ __forceinline__ ResponseWindow response_window(const int64_t* cu_seqlens, const int64_t* response_lens,
+                                                          int64_t b, int64_t B, int64_t n_rows, int64_t T_out,
+                                                          int* why) {
+  const int64_t begin = cu_seqlens[b];
+  const int64_t end = cu_seqlens[b + 1];
+  const int64_t resp = response_lens[b];
+  const bool span_ok = (begin >= 0) && (end <= n_rows) && (end >= begin) && (b != 0 || begin == 0) &&
+                       (b + 1 != B || end == n_rows);
+  ResponseWindow w;
+  w.resp = resp;
+  w.first = 0;
+  bool resp_ok = false;
+  if (span_ok && resp >= 0 && resp <= T_out) {  // only now is end - resp - 1 known not to wrap
+    w.first = end - resp - 1;
+    resp_ok = w.first >= begin;
+  }
+  w.ok = span_ok && resp_ok;
+  *why = span_ok ? (resp_ok ? 0 : 2) : 4;
+  return w;
+}
+
+template <int DT, int WAVES, int U, bool EXACT>
+__global__ __launch_bounds__(WAVES * 64) void score_responses_kernel(
+    const void* __restrict__ logits, int64_t n_rows, int64_t vocab, int64_t row_stride,
+    const int64_t* __restrict__ labels, const int64_t* __restrict__ input_ids,
+    const float* __restrict__ temperature, const int64_t* __restrict__ cu_seqlens,
+    const int64_t* __restrict__ response_lens, int64_t B, int64_t T_out, float* __restrict__ out_logprob,
+    float* __restrict__ out_entropy, float* __restrict__ resp_logprob, float* __restrict__ resp_entropy,
+    int32_t* err_flag) {
+  constexpr int NTHR = WAVES * 64;
+  const int64_t wg = blockIdx.x;
+  if (wg >= n_rows) {
+    // sequence workgroup: validation and the zeros of row b
+    const int64_t b = wg - n_rows;
+    int why = 0;
+    const ResponseWindow w = response_window(cu_seqlens, response_lens, b, B, n_rows, T_out, &why);
+    if (why != 0 && threadIdx.x == 0) atomicOr(err_flag, why);
+    const int64_t from = w.ok ? w.resp : 0;
+    for (int64_t j = from + threadIdx.x; j < T_out; j += NTHR) {
+      if (resp_logprob != nullptr) resp_logprob[b * T_out + j] = 0.f;
+      if (resp_entropy != nullptr) resp_entropy[b * T_out + j] = 0.f;
+    }
+    return;
+  }
+  const int64_t row = wg;
+  // sequence of this row: the largest b with cu[b] <= row (bisection; uniform over the workgroup)
+  int64_t lo = 0, hi = B;  // invariant: answer in [lo, hi)
+  while (hi - lo > 1) {
+    const int64_t mid = (lo + hi) >> 1;
+    if (cu_seqlens[mid] <= row) lo = mid; else hi = mid;
+  }
+  bool in_window = false;
+  int64_t col = 0;
+  const int64_t b = lo;
+  if (B > 0 && cu_seqlens[b] <= row && row < cu_seqlens[b + 1]) {
+    int why = 0;
+    const ResponseWindow w = response_window(cu_seqlens, response_lens, b, B, n_rows, T_out, &why);
+    if (w.ok) {
+      col = row - w.first;
+      in_window = col >= 0 && col < w.resp;
+    }
+  }
+  const bool per_token = (out_logprob != nullptr) || (out_entropy != nullptr);
+  if (!per_token && !in_window) return;  // the whole workgroup: this row's logits are never read
+
+  const char* rowp = static_cast<const char*>(logits) + row * row_stride * Elem<DT>::kBytes;
+  const Scale<EXACT> sc = make_scale<EXACT>(temperature, row);
+  const bool want_lp = (out_logprob != nullptr) || (resp_logprob != nullptr);
+  float xl = 0.f;
+  bool label_ok = true;
+  if (want_lp && threadIdx.x == 0) {
+    int64_t lab;
+    if (input_ids != nullptr) {
+      lab = input_ids[row + 1 < n_rows ? row + 1 : 0];
+    } else {
+      lab = labels[row];
+    }
+    label_ok = (lab >= 0) && (lab < vocab);
+    xl = label_ok ? Elem<DT>::load1(rowp, lab) : quiet_nan();
+  }
+  const Part w = block_reduce_range<DT, WAVES, U, EXACT, true, false>(rowp, 0, vocab, sc);
+  if (threadIdx.x == 0) {
+    if (want_lp && !label_ok && out_logprob == nullptr) atomicOr(err_flag, 1);  // finalize_row flags it otherwise
+    const RowResult r = finalize_row<EXACT, false>(w, xl, label_ok, sc, row, out_logprob, out_entropy, nullptr,
+                                                   nullptr, err_flag);
+    if (in_window) {
+      if (resp_logprob != nullptr) resp_logprob[b * T_out + col] = r.lp;
+      if (resp_entropy != nullptr) resp_entropy[b * T_out + col] = r.H;
+    }
+  }
 }
 
 // ---- few rows: several workgroups per row ------------------------------------

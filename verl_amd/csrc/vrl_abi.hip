@@ -204,6 +204,26 @@ int check_layout(const int64_t* cu_seqlens, int64_t B, int64_t T, int64_t n_toke
   return VRL_OK;
 }
 
+template <int DT, int W, int U, bool EXACT>
+void launch_score_responses(const void* logits, int64_t n_rows, int64_t vocab, int64_t row_stride,
+                            const int64_t* labels, const int64_t* input_ids, const float* temperature,
+                            const int64_t* cu_seqlens, const int64_t* response_lens, int64_t B, int64_t T_out,
+                            float* out_logprob, float* out_entropy, float* resp_logprob, float* resp_entropy,
+                            int32_t* err_flag, hipStream_t s) {
+  vrl::score_responses_kernel<DT, W, U, EXACT><<<dim3(static_cast<unsigned>(n_rows + B)), dim3(W * 64), 0, s>>>(
+      logits, n_rows, vocab, row_stride, labels, input_ids, temperature, cu_seqlens, response_lens, B, T_out,
+      out_logprob, out_entropy, resp_logprob, resp_entropy, err_flag);
+}
+
+template <int DT, bool EXACT, typename... Args>
+void launch_score_responses_shaped(int64_t n_rows, int64_t vocab, Args... a) {
+  // same workgroup shapes as the plain row kernel (see launch_rows)
+  if (n_rows < kWideRowsBelow && vocab >= kWideVocabFrom)
+    launch_score_responses<DT, 16, 2, EXACT>(a...);
+  else
+    launch_score_responses<DT, RowShape<DT>::kWaves, RowShape<DT>::kUnroll, EXACT>(a...);
+}
+
 int check_verify(const float* logp_new, const float* logp_old, const float* log_u, const uint8_t* mask,
                  const int64_t* cu_seqlens, int64_t B, int64_t T, int64_t n_tokens, const int32_t* err_flag,
                  const uint8_t* accept, const int32_t* first_reject, const int32_t* prefix_len,
@@ -313,6 +333,45 @@ int vrl_label_logprob(const void* logits, int dtype, int64_t n_rows, int64_t voc
     vrl::label_logprob_kernel<VRL_F16, false><<<grid, dim3(256), 0, s>>>(logits, n_rows, vocab, row_stride, labels,
                                                                          temperature, lse, out_logprob, err_flag);
   }
+  return launch_status();
+}
+
+int vrl_score_responses(const void* logits, int dtype, int64_t n_rows, int64_t vocab, int64_t row_stride,
+                        const int64_t* labels, const int64_t* input_ids, const float* temperature,
+                        const int64_t* cu_seqlens, const int64_t* response_lens, int64_t B, int64_t T_out,
+                        float* out_logprob, float* out_entropy, float* resp_logprob, float* resp_entropy,
+                        int32_t* err_flag, void* stream) {
+  if (!known_dtype(dtype)) return VRL_ERR_DTYPE;
+  if (n_rows < 0 || vocab <= 0 || row_stride < vocab || B < 0 || T_out < 0 || n_rows + B > kMaxGrid)
+    return VRL_ERR_SHAPE;
+  if (resp_logprob == nullptr && resp_entropy == nullptr) return VRL_ERR_ARG;
+  if (labels != nullptr && input_ids != nullptr) return VRL_ERR_ARG;   // one source of labels
+  if (out_logprob != nullptr && resp_logprob == nullptr) return VRL_ERR_ARG;
+  if (out_entropy != nullptr && resp_entropy == nullptr) return VRL_ERR_ARG;
+  if (B == 0) return (n_rows == 0) ? VRL_OK : VRL_ERR_SHAPE;          // rows that belong to no sequence
+  if (cu_seqlens == nullptr || response_lens == nullptr || err_flag == nullptr) return VRL_ERR_NULL;
+  if (n_rows > 0 && logits == nullptr) return VRL_ERR_NULL;
+  if (resp_logprob != nullptr && labels == nullptr && input_ids == nullptr && n_rows > 0) return VRL_ERR_NULL;
+  const uintptr_t esize = (dtype == VRL_F32) ? 4 : 2;
+  if (!aligned(logits, esize) || !aligned(labels, 8) || !aligned(input_ids, 8) || !aligned(temperature, 4) ||
+      !aligned(cu_seqlens, 8) || !aligned(response_lens, 8) || !aligned(out_logprob, 4) ||
+      !aligned(out_entropy, 4) || !aligned(resp_logprob, 4) || !aligned(resp_entropy, 4) || !aligned(err_flag, 4))
+    return VRL_ERR_ALIGN;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+#define VRL_SR_ARGS                                                                                               \
+  n_rows, vocab, logits, n_rows, vocab, row_stride, labels, input_ids, temperature, cu_seqlens, response_lens, B, \
+      T_out, out_logprob, out_entropy, resp_logprob, resp_entropy, err_flag, s
+  if (dtype == VRL_F32) {
+    if (temperature != nullptr)
+      launch_score_responses_shaped<VRL_F32, true>(VRL_SR_ARGS);
+    else
+      launch_score_responses_shaped<VRL_F32, false>(VRL_SR_ARGS);
+  } else if (dtype == VRL_BF16) {
+    launch_score_responses_shaped<VRL_BF16, false>(VRL_SR_ARGS);
+  } else {
+    launch_score_responses_shaped<VRL_F16, false>(VRL_SR_ARGS);
+  }
+#undef VRL_SR_ARGS
   return launch_status();
 }
 

@@ -34,6 +34,7 @@ __all__ = [
     "entropy_from_logits_with_chunking",
     "calculate_sum_pi_squared_from_logits",
     "fused_logprob_entropy",
+    "score_responses",
 ]
 
 # A label outside [0, vocab) makes that row's log-prob NaN and sets a bit in the kernel's error flag. How the flag
@@ -437,3 +438,94 @@ def fused_logprob_entropy(
     """
     return rowscore(logits, labels, temperature, check_labels=check_labels, want_sum_pi_sq=want_sum_pi_sq,
                     n_splits=n_splits, what="fused_logprob_entropy")
+
+
+def score_responses(
+    logits: torch.Tensor,
+    cu_seqlens: torch.Tensor,
+    response_lens: torch.Tensor,
+    max_response_len: int,
+    *,
+    labels: Optional[torch.Tensor] = None,
+    input_ids: Optional[torch.Tensor] = None,
+    temperature: Union[None, float, torch.Tensor] = None,
+    want_logprob: bool = True,
+    want_entropy: bool = True,
+    per_token: bool = False,
+    check=None,
+):
+    """Packed ``logits`` ``(total_nnz, V)`` -> padded ``(B, max_response_len)`` response log-probs and entropies in ONE
+    kernel launch (``vrl_score_responses``).
+
+    The engine's sequence on a packed micro-batch — ``labels = roll(input_ids, -1)``
+    (verl/workers/engine/fsdp/transformer_impl.py:1177), divide by the temperature (:1357), entropy and log-probs
+    (:1364-1399), then ``no_padding_2_padding`` (verl/workers/utils/padding.py:97-141: per sequence take
+    ``values[end - r - 1 : end - 1]`` and right-pad with zeros) — done by the row kernel itself: give ``input_ids``
+    (the packed ids, rolled inside the kernel) or ready ``labels``; ``temperature`` is a float or one value per token.
+
+    Returns ``(resp_logprob | None, resp_entropy | None)``; with ``per_token`` also the ``(total_nnz,)`` vectors, as
+    ``(resp_logprob, resp_entropy, logprob, entropy)``. Without ``per_token`` the logits of tokens outside every
+    response window (the prompts) are never read. Forward only. Device-side findings (a label outside the vocabulary:
+    IndexError; a sequence without a prompt token, a response longer than ``max_response_len``, offsets that do not
+    partition the rows: ValueError) follow ``check`` as in verl_amd.errors.
+    """
+    what = "score_responses"
+    _check_logits(logits, what)
+    _errors.poll()
+    if logits.dim() != 2:
+        raise ValueError(f"{what}: logits must be packed (total_nnz, vocab), got shape {tuple(logits.shape)}")
+    if torch.is_grad_enabled() and logits.requires_grad:
+        raise NotImplementedError(f"{what} is a forward-only step (compute_log_prob); use fused_logprob_entropy "
+                                  "followed by response_slice when gradients are needed")
+    if not (want_logprob or want_entropy):
+        raise ValueError(f"{what}: nothing to compute")
+    if want_logprob and (labels is None) == (input_ids is None):
+        raise ValueError(f"{what}: give exactly one of labels and input_ids for the log-probs")
+    x = _rows_2d(logits)
+    n, V = x.shape
+    dev = x.device
+    src = labels if labels is not None else input_ids
+    lab = None
+    if want_logprob:
+        if tuple(src.shape) != (n,):
+            raise ValueError(f"{what}: labels / input_ids must have shape ({n},), got {tuple(src.shape)}")
+        if src.dtype.is_floating_point or src.dtype == torch.bool:
+            raise TypeError(f"{what}: labels / input_ids must be an integer tensor, got {src.dtype}")
+        lab = src.to(device=dev, dtype=torch.int64).contiguous()
+    temp = _temperature_rows(temperature, (n,), n, dev)
+    cu = cu_seqlens.to(device=dev, dtype=torch.int64).contiguous()
+    rl = response_lens.to(device=dev, dtype=torch.int64).contiguous()
+    B = rl.numel()
+    if cu.dim() != 1 or cu.numel() != B + 1:
+        raise ValueError(f"{what}: cu_seqlens must have B+1 = {B + 1} entries, got {tuple(cu.shape)}")
+    T = int(max_response_len)
+    if T < 0:
+        raise ValueError(f"{what}: max_response_len must not be negative")
+    if B == 0 and n > 0:
+        raise ValueError(f"{what}: {n} rows but no sequence")
+    f32 = dict(dtype=torch.float32, device=dev)
+    r_lp = torch.empty((B, T), **f32) if want_logprob else None
+    r_h = torch.empty((B, T), **f32) if want_entropy else None
+    t_lp = torch.empty(n, **f32) if (per_token and want_logprob) else None
+    t_h = torch.empty(n, **f32) if (per_token and want_entropy) else None
+    if B > 0:
+        flag = torch.zeros(1, dtype=torch.int32, device=dev)
+        lib = _lib.load()
+        with torch.cuda.device(dev):
+            st = lib.vrl_score_responses(
+                x.data_ptr() if n else None, _DTYPE_CODES[x.dtype], n, V, x.stride(0) if n > 1 else V,
+                _ptr(lab) if labels is not None else None, _ptr(lab) if labels is None else None, _ptr(temp),
+                cu.data_ptr(), rl.data_ptr(), B, T, _ptr(t_lp), _ptr(t_h), _ptr(r_lp), _ptr(r_h), flag.data_ptr(),
+                _lib.stream_ptr(dev))
+        _lib.check("vrl_score_responses", st)
+        counters["forward_passes"] += 1
+        _errors.report(flag, {
+            _lib.VRL_FLAG_LABEL_OOB: (IndexError, f"{what}: a label is outside [0, {V})"),
+            _lib.VRL_FLAG_SEQ_RANGE: (ValueError, f"{what}: cu_seqlens is not a partition of the {n} rows "
+                                      "(it must start at 0, never decrease and end at the number of rows)"),
+            _lib.VRL_FLAG_SLICE_RANGE: (ValueError, f"{what}: a sequence has no prompt token, or a response length "
+                                        f"outside [0, {T}]"),
+        }, check)
+    if per_token:
+        return r_lp, r_h, t_lp, t_h
+    return r_lp, r_h
