@@ -157,30 +157,60 @@ class Step:
         _lib.check("vrl_fused_score_verify", st)
 
     def check_against_torch(self, rows: int = 1024):
-        """Guard: the first rows against torch's fp32 ops on the GPU (not timed)."""
+        """Guard, not timed: the first rows against torch on the GPU, in fp32 (what verl computes there) and in
+        fp64 (the value of the same formula on the same fp32 inputs). Returns a record with the maximum
+        distances and the number of rows whose distance from torch's fp32 result exceeds the plain bar
+        (1e-5 for fp32 logits, 2e-3 for 16-bit ones): torch's own fp32 entropy is up to ~1.3e-5 from the fp64
+        value at V ~ 128k, so a kernel that is closer to the fp64 value than torch can still sit outside 1e-5
+        of torch on a few rows; the record shows how many."""
         z = self.logits[:rows].float()
         if self.temp is not None:
             z = z / self.temp[:rows].clamp(min=1e-8).unsqueeze(-1)
+        lab = self.labels[:rows, None]
         lse = torch.logsumexp(z, -1)
-        ref_lp = z.gather(-1, self.labels[:rows, None]).squeeze(-1) - lse
+        ref_lp = z.gather(-1, lab).squeeze(-1) - lse
         ref_h = lse - (torch.softmax(z, -1) * z).sum(-1)
-        e1 = (self.lp[:rows] - ref_lp).abs().max().item()
-        e2 = (self.h[:rows] - ref_h).abs().max().item()
-        # A coarse guard, not the parity test: torch's own fp32 entropy on the GPU is up to ~1.3e-5 from the
-        # exact value at V ~ 128k (tests/_parity.py measures it against the fp64 oracle), hence 5e-5 there.
-        tol_lp, tol_h = (1e-5, 5e-5) if self.w.dtype == torch.float32 else (2e-3, 2e-3)
-        if not (e1 <= tol_lp and e2 <= tol_h):
-            raise SystemExit(f"bench: kernel disagrees with torch fp32 (logprob {e1} > {tol_lp} or entropy {e2} > {tol_h})")
+        z64 = z.double()
+        lse64 = torch.logsumexp(z64, -1)
+        t_lp = z64.gather(-1, lab).squeeze(-1) - lse64
+        t_h = lse64 - (torch.softmax(z64, -1) * z64).sum(-1)
+        del z64
+        lp, h = self.lp[:rows].double(), self.h[:rows].double()
+        tol = 1e-5 if self.w.dtype == torch.float32 else 2e-3
+        rec = {
+            "rows": rows,
+            "tolerance": tol,
+            "max_abs_err_logprob": (lp - ref_lp).abs().max().item(),
+            "max_abs_err_entropy": (h - ref_h).abs().max().item(),
+            "max_abs_err_logprob_vs_fp64": (lp - t_lp).abs().max().item(),
+            "max_abs_err_entropy_vs_fp64": (h - t_h).abs().max().item(),
+            "torch_fp32_own_err_logprob": (ref_lp.double() - t_lp).abs().max().item(),
+            "torch_fp32_own_err_entropy": (ref_h.double() - t_h).abs().max().item(),
+            "rows_over_plain_tol_logprob": int(((lp - ref_lp).abs() > tol).sum().item()),
+            "rows_over_plain_tol_entropy": int(((h - ref_h).abs() > tol).sum().item()),
+        }
+        # A coarse guard, not the parity test (tests/_parity.py is): 4e-6 of the fp64 value, and the bar widened
+        # per row only by torch's own distance from the fp64 value.
+        ok = (rec["max_abs_err_logprob_vs_fp64"] <= 4e-6 and rec["max_abs_err_entropy_vs_fp64"] <= 4e-6
+              and bool(((lp - ref_lp).abs() <= tol + (ref_lp.double() - t_lp).abs()).all())
+              and bool(((h - ref_h).abs() <= tol + (ref_h.double() - t_h).abs()).all()))
+        if not ok:
+            raise SystemExit(f"bench: kernel disagrees with torch: {rec}")
         if int(self.flag.item()) != 0:
-            raise SystemExit("bench: label out of range flagged")
-        return e1, e2
+            raise SystemExit("bench: an error flag is set after the guard run")
+        return rec
 
 
-def bench_backward(args, dev):
+# HBM bytes per launch of rowscore_backward_kernel from rocprofv3 --pmc (FETCH_SIZE, WRITE_SIZE; same scaling as above).
+MEASURED_BACKWARD_TRAFFIC_BYTES = {"c3": 4981794581}   # profiles/rowscore_backward_kernel_hbm_counters_c3.md
+
+
+def bench_backward(args, dev, workload=None):
     """Throughput of vrl_rowscore_backward (gradient of log-prob and entropy with respect to the logits) on the
     workload's rows: reads the logits once, writes the gradient once (2 * V * sizeof + per-row scalars)."""
-    w = synthetic.WORKLOADS[args.workload]
-    step = Step(w, dev, seed=1000 * int(args.workload[1]))
+    workload = workload or args.workload
+    w = synthetic.WORKLOADS[workload]
+    step = Step(w, dev, seed=1000 * int(workload[1]))
     lse = torch.empty(step.n, dtype=torch.float32, device=dev)
     st = step.lib.vrl_rowscore(step.logits.data_ptr(), step.dt, step.n, w.V, step.logits.stride(0), step.labels.data_ptr(),
                                step._tp(), step.lp.data_ptr(), step.h.data_ptr(), None, lse.data_ptr(),
@@ -197,6 +227,8 @@ def bench_backward(args, dev):
                                             gl.data_ptr(), gh.data_ptr(), dx.data_ptr(), dx.stride(0), step.stream)
         _lib.check("vrl_rowscore_backward", st)
 
+    if args.copy_calibration:
+        copy_calibration(dev)
     # guard: first rows against torch autograd in fp32
     run()
     rows = 256
@@ -229,7 +261,7 @@ def bench_backward(args, dev):
     esize = 2 if w.dtype == torch.bfloat16 else 4
     bytes_launch = step.n * (2 * w.V * esize + 8 + 4 + 4 + 4 + 4 + (4 if step.temp is not None else 0))
     achieved = bytes_launch / (avg_ms * 1e-3) / 1e9
-    print(json.dumps({
+    return {
         "metric": "tokens/sec of the backward of the row op + achieved HBM GB/s", "value": step.n * args.steps / wall,
         "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": wall * 1e3 / args.steps,
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
@@ -237,9 +269,10 @@ def bench_backward(args, dev):
         "config": {"workload": w.name, "layout": step.layout, "rows_per_step": step.n, "vocab": w.V,
                    "step": "vrl_rowscore_backward through the C ABI (gradients of log-prob and entropy)"},
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                     "frac": achieved / HBM_PEAK_GBPS, "traffic": None, "kernel": "rowscore_backward_kernel",
-                     "avg_kernel_ms": avg_ms, "algorithmic_bytes_per_launch": bytes_launch},
-    }), flush=True)
+                     "frac": achieved / HBM_PEAK_GBPS, "traffic": MEASURED_BACKWARD_TRAFFIC_BYTES.get(workload),
+                     "kernel": "rowscore_backward_kernel", "avg_kernel_ms": avg_ms,
+                     "algorithmic_bytes_per_launch": bytes_launch},
+    }
 
 
 class VerifyOnlyStep:
@@ -279,7 +312,7 @@ class VerifyOnlyStep:
         _lib.check("vrl_spec_verify", st)
 
 
-def bench_verify_only(args, dev):
+def bench_verify_only(args, dev, with_cpu_baseline=True):
     """tokens/s of vrl_spec_verify alone on the c5 workload; 4+4+4 in, 1 out per token, plus the truncated draft
     (8 in, 8+1 out) = 30 B/token with the draft, 14 B/token (13 + per-sequence outputs) without."""
     w = synthetic.WORKLOADS["c5"]
@@ -312,7 +345,7 @@ def bench_verify_only(args, dev):
                      "frac": achieved / HBM_PEAK_GBPS, "traffic": None, "kernel": "spec_verify_kernel",
                      "avg_kernel_ms": avg_ms, "algorithmic_bytes_per_launch": bytes_launch},
     }
-    if not args.no_cpu_baseline:
+    if with_cpu_baseline:
         from oracle import verify as overify  # baseline only
 
         ln, lo, lu, ids, cu = step.lp.cpu(), step.lp_old.cpu(), step.log_u.cpu(), step.ids.cpu(), step.cu.cpu()
@@ -324,7 +357,7 @@ def bench_verify_only(args, dev):
         out["cpu_baseline"] = {"value": step.n / statistics.median(times), "unit": "tokens/s",
                                "cores": torch.get_num_threads(), "kind": "port",
                                "sample": f"the whole workload ({step.n} tokens), median of 3 runs of the vectorised torch statement of the rule"}
-    print(json.dumps(out), flush=True)
+    return out
 
 
 def bench_lm_head(args, dev):
@@ -451,46 +484,61 @@ def cpu_baseline(step: Step, budget_s: float = 12.0, runs: int = 4):
     }
 
 
-def main():
-    ap = argparse.ArgumentParser()
-    ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=20)
-    ap.add_argument("--warmup", type=int, default=3)
-    ap.add_argument("--workload", default="c2", choices=["c1", "c2", "c3", "c4", "c5"],
-                    help="c5 times the verify kernel alone (its logits do not fit; they are scored like c3)")
-    ap.add_argument("--vocab", type=int, default=0, help="run the workload's recipe at another vocabulary size")
-    ap.add_argument("--seqs", type=int, default=0, help="... with another number of sequences")
-    ap.add_argument("--dtype", choices=["bf16", "f32"], default=None, help="... with another logits element type")
-    ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--backward", action="store_true",
-                    help="time vrl_rowscore_backward on the workload instead of the fused forward step")
-    ap.add_argument("--lm-head", action="store_true",
-                    help="time the LM head + scoring step (verl_amd.fused_linear) instead of the fused forward step")
-    ap.add_argument("--chunk", type=int, default=4096, help="--lm-head: tokens projected at a time")
-    ap.add_argument("--keep-logits", action="store_true", help="--lm-head: keep the logits for the backward")
-    ap.add_argument("--copy-calibration", action="store_true",
-                    help="also run a plain device copy of known size (for scaling rocprofv3 byte counters)")
-    args = ap.parse_args()
-    if args.gpus != 1:
-        print("bench.py: this build runs on one GPU only; "
-              f"--gpus {args.gpus} is not supported", file=sys.stderr)
-        sys.exit(2)
-    if not torch.cuda.is_available():
-        print("bench.py: no GPU visible; the HIP path has no CPU fallback", file=sys.stderr)
-        sys.exit(2)
+def copy_calibration(dev):
+    """A plain copy kernel of known size: reads 1 GiB, writes 1 GiB. Whatever FETCH_SIZE / WRITE_SIZE report for it
+    is the scale that converts the same counters of the row kernels into bytes."""
+    src = torch.empty(1 << 29, dtype=torch.int16, device=dev).fill_(3)
+    dst = torch.empty_like(src)
+    for _ in range(3):
+        dst.copy_(src)
+    torch.cuda.synchronize()
+    del src, dst
 
-    dev = torch.device("cuda:0")
-    torch.cuda.set_device(dev)
-    if args.lm_head:
-        bench_lm_head(args, dev)
-        return
-    if args.workload == "c5":
-        bench_verify_only(args, dev)
-        return
-    if args.backward:
-        bench_backward(args, dev)
-        return
-    w = synthetic.WORKLOADS[args.workload]
+
+def bench_ceilings(args, dev):
+    """The memory system's own ceilings for the row kernels' access pattern (vrl_stream_probe): a non-temporal read
+    of c3's rows (forward kernel) and a non-temporal copy of them (backward kernel), plus torch's device copy."""
+    lib = _lib.load()
+    stream = torch.cuda.current_stream(dev).cuda_stream
+    out = {"metric": "HBM GB/s delivered to the row kernels' access pattern without arithmetic", "unit": "GB/s",
+           "peak": HBM_PEAK_GBPS, "probes": []}
+    sink = torch.zeros(1, dtype=torch.int32, device=dev)
+    for name, rows, row_bytes in (("c3 micro-batch, 8192 x 151936 bf16", 8192, 151936 * 2),
+                                  ("c2, 65536 x 152064 bf16", 65536, 152064 * 2)):
+        src = torch.empty(rows * row_bytes // 2, dtype=torch.int16, device=dev).fill_(5)
+        for mode, what, factor in ((0, "non-temporal read", 1), (1, "non-temporal copy", 2)):
+            if mode == 1 and rows * row_bytes > (8 << 30):
+                continue
+            dst = torch.empty_like(src) if mode == 1 else None
+
+            def run():
+                st = lib.vrl_stream_probe(src.data_ptr(), None if dst is None else dst.data_ptr(), rows, row_bytes, mode,
+                                          sink.data_ptr(), stream)
+                _lib.check("vrl_stream_probe", st)
+
+            spin_up(run)
+            evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(args.steps)]
+            for a, b in evs:
+                a.record()
+                run()
+                b.record()
+            torch.cuda.synchronize()
+            ms = sum(a.elapsed_time(b) for a, b in evs) / len(evs)
+            if mode == 1 and not torch.equal(dst, src):
+                raise SystemExit("bench: the copy probe did not copy")
+            out["probes"].append({"buffer": name, "probe": what, "kernel": "stream_probe_kernel", "avg_kernel_ms": ms,
+                                  "bytes_per_launch": factor * rows * row_bytes,
+                                  "gbps": factor * rows * row_bytes / (ms * 1e-3) / 1e9,
+                                  "frac_of_peak": factor * rows * row_bytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBPS})
+            del dst
+        del src
+        torch.cuda.empty_cache()
+    print(json.dumps(out), flush=True)
+
+
+def bench_forward(args, dev, workload, steps, warmup, with_cpu_baseline):
+    """The fused score + verify step on one workload; returns the JSON record."""
+    w = synthetic.WORKLOADS[workload]
     if args.vocab or args.seqs or args.dtype:
         # the workload's recipe at another vocabulary / batch / element type (e.g. 32000, 128256, 129280, 262144)
         kw = {"name": w.name + "_resized"}
@@ -501,33 +549,26 @@ def main():
         if args.dtype:
             kw["dtype"] = {"bf16": torch.bfloat16, "f32": torch.float32}[args.dtype]
         w = w.scaled(**kw)
-    step = Step(w, dev, seed=1000 * int(args.workload[1]))
-    err_lp, err_h = step.check_against_torch()
+    step = Step(w, dev, seed=1000 * int(workload[1]))
+    guard = step.check_against_torch()
 
     if args.copy_calibration:
-        # A plain copy kernel of known size: reads 1 GiB, writes 1 GiB. Whatever FETCH_SIZE / WRITE_SIZE report
-        # for it is the scale that converts the same counters of the row kernel into bytes.
-        src = torch.empty(1 << 29, dtype=torch.int16, device=dev).fill_(3)
-        dst = torch.empty_like(src)
-        for _ in range(3):
-            dst.copy_(src)
-        torch.cuda.synchronize()
-        del src, dst
+        copy_calibration(dev)
 
     spin_up(step.fused)
-    for _ in range(args.warmup):
+    for _ in range(warmup):
         step.fused()
     torch.cuda.synchronize()
     t0 = time.perf_counter()
-    for _ in range(args.steps):
+    for _ in range(steps):
         step.fused()
     torch.cuda.synchronize()
     wall = time.perf_counter() - t0
-    ms_per_step = wall * 1e3 / args.steps
-    tokens_per_s = step.n_valid * args.steps / wall
+    ms_per_step = wall * 1e3 / steps
+    tokens_per_s = step.n_valid * steps / wall
 
     # Row kernel alone, one HIP event pair per launch on the launch stream.
-    evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(args.steps)]
+    evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(steps)]
     for a, b in evs:
         a.record()
         step.score()
@@ -539,14 +580,15 @@ def main():
     bytes_score = algorithmic_bytes_per_token(w.V, esize, step.temp is not None, False) * step.n
     achieved = bytes_score / (avg_kern_ms * 1e-3) / 1e9
     bytes_fused = algorithmic_bytes_per_token(w.V, esize, step.temp is not None, True) * step.n
+    resized = bool(args.vocab or args.seqs or args.dtype)
 
     out = {
         "metric": METRIC,
         "value": tokens_per_s,
         "unit": "tokens/s",
         "n_gpus": 1,
-        "steps": args.steps,
-        "warmup": args.warmup,
+        "steps": steps,
+        "warmup": warmup,
         "ms_per_step": ms_per_step,
         "higher_is_better": True,
         "scaling": "weak",
@@ -573,15 +615,177 @@ def main():
             "peak": HBM_PEAK_GBPS,
             "unit": "GB/s",
             "frac": achieved / HBM_PEAK_GBPS,
-            "traffic": None if (args.vocab or args.seqs or args.dtype) else MEASURED_TRAFFIC_BYTES.get(args.workload),
+            "traffic": None if resized else MEASURED_TRAFFIC_BYTES.get(workload),
+            "traffic_source": None if resized or workload not in MEASURED_TRAFFIC_BYTES else
+            "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of this kernel at this shape, profiles/rowscore_kernel_hbm_counters_c2_c3_c4.md",
             "kernel": "rowscore_kernel",
             "avg_kernel_ms": avg_kern_ms,
             "algorithmic_bytes_per_launch": bytes_score,
         },
-        "parity_guard": {"rows": 1024, "max_abs_err_logprob": err_lp, "max_abs_err_entropy": err_h},
+        "parity_guard": guard,
     }
-    if not args.no_cpu_baseline:
+    if with_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(step)
+    return out
+
+
+def bench_score_responses(args, dev, steps, warmup):
+    """c3's packed micro-batch through vrl_score_responses: label roll, scoring and the (B, T) response slicing in
+    one launch; only rows inside a response window are read. Sequences are prompt + response with the response
+    lengths of the workload and prompts of a quarter of that."""
+    w = synthetic.WORKLOADS["c3"]
+    budget = int(w.micro_batch_tokens)
+    resp_all = synthetic.draw_lengths(w, 3002).tolist()
+    seqs, total = [], 0
+    for r in resp_all:
+        p = max(1, r // 4)
+        if total + p + r > budget:
+            break
+        seqs.append((p, r))
+        total += p + r
+    seqs[-1] = (seqs[-1][0] + budget - total, seqs[-1][1])   # the last prompt takes up the rest of the budget
+    n = budget
+    cu = torch.zeros(len(seqs) + 1, dtype=torch.int64)
+    cu[1:] = torch.cumsum(torch.tensor([p + r for p, r in seqs]), 0)
+    resp = torch.tensor([r for _, r in seqs], dtype=torch.int64)
+    g = torch.Generator(device=dev).manual_seed(3001)
+    ids = torch.randint(0, w.V, (n,), generator=g, device=dev, dtype=torch.int64)
+    logits = synthetic.make_logits(n, w.V, w.dtype, w.sigma, torch.roll(ids, -1), dev, 3003, boost=w.boost,
+                                   boost_frac=w.boost_frac)
+    B, T = len(seqs), w.T
+    cu_d, resp_d = cu.to(dev), resp.to(dev)
+    r_lp = torch.empty((B, T), dtype=torch.float32, device=dev)
+    r_h = torch.empty_like(r_lp)
+    flag = torch.zeros(1, dtype=torch.int32, device=dev)
+    lib = _lib.load()
+    stream = torch.cuda.current_stream(dev).cuda_stream
+
+    def run():
+        st = lib.vrl_score_responses(logits.data_ptr(), _lib.VRL_BF16, n, w.V, logits.stride(0), None, ids.data_ptr(),
+                                     None, cu_d.data_ptr(), resp_d.data_ptr(), B, T, None, None, r_lp.data_ptr(),
+                                     r_h.data_ptr(), flag.data_ptr(), stream)
+        _lib.check("vrl_score_responses", st)
+
+    run()
+    # guard: equal to the separate entry points
+    lp, h = vf.fused_logprob_entropy(logits, torch.roll(ids, -1))
+    from verl_amd import layout
+    if not (torch.equal(r_lp, layout.response_slice(lp, cu_d, resp_d, T)) and torch.equal(r_h, layout.response_slice(h, cu_d, resp_d, T))):
+        raise SystemExit("bench: vrl_score_responses disagrees with vrl_rowscore + vrl_response_slice")
+    if int(flag.item()) != 0:
+        raise SystemExit("bench: vrl_score_responses set an error flag")
+    spin_up(run)
+    for _ in range(warmup):
+        run()
+    torch.cuda.synchronize()
+    evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(steps)]
+    t0 = time.perf_counter()
+    for a, b in evs:
+        a.record()
+        run()
+        b.record()
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    avg_ms = sum(a.elapsed_time(b) for a, b in evs) / len(evs)
+    n_resp = int(resp.sum())
+    bytes_launch = n_resp * (w.V * 2 + 8 + 4 + 4) + (B + 1) * 8 + B * 8 + B * T * 8 - n_resp * 8
+    achieved = bytes_launch / (avg_ms * 1e-3) / 1e9
+    return {
+        "metric": "response tokens/sec from packed logits to padded (B, T) log-probs and entropies, one launch",
+        "value": n_resp * steps / wall, "unit": "tokens/s", "ms_per_step": wall * 1e3 / steps, "dtype": "bf16",
+        "config": {"workload": "c3_grpo_packed_prompt_plus_response_v151936_bf16", "rows_per_step": n,
+                   "response_rows_per_step": n_resp, "sequences": B, "padded_response_len": T,
+                   "step": "vrl_score_responses through the C ABI (labels rolled in-kernel, prompt rows not read)"},
+        "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                     "frac": achieved / HBM_PEAK_GBPS, "traffic": None, "kernel": "score_responses_kernel",
+                     "avg_kernel_ms": avg_ms, "algorithmic_bytes_per_launch": bytes_launch},
+        "all_rows_equivalent_tokens_per_s": n * steps / wall,
+    }
+
+
+def compact(rec: dict) -> dict:
+    """The fields of a workload record that the headline line carries for every other workload."""
+    keep = ("value", "unit", "ms_per_step", "dtype", "hbm_gbps_fused_step", "parity_guard")
+    out = {"workload": rec["config"]["workload"], "step": rec["config"]["step"]}
+    out.update({k: rec[k] for k in keep if k in rec})
+    r = rec["roofline"]
+    out["roofline"] = {k: r[k] for k in ("bound", "achieved", "peak", "unit", "frac", "traffic", "kernel", "avg_kernel_ms",
+                                         "algorithmic_bytes_per_launch") if k in r}
+    return out
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--workload", default=None, choices=["c1", "c2", "c3", "c4", "c5"],
+                    help="time this workload only (c5 times the verify kernel alone: its logits do not fit, they are "
+                         "scored like c3). Default: c2 as the headline plus a short record of every other workload")
+    ap.add_argument("--vocab", type=int, default=0, help="run the workload's recipe at another vocabulary size")
+    ap.add_argument("--seqs", type=int, default=0, help="... with another number of sequences")
+    ap.add_argument("--dtype", choices=["bf16", "f32"], default=None, help="... with another logits element type")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--backward", action="store_true",
+                    help="time vrl_rowscore_backward on the workload instead of the fused forward step")
+    ap.add_argument("--score-responses", action="store_true",
+                    help="time vrl_score_responses (packed logits -> padded response blocks, one launch) on c3")
+    ap.add_argument("--lm-head", action="store_true",
+                    help="time the LM head + scoring step (verl_amd.fused_linear) instead of the fused forward step")
+    ap.add_argument("--chunk", type=int, default=4096, help="--lm-head: tokens projected at a time")
+    ap.add_argument("--keep-logits", action="store_true", help="--lm-head: keep the logits for the backward")
+    ap.add_argument("--ceilings", action="store_true",
+                    help="time plain non-temporal read / copy probes with the row kernels' access pattern")
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="also run a plain device copy of known size (for scaling rocprofv3 byte counters)")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build runs on one GPU only; "
+              f"--gpus {args.gpus} is not supported", file=sys.stderr)
+        sys.exit(2)
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible; the HIP path has no CPU fallback", file=sys.stderr)
+        sys.exit(2)
+
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    if args.lm_head:
+        bench_lm_head(args, dev)
+        return
+    if args.ceilings:
+        bench_ceilings(args, dev)
+        return
+    if args.score_responses:
+        print(json.dumps(bench_score_responses(args, dev, args.steps, args.warmup)), flush=True)
+        return
+    if args.backward:
+        args.workload = args.workload or "c2"
+        print(json.dumps(bench_backward(args, dev)), flush=True)
+        return
+    if args.workload == "c5":
+        print(json.dumps(bench_verify_only(args, dev, not args.no_cpu_baseline)), flush=True)
+        return
+    if args.workload is not None or args.vocab or args.seqs or args.dtype:
+        rec = bench_forward(args, dev, args.workload or "c2", args.steps, args.warmup, not args.no_cpu_baseline)
+        print(json.dumps(rec), flush=True)
+        return
+
+    # Default: the headline workload (c2, the configuration the metric is quoted on) in full, then every other
+    # workload with fewer steps and without a CPU leg, as short records under "workloads".
+    out = bench_forward(args, dev, "c2", args.steps, args.warmup, not args.no_cpu_baseline)
+    few = argparse.Namespace(**vars(args))
+    few.steps, few.warmup = min(args.steps, 10), min(args.warmup, 3)
+    others = []
+    for name in ("c3", "c4", "c1"):
+        torch.cuda.empty_cache()
+        others.append(compact(bench_forward(few, dev, name, few.steps, few.warmup, False)))
+    torch.cuda.empty_cache()
+    others.append(compact(bench_verify_only(few, dev, False)))
+    torch.cuda.empty_cache()
+    others.append(compact(bench_backward(few, dev, "c3")))
+    torch.cuda.empty_cache()
+    others.append(compact(bench_score_responses(few, dev, few.steps, few.warmup)))
+    out["workloads"] = others
     print(json.dumps(out), flush=True)
 
 

@@ -335,6 +335,17 @@ int vrl_fused_score_verify(const void* logits, int dtype, int64_t n_rows, int64_
                            int32_t* prefix_len, int32_t* near_count, const int64_t* draft_ids,
                            int64_t pad_id, int64_t* out_ids, uint8_t* out_mask, void* stream);
 
+/*
+ * vrl_stream_probe — what the memory system delivers for the row kernels' access pattern with no arithmetic in the
+ * way: the ceilings the kernels above are measured against. One workgroup per "row" of row_bytes (a multiple of 16)
+ * streams it with non-temporal 128-bit accesses exactly as vrl_rowscore's kernel does.
+ *   mode 0: read only (the data is XOR-folded; *sink is written only if the fold equals a constant)  -> forward ceiling
+ *   mode 1: read src, write dst (n_rows * row_bytes each, not overlapping)                           -> backward ceiling
+ * A measurement aid with no counterpart in the reference.
+ */
+int vrl_stream_probe(const void* src, void* dst, int64_t n_rows, int64_t row_bytes, int mode, uint32_t* sink,
+                     void* stream);
+
 /* Text for a VRL_* status code; never NULL. */
 const char* vrl_strerror(int status);
 

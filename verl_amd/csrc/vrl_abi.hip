@@ -12,6 +12,7 @@
 #include "backward_kernels.h"
 #include "layout_kernels.h"
 #include "lmhead_kernels.h"
+#include "probe_kernels.h"
 #include "rollout_corr_kernels.h"
 #include "rowscore_kernels.h"
 #include "transpose_kernels.h"
@@ -663,6 +664,27 @@ int vrl_fused_score_verify(const void* logits, int dtype, int64_t n_rows, int64_
   return vrl_spec_verify(out_logprob, logp_old, log_u, mask, cu_seqlens, B, T, n_rows, thresh_offset, near_eps,
                          accept, first_reject, prefix_len, near_count, draft_ids, pad_id, out_ids,
                          out_mask, err_flag, stream);
+}
+
+int vrl_stream_probe(const void* src, void* dst, int64_t n_rows, int64_t row_bytes, int mode, uint32_t* sink,
+                     void* stream) {
+  if (mode != 0 && mode != 1) return VRL_ERR_ARG;
+  if (n_rows < 0 || row_bytes < 0 || row_bytes % 16 != 0 || n_rows > kMaxGrid) return VRL_ERR_SHAPE;
+  if (n_rows == 0 || row_bytes == 0) return VRL_OK;
+  if (src == nullptr || (mode == 1 && dst == nullptr) || (mode == 0 && sink == nullptr)) return VRL_ERR_NULL;
+  if (!aligned(src, 16) || !aligned(dst, 16) || !aligned(sink, 4)) return VRL_ERR_ALIGN;
+  const dim3 grid(static_cast<unsigned>(n_rows));
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const int64_t vecs = row_bytes / 16;
+  // the forward / backward row kernels' workgroup shapes for 16-bit logits
+  if (mode == 0)
+    vrl::stream_probe_kernel<RowShape<VRL_BF16>::kWaves, RowShape<VRL_BF16>::kUnroll, false>
+        <<<grid, dim3(RowShape<VRL_BF16>::kWaves * 64), 0, s>>>(static_cast<const vrl::u32x4*>(src), nullptr, vecs,
+                                                                0x9e3779b9u, sink);
+  else
+    vrl::stream_probe_kernel<kBackwardWaves, kBackwardUnroll, true><<<grid, dim3(kBackwardWaves * 64), 0, s>>>(
+        static_cast<const vrl::u32x4*>(src), static_cast<vrl::u32x4*>(dst), vecs, 0u, nullptr);
+  return launch_status();
 }
 
 const char* vrl_strerror(int status) {
