@@ -410,9 +410,14 @@ def bench_lm_head(args, dev):
         return lm_head_score_mfma(hidden.detach(), weight.detach(), ids, temperature)
 
     lp_m, h_m = fwd_mfma()
-    e3 = (lp_m[:256] - torch.log_softmax(z, -1).gather(-1, ids[:256, None]).squeeze(-1)).abs().max().item()
-    if not e3 <= 3e-2:   # z holds bf16-rounded logits, the kernel keeps them in fp32
-        raise SystemExit(f"bench: matrix-core LM-head scores disagree with torch ({e3})")
+    # guard: 8 tokens out of every 256-token block (every workgroup's tile) against the fp32 composition
+    pick = (torch.arange(0, T, 256, device=dev)[:, None] + torch.tensor([0, 37, 64, 101, 128, 190, 222, 255], device=dev)).reshape(-1)
+    zz = (hidden.detach()[pick].float() @ weight.detach().float().t()) / temperature
+    e3 = (lp_m[pick] - torch.log_softmax(zz, -1).gather(-1, ids[pick, None]).squeeze(-1)).abs().max().item()
+    e4 = (h_m[pick] - (torch.logsumexp(zz, -1) - (torch.softmax(zz, -1) * zz).sum(-1))).abs().max().item()
+    del zz
+    if not (e3 <= 1e-4 and e4 <= 1e-4):   # fp32 sums of exact products on both sides; only the order differs
+        raise SystemExit(f"bench: matrix-core LM-head scores disagree with torch (log-prob {e3}, entropy {e4})")
     t_f = timed(fwd)
     t_fb = timed(fwd_bwd)
     t_m = timed(fwd_mfma)
@@ -435,7 +440,8 @@ def bench_lm_head(args, dev):
                      "forward_tflops": flops_f / t_f / 1e12},
         "single_kernel_forward": {"ms": t_m * 1e3, "tflops": flops_f / t_m / 1e12, "frac_of_mfma_peak": flops_f / t_m / 1e12 / 2500.0,
                                   "kernel": "lmhead_partial_kernel<bf16> + lmhead_finish_kernel (vrl_lmhead_score)",
-                                  "note": "hand-written MFMA kernel, logits never written; slower than the library GEMM path above"},
+                                  "parity_guard": {"rows": int(pick.numel()), "max_abs_err_logprob": e3, "max_abs_err_entropy": e4},
+                                  "note": "hand-written MFMA kernel, logits never written"},
         "weight_transpose": {"ms": t_tr * 1e3, "gbps": 2.0 * V * D * 2 / t_tr / 1e9, "kernel": "transpose_kernel<2>"},
         "parity_guard": {"rows": 256, "max_abs_err_logprob": e1, "max_abs_err_entropy": e2},
     }), flush=True)

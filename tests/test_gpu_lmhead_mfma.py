@@ -41,6 +41,41 @@ def test_matches_fp64_composition(dev, dtype, T, V, K, splits):
         assert (ent.double() - r_ent).abs().max().item() <= 2e-5
 
 
+def test_xcd_aware_workgroup_order_covers_every_token_block_and_split(dev):
+    """32 token blocks x 8 splits takes the XCD-aware (token block, split) mapping of the workgroups (it needs the
+    block count to divide by 8 and the split count by 4): every token of every block must come out right, which a
+    wrong mapping (a block or split served twice, another never) would not."""
+    T, V, K, splits = 8192, 8192, 256, 8
+    g = torch.Generator(device=dev).manual_seed(99)
+    h = (torch.randn(T, K, generator=g, device=dev) * 0.5).bfloat16()
+    w = (torch.randn(V, K, generator=g, device=dev) * 0.2).bfloat16()
+    ids = torch.randint(0, V, (T,), generator=g, device=dev)
+    temp = torch.rand(T, generator=g, device=dev) + 0.5
+    lp, ent = lm_head_score_mfma(h, w, ids, temp, n_splits=splits)
+    r_lp, r_ent = _reference(h, w, ids, temp)
+    assert (lp.double() - r_lp).abs().max().item() <= 2e-5
+    assert (ent.double() - r_ent).abs().max().item() <= 2e-5
+
+
+def test_benchmark_shape_against_the_chunked_fp64_composition(dev):
+    """8192 tokens x 3584 -> 152064 bf16 (the shape bench.py --lm-head times; 594 vocabulary tiles over 8 splits,
+    the last split shorter, XCD-aware order): all tokens against the fp64 composition, formed 256 tokens at a time."""
+    T, K, V = 8192, 3584, 152064
+    g = torch.Generator(device=dev).manual_seed(4000)
+    h = torch.empty(T, K, device=dev).uniform_(-0.5, 0.5, generator=g).bfloat16()
+    w = (torch.empty(V, K, device=dev).uniform_(-0.5, 0.5, generator=g) * 0.05).bfloat16()
+    ids = torch.randint(0, V, (T,), generator=g, device=dev)
+    lp, ent = lm_head_score_mfma(h, w, ids, 1.5)
+    w64 = w.double()
+    worst_lp = worst_ent = 0.0
+    for lo in range(0, T, 256):
+        r_lp, r_ent = _reference(h[lo:lo + 256], w64, ids[lo:lo + 256], 1.5)
+        worst_lp = max(worst_lp, (lp[lo:lo + 256].double() - r_lp).abs().max().item())
+        worst_ent = max(worst_ent, (ent[lo:lo + 256].double() - r_ent).abs().max().item())
+    print(f"[lmhead 8192x3584->152064] max abs err vs fp64: log-prob {worst_lp:.2e}, entropy {worst_ent:.2e}", flush=True)
+    assert worst_lp <= 2e-5 and worst_ent <= 2e-5
+
+
 def test_close_to_the_library_path_and_3d_inputs(dev):
     g = torch.Generator(device=dev).manual_seed(4)
     B, S, K, V = 2, 260, 256, 5003

@@ -1,12 +1,15 @@
 // LM head fused with the row reduction: logits[tok][v] = sum_k H[tok][k] * W[v][k] are formed on the matrix cores
 // and folded straight into the online-softmax partial (m, s, t) of their token; they never reach HBM.
 //
-// lmhead_partial_kernel: one workgroup (4 wavefronts) owns 256 tokens and walks a range of 256-row vocabulary
-// tiles (its "split"); per tile it runs the full contraction in steps of 64 (v_mfma_f32_32x32x16 on bf16 / fp16,
-// fp32 accumulators: 16 blocks of 32x32 per wavefront = 256 accumulator registers), then folds the 256 x 256
-// accumulators into per-lane running (m, s, t) states (a lane sees 4 token columns). Operands go global -> LDS
-// directly (128-bit loads, two 64 KiB stages = 128 KiB of LDS, one workgroup per CU), swizzled so that the
-// 128-bit fragment reads are free of bank conflicts (measured: SQ_LDS_BANK_CONFLICT = 0).
+// lmhead_partial_kernel: one workgroup of 8 wavefronts (two per SIMD) owns 256 tokens and walks a range of 256-row
+// vocabulary tiles (its "split"); per tile it runs the full contraction in steps of 64 (v_mfma_f32_32x32x16 on
+// bf16 / fp16, fp32 accumulators). A wavefront owns a 64 (vocabulary) x 128 (tokens) part of the tile: 8 blocks of
+// 32x32 = 128 accumulator registers, so two wavefronts fit a SIMD and one's matrix instructions cover the other's
+// waits. Operands go global -> LDS directly (128-bit loads, two 64 KiB stages = 128 KiB of LDS, one workgroup per CU),
+// swizzled so that the 128-bit fragment reads are free of bank conflicts (measured: SQ_LDS_BANK_CONFLICT = 0).
+// A step is four quarter steps of 16 contraction elements. The workgroup barrier sits before the LAST quarter's matrix
+// instructions: that quarter's fragments are already in registers, so behind the barrier the first fragments of the
+// next step are fetched and the loads of the step after are issued while the matrix cores still work on this step.
 // The MFMA is issued with the vocabulary on its row side so that a lane's 16 results of a block belong to ONE
 // token: the softmax state needs no cross-lane traffic until the very end.
 //
@@ -53,36 +56,39 @@ struct LmFrag<2> {
   }
 };
 
+constexpr int kLmWaves = 8;                       // wavefronts per workgroup: 4 vocabulary quarters x 2 token halves
+
 // One wave instruction moves 8 tile rows x 128 bytes into LDS (lane l lands at byte l*16 of the 1 KiB block):
 // lane l serves row r = l>>3 of the block and physical 16-byte slot p = l&7, and fetches the logical chunk that the
 // swizzle assigns to that slot (two lane offsets: blocks of 8 rows alternate in the swizzle's row bits).
+// Wavefront w brings tile rows [32w, 32w + 32) with four such instructions.
 // tile: uniform pointer to (first row of the tile, k step); row_block_bytes: 8 rows in bytes (uniform).
 __device__ __forceinline__ void load_tile(const char* __restrict__ tile, uint32_t lane_off_even, uint32_t lane_off_odd,
                                           int64_t row_block_bytes, char* lds_tile, int wave) {
 #pragma unroll
-  for (int i = 0; i < 8; ++i) {
+  for (int i = 0; i < 4; ++i) {
     // scalar base + 32-bit lane offset: tell the compiler the base is uniform so the address stays in SGPRs
-    const uint64_t u = reinterpret_cast<uint64_t>(tile + (wave * 8 + i) * row_block_bytes);
+    const uint64_t u = reinterpret_cast<uint64_t>(tile + (wave * 4 + i) * row_block_bytes);
     const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)u);
     const uint32_t hi = __builtin_amdgcn_readfirstlane((uint32_t)(u >> 32));
     const char* src = reinterpret_cast<const char*>(((uint64_t)hi << 32) | lo);
-    char* dst = lds_tile + (wave * 64 + i * 8) * kLmRowBytes;      // uniform
+    char* dst = lds_tile + (wave * 32 + i * 8) * kLmRowBytes;      // uniform
     __builtin_amdgcn_global_load_lds((const VRL_GLOBAL_AS void*)(src + ((i & 1) ? lane_off_odd : lane_off_even)), (VRL_LDS_AS void*)dst, 16, 0, 0);
   }
 }
 
 template <int DT>
-__global__ __launch_bounds__(256, 1) void lmhead_partial_kernel(
+__global__ __launch_bounds__(kLmWaves * 64, 1) void lmhead_partial_kernel(
     const uint16_t* __restrict__ W, const uint16_t* __restrict__ H, int64_t V, int64_t T, int64_t K, int64_t w_stride,
     int64_t h_stride, const float* __restrict__ temperature, int n_splits, int tiles_per_split,
     int xcd_map, float* __restrict__ partials) {
   extern __shared__ __attribute__((aligned(1024))) char lds[];  // [2 buffers][W tile, H tile]
-  __shared__ float red[2][256][3];
+  __shared__ float red[4][256][3];
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);   // uniform: keeps tile addressing in scalar registers
-  const int wv = wave >> 1;  // vocab half of the tile
+  const int wv = wave >> 1;  // vocab quarter of the tile (8 wavefronts: 4 vocab quarters x 2 token halves)
   const int wt = wave & 1;   // token half of the tile
   // Workgroup -> (token block, split). Hardware deals workgroups round-robin over the 8 XCDs (id % 8); the 32 that
   // are resident on one XCD together should share operands through its L2: 8 token blocks x 4 splits per XCD
@@ -130,7 +136,7 @@ __global__ __launch_bounds__(256, 1) void lmhead_partial_kernel(
   int phys[4];
 #pragma unroll
   for (int sb = 0; sb < 4; ++sb) phys[sb] = (((2 * sb + (lane >> 5)) ^ ((lane >> 1) & 7)) * 16);
-  const int fragoff_w = (wv * 128 + (lane & 31)) * kLmRowBytes;
+  const int fragoff_w = (wv * 64 + (lane & 31)) * kLmRowBytes;
   const int fragoff_h = kLmTileBytes + (wt * 128 + (lane & 31)) * kLmRowBytes;
 
   // Edge tiles are moved back so that all 256 rows exist (host guarantees V, T >= 256); the rows they share with
@@ -146,40 +152,45 @@ __global__ __launch_bounds__(256, 1) void lmhead_partial_kernel(
   const char* Wb = reinterpret_cast<const char*>(W);
   const char* Hb = reinterpret_cast<const char*>(H) + tok0_ld * h_stride * 2;
 
-  // prefetch cursor: global step (tile, k step), one step ahead of the compute cursor
+  // prefetch cursor: global step (tile, k step), two steps ahead of the compute cursor once the loop runs
   const int64_t total_steps = (vt_end > vt_begin ? (vt_end - vt_begin) : 0) * ksteps;
   int64_t pstep = 0, pvt = vt_begin;
   int pks = 0;
-  auto issue = [&]() {   // loads of global step `pstep` into buffer pstep & 1
+  // Loads of global step `pstep` into stage pstep & 1. Branch-free: past the last step the cursor stays on the last
+  // step, whose tile is loaded once more into the stage nobody will read (in bounds, harmless), so the main loop is
+  // one basic block.
+  auto issue_always = [&]() {
     char* st = lds + (int)(pstep & 1) * 2 * kLmTileBytes;
     const int64_t vrow = (pvt + 1) * kLmVocab <= V ? pvt * kLmVocab : V - kLmVocab;
     load_tile(Wb + vrow * w_stride * 2 + (int64_t)pks * kLmRowBytes, w_lane_e, w_lane_o, w_blk, st, wave);
     load_tile(Hb + (int64_t)pks * kLmRowBytes, h_lane_e, h_lane_o, h_blk, st + kLmTileBytes, wave);
+    const bool more = pstep + 1 < total_steps;
     ++pstep;
-    if (++pks == ksteps) {
-      pks = 0;
-      ++pvt;
-    }
+    const int nks = pks + 1;
+    const bool wrap = nks == ksteps;
+    pks = more ? (wrap ? 0 : nks) : pks;
+    pvt = more ? (wrap ? pvt + 1 : pvt) : pvt;
   };
-  typename LmFrag<DT>::type a[2][4], b[2][4];
+  typename LmFrag<DT>::type a[2][2], b[2][4];
   auto read_frags = [&](int set, const char* stage, int sb) {
 #pragma unroll
-    for (int i = 0; i < 4; ++i) a[set][i] = *reinterpret_cast<const typename LmFrag<DT>::type*>(stage + fragoff_w + i * 32 * kLmRowBytes + phys[sb]);
+    for (int i = 0; i < 2; ++i) a[set][i] = *reinterpret_cast<const typename LmFrag<DT>::type*>(stage + fragoff_w + i * 32 * kLmRowBytes + phys[sb]);
 #pragma unroll
     for (int j = 0; j < 4; ++j) b[set][j] = *reinterpret_cast<const typename LmFrag<DT>::type*>(stage + fragoff_h + j * 32 * kLmRowBytes + phys[sb]);
   };
   if (total_steps > 0) {
-    issue();
+    issue_always();   // step 0 -> stage 0
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
     read_frags(0, lds, 0);
+    issue_always();   // step 1 -> stage 1
   }
 
   int64_t step = 0;
   for (int64_t vt = vt_begin; vt < vt_end; ++vt) {
-    lm_f32x16 acc[4][4];
+    lm_f32x16 acc[2][4];
 #pragma unroll
-    for (int i = 0; i < 4; ++i)
+    for (int i = 0; i < 2; ++i)
 #pragma unroll
       for (int j = 0; j < 4; ++j)
 #pragma unroll
@@ -188,33 +199,42 @@ __global__ __launch_bounds__(256, 1) void lmhead_partial_kernel(
     for (int ks = 0; ks < ksteps; ++ks, ++step) {
       const char* cur = lds + (int)(step & 1) * 2 * kLmTileBytes;
       const char* nxt = lds + (int)((step + 1) & 1) * 2 * kLmTileBytes;
-      // the other buffer was last read before the barrier of the previous step
-      if (pstep < total_steps) issue();
+      // Quarter steps 0..2 compute from fragments and read the next quarter's fragments from `cur`.
 #pragma unroll
-      for (int sb = 0; sb < 4; ++sb) {
+      for (int sb = 0; sb < 3; ++sb) {
         const int cu = sb & 1, nx = cu ^ 1;
-        if (sb < 3) read_frags(nx, cur, sb + 1);
+        read_frags(nx, cur, sb + 1);
 #pragma unroll
-        for (int i = 0; i < 4; ++i)
+        for (int i = 0; i < 2; ++i)
 #pragma unroll
           for (int j = 0; j < 4; ++j)
             acc[i][j] = LmFrag<DT>::mfma(a[cu][i], b[cu][j], acc[i][j]);
       }
-      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+      // The barrier sits BEFORE the last quarter's matrix instructions: its fragments (set 1) are in registers, so
+      // every wavefront is done reading `cur`, and the next step's tile, requested a whole step ago, has landed in
+      // `nxt`. Behind the barrier the next step's first fragments are fetched and the loads of the step after are
+      // issued into `cur`, all underneath this quarter's matrix instructions.
+      asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
       __syncthreads();
-      if (step + 1 < total_steps) read_frags(0, nxt, 0);
+      read_frags(0, nxt, 0);
+      issue_always();
+#pragma unroll
+      for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+          acc[i][j] = LmFrag<DT>::mfma(a[1][i], b[1][j], acc[i][j]);
     }
 
     // epilogue of this vocab tile: fold 64 logits per token column into the running state (two passes over the
     // accumulators: maximum, then exponentials; nothing is buffered)
     const bool edge = (vt + 1) * kLmVocab > V;
-    const int64_t vrow0 = (edge ? V - kLmVocab : vt * kLmVocab) + wv * 128 + 4 * (lane >> 5);
+    const int64_t vrow0 = (edge ? V - kLmVocab : vt * kLmVocab) + wv * 64 + 4 * (lane >> 5);
     const int64_t vfirst = vt * kLmVocab;   // rows below belong to the tile before
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
       float bm = neg_inf();
 #pragma unroll
-      for (int i = 0; i < 4; ++i) {
+      for (int i = 0; i < 2; ++i) {
         // one 32x32 block (16 accumulator registers) at a time; the scheduling barrier keeps the compiler from
         // pulling the next blocks' accumulator copies forward, which would spill registers across the main loop
         float x[16];
@@ -242,7 +262,7 @@ __global__ __launch_bounds__(256, 1) void lmhead_partial_kernel(
       const float sub = (m[j] == neg_inf()) ? 0.f : m[j];
       float ps = 0.f, pt = 0.f;
 #pragma unroll
-      for (int i = 0; i < 4; ++i) {
+      for (int i = 0; i < 2; ++i) {
         float x[16];
 #pragma unroll
         for (int v = 0; v < 16; ++v) x[v] = acc[i][j][v];
@@ -267,6 +287,7 @@ __global__ __launch_bounds__(256, 1) void lmhead_partial_kernel(
     }
   }
 
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // the last, redundant loads still target the LDS stages
   // combine: lanes l and l^32 hold the same tokens (other vocab rows), then the two vocab-half waves via LDS
 #pragma unroll
   for (int j = 0; j < 4; ++j) {
@@ -290,19 +311,23 @@ __global__ __launch_bounds__(256, 1) void lmhead_partial_kernel(
     }
   }
   __syncthreads();
-  {
-    const int col = tid;  // 256 threads, 256 token columns
+  if (tid < 256) {
+    const int col = tid;  // 256 token columns
     const int64_t tok = tok0_ld + col;
     if (tok >= tok0) {
-      const float m0 = red[0][col][0], m1 = red[1][col][0];
-      const float M = __builtin_fmaxf(m0, m1);
+      float M = red[0][col][0];
+#pragma unroll
+      for (int q = 1; q < 4; ++q) M = __builtin_fmaxf(M, red[q][col][0]);
       float S = 0.f, Tt = 0.f;
       if (M != neg_inf()) {
-        const float a1 = hw_exp2(m0 - M), a2 = hw_exp2(m1 - M);
-        const float d1 = (m0 == neg_inf()) ? 0.f : m0 - M;
-        const float d2 = (m1 == neg_inf()) ? 0.f : m1 - M;
-        S = a1 * red[0][col][1] + a2 * red[1][col][1];
-        Tt = a1 * (red[0][col][2] + d1 * red[0][col][1]) + a2 * (red[1][col][2] + d2 * red[1][col][1]);
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          const float mq = red[q][col][0];
+          const float aq = hw_exp2(mq - M);
+          const float dq = (mq == neg_inf()) ? 0.f : mq - M;
+          S += aq * red[q][col][1];
+          Tt += aq * (red[q][col][2] + dq * red[q][col][1]);
+        }
       }
       float* p = partials + (tok * n_splits + split) * 4;
       p[0] = M;

@@ -280,7 +280,7 @@ int launch_lmhead(const void* hidden, const void* weight, int64_t T, int64_t V, 
       raised[dev].store(true, std::memory_order_release);
     }
   }
-  vrl::lmhead_partial_kernel<DT><<<dim3(static_cast<unsigned>(tblocks * n_splits)), dim3(256), vrl::kLmLdsBytes, s>>>(
+  vrl::lmhead_partial_kernel<DT><<<dim3(static_cast<unsigned>(tblocks * n_splits)), dim3(vrl::kLmWaves * 64), vrl::kLmLdsBytes, s>>>(
       static_cast<const uint16_t*>(weight), static_cast<const uint16_t*>(hidden), V, T, K, w_stride, h_stride,
       temperature, n_splits, tiles_per_split, xcd_map, partials);
   vrl::lmhead_finish_kernel<DT><<<dim3(static_cast<unsigned>((T + 3) / 4)), dim3(256), 0, s>>>(
