@@ -418,9 +418,21 @@ def bench_lm_head(args, dev):
     del zz
     if not (e3 <= 1e-4 and e4 <= 1e-4):   # fp32 sums of exact products on both sides; only the order differs
         raise SystemExit(f"bench: matrix-core LM-head scores disagree with torch (log-prob {e3}, entropy {e4})")
+    def fwd_bwd_mfma():
+        lp, h = fused_linear_for_ppo(hidden, weight, ids, temperature, chunk, False, "mfma")
+        return torch.autograd.grad((lp, h), (hidden, weight), (g_lp, g_h))
+
+    # guard: the matrix-core backward against the library one
+    ga, gb = fwd_bwd(), fwd_bwd_mfma()
+    for x, y, what in ((ga[0], gb[0], "d hidden"), (ga[1], gb[1], "d weight")):
+        err = (x.float() - y.float()).abs().max().item()
+        if not err <= 3e-2 * max(x.float().abs().max().item(), 1e-6):
+            raise SystemExit(f"bench: matrix-core backward disagrees with the library path on {what} ({err})")
+    del ga, gb
     t_f = timed(fwd)
     t_fb = timed(fwd_bwd)
     t_m = timed(fwd_mfma)
+    t_fb_m = timed(fwd_bwd_mfma)
     wt = torch.empty(D, V, dtype=weight.dtype, device=dev)
     t_tr = timed(lambda: transpose_2d(weight.detach(), wt))
     flops_f, flops_fb = 2.0 * T * D * V, 6.0 * T * D * V
@@ -442,6 +454,11 @@ def bench_lm_head(args, dev):
                                   "kernel": "lmhead_partial_kernel<bf16> + lmhead_finish_kernel (vrl_lmhead_score)",
                                   "parity_guard": {"rows": int(pick.numel()), "max_abs_err_logprob": e3, "max_abs_err_entropy": e4},
                                   "note": "hand-written MFMA kernel, logits never written"},
+        "matrix_core_backward": {"forward_backward_ms": t_fb_m * 1e3,
+                                 "kernel": "library GEMM forward, lmhead_dlogits_kernel<bf16> (vrl_lmhead_dlogits) + two library "
+                                           "GEMMs backward",
+                                 "note": "the logits are formed again by the hand-written MFMA kernel and their gradient "
+                                         "is written from registers (no GEMM into the buffer, no pass over it)"},
         "weight_transpose": {"ms": t_tr * 1e3, "gbps": 2.0 * V * D * 2 / t_tr / 1e9, "kernel": "transpose_kernel<2>"},
         "parity_guard": {"rows": 256, "max_abs_err_logprob": e1, "max_abs_err_entropy": e2},
     }), flush=True)

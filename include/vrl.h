@@ -243,6 +243,27 @@ int vrl_lmhead_score(const void* hidden, const void* weight, int dtype, int64_t 
                      int64_t hidden_size, int64_t h_stride, int64_t w_stride, const int64_t* labels,
                      const float* temperature, int n_splits, float* partials, float* out_logprob,
                      float* out_entropy, float* out_lse, int32_t* err_flag, void* stream);
+/*
+ * vrl_lmhead_dlogits — backward counterpart of vrl_lmhead_score: the logits are formed again on the matrix cores,
+ * tile by tile, and turned in registers into the gradient with respect to the logits,
+ *   dlogits[t, v] = ( g_logprob[t] * (1[v == label[t]] - p)  -  g_entropy[t] * p * (log p + entropy[t]) ) / T[t],
+ *   p = exp(z[t, v] - lse[t]),  z as in vrl_lmhead_score
+ * (the arithmetic of vrl_rowscore_backward on fp32 logits that were never rounded to the operand type), which is
+ * written in the operands' type to dlogits[t * d_stride + v], t < n_tokens, v < vocab. The caller forms
+ *   d hidden = dlogits @ weight,   d weight = dlogits^T @ hidden
+ * with its GEMM of choice, as the reference does (torch.matmul at verl/utils/kernel/kernels.py:1710-1720).
+ * lse and entropy are vrl_lmhead_score's outputs. g_logprob or g_entropy may be NULL (that term is then absent;
+ * labels / entropy may be NULL with it). Same shape rules as vrl_lmhead_score, plus vocab and d_stride multiples
+ * of 8 and a 16-byte aligned dlogits. n_splits as from vrl_lmhead_plan. No scratch.
+ *
+ * Replaces the reference's default backward kernel of the fused linear + cross-entropy op:
+ *   verl/utils/kernel/kernels.py:1229-1387 (efficient_entropy_backward_kernel_general_d_logits_split_N, Triton)
+ *   and its host loop :1663-1721 (BackwardEnum._Split_Dlogits_N).
+ */
+int vrl_lmhead_dlogits(const void* hidden, const void* weight, int dtype, int64_t n_tokens, int64_t vocab,
+                       int64_t hidden_size, int64_t h_stride, int64_t w_stride, const int64_t* labels,
+                       const float* temperature, const float* lse, const float* entropy, const float* g_logprob,
+                       const float* g_entropy, int n_splits, void* dlogits, int64_t d_stride, void* stream);
 /* Vocabulary splits per 256-token block that fill the part (about one workgroup per CU) for this shape. */
 int vrl_lmhead_plan(int64_t n_tokens, int64_t vocab);
 

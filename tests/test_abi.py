@@ -195,6 +195,32 @@ def test_score_responses_argument_errors(lib):
     assert call(n=0, B=0, x=None, cu=None, rl=None, flag=None) == _lib.VRL_OK
 
 
+def test_lmhead_dlogits_argument_errors(lib):
+    f = lib.vrl_lmhead_dlogits
+    ok = dict(h=P, w=P, dt=_lib.VRL_BF16, T=512, V=1024, K=128, hs=128, ws=128, lab=P, temp=None, lse=P, ent=P, gl=P, gh=P,
+              S=2, out=P, ds=1024)
+
+    def call(**kw):
+        a = {**ok, **kw}
+        return f(a["h"], a["w"], a["dt"], a["T"], a["V"], a["K"], a["hs"], a["ws"], a["lab"], a["temp"], a["lse"], a["ent"],
+                 a["gl"], a["gh"], a["S"], a["out"], a["ds"], None)
+
+    assert call(dt=_lib.VRL_F32) == _lib.VRL_ERR_DTYPE
+    assert call(T=100) == _lib.VRL_ERR_SHAPE
+    assert call(K=96, hs=96, ws=96) == _lib.VRL_ERR_SHAPE
+    assert call(V=1020, ds=1024) == _lib.VRL_ERR_SHAPE            # 8-byte stores need a vocabulary that is a multiple of 8
+    assert call(ds=1016) == _lib.VRL_ERR_SHAPE
+    assert call(ds=1028) == _lib.VRL_ERR_SHAPE
+    assert call(S=0) == _lib.VRL_ERR_SHAPE
+    assert call(gl=None, gh=None) == _lib.VRL_ERR_ARG
+    assert call(lse=None) == _lib.VRL_ERR_NULL
+    assert call(out=None) == _lib.VRL_ERR_NULL
+    assert call(lab=None) == _lib.VRL_ERR_NULL
+    assert call(ent=None) == _lib.VRL_ERR_NULL
+    assert call(out=P + 8) == _lib.VRL_ERR_ALIGN
+    assert call(lse=P + 2) == _lib.VRL_ERR_ALIGN
+
+
 def test_response_pack_argument_errors(lib):
     g = lib.vrl_response_pack      # (values, cu, response_lens, out_offsets, B, n_tokens, out_total, out, err_flag, stream)
     assert g(P, P, P, P, -1, 9, 4, P, P, None) == _lib.VRL_ERR_SHAPE

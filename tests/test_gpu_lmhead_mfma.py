@@ -76,6 +76,94 @@ def test_benchmark_shape_against_the_chunked_fp64_composition(dev):
     assert worst_lp <= 2e-5 and worst_ent <= 2e-5
 
 
+def _dlogits_reference(h, w, ids, temp, g_lp, g_h):
+    """fp64 gradient of sum(g_lp * logprob + g_h * entropy) with respect to the logits, by autograd."""
+    z = (h.double() @ w.double().t()).requires_grad_(True)
+    zt = z if temp is None else z / (temp.double().clamp(min=1e-8)[:, None] if isinstance(temp, torch.Tensor) else float(temp))
+    lse = torch.logsumexp(zt, -1)
+    lp = zt.gather(-1, ids[:, None]).squeeze(-1) - lse
+    ent = lse - (torch.softmax(zt, -1) * zt).sum(-1)
+    loss = 0.0
+    if g_lp is not None:
+        loss = loss + (lp * g_lp.double()).sum()
+    if g_h is not None:
+        loss = loss + (ent * g_h.double()).sum()
+    loss.backward()
+    return z.grad, lse.detach(), ent.detach()
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("T,V,K,splits", [(256, 256, 64, 1), (300, 704, 192, 2), (512, 1024, 256, 3), (1000, 304, 64, 1),
+                                          (257, 18992, 512, None), (2048, 4104, 320, None)])
+def test_dlogits_matches_fp64_autograd(dev, dtype, T, V, K, splits):
+    """vrl_lmhead_dlogits (logits formed again on the matrix cores, gradient written from registers) against the fp64
+    gradient: the result is the fp32 formula rounded once to the operand type (half an ulp of it, 2^-9 relative for
+    bf16, 2^-12 for fp16) plus the fp32 arithmetic's own 1e-6. Edge tiles in both directions, every combination of
+    incoming gradients, per-token temperatures."""
+    lib = _lib.load()
+    g = torch.Generator(device=dev).manual_seed(T * 3 + V + K)
+    h = (torch.randn(T, K, generator=g, device=dev) * 0.5).to(dtype)
+    w = (torch.randn(V, K, generator=g, device=dev) * 0.2).to(dtype)
+    ids = torch.randint(0, V, (T,), generator=g, device=dev)
+    temp = torch.rand(T, generator=g, device=dev) + 0.5
+    g_lp = torch.randn(T, generator=g, device=dev)
+    g_h = torch.randn(T, generator=g, device=dev) * 0.3
+    code = _lib.VRL_BF16 if dtype == torch.bfloat16 else _lib.VRL_F16
+    n_splits = lib.vrl_lmhead_plan(T, V) if splits is None else splits
+    pitch = V + 8     # rows of the output need not be dense
+    for gl, gh, tt in ((g_lp, g_h, temp), (g_lp, None, None), (None, g_h, temp)):
+        want, lse, ent = _dlogits_reference(h, w, ids, tt, gl, gh)
+        lse32, ent32 = lse.float().contiguous(), ent.float().contiguous()
+        out = torch.full((T, pitch), float("nan"), dtype=dtype, device=dev)
+        with torch.cuda.device(dev):
+            st = lib.vrl_lmhead_dlogits(h.data_ptr(), w.data_ptr(), code, T, V, K, K, K, ids.data_ptr(),
+                                        None if tt is None else tt.data_ptr(), lse32.data_ptr(), ent32.data_ptr(),
+                                        None if gl is None else gl.data_ptr(), None if gh is None else gh.data_ptr(),
+                                        n_splits, out.data_ptr(), pitch, _lib.stream_ptr(dev))
+        assert st == _lib.VRL_OK, lib.vrl_strerror(st)
+        got = out[:, :V].double()
+        assert torch.isfinite(got).all()                       # every element of the (T, V) block was written
+        assert torch.isnan(out[:, V:].float()).all()           # and nothing beyond it
+        rel = 2.0 ** -8 if dtype == torch.bfloat16 else 2.0 ** -11
+        err = (got - want).abs()
+        assert bool((err <= rel * want.abs() + 2e-6).all()), err.max().item()
+
+
+def test_fused_linear_with_the_matrix_core_kernels(dev):
+    """fused_linear_for_ppo(kernels="mfma"): forward from vrl_lmhead_score, backward through vrl_lmhead_dlogits and the
+    two products, against torch autograd on the fp32 composition at the reference's tolerances
+    (tests/utils/test_linear_cross_entropy.py:261-276) and against the library-GEMM path."""
+    g = torch.Generator(device=dev).manual_seed(77)
+    T, D, V = 1200, 256, 32256
+    hidden = torch.empty(T, D, device=dev).uniform_(-0.5, 0.5, generator=g).bfloat16().requires_grad_()
+    weight = torch.empty(V, D, device=dev).uniform_(-0.5, 0.5, generator=g).bfloat16().requires_grad_()
+    labels = torch.randint(0, V, (T,), generator=g, device=dev)
+    g_ent = torch.empty(T, device=dev).uniform_(-0.5, 0.5, generator=g)
+    g_lp = torch.empty(T, device=dev).uniform_(-1, 1, generator=g)
+    logits = torch.matmul(hidden.float(), weight.float().t()) / 1.5
+    ref_ent = torch.logsumexp(logits, -1) - (torch.softmax(logits, -1) * logits).sum(-1)
+    ref_lp = -torch.nn.functional.cross_entropy(logits, labels, reduction="none")
+    d_ref_h, d_ref_w = torch.autograd.grad((ref_ent, ref_lp), (hidden, weight), (g_ent, g_lp))
+    for chunk in (512, 4096):
+        lp, ent = fused_linear_for_ppo(hidden, weight, labels, 1.5, chunk_size=chunk, kernels="mfma")
+        torch.testing.assert_close(ref_lp, lp, atol=3e-2, rtol=1e-4)     # the forward with gradients rounds the logits to bf16 (library GEMM)
+        d_h, d_w = torch.autograd.grad((ent, lp), (hidden, weight), (g_ent, g_lp))
+        assert d_h.dtype == torch.bfloat16 and d_w.dtype == torch.bfloat16
+        torch.testing.assert_close(d_ref_h.float(), d_h.float(), atol=1e-2, rtol=1e-2)
+        torch.testing.assert_close(d_ref_w.float(), d_w.float(), atol=1e-2, rtol=1e-2)
+        lp2, ent2 = fused_linear_for_ppo(hidden, weight, labels, 1.5, chunk_size=chunk, kernels="library")
+        d_h2, d_w2 = torch.autograd.grad((ent2, lp2), (hidden, weight), (g_ent, g_lp))
+        assert (d_h.float() - d_h2.float()).abs().max().item() <= 2e-2 * max(d_h2.float().abs().max().item(), 1e-3)
+        assert (d_w.float() - d_w2.float()).abs().max().item() <= 2e-2 * max(d_w2.float().abs().max().item(), 1e-3)
+    # without gradients the same switch takes the single forward kernel: fp32 logits, no buffer
+    with torch.no_grad():
+        lp, ent = fused_linear_for_ppo(hidden, weight, labels, 1.5, kernels="mfma")
+    torch.testing.assert_close(ref_lp, lp, atol=1e-4, rtol=1e-4)
+    torch.testing.assert_close(ref_ent, ent, atol=1e-4, rtol=1e-4)
+    with pytest.raises(ValueError):
+        fused_linear_for_ppo(hidden, weight, labels, 1.5, kernels="cublas")
+
+
 def test_close_to_the_library_path_and_3d_inputs(dev):
     g = torch.Generator(device=dev).manual_seed(4)
     B, S, K, V = 2, 260, 256, 5003

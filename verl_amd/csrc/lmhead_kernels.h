@@ -13,6 +13,11 @@
 // The MFMA is issued with the vocabulary on its row side so that a lane's 16 results of a block belong to ONE
 // token: the softmax state needs no cross-lane traffic until the very end.
 //
+// lmhead_dlogits_kernel: the same walk over (token block, vocabulary tiles) for the backward pass. The logits tile is
+// recomputed on the matrix cores and turned, in registers, into the gradient with respect to the logits
+// (the row-backward arithmetic of backward_kernels.h), which is stored in the operands' type; the two products that
+// follow (d hidden, d W) are plain GEMMs over that buffer.
+//
 // lmhead_finish_kernel: one wavefront per token forms the label's logit as a dot product in fp32, merges the
 // token's partials over the splits and writes log-prob, entropy and logsumexp (same finish as the row kernel).
 //
@@ -22,6 +27,7 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include "backward_kernels.h"
 #include "rowscore_kernels.h"
 
 namespace vrl {
@@ -58,79 +64,64 @@ struct LmFrag<2> {
 
 constexpr int kLmWaves = 8;                       // wavefronts per workgroup: 4 vocabulary quarters x 2 token halves
 
-// One wave instruction moves 8 tile rows x 128 bytes into LDS (lane l lands at byte l*16 of the 1 KiB block):
-// lane l serves row r = l>>3 of the block and physical 16-byte slot p = l&7, and fetches the logical chunk that the
-// swizzle assigns to that slot (two lane offsets: blocks of 8 rows alternate in the swizzle's row bits).
-// Wavefront w brings tile rows [32w, 32w + 32) with four such instructions.
-// tile: uniform pointer to (first row of the tile, k step); row_block_bytes: 8 rows in bytes (uniform).
-__device__ __forceinline__ void load_tile(const char* __restrict__ tile, uint32_t lane_off_even, uint32_t lane_off_odd,
-                                          int64_t row_block_bytes, char* lds_tile, int wave) {
-#pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    // scalar base + 32-bit lane offset: tell the compiler the base is uniform so the address stays in SGPRs
-    const uint64_t u = reinterpret_cast<uint64_t>(tile + (wave * 4 + i) * row_block_bytes);
-    const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)u);
-    const uint32_t hi = __builtin_amdgcn_readfirstlane((uint32_t)(u >> 32));
-    const char* src = reinterpret_cast<const char*>(((uint64_t)hi << 32) | lo);
-    char* dst = lds_tile + (wave * 32 + i * 8) * kLmRowBytes;      // uniform
-    __builtin_amdgcn_global_load_lds((const VRL_GLOBAL_AS void*)(src + ((i & 1) ? lane_off_odd : lane_off_even)), (VRL_LDS_AS void*)dst, 16, 0, 0);
+// Which (token block, vocabulary split) a workgroup serves. Hardware deals workgroups round-robin over the 8 XCDs
+// (id % 8); the 32 that are resident on one XCD together should share operands through its L2: 8 token blocks x 4
+// splits per XCD (each W slice read by 8 workgroups, each H slice by 4) when the grid has that shape (xcd_map), plain
+// order otherwise.
+struct LmWork {
+  int split;
+  int64_t tok0;      // first token of the block
+  int64_t tok0_ld;   // first token of the 256 rows that are loaded (an edge block is moved back so all rows exist)
+  int64_t vt_begin;  // vocabulary tiles [vt_begin, vt_end)
+  int64_t vt_end;
+};
+
+__device__ __forceinline__ LmWork lm_work(int64_t V, int64_t T, int n_splits, int tiles_per_split, int xcd_map) {
+  LmWork w;
+  int64_t tb;
+  const int64_t tblocks = (T + kLmTokens - 1) / kLmTokens;
+  const int64_t id = blockIdx.x;
+  if (xcd_map) {
+    const int x = (int)(id & 7);
+    const int64_t local = id >> 3;            // 0 .. tblocks*n_splits/8
+    const int64_t tgroups = tblocks / 8;      // groups of 8 token blocks
+    // super index over (tgroup, sgroup) pairs: 8 consecutive ones run at a time (one per XCD)
+    const int64_t super = (local / 32) * 8 + x;
+    const int64_t within = local % 32;
+    const int64_t tg = super % tgroups;
+    const int sg = (int)(super / tgroups);
+    tb = tg * 8 + (within & 7);
+    w.split = sg * 4 + (int)(within >> 3);
+  } else {
+    w.split = (int)(id % n_splits);
+    tb = id / n_splits;
   }
+  w.tok0 = tb * kLmTokens;
+  w.tok0_ld = w.tok0 + kLmTokens <= T ? w.tok0 : T - kLmTokens;
+  const int64_t n_vtiles = (V + kLmVocab - 1) / kLmVocab;
+  w.vt_begin = (int64_t)w.split * tiles_per_split;
+  w.vt_end = w.vt_begin + tiles_per_split;
+  if (w.vt_end > n_vtiles) w.vt_end = n_vtiles;
+  return w;
 }
 
-template <int DT>
-__global__ __launch_bounds__(kLmWaves * 64, 1) void lmhead_partial_kernel(
-    const uint16_t* __restrict__ W, const uint16_t* __restrict__ H, int64_t V, int64_t T, int64_t K, int64_t w_stride,
-    int64_t h_stride, const float* __restrict__ temperature, int n_splits, int tiles_per_split,
-    int xcd_map, float* __restrict__ partials) {
-  extern __shared__ __attribute__((aligned(1024))) char lds[];  // [2 buffers][W tile, H tile]
-  __shared__ float red[4][256][3];
-
+// The matrix-core walk shared by the forward and backward kernels. All 512 threads call it. For every vocabulary
+// tile of `work` it forms the 256 x 256 block of logits of tokens [tok0_ld, tok0_ld + 256) and hands this wavefront's
+// 64 (vocabulary) x 128 (tokens) part to on_tile(vt, acc): acc[i][j][v] is the logit of
+//   vocabulary row  tile_row0 + wv*64 + i*32 + 8*(v>>2) + 4*(lane>>5) + (v&3)
+//   token           tok0_ld + wt*128 + j*32 + (lane&31)
+// with wv = wave>>1, wt = wave&1 and tile_row0 = vt*256 (V-256 for an edge tile, whose rows below vt*256 repeat the
+// tile before). `lds` is 128 KiB, 1 KiB aligned. On return no load is in flight.
+template <int DT, class OnTile>
+__device__ __forceinline__ void lm_walk_tiles(const uint16_t* __restrict__ W, const uint16_t* __restrict__ H, int64_t V,
+                                              int64_t K, int64_t w_stride, int64_t h_stride, const LmWork& work,
+                                              char* lds, OnTile&& on_tile) {
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);   // uniform: keeps tile addressing in scalar registers
-  const int wv = wave >> 1;  // vocab quarter of the tile (8 wavefronts: 4 vocab quarters x 2 token halves)
+  const int wv = wave >> 1;  // vocabulary quarter of the tile
   const int wt = wave & 1;   // token half of the tile
-  // Workgroup -> (token block, split). Hardware deals workgroups round-robin over the 8 XCDs (id % 8); the 32 that
-  // are resident on one XCD together should share operands through its L2: 8 token blocks x 4 splits per XCD
-  // (each W slice read by 8 workgroups, each H slice by 4) when the grid has that shape, plain order otherwise.
-  int split;
-  int64_t tb;
-  {
-    const int64_t tblocks = (T + kLmTokens - 1) / kLmTokens;
-    const int64_t id = blockIdx.x;
-    if (xcd_map) {
-      const int x = (int)(id & 7);
-      const int64_t local = id >> 3;            // 0 .. tblocks*n_splits/8
-      const int64_t tgroups = tblocks / 8;      // groups of 8 token blocks
-      // super index over (tgroup, sgroup) pairs: 8 consecutive ones run at a time (one per XCD)
-      const int64_t super = (local / 32) * 8 + x;
-      const int64_t within = local % 32;
-      const int64_t tg = super % tgroups;
-      const int sg = (int)(super / tgroups);
-      tb = tg * 8 + (within & 7);
-      split = sg * 4 + (int)(within >> 3);
-    } else {
-      split = (int)(id % n_splits);
-      tb = id / n_splits;
-    }
-  }
-  const int64_t tok0 = tb * kLmTokens;
-  const int64_t n_vtiles = (V + kLmVocab - 1) / kLmVocab;
-  const int64_t vt_begin = (int64_t)split * tiles_per_split;
-  int64_t vt_end = vt_begin + tiles_per_split;
-  if (vt_end > n_vtiles) vt_end = n_vtiles;
   const int ksteps = (int)(K / kLmK);
-
-  // per-lane softmax state for the 4 token columns this lane sees
-  float m[4], s[4], t[4], c[4];
-#pragma unroll
-  for (int j = 0; j < 4; ++j) {
-    m[j] = neg_inf();
-    s[j] = 0.f;
-    t[j] = 0.f;
-    const int64_t tok = (tok0 + kLmTokens <= T ? tok0 : T - kLmTokens) + wt * 128 + j * 32 + (lane & 31);
-    c[j] = make_scale<false>(temperature, tok).c;   // log2(e) / max(T, 1e-8), exactly what the finishing kernel uses
-  }
 
   // fragment addressing: row (within its 32-row block) = lane&31, logical chunk = 2*sub + (lane>>5), sub in 0..3
   int phys[4];
@@ -139,37 +130,61 @@ __global__ __launch_bounds__(kLmWaves * 64, 1) void lmhead_partial_kernel(
   const int fragoff_w = (wv * 64 + (lane & 31)) * kLmRowBytes;
   const int fragoff_h = kLmTileBytes + (wt * 128 + (lane & 31)) * kLmRowBytes;
 
-  // Edge tiles are moved back so that all 256 rows exist (host guarantees V, T >= 256); the rows they share with
-  // the tile before are masked in the epilogue (vocab) or not written (tokens).
-  const int64_t tok0_ld = tok0 + kLmTokens <= T ? tok0 : T - kLmTokens;
-  // physical 16-byte slot p of tile row R holds logical chunk p ^ ((R >> 1) & 7): 16 consecutive rows then cover
-  // 16 distinct (row parity, slot) pairs, i.e. all 64 banks once per 16 lanes of a 128-bit read
+  // One wave instruction moves 8 tile rows x 128 bytes into LDS (lane l lands at byte l*16 of the 1 KiB block): lane l
+  // serves row r = l>>3 of the block and physical 16-byte slot p = l&7, and fetches the logical chunk that the swizzle
+  // assigns to that slot. Physical slot p of tile row R holds logical chunk p ^ ((R >> 1) & 7): 16 consecutive rows
+  // then cover 16 distinct (row parity, slot) pairs, i.e. all 64 banks once per 16 lanes of a 128-bit read. Blocks of
+  // 8 rows alternate in the swizzle's row bits, hence two lane offsets.
   const int lr = lane >> 3;
   const int lc_e = (lane & 7) ^ (lr >> 1), lc_o = (lane & 7) ^ (4 + (lr >> 1));
   const uint32_t w_lane_e = (uint32_t)((lr * w_stride + lc_e * 8) * 2), w_lane_o = (uint32_t)((lr * w_stride + lc_o * 8) * 2);
   const uint32_t h_lane_e = (uint32_t)((lr * h_stride + lc_e * 8) * 2), h_lane_o = (uint32_t)((lr * h_stride + lc_o * 8) * 2);
-  const int64_t w_blk = 8 * w_stride * 2, h_blk = 8 * h_stride * 2;
-  const char* Wb = reinterpret_cast<const char*>(W);
-  const char* Hb = reinterpret_cast<const char*>(H) + tok0_ld * h_stride * 2;
+  const uint64_t w_blk = (uint64_t)(8 * w_stride * 2), h_blk = (uint64_t)(8 * h_stride * 2);   // 8 rows in bytes
 
-  // prefetch cursor: global step (tile, k step), two steps ahead of the compute cursor once the loop runs
-  const int64_t total_steps = (vt_end > vt_begin ? (vt_end - vt_begin) : 0) * ksteps;
-  int64_t pstep = 0, pvt = vt_begin;
+  // Load cursor: global step (tile, k step); it runs two steps ahead of the compute cursor once the loop is going.
+  // wp / hp are uniform byte pointers to this wavefront's first row (it brings rows [32*wave, 32*wave + 32) with four
+  // instructions per operand) of the W and H tiles of the step to load next. A step advances both by one k step
+  // (128 bytes); at the end of a vocabulary tile W jumps to the next tile's rows and H returns to k = 0. Past the last
+  // step they stay put: the last tile is loaded once more into the stage nobody reads (in bounds, harmless), so the
+  // main loop needs no "is there more" branch around its loads.
+  const int64_t total_steps = (work.vt_end > work.vt_begin ? (work.vt_end - work.vt_begin) : 0) * ksteps;
+  auto uniform64 = [](uint64_t v) {
+    const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)v);
+    const uint32_t hi = __builtin_amdgcn_readfirstlane((uint32_t)(v >> 32));
+    return ((uint64_t)hi << 32) | lo;
+  };
+  auto vrow_of = [&](int64_t vt) { return (vt + 1) * kLmVocab <= V ? vt * kLmVocab : V - kLmVocab; };
+  uint64_t wp = uniform64(reinterpret_cast<uint64_t>(W) + (uint64_t)(vrow_of(work.vt_begin) * w_stride * 2) + wave * 4 * w_blk);
+  uint64_t hp = uniform64(reinterpret_cast<uint64_t>(H) + (uint64_t)(work.tok0_ld * h_stride * 2) + wave * 4 * h_blk);
+  int64_t pstep = 0, pvt = work.vt_begin;
   int pks = 0;
-  // Loads of global step `pstep` into stage pstep & 1. Branch-free: past the last step the cursor stays on the last
-  // step, whose tile is loaded once more into the stage nobody will read (in bounds, harmless), so the main loop is
-  // one basic block.
-  auto issue_always = [&]() {
-    char* st = lds + (int)(pstep & 1) * 2 * kLmTileBytes;
-    const int64_t vrow = (pvt + 1) * kLmVocab <= V ? pvt * kLmVocab : V - kLmVocab;
-    load_tile(Wb + vrow * w_stride * 2 + (int64_t)pks * kLmRowBytes, w_lane_e, w_lane_o, w_blk, st, wave);
-    load_tile(Hb + (int64_t)pks * kLmRowBytes, h_lane_e, h_lane_o, h_blk, st + kLmTileBytes, wave);
+  auto load4 = [&](uint64_t base, uint64_t blk, uint32_t off_e, uint32_t off_o, char* dst) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const char* src = reinterpret_cast<const char*>(base + i * blk);
+      __builtin_amdgcn_global_load_lds((const VRL_GLOBAL_AS void*)(src + ((i & 1) ? off_o : off_e)),
+                                       (VRL_LDS_AS void*)(dst + i * 8 * kLmRowBytes), 16, 0, 0);
+    }
+  };
+  auto issue = [&]() {   // loads of global step `pstep` into stage pstep & 1
+    char* st = lds + (int)(pstep & 1) * 2 * kLmTileBytes + wave * 32 * kLmRowBytes;
+    load4(wp, w_blk, w_lane_e, w_lane_o, st);
+    load4(hp, h_blk, h_lane_e, h_lane_o, st + kLmTileBytes);
     const bool more = pstep + 1 < total_steps;
     ++pstep;
-    const int nks = pks + 1;
-    const bool wrap = nks == ksteps;
-    pks = more ? (wrap ? 0 : nks) : pks;
-    pvt = more ? (wrap ? pvt + 1 : pvt) : pvt;
+    if (more) {
+      if (pks + 1 == ksteps) {
+        const int64_t dv = vrow_of(pvt + 1) - vrow_of(pvt);
+        wp += (uint64_t)(dv * w_stride * 2) - (uint64_t)(ksteps - 1) * kLmRowBytes;
+        hp -= (uint64_t)(ksteps - 1) * kLmRowBytes;
+        pks = 0;
+        ++pvt;
+      } else {
+        wp += kLmRowBytes;
+        hp += kLmRowBytes;
+        ++pks;
+      }
+    }
   };
   typename LmFrag<DT>::type a[2][2], b[2][4];
   auto read_frags = [&](int set, const char* stage, int sb) {
@@ -179,15 +194,15 @@ __global__ __launch_bounds__(kLmWaves * 64, 1) void lmhead_partial_kernel(
     for (int j = 0; j < 4; ++j) b[set][j] = *reinterpret_cast<const typename LmFrag<DT>::type*>(stage + fragoff_h + j * 32 * kLmRowBytes + phys[sb]);
   };
   if (total_steps > 0) {
-    issue_always();   // step 0 -> stage 0
+    issue();   // step 0 -> stage 0
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
     read_frags(0, lds, 0);
-    issue_always();   // step 1 -> stage 1
+    issue();   // step 1 -> stage 1
   }
 
   int64_t step = 0;
-  for (int64_t vt = vt_begin; vt < vt_end; ++vt) {
+  for (int64_t vt = work.vt_begin; vt < work.vt_end; ++vt) {
     lm_f32x16 acc[2][4];
 #pragma unroll
     for (int i = 0; i < 2; ++i)
@@ -217,16 +232,49 @@ __global__ __launch_bounds__(kLmWaves * 64, 1) void lmhead_partial_kernel(
       asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
       __syncthreads();
       read_frags(0, nxt, 0);
-      issue_always();
+      issue();
 #pragma unroll
       for (int i = 0; i < 2; ++i)
 #pragma unroll
         for (int j = 0; j < 4; ++j)
           acc[i][j] = LmFrag<DT>::mfma(a[1][i], b[1][j], acc[i][j]);
     }
+    on_tile(vt, acc);
+  }
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // the last, redundant loads still target the LDS stages
+}
 
-    // epilogue of this vocab tile: fold 64 logits per token column into the running state (two passes over the
-    // accumulators: maximum, then exponentials; nothing is buffered)
+// grid.x = token blocks * n_splits, block = 512, dynamic LDS = kLmLdsBytes. Writes, per (token, split), the online-softmax
+// partial (m, s, t, 0) of the split's vocabulary tiles to partials[(token * n_splits + split) * 4 ...].
+template <int DT>
+__global__ __launch_bounds__(kLmWaves * 64, 1) void lmhead_partial_kernel(
+    const uint16_t* __restrict__ W, const uint16_t* __restrict__ H, int64_t V, int64_t T, int64_t K, int64_t w_stride,
+    int64_t h_stride, const float* __restrict__ temperature, int n_splits, int tiles_per_split,
+    int xcd_map, float* __restrict__ partials) {
+  extern __shared__ __attribute__((aligned(1024))) char lds[];  // [2 stages][W tile, H tile]
+  __shared__ float red[4][256][3];
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wv = wave >> 1;
+  const int wt = wave & 1;
+  const LmWork work = lm_work(V, T, n_splits, tiles_per_split, xcd_map);
+
+  // per-lane softmax state for the 4 token columns this lane sees
+  float m[4], s[4], t[4], c[4];
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    m[j] = neg_inf();
+    s[j] = 0.f;
+    t[j] = 0.f;
+    const int64_t tok = work.tok0_ld + wt * 128 + j * 32 + (lane & 31);
+    c[j] = make_scale<false>(temperature, tok).c;   // log2(e) / max(T, 1e-8), exactly what the finishing kernel uses
+  }
+
+  lm_walk_tiles<DT>(W, H, V, K, w_stride, h_stride, work, lds, [&](int64_t vt, lm_f32x16 (&acc)[2][4]) {
+    // fold 64 logits per token column into the running state (two passes over the accumulators: maximum, then
+    // exponentials; nothing is buffered)
     const bool edge = (vt + 1) * kLmVocab > V;
     const int64_t vrow0 = (edge ? V - kLmVocab : vt * kLmVocab) + wv * 64 + 4 * (lane >> 5);
     const int64_t vfirst = vt * kLmVocab;   // rows below belong to the tile before
@@ -236,7 +284,7 @@ __global__ __launch_bounds__(kLmWaves * 64, 1) void lmhead_partial_kernel(
 #pragma unroll
       for (int i = 0; i < 2; ++i) {
         // one 32x32 block (16 accumulator registers) at a time; the scheduling barrier keeps the compiler from
-        // pulling the next blocks' accumulator copies forward, which would spill registers across the main loop
+        // pulling the next blocks' accumulator copies forward
         float x[16];
 #pragma unroll
         for (int v = 0; v < 16; ++v) x[v] = acc[i][j][v];
@@ -285,10 +333,10 @@ __global__ __launch_bounds__(kLmWaves * 64, 1) void lmhead_partial_kernel(
       s[j] += ps;
       t[j] += pt;
     }
-  }
+  });
 
-  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // the last, redundant loads still target the LDS stages
-  // combine: lanes l and l^32 hold the same tokens (other vocab rows), then the two vocab-half waves via LDS
+  // combine: lanes l and l^32 hold the same tokens (other vocabulary rows), then the four vocabulary-quarter
+  // wavefronts of a token half through LDS
 #pragma unroll
   for (int j = 0; j < 4; ++j) {
     const float om = __shfl_xor(m[j], 32);
@@ -313,8 +361,8 @@ __global__ __launch_bounds__(kLmWaves * 64, 1) void lmhead_partial_kernel(
   __syncthreads();
   if (tid < 256) {
     const int col = tid;  // 256 token columns
-    const int64_t tok = tok0_ld + col;
-    if (tok >= tok0) {
+    const int64_t tok = work.tok0_ld + col;
+    if (tok >= work.tok0) {
       float M = red[0][col][0];
 #pragma unroll
       for (int q = 1; q < 4; ++q) M = __builtin_fmaxf(M, red[q][col][0]);
@@ -329,13 +377,92 @@ __global__ __launch_bounds__(kLmWaves * 64, 1) void lmhead_partial_kernel(
           Tt += aq * (red[q][col][2] + dq * red[q][col][1]);
         }
       }
-      float* p = partials + (tok * n_splits + split) * 4;
+      float* p = partials + (tok * n_splits + work.split) * 4;
       p[0] = M;
       p[1] = S;
       p[2] = Tt;
       p[3] = 0.f;
     }
   }
+}
+
+// Backward: dlogits[tok, v] = (g_logprob[tok] * (1[v == label[tok]] - p) - g_entropy[tok] * p * (log p + entropy[tok])) / T[tok]
+// with p = exp(z - lse[tok]), z = logits / T, for all tokens and the vocabulary tiles of each split, written in the
+// operands' type to dlogits[tok * d_stride + v] (d_stride, V multiples of 8; 16-byte aligned base). Same grid and LDS as
+// lmhead_partial_kernel. A lane holds 4 consecutive vocabulary entries of one token per accumulator quad, i.e. one
+// 8-byte store; lanes l and l+32 complete 16 contiguous bytes, the four quads of a block 64.
+template <int DT>
+__global__ __launch_bounds__(kLmWaves * 64, 1) void lmhead_dlogits_kernel(
+    const uint16_t* __restrict__ W, const uint16_t* __restrict__ H, int64_t V, int64_t T, int64_t K, int64_t w_stride,
+    int64_t h_stride, const int64_t* __restrict__ labels, const float* __restrict__ temperature,
+    const float* __restrict__ lse, const float* __restrict__ entropy, const float* __restrict__ g_logprob,
+    const float* __restrict__ g_entropy, int n_splits, int tiles_per_split, int xcd_map, uint16_t* __restrict__ dlogits,
+    int64_t d_stride) {
+  extern __shared__ __attribute__((aligned(1024))) char lds[];  // [2 stages][W tile, H tile]
+  using O = ElemOut<DT>;
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wv = wave >> 1;
+  const int wt = wave & 1;
+  const LmWork work = lm_work(V, T, n_splits, tiles_per_split, xcd_map);
+
+  // the row constants of the 4 token columns this lane sees
+  RowGrad f[4];
+  int label[4];       // -1: no label term
+  bool tok_mine[4];   // false for the rows an edge block shares with the block before
+  uint16_t* out[4];
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    const int64_t tok = work.tok0_ld + wt * 128 + j * 32 + (lane & 31);
+    tok_mine[j] = tok >= work.tok0;
+    float Tm = 1.f;
+    if (temperature != nullptr) {
+      Tm = temperature[tok];
+      Tm = (Tm < kMinTemperature) ? kMinTemperature : Tm;
+    }
+    const float rT = 1.0f / Tm;
+    const float gl = (g_logprob != nullptr) ? g_logprob[tok] : 0.f;
+    const float gh = (g_entropy != nullptr) ? g_entropy[tok] : 0.f;
+    const float Hh = (g_entropy != nullptr) ? entropy[tok] : 0.f;
+    f[j].c = kLog2e * rT;
+    f[j].lse2 = lse[tok] * kLog2e;
+    f[j].a = -(gh * kLn2f) * rT;
+    f[j].b = -(gl + gh * Hh) * rT;
+    f[j].lab = gl * rT;
+    const int64_t lab = (g_logprob != nullptr) ? labels[tok] : -1;
+    label[j] = (lab >= 0 && lab < V) ? (int)lab : -1;   // an out-of-range label was reported by the forward pass
+    out[j] = dlogits + tok * d_stride;
+  }
+
+  lm_walk_tiles<DT>(W, H, V, K, w_stride, h_stride, work, lds, [&](int64_t vt, lm_f32x16 (&acc)[2][4]) {
+    const bool edge = (vt + 1) * kLmVocab > V;
+    const int vrow0 = (int)(edge ? V - kLmVocab : vt * kLmVocab) + wv * 64 + 4 * (lane >> 5);
+    const int vfirst = (int)(vt * kLmVocab);   // rows below belong to the tile before
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+#pragma unroll
+      for (int i = 0; i < 2; ++i) {
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          const int vr = vrow0 + i * 32 + 8 * q;   // first of 4 consecutive vocabulary entries (a multiple of 4)
+          float y[4];
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            y[e] = f[j](acc[i][j][q * 4 + e]);
+            if (vr + e == label[j]) y[e] += f[j].lab;
+          }
+          if (tok_mine[j] && vr >= vfirst) {
+            uint2 pk;
+            pk.x = O::pack2(y[0], y[1]);
+            pk.y = O::pack2(y[2], y[3]);
+            *reinterpret_cast<uint2*>(out[j] + vr) = pk;
+          }
+        }
+        __builtin_amdgcn_sched_barrier(0);
+      }
+    }
+  });
 }
 
 

@@ -258,35 +258,83 @@ int verify_waves(const int64_t* cu_seqlens, int64_t B, int64_t T) {
   return B <= 4096 ? 16 : 4;
 }
 
+struct LmGrid {
+  int64_t tblocks;
+  int tiles_per_split;
+  int xcd_map;
+};
+
+LmGrid lm_grid(int64_t T, int64_t V, int n_splits) {
+  LmGrid g;
+  g.tblocks = (T + vrl::kLmTokens - 1) / vrl::kLmTokens;
+  const int64_t vtiles = (V + vrl::kLmVocab - 1) / vrl::kLmVocab;
+  g.tiles_per_split = static_cast<int>((vtiles + n_splits - 1) / n_splits);
+  // 8 token blocks x 4 splits per XCD when the grid divides that way (see vrl::lm_work)
+  g.xcd_map = (g.tblocks % 8 == 0 && n_splits % 4 == 0 && ((g.tblocks / 8) * (n_splits / 4)) % 8 == 0) ? 1 : 0;
+  return g;
+}
+
+// The matrix-core kernels ask for more LDS than the default limit: raise it once per device and kernel, not per launch.
+int raise_lds_limit(const void* kernel, std::atomic<bool>* raised) {
+  int dev = -1;
+  if (hipGetDevice(&dev) != hipSuccess) return launch_status();
+  if (dev < 0 || dev >= kMaxDevices) return VRL_ERR_SHAPE;
+  if (!raised[dev].load(std::memory_order_acquire)) {
+    if (hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, vrl::kLmLdsBytes) != hipSuccess)
+      return launch_status();
+    raised[dev].store(true, std::memory_order_release);
+  }
+  return VRL_OK;
+}
+
 template <int DT>
 int launch_lmhead(const void* hidden, const void* weight, int64_t T, int64_t V, int64_t K, int64_t h_stride,
-                         int64_t w_stride, const int64_t* labels, const float* temperature, int n_splits,
-                         float* partials, float* out_logprob, float* out_entropy, float* out_lse,
-                         int32_t* err_flag, hipStream_t s) {
-  const int64_t tblocks = (T + vrl::kLmTokens - 1) / vrl::kLmTokens;
-  const int64_t vtiles = (V + vrl::kLmVocab - 1) / vrl::kLmVocab;
-  const int tiles_per_split = static_cast<int>((vtiles + n_splits - 1) / n_splits);
-  // 8 token blocks x 4 splits per XCD when the grid divides that way (see the kernel's mapping)
-  const int xcd_map = (tblocks % 8 == 0 && n_splits % 4 == 0 && ((tblocks / 8) * (n_splits / 4)) % 8 == 0) ? 1 : 0;
-  {  // the kernel's LDS request is above the default limit: raise it once per device, not per launch
-    static std::atomic<bool> raised[kMaxDevices];
-    int dev = -1;
-    if (hipGetDevice(&dev) != hipSuccess) return launch_status();
-    if (dev < 0 || dev >= kMaxDevices) return VRL_ERR_SHAPE;
-    if (!raised[dev].load(std::memory_order_acquire)) {
-      if (hipFuncSetAttribute(reinterpret_cast<const void*>(vrl::lmhead_partial_kernel<DT>),
-                              hipFuncAttributeMaxDynamicSharedMemorySize, vrl::kLmLdsBytes) != hipSuccess)
-        return launch_status();
-      raised[dev].store(true, std::memory_order_release);
-    }
-  }
-  vrl::lmhead_partial_kernel<DT><<<dim3(static_cast<unsigned>(tblocks * n_splits)), dim3(vrl::kLmWaves * 64), vrl::kLmLdsBytes, s>>>(
+                  int64_t w_stride, const int64_t* labels, const float* temperature, int n_splits, float* partials,
+                  float* out_logprob, float* out_entropy, float* out_lse, int32_t* err_flag, hipStream_t s) {
+  const LmGrid g = lm_grid(T, V, n_splits);
+  static std::atomic<bool> raised[kMaxDevices];
+  const int rs = raise_lds_limit(reinterpret_cast<const void*>(vrl::lmhead_partial_kernel<DT>), raised);
+  if (rs != VRL_OK) return rs;
+  vrl::lmhead_partial_kernel<DT><<<dim3(static_cast<unsigned>(g.tblocks * n_splits)), dim3(vrl::kLmWaves * 64),
+                                   vrl::kLmLdsBytes, s>>>(
       static_cast<const uint16_t*>(weight), static_cast<const uint16_t*>(hidden), V, T, K, w_stride, h_stride,
-      temperature, n_splits, tiles_per_split, xcd_map, partials);
+      temperature, n_splits, g.tiles_per_split, g.xcd_map, partials);
   vrl::lmhead_finish_kernel<DT><<<dim3(static_cast<unsigned>((T + 3) / 4)), dim3(256), 0, s>>>(
       static_cast<const char*>(weight), static_cast<const char*>(hidden), V, T, K, w_stride, h_stride, labels,
       temperature, n_splits, partials, out_logprob, out_entropy, out_lse, err_flag);
   return launch_status();
+}
+
+template <int DT>
+int launch_lmhead_dlogits(const void* hidden, const void* weight, int64_t T, int64_t V, int64_t K, int64_t h_stride,
+                          int64_t w_stride, const int64_t* labels, const float* temperature, const float* lse,
+                          const float* entropy, const float* g_logprob, const float* g_entropy, int n_splits,
+                          void* dlogits, int64_t d_stride, hipStream_t s) {
+  const LmGrid g = lm_grid(T, V, n_splits);
+  static std::atomic<bool> raised[kMaxDevices];
+  const int rs = raise_lds_limit(reinterpret_cast<const void*>(vrl::lmhead_dlogits_kernel<DT>), raised);
+  if (rs != VRL_OK) return rs;
+  vrl::lmhead_dlogits_kernel<DT><<<dim3(static_cast<unsigned>(g.tblocks * n_splits)), dim3(vrl::kLmWaves * 64),
+                                   vrl::kLmLdsBytes, s>>>(
+      static_cast<const uint16_t*>(weight), static_cast<const uint16_t*>(hidden), V, T, K, w_stride, h_stride, labels,
+      temperature, lse, entropy, g_logprob, g_entropy, n_splits, g.tiles_per_split, g.xcd_map,
+      static_cast<uint16_t*>(dlogits), d_stride);
+  return launch_status();
+}
+
+// Shape rules the matrix-core kernels share.
+int check_lmhead_shape(int dtype, int64_t n_tokens, int64_t vocab, int64_t hidden_size, int64_t h_stride,
+                       int64_t w_stride, int n_splits) {
+  if (dtype != VRL_BF16 && dtype != VRL_F16) return VRL_ERR_DTYPE;
+  if (n_tokens < vrl::kLmTokens || vocab < vrl::kLmVocab || hidden_size <= 0 || hidden_size % vrl::kLmK != 0 ||
+      h_stride < hidden_size || w_stride < hidden_size || h_stride % 8 != 0 || w_stride % 8 != 0 ||
+      n_splits < 1 || n_splits > vrl::kLmMaxSplits)
+    return VRL_ERR_SHAPE;
+  // 32-bit byte offsets inside each operand; grid size
+  if (vocab * w_stride * 2 >= (1LL << 32) || n_tokens * h_stride * 2 >= (1LL << 32)) return VRL_ERR_SHAPE;
+  if (((n_tokens + vrl::kLmTokens - 1) / vrl::kLmTokens) * n_splits > kMaxGrid || (n_tokens + 3) / 4 > kMaxGrid)
+    return VRL_ERR_SHAPE;
+  return VRL_OK;
 }
 
 }  // namespace
@@ -545,15 +593,8 @@ int vrl_lmhead_score(const void* hidden, const void* weight, int dtype, int64_t 
                      int64_t hidden_size, int64_t h_stride, int64_t w_stride, const int64_t* labels,
                      const float* temperature, int n_splits, float* partials, float* out_logprob,
                      float* out_entropy, float* out_lse, int32_t* err_flag, void* stream) {
-  if (dtype != VRL_BF16 && dtype != VRL_F16) return VRL_ERR_DTYPE;
-  if (n_tokens < vrl::kLmTokens || vocab < vrl::kLmVocab || hidden_size <= 0 || hidden_size % vrl::kLmK != 0 ||
-      h_stride < hidden_size || w_stride < hidden_size || h_stride % 8 != 0 || w_stride % 8 != 0 ||
-      n_splits < 1 || n_splits > vrl::kLmMaxSplits)
-    return VRL_ERR_SHAPE;
-  // 32-bit byte offsets inside each operand; grid size
-  if (vocab * w_stride * 2 >= (1LL << 32) || n_tokens * h_stride * 2 >= (1LL << 32)) return VRL_ERR_SHAPE;
-  if (((n_tokens + vrl::kLmTokens - 1) / vrl::kLmTokens) * n_splits > kMaxGrid || (n_tokens + 3) / 4 > kMaxGrid)
-    return VRL_ERR_SHAPE;
+  const int cs = check_lmhead_shape(dtype, n_tokens, vocab, hidden_size, h_stride, w_stride, n_splits);
+  if (cs != VRL_OK) return cs;
   if (out_logprob == nullptr && out_entropy == nullptr && out_lse == nullptr) return VRL_ERR_ARG;
   if (hidden == nullptr || weight == nullptr || partials == nullptr) return VRL_ERR_NULL;
   if (out_logprob != nullptr && (labels == nullptr || err_flag == nullptr)) return VRL_ERR_NULL;
@@ -567,6 +608,31 @@ int vrl_lmhead_score(const void* hidden, const void* weight, int dtype, int64_t 
                                    n_splits, partials, out_logprob, out_entropy, out_lse, err_flag, s);
   return launch_lmhead<VRL_F16>(hidden, weight, n_tokens, vocab, hidden_size, h_stride, w_stride, labels, temperature,
                                 n_splits, partials, out_logprob, out_entropy, out_lse, err_flag, s);
+}
+
+int vrl_lmhead_dlogits(const void* hidden, const void* weight, int dtype, int64_t n_tokens, int64_t vocab,
+                       int64_t hidden_size, int64_t h_stride, int64_t w_stride, const int64_t* labels,
+                       const float* temperature, const float* lse, const float* entropy, const float* g_logprob,
+                       const float* g_entropy, int n_splits, void* dlogits, int64_t d_stride, void* stream) {
+  const int cs = check_lmhead_shape(dtype, n_tokens, vocab, hidden_size, h_stride, w_stride, n_splits);
+  if (cs != VRL_OK) return cs;
+  // 8-byte stores of 4 consecutive vocabulary entries: the vocabulary and the output pitch must keep them aligned
+  if (vocab % 8 != 0 || d_stride < vocab || d_stride % 8 != 0) return VRL_ERR_SHAPE;
+  if (g_logprob == nullptr && g_entropy == nullptr) return VRL_ERR_ARG;
+  if (hidden == nullptr || weight == nullptr || lse == nullptr || dlogits == nullptr) return VRL_ERR_NULL;
+  if (g_logprob != nullptr && labels == nullptr) return VRL_ERR_NULL;
+  if (g_entropy != nullptr && entropy == nullptr) return VRL_ERR_NULL;
+  if (!aligned(hidden, 16) || !aligned(weight, 16) || !aligned(dlogits, 16) || !aligned(labels, 8) ||
+      !aligned(temperature, 4) || !aligned(lse, 4) || !aligned(entropy, 4) || !aligned(g_logprob, 4) ||
+      !aligned(g_entropy, 4))
+    return VRL_ERR_ALIGN;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  if (dtype == VRL_BF16)
+    return launch_lmhead_dlogits<VRL_BF16>(hidden, weight, n_tokens, vocab, hidden_size, h_stride, w_stride, labels,
+                                           temperature, lse, entropy, g_logprob, g_entropy, n_splits, dlogits, d_stride,
+                                           s);
+  return launch_lmhead_dlogits<VRL_F16>(hidden, weight, n_tokens, vocab, hidden_size, h_stride, w_stride, labels,
+                                        temperature, lse, entropy, g_logprob, g_entropy, n_splits, dlogits, d_stride, s);
 }
 
 int vrl_transpose(const void* src, int elem_size, int64_t rows, int64_t cols, int64_t src_stride,

@@ -12,6 +12,7 @@ gather, scatter, ...; :27-79); peak extra memory here is one ``(chunk, vocab)`` 
 
 from __future__ import annotations
 
+import os
 from typing import Optional
 
 import torch
@@ -28,6 +29,25 @@ __all__ = ["FusedLinearForPPO", "fused_linear_for_ppo", "linear_cross_entropy", 
 # projection reaches 1.4 PFLOP/s instead of 0.86 at 512, and the weight gradient is accumulated 8x less often.
 DEFAULT_CHUNK_TOKENS = 4096
 
+# Who forms the logits of a chunk. "library": torch.matmul (hipBLASLt) into the chunk buffer, then the row kernels over
+# it. "mfma": this package's own matrix-core kernels, which never round the logits to the operand type: forward
+# vrl_lmhead_score (no buffer at all, only when no gradient is recorded), backward vrl_lmhead_dlogits (logits formed
+# again on the matrix cores and turned into their gradient in registers; the buffer receives the gradient directly).
+# The default is what is faster on MI355X today (the library GEMM by ~10 %); VERL_AMD_LMHEAD_KERNELS or the
+# ``kernels`` argument select the other. Shapes the matrix-core kernels do not take always go to the library.
+DEFAULT_KERNELS = os.environ.get("VERL_AMD_LMHEAD_KERNELS", "library")
+
+
+def _mfma_takes(hidden: torch.Tensor, weight: torch.Tensor, n_tokens: int) -> bool:
+    """Shape rules of vrl_lmhead_score / vrl_lmhead_dlogits (include/vrl.h)."""
+    V, K = weight.shape
+    return (hidden.dtype in (torch.bfloat16, torch.float16) and n_tokens >= 256 and V >= 256 and V % 8 == 0
+            and K % 64 == 0 and hidden.stride(-1) == 1 and weight.stride(-1) == 1
+            and hidden.stride(0) % 8 == 0 and weight.stride(0) % 8 == 0
+            and V * weight.stride(0) * 2 < (1 << 32) and n_tokens * hidden.stride(0) * 2 < (1 << 32)
+            and hidden.data_ptr() % 16 == 0 and weight.data_ptr() % 16 == 0)
+
+
 # From this many tokens on, one transposed copy of the weight per backward (0.44 ms for 152064 x 3584 bf16) is
 # repaid by the faster `d hidden` product.
 _WEIGHT_TRANSPOSE_MIN_TOKENS = 2048
@@ -43,8 +63,9 @@ def _score_chunk(lib, logits, labels, temp, lp, h, lse, flag, stream):
 
 class _FusedLinearForPPOFunction(torch.autograd.Function):
     @staticmethod
-    def forward(ctx, hidden, weight, input_ids, temperature, chunk_size, keep_logits):
+    def forward(ctx, hidden, weight, input_ids, temperature, chunk_size, keep_logits, kernels):
         ctx.set_materialize_grads(False)
+        ctx.kernels = kernels
         T, D = hidden.shape
         V = weight.shape[0]
         dev = hidden.device
@@ -78,7 +99,7 @@ class _FusedLinearForPPOFunction(torch.autograd.Function):
     def backward(ctx, g_lp: Optional[torch.Tensor], g_h: Optional[torch.Tensor]):
         hidden, weight, input_ids, lse, h = ctx.saved_tensors
         if g_lp is None and g_h is None:
-            return None, None, None, None, None, None
+            return None, None, None, None, None, None, None
         kept = ctx.kept_logits
         if kept is not None:
             ctx.kept_logits = None        # the gradient is written over them: they serve one backward
@@ -109,6 +130,21 @@ class _FusedLinearForPPOFunction(torch.autograd.Function):
             for lo in range(0, T, chunk):
                 hi = min(lo + chunk, T)
                 n = hi - lo
+                if kept is None and ctx.kernels == "mfma" and _mfma_takes(hidden[lo:hi], weight, n) and V % 8 == 0:
+                    # logits formed again on the matrix cores, their gradient written straight into the buffer
+                    logits = buf[:n]
+                    st = lib.vrl_lmhead_dlogits(
+                        hidden[lo:hi].data_ptr(), weight.data_ptr(), dt, n, V, D, hidden.stride(0), weight.stride(0),
+                        input_ids[lo:hi].data_ptr(), None if temp is None else temp.data_ptr(), lse[lo:hi].data_ptr(),
+                        h[lo:hi].data_ptr(), None if gl is None else gl[lo:hi].data_ptr(),
+                        None if gh is None else gh[lo:hi].data_ptr(), lib.vrl_lmhead_plan(n, V), logits.data_ptr(),
+                        logits.stride(0), stream)
+                    _lib.check("vrl_lmhead_dlogits", st)
+                    if need_dh:
+                        torch.matmul(logits, weight if weight_t is None else weight_t.t(), out=d_hidden[lo:hi])
+                    if need_dw:
+                        d_weight.addmm_(logits.t(), transpose_2d(hidden[lo:hi]).t() if half else hidden[lo:hi])
+                    continue
                 if kept is not None:
                     logits = buf[lo:hi]
                 else:
@@ -132,11 +168,12 @@ class _FusedLinearForPPOFunction(torch.autograd.Function):
                     torch.matmul(kept, weight if weight_t is None else weight_t.t(), out=d_hidden)
                 if need_dw:
                     torch.matmul(kept.t(), transpose_2d(hidden).t() if half else hidden, out=d_weight)
-        return d_hidden, d_weight, None, None, None, None
+        return d_hidden, d_weight, None, None, None, None, None
 
 
 def fused_linear_for_ppo(hidden_states: torch.Tensor, vocab_weights: torch.Tensor, input_ids: torch.Tensor,
-                         temperature: float = 1.0, chunk_size: int = DEFAULT_CHUNK_TOKENS, keep_logits: bool = False):
+                         temperature: float = 1.0, chunk_size: int = DEFAULT_CHUNK_TOKENS, keep_logits: bool = False,
+                         kernels: Optional[str] = None):
     """(log_probs fp32, entropy fp32) of ``softmax((hidden_states @ vocab_weights.T) / temperature)`` at ``input_ids``.
 
     ``hidden_states`` is ``(tokens, hidden)`` or ``(batch, seq, hidden)`` with ``input_ids`` of the matching leading
@@ -148,7 +185,14 @@ def fused_linear_for_ppo(hidden_states: torch.Tensor, vocab_weights: torch.Tenso
     ``keep_logits=True`` trades memory for time when gradients are needed: the forward keeps all
     ``tokens x vocab`` logits (2.5 GB for 8192 x 152064 bf16), the backward writes their gradient over them instead of
     projecting again and forms ``d hidden`` and ``d W`` with one product each. Such a graph can be differentiated once.
+
+    ``kernels`` chooses who forms the logits: ``"library"`` (a GEMM per chunk into the buffer) or ``"mfma"`` (this
+    package's matrix-core kernels: no buffer at all when no gradient is recorded, and a backward that writes the
+    gradient of the logits straight from registers); None takes ``DEFAULT_KERNELS``.
     """
+    kernels = DEFAULT_KERNELS if kernels is None else kernels
+    if kernels not in ("library", "mfma"):
+        raise ValueError(f"kernels must be 'library' or 'mfma', got {kernels!r}")
     if not hidden_states.is_cuda or not vocab_weights.is_cuda:
         raise RuntimeError("fused_linear_for_ppo: tensors must be on the GPU; verl_amd has no CPU implementation")
     if hidden_states.dtype != vocab_weights.dtype or hidden_states.dtype not in _DTYPE_CODES:
@@ -170,8 +214,13 @@ def fused_linear_for_ppo(hidden_states: torch.Tensor, vocab_weights: torch.Tenso
     h2 = hidden_states.reshape(-1, hidden_states.shape[-1]).contiguous()
     # the kernels read the ids through a raw device pointer: they must live next to the hidden states
     ids = input_ids.reshape(-1).to(device=h2.device, dtype=torch.int64).contiguous()
-    lp, ent = _FusedLinearForPPOFunction.apply(h2, vocab_weights.contiguous(), ids, float(temperature), int(chunk_size),
-                                               bool(keep_logits))
+    w2 = vocab_weights.contiguous()
+    needs_grad = torch.is_grad_enabled() and (h2.requires_grad or w2.requires_grad)
+    if kernels == "mfma" and not needs_grad and _mfma_takes(h2, w2, h2.shape[0]):
+        lp, ent = lm_head_score_mfma(h2, w2, ids, float(temperature))
+        return lp.reshape(lead), ent.reshape(lead)
+    lp, ent = _FusedLinearForPPOFunction.apply(h2, w2, ids, float(temperature), int(chunk_size), bool(keep_logits),
+                                               kernels)
     return lp.reshape(lead), ent.reshape(lead)
 
 
@@ -259,11 +308,12 @@ def linear_cross_entropy(hidden: torch.Tensor, weight: torch.Tensor, labels: tor
 class FusedLinearForPPO(torch.nn.Module):
     """Module form, constructed and called like verl's (verl/utils/experimental/torch_functional.py:211-231)."""
 
-    def __init__(self, chunk_size: int = DEFAULT_CHUNK_TOKENS, keep_logits: bool = False):
+    def __init__(self, chunk_size: int = DEFAULT_CHUNK_TOKENS, keep_logits: bool = False, kernels: Optional[str] = None):
         super().__init__()
         self.chunk_size = chunk_size
         self.keep_logits = keep_logits
+        self.kernels = kernels
 
     def forward(self, hidden_states, vocab_weights, input_ids, temperature: float = 1.0):
         return fused_linear_for_ppo(hidden_states, vocab_weights, input_ids, temperature, self.chunk_size,
-                                    self.keep_logits)
+                                    self.keep_logits, self.kernels)
