@@ -55,4 +55,26 @@ __global__ __launch_bounds__(WAVES * 64) void stream_probe_kernel(const u32x4* _
   }
 }
 
+// The same copy without rows: a fixed number of workgroups of 4 wavefronts walk the whole buffer, each wavefront moving
+// 8 KiB (8 non-temporal 128-bit loads per lane, then 8 stores) per trip. The best of the shapes tried for a read+write
+// stream on this part; it bounds what any row-shaped kernel that reads N bytes and writes N bytes can reach.
+__global__ __launch_bounds__(256) void stream_probe_flat_copy_kernel(const u32x4* __restrict__ src, u32x4* __restrict__ dst,
+                                                                     int64_t nvec) {
+  constexpr int U = 8;
+  const int64_t stride = static_cast<int64_t>(gridDim.x) * 256 * U;
+  int64_t base = (static_cast<int64_t>(blockIdx.x) * 256 + (threadIdx.x >> 6) * 64) * U + (threadIdx.x & 63);
+  for (; base + (U - 1) * 64 < nvec; base += stride) {
+    u32x4 v[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) v[u] = __builtin_nontemporal_load(src + base + u * 64);
+#pragma unroll
+    for (int u = 0; u < U; ++u) __builtin_nontemporal_store(v[u], dst + base + u * 64);
+  }
+  // what is left of the last, partial trip of this wavefront's slot
+  for (int u = 0; u < U; ++u) {
+    const int64_t k = base + u * 64;
+    if (k < nvec) __builtin_nontemporal_store(__builtin_nontemporal_load(src + k), dst + k);
+  }
+}
+
 }  // namespace vrl
