@@ -687,7 +687,7 @@ def bench_score_responses(args, dev, steps, warmup):
     def run():
         st = lib.vrl_score_responses(logits.data_ptr(), _lib.VRL_BF16, n, w.V, logits.stride(0), None, ids.data_ptr(),
                                      None, cu_d.data_ptr(), resp_d.data_ptr(), B, T, None, None, r_lp.data_ptr(),
-                                     r_h.data_ptr(), flag.data_ptr(), stream)
+                                     r_h.data_ptr(), None, flag.data_ptr(), stream)
         _lib.check("vrl_score_responses", st)
 
     run()
@@ -714,6 +714,55 @@ def bench_score_responses(args, dev, steps, warmup):
     n_resp = int(resp.sum())
     bytes_launch = n_resp * (w.V * 2 + 8 + 4 + 4) + (B + 1) * 8 + B * 8 + B * T * 8 - n_resp * 8
     achieved = bytes_launch / (avg_ms * 1e-3) / 1e9
+
+    # The gradient of the same blocks (vrl_score_responses_backward): response rows are read once and their gradient
+    # written, every other row of the gradient is written as zeros without being read.
+    r_lse = torch.empty_like(r_lp)
+    st = lib.vrl_score_responses(logits.data_ptr(), _lib.VRL_BF16, n, w.V, logits.stride(0), None, ids.data_ptr(),
+                                 None, cu_d.data_ptr(), resp_d.data_ptr(), B, T, None, None, r_lp.data_ptr(),
+                                 r_h.data_ptr(), r_lse.data_ptr(), flag.data_ptr(), stream)
+    _lib.check("vrl_score_responses", st)
+    gg = torch.Generator(device=dev).manual_seed(3004)
+    g_lp = torch.randn((B, T), generator=gg, device=dev)
+    g_h = torch.randn((B, T), generator=gg, device=dev)
+    dlogits = torch.empty_like(logits)
+
+    def run_backward():
+        st = lib.vrl_score_responses_backward(
+            logits.data_ptr(), _lib.VRL_BF16, n, w.V, logits.stride(0), None, ids.data_ptr(), None, cu_d.data_ptr(),
+            resp_d.data_ptr(), B, T, r_lse.data_ptr(), r_h.data_ptr(), g_lp.data_ptr(), g_h.data_ptr(),
+            dlogits.data_ptr(), dlogits.stride(0), stream)
+        _lib.check("vrl_score_responses_backward", st)
+
+    run_backward()
+    # guard: equal to the row op's backward fed with the per-token gradients (zero outside the response windows)
+    tok_lp = torch.zeros(n, device=dev)
+    tok_h = torch.zeros(n, device=dev)
+    for b in range(B):
+        end, r = int(cu[b + 1]), int(resp[b])
+        tok_lp[end - r - 1:end - 1] = g_lp[b, :r]
+        tok_h[end - r - 1:end - 1] = g_h[b, :r]
+    x = logits.detach().clone().requires_grad_(True)
+    lp2, h2 = vf.fused_logprob_entropy(x, torch.roll(ids, -1))
+    torch.autograd.backward([lp2, h2], [tok_lp, tok_h])
+    if not torch.equal(x.grad, dlogits):
+        raise SystemExit("bench: vrl_score_responses_backward disagrees with vrl_rowscore_backward")
+    del x, lp2, h2
+    for _ in range(warmup):
+        run_backward()
+    torch.cuda.synchronize()
+    evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(steps)]
+    for a, b in evs:
+        a.record()
+        run_backward()
+        b.record()
+    torch.cuda.synchronize()
+    bwd_ms = sum(a.elapsed_time(b) for a, b in evs) / len(evs)
+    bwd_bytes = n_resp * (w.V * 2 + 8 + 16) + n * w.V * 2 + (B + 1) * 8 + B * 8
+    backward = {"avg_kernel_ms": bwd_ms, "kernel": "score_responses_backward_kernel",
+                "algorithmic_bytes_per_launch": bwd_bytes, "achieved_gbps": bwd_bytes / (bwd_ms * 1e-3) / 1e9,
+                "all_rows_backward_bytes": n * (w.V * 4 + 8 + 16),
+                "parity_guard": "bit-equal to vrl_rowscore_backward with per-token gradients"}
     return {
         "metric": "response tokens/sec from packed logits to padded (B, T) log-probs and entropies, one launch",
         "value": n_resp * steps / wall, "unit": "tokens/s", "ms_per_step": wall * 1e3 / steps, "dtype": "bf16",
@@ -724,6 +773,7 @@ def bench_score_responses(args, dev, steps, warmup):
                      "frac": achieved / HBM_PEAK_GBPS, "traffic": None, "kernel": "score_responses_kernel",
                      "avg_kernel_ms": avg_ms, "algorithmic_bytes_per_launch": bytes_launch},
         "all_rows_equivalent_tokens_per_s": n * steps / wall,
+        "backward": backward,
     }
 
 

@@ -160,7 +160,8 @@ int vrl_rowscore_backward(const void* logits, int dtype, int64_t n_rows, int64_t
  *   logprob / entropy  as vrl_rowscore
  *   resp_logprob[b, j] = logprob[cu_seqlens[b+1] - response_lens[b] - 1 + j]  for j < response_lens[b], else 0
  *   resp_entropy[b, j] likewise            (the left shift by one of verl/workers/utils/padding.py:135-138)
- * resp_logprob / resp_entropy: at least one. out_logprob / out_entropy (n_rows, per token) are optional extras of the
+ * resp_logprob / resp_entropy: at least one; resp_lse (optional) receives the logsumexp in the same layout, which is what
+ * vrl_score_responses_backward needs. out_logprob / out_entropy (n_rows, per token) are optional extras of the
  * block of the same kind; when neither is given, rows outside every response window are not read at all (a prompt
  * token's logits cost no memory traffic).
  * Device-side checks, reported through *err_flag: a label outside [0, vocab) (VRL_FLAG_LABEL_OOB, that entry NaN);
@@ -176,7 +177,26 @@ int vrl_score_responses(const void* logits, int dtype, int64_t n_rows, int64_t v
                         const int64_t* labels, const int64_t* input_ids, const float* temperature,
                         const int64_t* cu_seqlens, const int64_t* response_lens, int64_t B, int64_t T_out,
                         float* out_logprob, float* out_entropy, float* resp_logprob, float* resp_entropy,
-                        int32_t* err_flag, void* stream);
+                        float* resp_lse, int32_t* err_flag, void* stream);
+
+/*
+ * vrl_score_responses_backward — gradient of vrl_score_responses with respect to the logits, from the gradients of the
+ * two (B, T_out) blocks: row r inside the response window of sequence b (column j) gets
+ *   dlogits[r, :] = vrl_rowscore_backward's row for g_logprob = g_resp_logprob[b, j], g_entropy = g_resp_entropy[b, j],
+ *                   lse = resp_lse[b, j], entropy = resp_entropy[b, j]
+ * (resp_lse is the optional logsumexp block of the forward call), every other row zeros, written without reading that
+ * row's logits. dlogits has the logits' type and may be the logits buffer itself. g_resp_logprob or g_resp_entropy
+ * may be NULL. Labels as in the forward call (labels, or input_ids rolled by one). Offsets that fail the forward call's
+ * validation give zero rows here; they were reported there.
+ *
+ * Replaces what autograd builds for verl/workers/engine/fsdp/transformer_impl.py:1177,1357-1418 +
+ * verl/workers/utils/padding.py:97-141 under update_actor.
+ */
+int vrl_score_responses_backward(const void* logits, int dtype, int64_t n_rows, int64_t vocab, int64_t row_stride,
+                                 const int64_t* labels, const int64_t* input_ids, const float* temperature,
+                                 const int64_t* cu_seqlens, const int64_t* response_lens, int64_t B, int64_t T_out,
+                                 const float* resp_lse, const float* resp_entropy, const float* g_resp_logprob,
+                                 const float* g_resp_entropy, void* dlogits, int64_t d_row_stride, void* stream);
 
 /*
  * vrl_response_slice — packed per-token values (total_nnz,) -> padded (B, T_out)

@@ -168,12 +168,12 @@ def test_label_logprob_argument_errors_and_flag_values(lib):
 def test_score_responses_argument_errors(lib):
     f = lib.vrl_score_responses
     ok = dict(x=P, dt=_lib.VRL_BF16, n=8, V=100, stride=100, lab=None, ids=P, temp=None, cu=P, rl=P, B=2, T=4, tlp=None,
-              th=None, rlp=P, rh=P, flag=P)
+              th=None, rlp=P, rh=P, rlse=None, flag=P)
 
     def call(**kw):
         a = {**ok, **kw}
         return f(a["x"], a["dt"], a["n"], a["V"], a["stride"], a["lab"], a["ids"], a["temp"], a["cu"], a["rl"], a["B"],
-                 a["T"], a["tlp"], a["th"], a["rlp"], a["rh"], a["flag"], None)
+                 a["T"], a["tlp"], a["th"], a["rlp"], a["rh"], a["rlse"], a["flag"], None)
 
     assert call(dt=4) == _lib.VRL_ERR_DTYPE
     assert call(n=-1) == _lib.VRL_ERR_SHAPE
@@ -192,7 +192,37 @@ def test_score_responses_argument_errors(lib):
     assert call(ids=None) == _lib.VRL_ERR_NULL                     # log-probs asked for, no source of labels
     assert call(cu=P + 4) == _lib.VRL_ERR_ALIGN
     assert call(rh=P + 2) == _lib.VRL_ERR_ALIGN
+    assert call(rlse=P + 2) == _lib.VRL_ERR_ALIGN
     assert call(n=0, B=0, x=None, cu=None, rl=None, flag=None) == _lib.VRL_OK
+
+
+def test_score_responses_backward_argument_errors(lib):
+    f = lib.vrl_score_responses_backward
+    ok = dict(x=P, dt=_lib.VRL_BF16, n=8, V=100, stride=100, lab=None, ids=P, temp=None, cu=P, rl=P, B=2, T=4, lse=P,
+              ent=P, gl=P, gh=P, out=P, ds=100)
+
+    def call(**kw):
+        a = {**ok, **kw}
+        return f(a["x"], a["dt"], a["n"], a["V"], a["stride"], a["lab"], a["ids"], a["temp"], a["cu"], a["rl"], a["B"],
+                 a["T"], a["lse"], a["ent"], a["gl"], a["gh"], a["out"], a["ds"], None)
+
+    assert call(dt=7) == _lib.VRL_ERR_DTYPE
+    assert call(n=-1) == _lib.VRL_ERR_SHAPE
+    assert call(stride=50) == _lib.VRL_ERR_SHAPE
+    assert call(ds=50) == _lib.VRL_ERR_SHAPE
+    assert call(T=-1) == _lib.VRL_ERR_SHAPE
+    assert call(gl=None, gh=None) == _lib.VRL_ERR_ARG
+    assert call(lab=P) == _lib.VRL_ERR_ARG                         # labels and input_ids together
+    assert call(x=None) == _lib.VRL_ERR_NULL
+    assert call(out=None) == _lib.VRL_ERR_NULL
+    assert call(cu=None) == _lib.VRL_ERR_NULL
+    assert call(lse=None) == _lib.VRL_ERR_NULL
+    assert call(ids=None) == _lib.VRL_ERR_NULL                     # a log-prob gradient without a source of labels
+    assert call(ent=None) == _lib.VRL_ERR_NULL                     # an entropy gradient without the entropies
+    assert call(B=0) == _lib.VRL_ERR_SHAPE                         # rows that belong to no sequence
+    assert call(out=P + 1) == _lib.VRL_ERR_ALIGN
+    assert call(gl=P + 2) == _lib.VRL_ERR_ALIGN
+    assert call(n=0, x=None, out=None) == _lib.VRL_OK
 
 
 def test_lmhead_dlogits_argument_errors(lib):

@@ -154,10 +154,97 @@ def test_device_side_checks(dev):
         verl_amd.score_responses(logits, cud[:-1], rd, T, input_ids=ids)
     with pytest.raises(ValueError):
         verl_amd.score_responses(logits.view(1, n, V), cud, rd, T, input_ids=ids)
-    with pytest.raises(NotImplementedError):
-        verl_amd.score_responses(logits.clone().requires_grad_(True), cud, rd, T, input_ids=ids)
     empty = verl_amd.score_responses(logits[:0], cud[:1], rd[:0], 4, input_ids=ids[:0])
     assert empty[0].shape == (0, 4)
+
+
+def _separate_steps(logits, labels, temp, cu, resp, T):
+    """The same blocks from this library's row op (its own, separately tested, backward) and torch slicing."""
+    lp, h = vf.fused_logprob_entropy(logits, labels, temp)
+    rows_lp, rows_h = [], []
+    for b in range(resp.numel()):
+        end, r = int(cu[b + 1]), int(resp[b])
+        rows_lp.append(torch.nn.functional.pad(lp[end - r - 1:end - 1], (0, T - r)))
+        rows_h.append(torch.nn.functional.pad(h[end - r - 1:end - 1], (0, T - r)))
+    return torch.stack(rows_lp), torch.stack(rows_h)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("which", ["both", "logprob", "entropy"])
+def test_gradient_equals_the_separate_steps_bit_for_bit(dev, dtype, which):
+    """d(blocks)/d(logits) from vrl_score_responses_backward equals what autograd builds from the row op's backward and
+    torch's slicing and padding; prompt rows and each sequence's last row get exact zeros."""
+    B, V = 11, 4099
+    prompt, resp, cu, ids, logits = _batch(dev, 123, B, V, dtype)
+    n = logits.shape[0]
+    T = int(resp.max()) + 3
+    per_seq = 0.5 + torch.rand(B, generator=torch.Generator().manual_seed(4))
+    temp = torch.repeat_interleave(per_seq, prompt + resp).to(dev)
+    gd = torch.Generator(device=dev).manual_seed(5)
+    w_lp = torch.randn(B, T, generator=gd, device=dev)
+    w_h = torch.randn(B, T, generator=gd, device=dev)
+    labels = layout.roll_labels(ids)
+
+    def loss(r_lp, r_h):
+        out = 0.0
+        if which in ("both", "logprob"):
+            out = out + (r_lp * w_lp).sum()
+        if which in ("both", "entropy"):
+            out = out + (r_h * w_h).sum()
+        return out
+
+    a = logits.clone().requires_grad_(True)
+    got = verl_amd.score_responses(a, cu.to(dev), resp.to(dev), T, input_ids=ids, temperature=temp,
+                                   want_logprob=which != "entropy", want_entropy=which != "logprob")
+    before = dict(vf.counters)
+    loss(*got).backward()
+    assert vf.counters["backward_passes"] == before["backward_passes"] + 1
+    b = logits.clone().requires_grad_(True)
+    want = _separate_steps(b, labels, temp, cu, resp, T)
+    if which != "entropy":
+        assert torch.equal(got[0], want[0])
+    if which != "logprob":
+        assert torch.equal(got[1], want[1])
+    loss(*want).backward()
+    assert torch.equal(a.grad, b.grad)
+    for s in range(B):
+        begin, end, r = int(cu[s]), int(cu[s + 1]), int(resp[s])
+        assert not a.grad[begin:end - r - 1].any() and not a.grad[end - 1].any()
+    # ready labels instead of ids, and the gradient written over the logits' own storage
+    c = logits.clone().requires_grad_(True)
+    c2 = c * 1.0
+    got2 = verl_amd.score_responses(c2, cu.to(dev), resp.to(dev), T, labels=labels if which != "entropy" else None,
+                                    temperature=temp, want_logprob=which != "entropy", want_entropy=which != "logprob",
+                                    inplace_backward=True)
+    loss(*got2).backward()
+    assert torch.equal(c.grad, a.grad)
+    assert torch.equal(c2.detach(), a.grad)                  # c2's storage now holds the gradient
+
+
+def test_gradient_against_fp64_autograd(dev):
+    """The gradient itself against torch's fp64 autograd of the reference's sequence of steps (roll, divide, log-softmax
+    gather, entropy, slice, pad), fp32 logits: |diff| <= 2e-6 * max|grad|."""
+    B, V = 5, 1237
+    prompt, resp, cu, ids, logits = _batch(dev, 9, B, V, torch.float32, max_prompt=9, max_resp=20)
+    T = int(resp.max())
+    gd = torch.Generator(device=dev).manual_seed(6)
+    w_lp = torch.randn(B, T, generator=gd, device=dev)
+    w_h = torch.randn(B, T, generator=gd, device=dev)
+    a = logits.clone().requires_grad_(True)
+    r_lp, r_h = verl_amd.score_responses(a, cu.to(dev), resp.to(dev), T, input_ids=ids, temperature=0.7)
+    ((r_lp * w_lp).sum() + (r_h * w_h).sum()).backward()
+    x = logits.double().cpu().requires_grad_(True)
+    z = x / 0.7
+    logp = torch.log_softmax(z, -1)
+    lp = logp.gather(-1, torch.roll(ids.cpu(), -1)[:, None])[:, 0]
+    h = -(logp.exp() * logp).sum(-1)
+    total = 0.0
+    for s in range(B):
+        end, r = int(cu[s + 1]), int(resp[s])
+        total = total + (lp[end - r - 1:end - 1] * w_lp[s, :r].double().cpu()).sum()
+        total = total + (h[end - r - 1:end - 1] * w_h[s, :r].double().cpu()).sum()
+    total.backward()
+    assert (a.grad.double().cpu() - x.grad).abs().max().item() <= 2e-6 * x.grad.abs().max().item()
 
 
 def test_bad_offsets_leave_the_guard_regions_alone(dev):
@@ -176,6 +263,10 @@ def test_bad_offsets_leave_the_guard_regions_alone(dev):
         t_h = ar.make(N, torch.float32)
         r_lp = ar.make(B * T, torch.float32)
         r_h = ar.make(B * T, torch.float32)
+        r_lse = ar.make(B * T, torch.float32)
+        g_lp = ar.make(B * T, torch.float32, torch.randn(B * T, generator=g))
+        g_h = ar.make(B * T, torch.float32, torch.randn(B * T, generator=g))
+        dlogits = ar.make(N * V, torch.bfloat16)
         flag = ar.make(1, torch.int32, torch.zeros(1, dtype=torch.int32))
         print(f"[score_responses] cu_seqlens={offsets} over {N} rows", flush=True)
         for per_token in (True, False):
@@ -184,12 +275,22 @@ def test_bad_offsets_leave_the_guard_regions_alone(dev):
                 st = lib.vrl_score_responses(logits.data_ptr(), _lib.VRL_BF16, N, V, V, None, ids.data_ptr(), None,
                                              cu.data_ptr(), rl.data_ptr(), B, T, t_lp.data_ptr() if per_token else None,
                                              t_h.data_ptr() if per_token else None, r_lp.data_ptr(), r_h.data_ptr(),
-                                             flag.data_ptr(), _lib.stream_ptr(dev))
+                                             r_lse.data_ptr(), flag.data_ptr(), _lib.stream_ptr(dev))
             assert st == _lib.VRL_OK
             torch.cuda.synchronize(dev)
             assert int(flag.item()) & _lib.VRL_FLAG_SEQ_RANGE, case
             assert ar.guards_intact(), case
             assert torch.isfinite(r_lp).all() and torch.isfinite(r_h).all(), case   # every block element was written
+        # the backward over the same offsets: every row of the gradient is written, nothing else is
+        with torch.cuda.device(dev):
+            st = lib.vrl_score_responses_backward(logits.data_ptr(), _lib.VRL_BF16, N, V, V, None, ids.data_ptr(), None,
+                                                  cu.data_ptr(), rl.data_ptr(), B, T, r_lse.data_ptr(), r_h.data_ptr(),
+                                                  g_lp.data_ptr(), g_h.data_ptr(), dlogits.data_ptr(), V,
+                                                  _lib.stream_ptr(dev))
+        assert st == _lib.VRL_OK
+        torch.cuda.synchronize(dev)
+        assert ar.guards_intact(), case
+        assert torch.isfinite(dlogits.float()).all(), case
 
 
 def test_c3_micro_batch_full_size(dev):

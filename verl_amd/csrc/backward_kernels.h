@@ -117,13 +117,10 @@ struct RowGradExact {
   }
 };
 
-// grid.x = n_rows, block = WAVES*64. EXACT selects RowGradExact (fp32 logits).
-template <int DT, int WAVES, int U, bool EXACT = (DT == 0)>
-__global__ __launch_bounds__(WAVES * 64) void rowscore_backward_kernel(
-    const void* logits, int64_t vocab, int64_t row_stride, const int64_t* __restrict__ labels,
-    const float* __restrict__ temperature, const float* __restrict__ lse, const float* __restrict__ entropy,
-    const float* __restrict__ g_logprob, const float* __restrict__ g_entropy, void* dlogits,
-    int64_t d_row_stride) {
+// The whole workgroup (WAVES*64 threads) writes the gradient of one row: out[v] = f(in[v]) (+ f.lab at v == label).
+// Rows need not be 16-byte aligned; the vector path is taken when input and output rows share their 16-byte phase.
+template <int DT, int WAVES, int U, class F>
+__device__ __forceinline__ void backward_row(const char* rowp, char* outp, int64_t vocab, const F& f, int64_t label) {
   using E = Elem<DT>;
   using O = ElemOut<DT>;
   constexpr int NTHR = WAVES * 64;
@@ -131,37 +128,6 @@ __global__ __launch_bounds__(WAVES * 64) void rowscore_backward_kernel(
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = tid >> 6;
-  const int64_t row = blockIdx.x;
-  const char* rowp = static_cast<const char*>(logits) + row * row_stride * E::kBytes;
-  char* outp = static_cast<char*>(dlogits) + row * d_row_stride * E::kBytes;
-
-  float T = 1.f;
-  if (temperature != nullptr) {
-    T = temperature[row];
-    T = (T < kMinTemperature) ? kMinTemperature : T;
-  }
-  const float rT = 1.0f / T;
-  const float gl = (g_logprob != nullptr) ? g_logprob[row] : 0.f;
-  const float gh = (g_entropy != nullptr) ? g_entropy[row] : 0.f;
-  const float H = (g_entropy != nullptr) ? entropy[row] : 0.f;
-  typename std::conditional<EXACT, RowGradExact, RowGrad>::type f;
-  if constexpr (EXACT) {
-    f.sc.c = kLog2e;
-    f.sc.T = T;
-    f.sc.r = rT;
-    f.lse = lse[row];
-    f.a = -gh * rT;
-  } else {
-    f.c = kLog2e * rT;
-    f.lse2 = lse[row] * kLog2e;
-    f.a = -(gh * kLn2f) * rT;
-  }
-  f.b = -(gl + gh * H) * rT;
-  f.lab = gl * rT;
-  // a label outside [0, vocab) was reported by the forward pass; here it simply matches nothing
-  const int64_t label = (g_logprob != nullptr) ? labels[row] : -1;
-
-  // Vector path only when the input and output rows have the same 16-byte phase.
   const uintptr_t ain = reinterpret_cast<uintptr_t>(rowp);
   const uintptr_t aout = reinterpret_cast<uintptr_t>(outp);
   const bool same_phase = ((ain ^ aout) & 15u) == 0;
@@ -205,6 +171,124 @@ __global__ __launch_bounds__(WAVES * 64) void rowscore_backward_kernel(
     if (idx == label) y += f.lab;
     O::store1(outp, idx, y);
   }
+}
+
+// The whole workgroup fills one output row with zeros without reading anything.
+template <int DT, int WAVES>
+__device__ __forceinline__ void zero_row(char* outp, int64_t vocab) {
+  using E = Elem<DT>;
+  using O = ElemOut<DT>;
+  constexpr int NTHR = WAVES * 64;
+  constexpr int PV = E::kPerVec;
+  const int tid = threadIdx.x;
+  const uintptr_t aout = reinterpret_cast<uintptr_t>(outp);
+  int64_t head = static_cast<int64_t>(((16u - (aout & 15u)) & 15u) / E::kBytes);
+  if (head > vocab) head = vocab;
+  const int64_t nvec = (vocab - head) / PV;
+  const int64_t tail0 = head + nvec * PV;
+  u32x4* vout = reinterpret_cast<u32x4*>(outp + head * E::kBytes);
+  const u32x4 z = {0u, 0u, 0u, 0u};
+  for (int64_t k = tid; k < nvec; k += NTHR) __builtin_nontemporal_store(z, vout + k);
+  for (int64_t i = tid; i < head + (vocab - tail0); i += NTHR) O::store1(outp, (i < head) ? i : tail0 + (i - head), 0.f);
+}
+
+// The row constants of the gradient from what the forward pass left and the incoming gradients.
+template <bool EXACT>
+__device__ __forceinline__ typename std::conditional<EXACT, RowGradExact, RowGrad>::type make_row_grad(
+    float T, float lse, float H, float gl, float gh) {
+  typename std::conditional<EXACT, RowGradExact, RowGrad>::type f;
+  const float rT = 1.0f / T;
+  if constexpr (EXACT) {
+    f.sc.c = kLog2e;
+    f.sc.T = T;
+    f.sc.r = rT;
+    f.lse = lse;
+    f.a = -gh * rT;
+  } else {
+    f.c = kLog2e * rT;
+    f.lse2 = lse * kLog2e;
+    f.a = -(gh * kLn2f) * rT;
+  }
+  f.b = -(gl + gh * H) * rT;
+  f.lab = gl * rT;
+  return f;
+}
+
+// grid.x = n_rows, block = WAVES*64. EXACT selects RowGradExact (fp32 logits).
+template <int DT, int WAVES, int U, bool EXACT = (DT == 0)>
+__global__ __launch_bounds__(WAVES * 64) void rowscore_backward_kernel(
+    const void* logits, int64_t vocab, int64_t row_stride, const int64_t* __restrict__ labels,
+    const float* __restrict__ temperature, const float* __restrict__ lse, const float* __restrict__ entropy,
+    const float* __restrict__ g_logprob, const float* __restrict__ g_entropy, void* dlogits,
+    int64_t d_row_stride) {
+  using E = Elem<DT>;
+  const int64_t row = blockIdx.x;
+  const char* rowp = static_cast<const char*>(logits) + row * row_stride * E::kBytes;
+  char* outp = static_cast<char*>(dlogits) + row * d_row_stride * E::kBytes;
+
+  float T = 1.f;
+  if (temperature != nullptr) {
+    T = temperature[row];
+    T = (T < kMinTemperature) ? kMinTemperature : T;
+  }
+  const float gl = (g_logprob != nullptr) ? g_logprob[row] : 0.f;
+  const float gh = (g_entropy != nullptr) ? g_entropy[row] : 0.f;
+  const float H = (g_entropy != nullptr) ? entropy[row] : 0.f;
+  const auto f = make_row_grad<EXACT>(T, lse[row], H, gl, gh);
+  // a label outside [0, vocab) was reported by the forward pass; here it simply matches nothing
+  const int64_t label = (g_logprob != nullptr) ? labels[row] : -1;
+  backward_row<DT, WAVES, U>(rowp, outp, vocab, f, label);
+}
+
+// Backward of score_responses_kernel (rowscore_kernels.h). grid.x = n_rows, block = WAVES*64. Row r finds its
+// sequence by bisection like the forward kernel; inside a valid response window it reads the forward's logsumexp and
+// entropy and the incoming gradients at (b, col) of the (B, T_out) blocks and writes its gradient row; every other row
+// (prompts, sequences that failed validation, rows no sequence owns) gets zeros without its logits being read.
+template <int DT, int WAVES, int U, bool EXACT = (DT == 0)>
+__global__ __launch_bounds__(WAVES * 64) void score_responses_backward_kernel(
+    const void* logits, int64_t n_rows, int64_t vocab, int64_t row_stride, const int64_t* __restrict__ labels,
+    const int64_t* __restrict__ input_ids, const float* __restrict__ temperature,
+    const int64_t* __restrict__ cu_seqlens, const int64_t* __restrict__ response_lens, int64_t B, int64_t T_out,
+    const float* __restrict__ resp_lse, const float* __restrict__ resp_entropy,
+    const float* __restrict__ g_resp_logprob, const float* __restrict__ g_resp_entropy, void* dlogits,
+    int64_t d_row_stride) {
+  using E = Elem<DT>;
+  const int64_t row = blockIdx.x;
+  char* outp = static_cast<char*>(dlogits) + row * d_row_stride * E::kBytes;
+  int64_t lo = 0, hi = B;
+  while (hi - lo > 1) {
+    const int64_t mid = (lo + hi) >> 1;
+    if (cu_seqlens[mid] <= row) lo = mid; else hi = mid;
+  }
+  const int64_t b = lo;
+  bool in_window = false;
+  int64_t col = 0;
+  if (B > 0 && cu_seqlens[b] <= row && row < cu_seqlens[b + 1]) {
+    int why = 0;
+    const ResponseWindow w = response_window(cu_seqlens, response_lens, b, B, n_rows, T_out, &why);
+    if (w.ok) {
+      col = row - w.first;
+      in_window = col >= 0 && col < w.resp;
+    }
+  }
+  if (!in_window) {   // the whole workgroup
+    zero_row<DT, WAVES>(outp, vocab);
+    return;
+  }
+  const char* rowp = static_cast<const char*>(logits) + row * row_stride * E::kBytes;
+  float T = 1.f;
+  if (temperature != nullptr) {
+    T = temperature[row];
+    T = (T < kMinTemperature) ? kMinTemperature : T;
+  }
+  const int64_t at = b * T_out + col;
+  const float gl = (g_resp_logprob != nullptr) ? g_resp_logprob[at] : 0.f;
+  const float gh = (g_resp_entropy != nullptr) ? g_resp_entropy[at] : 0.f;
+  const float H = (g_resp_entropy != nullptr) ? resp_entropy[at] : 0.f;
+  const auto f = make_row_grad<EXACT>(T, resp_lse[at], H, gl, gh);
+  int64_t label = -1;
+  if (g_resp_logprob != nullptr) label = (input_ids != nullptr) ? input_ids[row + 1 < n_rows ? row + 1 : 0] : labels[row];
+  backward_row<DT, WAVES, U>(rowp, outp, vocab, f, label);
 }
 
 }  // namespace vrl

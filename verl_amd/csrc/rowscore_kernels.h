@@ -449,7 +449,7 @@ __global__ __launch_bounds__(WAVES * 64) void score_responses_kernel(
     const float* __restrict__ temperature, const int64_t* __restrict__ cu_seqlens,
     const int64_t* __restrict__ response_lens, int64_t B, int64_t T_out, float* __restrict__ out_logprob,
     float* __restrict__ out_entropy, float* __restrict__ resp_logprob, float* __restrict__ resp_entropy,
-    int32_t* err_flag) {
+    float* __restrict__ resp_lse, int32_t* err_flag) {
   constexpr int NTHR = WAVES * 64;
   const int64_t wg = blockIdx.x;
   if (wg >= n_rows) {
@@ -462,6 +462,7 @@ __global__ __launch_bounds__(WAVES * 64) void score_responses_kernel(
     for (int64_t j = from + threadIdx.x; j < T_out; j += NTHR) {
       if (resp_logprob != nullptr) resp_logprob[b * T_out + j] = 0.f;
       if (resp_entropy != nullptr) resp_entropy[b * T_out + j] = 0.f;
+      if (resp_lse != nullptr) resp_lse[b * T_out + j] = 0.f;
     }
     return;
   }
@@ -509,6 +510,7 @@ __global__ __launch_bounds__(WAVES * 64) void score_responses_kernel(
     if (in_window) {
       if (resp_logprob != nullptr) resp_logprob[b * T_out + col] = r.lp;
       if (resp_entropy != nullptr) resp_entropy[b * T_out + col] = r.H;
+      if (resp_lse != nullptr) resp_lse[b * T_out + col] = r.lse;
     }
   }
 }

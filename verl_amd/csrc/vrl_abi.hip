@@ -210,10 +210,10 @@ void launch_score_responses(const void* logits, int64_t n_rows, int64_t vocab, i
                             const int64_t* labels, const int64_t* input_ids, const float* temperature,
                             const int64_t* cu_seqlens, const int64_t* response_lens, int64_t B, int64_t T_out,
                             float* out_logprob, float* out_entropy, float* resp_logprob, float* resp_entropy,
-                            int32_t* err_flag, hipStream_t s) {
+                            float* resp_lse, int32_t* err_flag, hipStream_t s) {
   vrl::score_responses_kernel<DT, W, U, EXACT><<<dim3(static_cast<unsigned>(n_rows + B)), dim3(W * 64), 0, s>>>(
       logits, n_rows, vocab, row_stride, labels, input_ids, temperature, cu_seqlens, response_lens, B, T_out,
-      out_logprob, out_entropy, resp_logprob, resp_entropy, err_flag);
+      out_logprob, out_entropy, resp_logprob, resp_entropy, resp_lse, err_flag);
 }
 
 template <int DT, bool EXACT, typename... Args>
@@ -389,11 +389,11 @@ int vrl_score_responses(const void* logits, int dtype, int64_t n_rows, int64_t v
                         const int64_t* labels, const int64_t* input_ids, const float* temperature,
                         const int64_t* cu_seqlens, const int64_t* response_lens, int64_t B, int64_t T_out,
                         float* out_logprob, float* out_entropy, float* resp_logprob, float* resp_entropy,
-                        int32_t* err_flag, void* stream) {
+                        float* resp_lse, int32_t* err_flag, void* stream) {
   if (!known_dtype(dtype)) return VRL_ERR_DTYPE;
   if (n_rows < 0 || vocab <= 0 || row_stride < vocab || B < 0 || T_out < 0 || n_rows + B > kMaxGrid)
     return VRL_ERR_SHAPE;
-  if (resp_logprob == nullptr && resp_entropy == nullptr) return VRL_ERR_ARG;
+  if (resp_logprob == nullptr && resp_entropy == nullptr && resp_lse == nullptr) return VRL_ERR_ARG;
   if (labels != nullptr && input_ids != nullptr) return VRL_ERR_ARG;   // one source of labels
   if (out_logprob != nullptr && resp_logprob == nullptr) return VRL_ERR_ARG;
   if (out_entropy != nullptr && resp_entropy == nullptr) return VRL_ERR_ARG;
@@ -404,12 +404,13 @@ int vrl_score_responses(const void* logits, int dtype, int64_t n_rows, int64_t v
   const uintptr_t esize = (dtype == VRL_F32) ? 4 : 2;
   if (!aligned(logits, esize) || !aligned(labels, 8) || !aligned(input_ids, 8) || !aligned(temperature, 4) ||
       !aligned(cu_seqlens, 8) || !aligned(response_lens, 8) || !aligned(out_logprob, 4) ||
-      !aligned(out_entropy, 4) || !aligned(resp_logprob, 4) || !aligned(resp_entropy, 4) || !aligned(err_flag, 4))
+      !aligned(out_entropy, 4) || !aligned(resp_logprob, 4) || !aligned(resp_entropy, 4) || !aligned(resp_lse, 4) ||
+      !aligned(err_flag, 4))
     return VRL_ERR_ALIGN;
   hipStream_t s = static_cast<hipStream_t>(stream);
 #define VRL_SR_ARGS                                                                                               \
   n_rows, vocab, logits, n_rows, vocab, row_stride, labels, input_ids, temperature, cu_seqlens, response_lens, B, \
-      T_out, out_logprob, out_entropy, resp_logprob, resp_entropy, err_flag, s
+      T_out, out_logprob, out_entropy, resp_logprob, resp_entropy, resp_lse, err_flag, s
   if (dtype == VRL_F32) {
     if (temperature != nullptr)
       launch_score_responses_shaped<VRL_F32, true>(VRL_SR_ARGS);
@@ -421,6 +422,44 @@ int vrl_score_responses(const void* logits, int dtype, int64_t n_rows, int64_t v
     launch_score_responses_shaped<VRL_F16, false>(VRL_SR_ARGS);
   }
 #undef VRL_SR_ARGS
+  return launch_status();
+}
+
+int vrl_score_responses_backward(const void* logits, int dtype, int64_t n_rows, int64_t vocab, int64_t row_stride,
+                                 const int64_t* labels, const int64_t* input_ids, const float* temperature,
+                                 const int64_t* cu_seqlens, const int64_t* response_lens, int64_t B, int64_t T_out,
+                                 const float* resp_lse, const float* resp_entropy, const float* g_resp_logprob,
+                                 const float* g_resp_entropy, void* dlogits, int64_t d_row_stride, void* stream) {
+  if (!known_dtype(dtype)) return VRL_ERR_DTYPE;
+  if (n_rows < 0 || vocab <= 0 || row_stride < vocab || d_row_stride < vocab || B < 0 || T_out < 0 ||
+      n_rows > kMaxGrid)
+    return VRL_ERR_SHAPE;
+  if (B == 0 && n_rows > 0) return VRL_ERR_SHAPE;  // rows that belong to no sequence
+  if (g_resp_logprob == nullptr && g_resp_entropy == nullptr) return VRL_ERR_ARG;
+  if (labels != nullptr && input_ids != nullptr) return VRL_ERR_ARG;
+  if (n_rows == 0) return VRL_OK;
+  if (logits == nullptr || dlogits == nullptr) return VRL_ERR_NULL;
+  if (B > 0 && (cu_seqlens == nullptr || response_lens == nullptr || resp_lse == nullptr)) return VRL_ERR_NULL;
+  if (g_resp_logprob != nullptr && labels == nullptr && input_ids == nullptr) return VRL_ERR_NULL;
+  if (g_resp_entropy != nullptr && resp_entropy == nullptr && B > 0) return VRL_ERR_NULL;
+  const uintptr_t esize = (dtype == VRL_F32) ? 4 : 2;
+  if (!aligned(logits, esize) || !aligned(dlogits, esize) || !aligned(labels, 8) || !aligned(input_ids, 8) ||
+      !aligned(temperature, 4) || !aligned(cu_seqlens, 8) || !aligned(response_lens, 8) || !aligned(resp_lse, 4) ||
+      !aligned(resp_entropy, 4) || !aligned(g_resp_logprob, 4) || !aligned(g_resp_entropy, 4))
+    return VRL_ERR_ALIGN;
+  const dim3 grid(static_cast<unsigned>(n_rows));
+  const dim3 block(kBackwardWaves * 64);
+  hipStream_t s = static_cast<hipStream_t>(stream);
+#define VRL_SRB_ARGS                                                                                                  \
+  logits, n_rows, vocab, row_stride, labels, input_ids, temperature, cu_seqlens, response_lens, B, T_out, resp_lse, \
+      resp_entropy, g_resp_logprob, g_resp_entropy, dlogits, d_row_stride
+  if (dtype == VRL_F32)
+    vrl::score_responses_backward_kernel<VRL_F32, kBackwardWaves, kBackwardUnroll><<<grid, block, 0, s>>>(VRL_SRB_ARGS);
+  else if (dtype == VRL_BF16)
+    vrl::score_responses_backward_kernel<VRL_BF16, kBackwardWaves, kBackwardUnroll><<<grid, block, 0, s>>>(VRL_SRB_ARGS);
+  else
+    vrl::score_responses_backward_kernel<VRL_F16, kBackwardWaves, kBackwardUnroll><<<grid, block, 0, s>>>(VRL_SRB_ARGS);
+#undef VRL_SRB_ARGS
   return launch_status();
 }
 

@@ -440,6 +440,77 @@ def fused_logprob_entropy(
                     n_splits=n_splits, what="fused_logprob_entropy")
 
 
+def _score_responses_launch(x, lab, rolled, temp, cu, rl, T, want_logprob, want_entropy, per_token, want_lse, flag):
+    """One vrl_score_responses launch; returns (resp_logprob, resp_entropy, logprob, entropy, resp_lse)."""
+    n, V = x.shape
+    dev = x.device
+    B = rl.numel()
+    f32 = dict(dtype=torch.float32, device=dev)
+    r_lp = torch.empty((B, T), **f32) if want_logprob else None
+    r_h = torch.empty((B, T), **f32) if want_entropy else None
+    r_lse = torch.empty((B, T), **f32) if want_lse else None
+    t_lp = torch.empty(n, **f32) if (per_token and want_logprob) else None
+    t_h = torch.empty(n, **f32) if (per_token and want_entropy) else None
+    if B > 0:
+        lib = _lib.load()
+        with torch.cuda.device(dev):
+            st = lib.vrl_score_responses(
+                x.data_ptr() if n else None, _DTYPE_CODES[x.dtype], n, V, x.stride(0) if n > 1 else V,
+                _ptr(lab) if not rolled else None, _ptr(lab) if rolled else None, _ptr(temp),
+                cu.data_ptr(), rl.data_ptr(), B, T, _ptr(t_lp), _ptr(t_h), _ptr(r_lp), _ptr(r_h), _ptr(r_lse),
+                flag.data_ptr(), _lib.stream_ptr(dev))
+        _lib.check("vrl_score_responses", st)
+        counters["forward_passes"] += 1
+    return r_lp, r_h, t_lp, t_h, r_lse
+
+
+class _ScoreResponsesFunction(torch.autograd.Function):
+    """Differentiable padded response blocks of packed logits: vrl_score_responses forward (which also leaves the
+    logsumexp block), vrl_score_responses_backward for the logits' gradient — one pass each; rows outside every
+    response window get a zero gradient without their logits being read."""
+
+    @staticmethod
+    def forward(ctx, x, lab, rolled, temp, cu, rl, T, want_logprob, want_entropy, per_token, inplace, flag):
+        ctx.set_materialize_grads(False)
+        r_lp, r_h, t_lp, t_h, r_lse = _score_responses_launch(x, lab, rolled, temp, cu, rl, T, want_logprob, True,
+                                                              per_token, True, flag)
+        ctx.save_for_backward(x, lab, temp, cu, rl, r_lse, r_h)
+        ctx.rolled, ctx.T, ctx.inplace = bool(rolled), int(T), bool(inplace)
+        if not want_entropy:
+            r_h_out = None
+        else:
+            r_h_out = r_h
+        for t in (t_lp, t_h):
+            if t is not None:
+                ctx.mark_non_differentiable(t)
+        return r_lp, r_h_out, t_lp, (t_h if want_entropy else None)
+
+    @staticmethod
+    def backward(ctx, g_lp, g_h, _g_tlp, _g_th):
+        none = (None,) * 12
+        if g_lp is None and g_h is None:
+            return none
+        x, lab, temp, cu, rl, r_lse, r_h = ctx.saved_tensors
+        n, V = x.shape
+        dev = x.device
+        B = rl.numel()
+        dx = x if ctx.inplace else torch.empty((n, V), dtype=x.dtype, device=dev)
+        if n > 0:
+            gl = None if g_lp is None else g_lp.to(torch.float32).contiguous()
+            gh = None if g_h is None else g_h.to(torch.float32).contiguous()
+            use_lab = lab if gl is not None else None
+            lib = _lib.load()
+            with torch.cuda.device(dev):
+                st = lib.vrl_score_responses_backward(
+                    x.data_ptr(), _DTYPE_CODES[x.dtype], n, V, x.stride(0) if n > 1 else V,
+                    _ptr(use_lab) if not ctx.rolled else None, _ptr(use_lab) if ctx.rolled else None, _ptr(temp),
+                    cu.data_ptr(), rl.data_ptr(), B, ctx.T, r_lse.data_ptr(), r_h.data_ptr(), _ptr(gl), _ptr(gh),
+                    dx.data_ptr(), dx.stride(0) if n > 1 else V, _lib.stream_ptr(dev))
+            _lib.check("vrl_score_responses_backward", st)
+            counters["backward_passes"] += 1
+        return (dx,) + none[1:]
+
+
 def score_responses(
     logits: torch.Tensor,
     cu_seqlens: torch.Tensor,
@@ -452,6 +523,7 @@ def score_responses(
     want_logprob: bool = True,
     want_entropy: bool = True,
     per_token: bool = False,
+    inplace_backward: bool = False,
     check=None,
 ):
     """Packed ``logits`` ``(total_nnz, V)`` -> padded ``(B, max_response_len)`` response log-probs and entropies in ONE
@@ -465,18 +537,17 @@ def score_responses(
 
     Returns ``(resp_logprob | None, resp_entropy | None)``; with ``per_token`` also the ``(total_nnz,)`` vectors, as
     ``(resp_logprob, resp_entropy, logprob, entropy)``. Without ``per_token`` the logits of tokens outside every
-    response window (the prompts) are never read. Forward only. Device-side findings (a label outside the vocabulary:
-    IndexError; a sequence without a prompt token, a response longer than ``max_response_len``, offsets that do not
-    partition the rows: ValueError) follow ``check`` as in verl_amd.errors.
+    response window (the prompts) are never read. When grad is enabled and the logits require it, the two blocks are
+    differentiable with respect to the logits (``vrl_score_responses_backward``: one pass, zero rows for the prompts,
+    over the logits' own storage with ``inplace_backward``); the per-token vectors are not. Device-side findings (a
+    label outside the vocabulary: IndexError; a sequence without a prompt token, a response longer than
+    ``max_response_len``, offsets that do not partition the rows: ValueError) follow ``check`` as in verl_amd.errors.
     """
     what = "score_responses"
     _check_logits(logits, what)
     _errors.poll()
     if logits.dim() != 2:
         raise ValueError(f"{what}: logits must be packed (total_nnz, vocab), got shape {tuple(logits.shape)}")
-    if torch.is_grad_enabled() and logits.requires_grad:
-        raise NotImplementedError(f"{what} is a forward-only step (compute_log_prob); use fused_logprob_entropy "
-                                  "followed by response_slice when gradients are needed")
     if not (want_logprob or want_entropy):
         raise ValueError(f"{what}: nothing to compute")
     if want_logprob and (labels is None) == (input_ids is None):
@@ -484,6 +555,7 @@ def score_responses(
     x = _rows_2d(logits)
     n, V = x.shape
     dev = x.device
+    rolled = labels is None
     src = labels if labels is not None else input_ids
     lab = None
     if want_logprob:
@@ -503,22 +575,16 @@ def score_responses(
         raise ValueError(f"{what}: max_response_len must not be negative")
     if B == 0 and n > 0:
         raise ValueError(f"{what}: {n} rows but no sequence")
-    f32 = dict(dtype=torch.float32, device=dev)
-    r_lp = torch.empty((B, T), **f32) if want_logprob else None
-    r_h = torch.empty((B, T), **f32) if want_entropy else None
-    t_lp = torch.empty(n, **f32) if (per_token and want_logprob) else None
-    t_h = torch.empty(n, **f32) if (per_token and want_entropy) else None
+    flag = torch.zeros(1, dtype=torch.int32, device=dev)
+    if torch.is_grad_enabled() and logits.requires_grad:
+        r_lp, r_h, t_lp, t_h = _ScoreResponsesFunction.apply(
+            x, lab, rolled, temp, cu, rl, T, want_logprob, want_entropy, per_token,
+            inplace_backward and _is_view_safe(logits), flag)
+    else:
+        with torch.no_grad():
+            r_lp, r_h, t_lp, t_h, _ = _score_responses_launch(x, lab, rolled, temp, cu, rl, T, want_logprob,
+                                                              want_entropy, per_token, False, flag)
     if B > 0:
-        flag = torch.zeros(1, dtype=torch.int32, device=dev)
-        lib = _lib.load()
-        with torch.cuda.device(dev):
-            st = lib.vrl_score_responses(
-                x.data_ptr() if n else None, _DTYPE_CODES[x.dtype], n, V, x.stride(0) if n > 1 else V,
-                _ptr(lab) if labels is not None else None, _ptr(lab) if labels is None else None, _ptr(temp),
-                cu.data_ptr(), rl.data_ptr(), B, T, _ptr(t_lp), _ptr(t_h), _ptr(r_lp), _ptr(r_h), flag.data_ptr(),
-                _lib.stream_ptr(dev))
-        _lib.check("vrl_score_responses", st)
-        counters["forward_passes"] += 1
         _errors.report(flag, {
             _lib.VRL_FLAG_LABEL_OOB: (IndexError, f"{what}: a label is outside [0, {V})"),
             _lib.VRL_FLAG_SEQ_RANGE: (ValueError, f"{what}: cu_seqlens is not a partition of the {n} rows "
