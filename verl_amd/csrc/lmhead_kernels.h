@@ -5,11 +5,11 @@
 // vocabulary tiles (its "split"); per tile it runs the full contraction in steps of 64 (v_mfma_f32_32x32x16 on
 // bf16 / fp16, fp32 accumulators). A wavefront owns a 64 (vocabulary) x 128 (tokens) part of the tile: 8 blocks of
 // 32x32 = 128 accumulator registers, so two wavefronts fit a SIMD and one's matrix instructions cover the other's
-// waits. Operands go global -> LDS directly (128-bit loads, two 64 KiB stages = 128 KiB of LDS, one workgroup per CU),
-// swizzled so that the 128-bit fragment reads are free of bank conflicts (measured: SQ_LDS_BANK_CONFLICT = 0).
-// A step is four quarter steps of 16 contraction elements. The workgroup barrier sits before the LAST quarter's matrix
-// instructions: that quarter's fragments are already in registers, so behind the barrier the first fragments of the
-// next step are fetched and the loads of the step after are issued while the matrix cores still work on this step.
+// waits. Operands go global -> LDS directly (128-bit loads) into a ring of five 32 KiB operand tiles (all 160 KiB of a
+// CU's LDS, one workgroup per CU), swizzled so that the 128-bit fragment reads are free of bank conflicts (measured:
+// SQ_LDS_BANK_CONFLICT = 0). A step is four quarter steps of 16 contraction elements with one workgroup barrier, placed
+// before the LAST quarter's matrix instructions; the loads of the tiles two steps ahead are spread over the step
+// (lm_walk_tiles).
 // The MFMA is issued with the vocabulary on its row side so that a lane's 16 results of a block belong to ONE
 // token: the softmax state needs no cross-lane traffic until the very end.
 //
@@ -42,7 +42,8 @@ constexpr int kLmVocab = 256;                     // vocabulary rows per tile
 constexpr int kLmK = 64;                          // contraction elements per step: 128 bytes per tile row, whole cache lines
 constexpr int kLmRowBytes = kLmK * 2;
 constexpr int kLmTileBytes = 256 * kLmRowBytes;   // one operand tile in LDS (32 KiB)
-constexpr int kLmLdsBytes = 4 * kLmTileBytes;     // two stages of (W tile, H tile)
+constexpr int kLmRingSlots = 5;                   // operand tiles resident in LDS
+constexpr int kLmLdsBytes = kLmRingSlots * kLmTileBytes;   // 160 KiB: all of a CU's LDS
 constexpr int kLmMaxSplits = 64;
 
 template <int DT>
@@ -105,17 +106,43 @@ __device__ __forceinline__ LmWork lm_work(int64_t V, int64_t T, int n_splits, in
   return w;
 }
 
+// Which load a wavefront issues behind matrix instruction `mm` (0..7) of quarter step `sb` (0..3) of a step:
+// 0 none, 1..4 part 0..3 of the W tile two steps ahead, 5..8 part 0..3 of the H tile two steps ahead.
+__device__ constexpr int lm_load_slot(int sb, int mm) {
+  if (sb == 3) return (mm & 1) ? 5 + (mm >> 1) : 0;
+  if (sb == 0) return mm == 1 ? 1 : mm == 5 ? 2 : 0;
+  if (sb == 1) return mm == 1 ? 3 : mm == 5 ? 4 : 0;
+  return 0;
+}
+
 // The matrix-core walk shared by the forward and backward kernels. All 512 threads call it. For every vocabulary
 // tile of `work` it forms the 256 x 256 block of logits of tokens [tok0_ld, tok0_ld + 256) and hands this wavefront's
 // 64 (vocabulary) x 128 (tokens) part to on_tile(vt, acc): acc[i][j][v] is the logit of
 //   vocabulary row  tile_row0 + wv*64 + i*32 + 8*(v>>2) + 4*(lane>>5) + (v&3)
 //   token           tok0_ld + wt*128 + j*32 + (lane&31)
 // with wv = wave>>1, wt = wave&1 and tile_row0 = vt*256 (V-256 for an edge tile, whose rows below vt*256 repeat the
-// tile before). `lds` is 128 KiB, 1 KiB aligned. On return no load is in flight.
-template <int DT, class OnTile>
+// tile before). `lds` is kLmLdsBytes (160 KiB), 1 KiB aligned. On return no load is in flight; callers that reuse
+// `lds` afterwards put a workgroup barrier first.
+//
+// LDS is a ring of five 32 KiB operand tiles. Item 2s is the W tile of global step s (a step = 64 contraction elements
+// of one vocabulary tile), item 2s+1 its H tile; item n lives in slot n mod 5. During step s:
+//   quarters 0, 1   request W(s+2) into the slot H(s-1) left (two loads per quarter and wavefront)
+//   quarter 2       no loads; its end is the step's only workgroup barrier: every wavefront holds the fragments of
+//                   quarter 3 in registers, so W(s) and H(s) are dead, and W(s+1), H(s+1) have landed (vmcnt(4): only
+//                   the four W(s+2) loads may still be in flight)
+//   quarter 3       requests H(s+2) into the slot W(s) left, reads the first fragments of step s+1
+// so the 64 loads a step needs are spread over it instead of arriving at the address unit in one burst, a W tile (the
+// operand that comes from HBM) has five quarters to land and an H tile (L2 / infinity cache) three. Within a quarter
+// every matrix instruction is followed by at most one fragment read and one load; the scheduling-group barriers pin
+// that interleave (left alone, the compiler gathers the reads in front of the barrier, where all eight wavefronts
+// then wait for them together).
+// EPILOGUE_STORES: on_tile writes to global memory. Stores count in vmcnt like loads but complete in their own order,
+// so the first barrier after on_tile waits for everything.
+template <int DT, bool EPILOGUE_STORES, class OnTile>
 __device__ __forceinline__ void lm_walk_tiles(const uint16_t* __restrict__ W, const uint16_t* __restrict__ H, int64_t V,
                                               int64_t K, int64_t w_stride, int64_t h_stride, const LmWork& work,
                                               char* lds, OnTile&& on_tile) {
+  using FragT = typename LmFrag<DT>::type;
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);   // uniform: keeps tile addressing in scalar registers
@@ -127,8 +154,8 @@ __device__ __forceinline__ void lm_walk_tiles(const uint16_t* __restrict__ W, co
   int phys[4];
 #pragma unroll
   for (int sb = 0; sb < 4; ++sb) phys[sb] = (((2 * sb + (lane >> 5)) ^ ((lane >> 1) & 7)) * 16);
-  const int fragoff_w = (wv * 64 + (lane & 31)) * kLmRowBytes;
-  const int fragoff_h = kLmTileBytes + (wt * 128 + (lane & 31)) * kLmRowBytes;
+  const int fragoff_w = (wv * 64 + (lane & 31)) * kLmRowBytes;    // within a W slot
+  const int fragoff_h = (wt * 128 + (lane & 31)) * kLmRowBytes;   // within an H slot
 
   // One wave instruction moves 8 tile rows x 128 bytes into LDS (lane l lands at byte l*16 of the 1 KiB block): lane l
   // serves row r = l>>3 of the block and physical 16-byte slot p = l&7, and fetches the logical chunk that the swizzle
@@ -141,12 +168,11 @@ __device__ __forceinline__ void lm_walk_tiles(const uint16_t* __restrict__ W, co
   const uint32_t h_lane_e = (uint32_t)((lr * h_stride + lc_e * 8) * 2), h_lane_o = (uint32_t)((lr * h_stride + lc_o * 8) * 2);
   const uint64_t w_blk = (uint64_t)(8 * w_stride * 2), h_blk = (uint64_t)(8 * h_stride * 2);   // 8 rows in bytes
 
-  // Load cursor: global step (tile, k step); it runs two steps ahead of the compute cursor once the loop is going.
-  // wp / hp are uniform byte pointers to this wavefront's first row (it brings rows [32*wave, 32*wave + 32) with four
-  // instructions per operand) of the W and H tiles of the step to load next. A step advances both by one k step
-  // (128 bytes); at the end of a vocabulary tile W jumps to the next tile's rows and H returns to k = 0. Past the last
-  // step they stay put: the last tile is loaded once more into the stage nobody reads (in bounds, harmless), so the
-  // main loop needs no "is there more" branch around its loads.
+  // Two load cursors, one per operand: uniform byte pointers to this wavefront's first row (it brings rows
+  // [32*wave, 32*wave + 32) of a tile with four instructions) of the W / H tile to request next, and the ring slot it
+  // goes to. A step advances a pointer by 128 bytes; at the end of a vocabulary tile W jumps to the next tile's rows
+  // and H returns to k = 0. Past the last step the pointers stay put: the last tiles are requested again into slots
+  // nobody reads any more (in bounds, harmless), so the main loop needs no "is there more" branch around its loads.
   const int64_t total_steps = (work.vt_end > work.vt_begin ? (work.vt_end - work.vt_begin) : 0) * ksteps;
   auto uniform64 = [](uint64_t v) {
     const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)v);
@@ -156,52 +182,74 @@ __device__ __forceinline__ void lm_walk_tiles(const uint16_t* __restrict__ W, co
   auto vrow_of = [&](int64_t vt) { return (vt + 1) * kLmVocab <= V ? vt * kLmVocab : V - kLmVocab; };
   uint64_t wp = uniform64(reinterpret_cast<uint64_t>(W) + (uint64_t)(vrow_of(work.vt_begin) * w_stride * 2) + wave * 4 * w_blk);
   uint64_t hp = uniform64(reinterpret_cast<uint64_t>(H) + (uint64_t)(work.tok0_ld * h_stride * 2) + wave * 4 * h_blk);
-  int64_t pstep = 0, pvt = work.vt_begin;
-  int pks = 0;
-  auto load4 = [&](uint64_t base, uint64_t blk, uint32_t off_e, uint32_t off_o, char* dst) {
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const char* src = reinterpret_cast<const char*>(base + i * blk);
-      __builtin_amdgcn_global_load_lds((const VRL_GLOBAL_AS void*)(src + ((i & 1) ? off_o : off_e)),
-                                       (VRL_LDS_AS void*)(dst + i * 8 * kLmRowBytes), 16, 0, 0);
-    }
+  int64_t w_step = 0, w_vt = work.vt_begin, h_step = 0;
+  int w_ks = 0, h_ks = 0;
+  int w_slot = 0, h_slot = 1;
+  const int wave_rows = wave * 32 * kLmRowBytes;
+  auto load_w = [&](int i) {
+    const char* src = reinterpret_cast<const char*>(wp + i * w_blk);
+    __builtin_amdgcn_global_load_lds((const VRL_GLOBAL_AS void*)(src + ((i & 1) ? w_lane_o : w_lane_e)),
+                                     (VRL_LDS_AS void*)(lds + w_slot * kLmTileBytes + wave_rows + i * 8 * kLmRowBytes), 16, 0, 0);
   };
-  auto issue = [&]() {   // loads of global step `pstep` into stage pstep & 1
-    char* st = lds + (int)(pstep & 1) * 2 * kLmTileBytes + wave * 32 * kLmRowBytes;
-    load4(wp, w_blk, w_lane_e, w_lane_o, st);
-    load4(hp, h_blk, h_lane_e, h_lane_o, st + kLmTileBytes);
-    const bool more = pstep + 1 < total_steps;
-    ++pstep;
+  auto load_h = [&](int i) {
+    const char* src = reinterpret_cast<const char*>(hp + i * h_blk);
+    __builtin_amdgcn_global_load_lds((const VRL_GLOBAL_AS void*)(src + ((i & 1) ? h_lane_o : h_lane_e)),
+                                     (VRL_LDS_AS void*)(lds + h_slot * kLmTileBytes + wave_rows + i * 8 * kLmRowBytes), 16, 0, 0);
+  };
+  auto next_slot = [](int slot) { return slot + 2 >= kLmRingSlots ? slot + 2 - kLmRingSlots : slot + 2; };
+  auto advance_w = [&]() {
+    w_slot = next_slot(w_slot);
+    const bool more = w_step + 1 < total_steps;
+    ++w_step;
     if (more) {
-      if (pks + 1 == ksteps) {
-        const int64_t dv = vrow_of(pvt + 1) - vrow_of(pvt);
+      if (w_ks + 1 == ksteps) {
+        const int64_t dv = vrow_of(w_vt + 1) - vrow_of(w_vt);
         wp += (uint64_t)(dv * w_stride * 2) - (uint64_t)(ksteps - 1) * kLmRowBytes;
-        hp -= (uint64_t)(ksteps - 1) * kLmRowBytes;
-        pks = 0;
-        ++pvt;
+        w_ks = 0;
+        ++w_vt;
       } else {
         wp += kLmRowBytes;
-        hp += kLmRowBytes;
-        ++pks;
+        ++w_ks;
       }
     }
   };
-  typename LmFrag<DT>::type a[2][2], b[2][4];
-  auto read_frags = [&](int set, const char* stage, int sb) {
-#pragma unroll
-    for (int i = 0; i < 2; ++i) a[set][i] = *reinterpret_cast<const typename LmFrag<DT>::type*>(stage + fragoff_w + i * 32 * kLmRowBytes + phys[sb]);
-#pragma unroll
-    for (int j = 0; j < 4; ++j) b[set][j] = *reinterpret_cast<const typename LmFrag<DT>::type*>(stage + fragoff_h + j * 32 * kLmRowBytes + phys[sb]);
+  auto advance_h = [&]() {
+    h_slot = next_slot(h_slot);
+    const bool more = h_step + 1 < total_steps;
+    ++h_step;
+    if (more) {
+      if (h_ks + 1 == ksteps) {
+        hp -= (uint64_t)(ksteps - 1) * kLmRowBytes;
+        h_ks = 0;
+      } else {
+        hp += kLmRowBytes;
+        ++h_ks;
+      }
+    }
   };
+
+  FragT a[2][2], b[2][4];
   if (total_steps > 0) {
-    issue();   // step 0 -> stage 0
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-    __syncthreads();
-    read_frags(0, lds, 0);
-    issue();   // step 1 -> stage 1
+    // W(0), H(0), W(1), H(1); the first two have to land before anything is read
+#pragma unroll
+    for (int rep = 0; rep < 2; ++rep) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) load_w(i);
+      advance_w();
+#pragma unroll
+      for (int i = 0; i < 4; ++i) load_h(i);
+      advance_h();
+    }
+    asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
+    __builtin_amdgcn_s_barrier();
+#pragma unroll
+    for (int i = 0; i < 2; ++i) a[0][i] = *reinterpret_cast<const FragT*>(lds + fragoff_w + i * 32 * kLmRowBytes + phys[0]);
+#pragma unroll
+    for (int j = 0; j < 4; ++j) b[0][j] = *reinterpret_cast<const FragT*>(lds + kLmTileBytes + fragoff_h + j * 32 * kLmRowBytes + phys[0]);
   }
 
-  int64_t step = 0;
+  int cw = 0, ch = 1;   // ring slots of the step being computed
+  bool after_epilogue = false;
   for (int64_t vt = work.vt_begin; vt < work.vt_end; ++vt) {
     lm_f32x16 acc[2][4];
 #pragma unroll
@@ -211,37 +259,53 @@ __device__ __forceinline__ void lm_walk_tiles(const uint16_t* __restrict__ W, co
 #pragma unroll
         for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
 
-    for (int ks = 0; ks < ksteps; ++ks, ++step) {
-      const char* cur = lds + (int)(step & 1) * 2 * kLmTileBytes;
-      const char* nxt = lds + (int)((step + 1) & 1) * 2 * kLmTileBytes;
-      // Quarter steps 0..2 compute from fragments and read the next quarter's fragments from `cur`.
+    for (int ks = 0; ks < ksteps; ++ks) {
+      const int nw = next_slot(cw), nh = next_slot(ch);
 #pragma unroll
-      for (int sb = 0; sb < 3; ++sb) {
+      for (int sb = 0; sb < 4; ++sb) {
         const int cu = sb & 1, nx = cu ^ 1;
-        read_frags(nx, cur, sb + 1);
+        if (sb == 3) {
+          if (EPILOGUE_STORES && after_epilogue) {
+            asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+          } else {
+            asm volatile("s_waitcnt vmcnt(4) lgkmcnt(0)" ::: "memory");
+          }
+          __builtin_amdgcn_s_barrier();
+          after_epilogue = false;
+        }
+        // this quarter's matrix instructions run on fragment set `cu`; the reads fill set `nx` for the next quarter
+        // (of this step's tiles, or, in quarter 3, the first of the next step's)
+        const char* rw = lds + ((sb == 3) ? nw : cw) * kLmTileBytes + fragoff_w;
+        const char* rh = lds + ((sb == 3) ? nh : ch) * kLmTileBytes + fragoff_h;
+        const int rq = (sb + 1) & 3;
 #pragma unroll
-        for (int i = 0; i < 2; ++i)
+        for (int mm = 0; mm < 8; ++mm) {
+          const int i = mm >> 2, j = mm & 3;
+          acc[i][j] = LmFrag<DT>::mfma(a[cu][i], b[cu][j], acc[i][j]);
+          if (mm == 0) a[nx][0] = *reinterpret_cast<const FragT*>(rw + phys[rq]);
+          else if (mm < 5) b[nx][mm - 1] = *reinterpret_cast<const FragT*>(rh + (mm - 1) * 32 * kLmRowBytes + phys[rq]);
+          else if (mm == 5) a[nx][1] = *reinterpret_cast<const FragT*>(rw + 32 * kLmRowBytes + phys[rq]);
+          const int op = lm_load_slot(sb, mm);
+          if (op >= 5) load_h(op - 5);
+          else if (op >= 1) load_w(op - 1);
+        }
 #pragma unroll
-          for (int j = 0; j < 4; ++j)
-            acc[i][j] = LmFrag<DT>::mfma(a[cu][i], b[cu][j], acc[i][j]);
+        for (int mm = 0; mm < 8; ++mm) {
+          __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                                   // one matrix instruction
+          if (mm < 6) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);                       // one LDS read
+          if (lm_load_slot(sb, mm) != 0) __builtin_amdgcn_sched_group_barrier(0x010, 1, 0);   // one load
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        if (sb == 1) advance_w();
+        if (sb == 3) advance_h();
       }
-      // The barrier sits BEFORE the last quarter's matrix instructions: its fragments (set 1) are in registers, so
-      // every wavefront is done reading `cur`, and the next step's tile, requested a whole step ago, has landed in
-      // `nxt`. Behind the barrier the next step's first fragments are fetched and the loads of the step after are
-      // issued into `cur`, all underneath this quarter's matrix instructions.
-      asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
-      __syncthreads();
-      read_frags(0, nxt, 0);
-      issue();
-#pragma unroll
-      for (int i = 0; i < 2; ++i)
-#pragma unroll
-        for (int j = 0; j < 4; ++j)
-          acc[i][j] = LmFrag<DT>::mfma(a[1][i], b[1][j], acc[i][j]);
+      cw = nw;
+      ch = nh;
     }
     on_tile(vt, acc);
+    after_epilogue = true;
   }
-  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // the last, redundant loads still target the LDS stages
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // the last, redundant loads still target the ring
 }
 
 // grid.x = token blocks * n_splits, block = 512, dynamic LDS = kLmLdsBytes. Writes, per (token, split), the online-softmax
@@ -251,8 +315,8 @@ __global__ __launch_bounds__(kLmWaves * 64, 1) void lmhead_partial_kernel(
     const uint16_t* __restrict__ W, const uint16_t* __restrict__ H, int64_t V, int64_t T, int64_t K, int64_t w_stride,
     int64_t h_stride, const float* __restrict__ temperature, int n_splits, int tiles_per_split,
     int xcd_map, float* __restrict__ partials) {
-  extern __shared__ __attribute__((aligned(1024))) char lds[];  // [2 stages][W tile, H tile]
-  __shared__ float red[4][256][3];
+  extern __shared__ __attribute__((aligned(1024))) char lds[];  // the operand ring; its start serves the final merge
+  float (*red)[256][3] = reinterpret_cast<float (*)[256][3]>(lds);   // [4][256][3], used once the walk is over
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -272,7 +336,7 @@ __global__ __launch_bounds__(kLmWaves * 64, 1) void lmhead_partial_kernel(
     c[j] = make_scale<false>(temperature, tok).c;   // log2(e) / max(T, 1e-8), exactly what the finishing kernel uses
   }
 
-  lm_walk_tiles<DT>(W, H, V, K, w_stride, h_stride, work, lds, [&](int64_t vt, lm_f32x16 (&acc)[2][4]) {
+  lm_walk_tiles<DT, false>(W, H, V, K, w_stride, h_stride, work, lds, [&](int64_t vt, lm_f32x16 (&acc)[2][4]) {
     // fold 64 logits per token column into the running state (two passes over the accumulators: maximum, then
     // exponentials; nothing is buffered)
     const bool edge = (vt + 1) * kLmVocab > V;
@@ -335,6 +399,7 @@ __global__ __launch_bounds__(kLmWaves * 64, 1) void lmhead_partial_kernel(
     }
   });
 
+  __syncthreads();   // every wavefront has left the ring: its memory now serves the merge
   // combine: lanes l and l^32 hold the same tokens (other vocabulary rows), then the four vocabulary-quarter
   // wavefronts of a token half through LDS
 #pragma unroll
@@ -398,7 +463,7 @@ __global__ __launch_bounds__(kLmWaves * 64, 1) void lmhead_dlogits_kernel(
     const float* __restrict__ lse, const float* __restrict__ entropy, const float* __restrict__ g_logprob,
     const float* __restrict__ g_entropy, int n_splits, int tiles_per_split, int xcd_map, uint16_t* __restrict__ dlogits,
     int64_t d_stride) {
-  extern __shared__ __attribute__((aligned(1024))) char lds[];  // [2 stages][W tile, H tile]
+  extern __shared__ __attribute__((aligned(1024))) char lds[];  // the operand ring
   using O = ElemOut<DT>;
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -435,7 +500,7 @@ __global__ __launch_bounds__(kLmWaves * 64, 1) void lmhead_dlogits_kernel(
     out[j] = dlogits + tok * d_stride;
   }
 
-  lm_walk_tiles<DT>(W, H, V, K, w_stride, h_stride, work, lds, [&](int64_t vt, lm_f32x16 (&acc)[2][4]) {
+  lm_walk_tiles<DT, true>(W, H, V, K, w_stride, h_stride, work, lds, [&](int64_t vt, lm_f32x16 (&acc)[2][4]) {
     const bool edge = (vt + 1) * kLmVocab > V;
     const int vrow0 = (int)(edge ? V - kLmVocab : vt * kLmVocab) + wv * 64 + 4 * (lane >> 5);
     const int vfirst = (int)(vt * kLmVocab);   // rows below belong to the tile before
