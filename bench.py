@@ -15,6 +15,7 @@ launch stream), and the same computation in torch on the host cores (bounded sam
 from __future__ import annotations
 
 import argparse
+import ctypes
 import json
 import os
 import statistics
@@ -32,6 +33,7 @@ from verl_amd import spec_rl as sv  # noqa: E402
 from verl_amd import torch_functional as vf  # noqa: E402
 
 HBM_PEAK_GBPS = 8000.0
+MFMA_BF16_PEAK_TFLOPS = 2500.0
 # HBM bytes per row-kernel launch measured with rocprofv3 (--pmc FETCH_SIZE and --pmc WRITE_SIZE, one run each,
 # both scaled by what the same counter reads for a plain 1 GiB device copy: x1.999956 and x1.0). The workload
 # shapes are fixed, so the figure is a property of (kernel, shape); the counter summary is kept under profiles/.
@@ -436,6 +438,7 @@ def bench_lm_head(args, dev):
     wt = torch.empty(D, V, dtype=weight.dtype, device=dev)
     t_tr = timed(lambda: transpose_2d(weight.detach(), wt))
     flops_f, flops_fb = 2.0 * T * D * V, 6.0 * T * D * V
+    ceiling = mfma_ceiling(dev, args.steps)
     print(json.dumps({
         "metric": "tokens/sec of LM head + scoring, forward + backward, never holding more than one chunk of logits",
         "value": T / t_fb, "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
@@ -446,14 +449,16 @@ def bench_lm_head(args, dev):
                    "step": "verl_amd.fused_linear_for_ppo forward + torch.autograd.grad for hidden and weight"},
         "forward_ms": t_f * 1e3,
         "forward_tokens_per_s": T / t_f,
-        "roofline": {"bound": "mfma", "achieved": flops_fb / t_fb / 1e12, "peak": 2500.0, "unit": "TFLOP/s",
-                     "frac": flops_fb / t_fb / 1e12 / 2500.0, "traffic": None,
+        "roofline": {"bound": "mfma", "achieved": flops_fb / t_fb / 1e12, "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
+                     "frac": flops_fb / t_fb / 1e12 / MFMA_BF16_PEAK_TFLOPS, "traffic": None,
                      "kernel": "hipBLASLt bf16 GEMMs (library) + rowscore_kernel + rowscore_backward_kernel",
                      "forward_tflops": flops_f / t_f / 1e12},
-        "single_kernel_forward": {"ms": t_m * 1e3, "tflops": flops_f / t_m / 1e12, "frac_of_mfma_peak": flops_f / t_m / 1e12 / 2500.0,
+        "single_kernel_forward": {"ms": t_m * 1e3, "tflops": flops_f / t_m / 1e12, "frac_of_mfma_peak": flops_f / t_m / 1e12 / MFMA_BF16_PEAK_TFLOPS,
                                   "kernel": "lmhead_partial_kernel<bf16> + lmhead_finish_kernel (vrl_lmhead_score)",
                                   "parity_guard": {"rows": int(pick.numel()), "max_abs_err_logprob": e3, "max_abs_err_entropy": e4},
+                                  "frac_of_sustained_mfma_rate": flops_f / t_m / 1e12 / ceiling["tflops"],
                                   "note": "hand-written MFMA kernel, logits never written"},
+        "matrix_core_ceiling": ceiling,
         "matrix_core_backward": {"forward_backward_ms": t_fb_m * 1e3,
                                  "kernel": "library GEMM forward, lmhead_dlogits_kernel<bf16> (vrl_lmhead_dlogits) + two library "
                                            "GEMMs backward",
@@ -557,7 +562,48 @@ def bench_ceilings(args, dev):
             del dst
         del src
         torch.cuda.empty_cache()
+    out["matrix_cores"] = mfma_ceiling(dev, args.steps)
     print(json.dumps(out), flush=True)
+
+
+def mfma_ceiling(dev, steps):
+    """What the part sustains on bf16 32x32x16 matrix instructions alone (vrl_mfma_probe: one workgroup of 8 wavefronts
+    per CU, register operands, no memory traffic), with the shader clock it ran at: once on pseudo-random operands (what
+    the LM-head kernels' matrix time is measured against: the part holds a lower clock when the operand bits toggle),
+    once on small constants (the nominal rate). Returns the record of the random-operand run with the other inside."""
+    lib = _lib.load()
+    stream = torch.cuda.current_stream(dev).cuda_stream
+    n_wg = torch.cuda.get_device_properties(dev).multi_processor_count
+    iters = 20000   # 8 products per round: about as many per wavefront as the LM-head kernel issues at 8192 tokens
+    sink = torch.zeros(1, dtype=torch.float32, device=dev)
+    clocks = torch.zeros(2, dtype=torch.int64, device=dev)
+    khz = ctypes.c_int64(0)
+    records = []
+    for random_operands in (1, 0):
+        def run():
+            st = lib.vrl_mfma_probe(n_wg, iters, random_operands, sink.data_ptr(), clocks.data_ptr(), ctypes.addressof(khz),
+                                    stream)
+            _lib.check("vrl_mfma_probe", st)
+
+        spin_up(run)
+        evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(steps)]
+        for a, b in evs:
+            a.record()
+            run()
+            b.record()
+        torch.cuda.synchronize()
+        ms = sum(a.elapsed_time(b) for a, b in evs) / len(evs)
+        flops = n_wg * 8 * iters * 8 * 2.0 * 32 * 32 * 16
+        cyc, ticks = clocks.tolist()
+        records.append({"operands": "pseudo-random bf16 in (-1, 1)" if random_operands else "small constants",
+                        "avg_kernel_ms": ms, "tflops": flops / (ms * 1e-3) / 1e12,
+                        "frac_of_peak": flops / (ms * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS,
+                        "shader_clock_ghz": (cyc / ticks) * khz.value * 1e-6 if ticks else None})
+    out = {"probe": "v_mfma_f32_32x32x16_bf16 on register operands, 8 wavefronts per CU, nothing else",
+           "kernel": "mfma_probe_kernel", "workgroups": n_wg}
+    out.update(records[0])
+    out["with_constant_operands"] = records[1]
+    return out
 
 
 def bench_forward(args, dev, workload, steps, warmup, with_cpu_baseline):

@@ -225,6 +225,16 @@ def test_score_responses_backward_argument_errors(lib):
     assert call(n=0, x=None, out=None) == _lib.VRL_OK
 
 
+def test_mfma_probe_argument_errors(lib):
+    f = lib.vrl_mfma_probe
+    assert f(-1, 10, 1, P, None, None, None) == _lib.VRL_ERR_SHAPE
+    assert f(4, -1, 1, P, None, None, None) == _lib.VRL_ERR_SHAPE
+    assert f(4, 10, 1, None, None, None, None) == _lib.VRL_ERR_NULL
+    assert f(4, 10, 0, P + 2, None, None, None) == _lib.VRL_ERR_ALIGN
+    assert f(4, 10, 0, P, P + 4, None, None) == _lib.VRL_ERR_ALIGN
+    assert f(0, 10, 1, None, None, None, None) == _lib.VRL_OK
+
+
 def test_lmhead_dlogits_argument_errors(lib):
     f = lib.vrl_lmhead_dlogits
     ok = dict(h=P, w=P, dt=_lib.VRL_BF16, T=512, V=1024, K=128, hs=128, ws=128, lab=P, temp=None, lse=P, ent=P, gl=P, gh=P,

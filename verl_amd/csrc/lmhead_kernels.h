@@ -197,35 +197,27 @@ __device__ __forceinline__ void lm_walk_tiles(const uint16_t* __restrict__ W, co
                                      (VRL_LDS_AS void*)(lds + h_slot * kLmTileBytes + wave_rows + i * 8 * kLmRowBytes), 16, 0, 0);
   };
   auto next_slot = [](int slot) { return slot + 2 >= kLmRingSlots ? slot + 2 - kLmRingSlots : slot + 2; };
+  // (branch-free: the quarter steps of a step stay one basic block, which lets the compiler count outstanding LDS
+  // reads exactly instead of waiting for all of them at every block boundary)
   auto advance_w = [&]() {
     w_slot = next_slot(w_slot);
     const bool more = w_step + 1 < total_steps;
+    const bool tile_end = w_ks + 1 == ksteps;
+    const int64_t dv = vrow_of(w_vt + 1) - vrow_of(w_vt);
+    const uint64_t jump = (uint64_t)(dv * w_stride * 2) - (uint64_t)(ksteps - 1) * kLmRowBytes;
+    wp += more ? (tile_end ? jump : (uint64_t)kLmRowBytes) : (uint64_t)0;
+    w_vt += (more && tile_end) ? 1 : 0;
+    w_ks = more ? (tile_end ? 0 : w_ks + 1) : w_ks;
     ++w_step;
-    if (more) {
-      if (w_ks + 1 == ksteps) {
-        const int64_t dv = vrow_of(w_vt + 1) - vrow_of(w_vt);
-        wp += (uint64_t)(dv * w_stride * 2) - (uint64_t)(ksteps - 1) * kLmRowBytes;
-        w_ks = 0;
-        ++w_vt;
-      } else {
-        wp += kLmRowBytes;
-        ++w_ks;
-      }
-    }
   };
   auto advance_h = [&]() {
     h_slot = next_slot(h_slot);
     const bool more = h_step + 1 < total_steps;
+    const bool tile_end = h_ks + 1 == ksteps;
+    const uint64_t back = (uint64_t)0 - (uint64_t)(ksteps - 1) * kLmRowBytes;
+    hp += more ? (tile_end ? back : (uint64_t)kLmRowBytes) : (uint64_t)0;
+    h_ks = more ? (tile_end ? 0 : h_ks + 1) : h_ks;
     ++h_step;
-    if (more) {
-      if (h_ks + 1 == ksteps) {
-        hp -= (uint64_t)(ksteps - 1) * kLmRowBytes;
-        h_ks = 0;
-      } else {
-        hp += kLmRowBytes;
-        ++h_ks;
-      }
-    }
   };
 
   FragT a[2][2], b[2][4];

@@ -77,4 +77,63 @@ __global__ __launch_bounds__(256) void stream_probe_flat_copy_kernel(const u32x4
   }
 }
 
+// Matrix-core probe: what the part sustains on v_mfma_f32_32x32x16_bf16 with nothing else in the way. 512 threads per
+// workgroup (two wavefronts per SIMD, like the LM-head kernels), every wavefront issues `iters` rounds of the 8 products
+// of a 64 x 128 wavefront tile (2 A fragments x 4 B fragments) on register operands. `random_operands` fills the
+// fragments with pseudo-random bf16 values in (-1, 1) (what real activations and weights look like to the multipliers);
+// otherwise every element is a small integer multiple of 1/8, the same in all products. The part is power-managed: the
+// clock it holds, and with it the rate, depends on how much the operand bits toggle. Thread 0 of workgroup 0 reports how
+// many shader clocks and how many ticks of the constant-rate wall clock its loop took, i.e. the clock the part ran at.
+typedef __bf16 probe_bf16x8 __attribute__((ext_vector_type(8)));
+typedef float probe_f32x16 __attribute__((ext_vector_type(16)));
+
+__device__ __forceinline__ float probe_uniform(uint32_t x) {   // (-1, 1), from a 32-bit mix
+  x ^= x >> 16;
+  x *= 0x7feb352dU;
+  x ^= x >> 15;
+  x *= 0x846ca68bU;
+  x ^= x >> 16;
+  return static_cast<float>(static_cast<int32_t>(x)) * (1.0f / 2147483648.0f);
+}
+
+__global__ __launch_bounds__(512, 1) void mfma_probe_kernel(int64_t iters, int random_operands, float* __restrict__ sink,
+                                                            int64_t* __restrict__ clocks) {
+  probe_bf16x8 a[2], b[4];
+  const uint32_t me = blockIdx.x * 512u + threadIdx.x;
+#pragma unroll
+  for (int f = 0; f < 6; ++f)
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const float v = random_operands ? probe_uniform(me * 48u + f * 8u + i) : 0.125f * static_cast<float>((threadIdx.x + i) & 7);
+      if (f < 2) a[f][i] = static_cast<__bf16>(v); else b[f - 2][i] = static_cast<__bf16>(v);
+    }
+  probe_f32x16 acc[2][4];
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
+  const long long c0 = clock64();
+  const long long w0 = wall_clock64();
+  for (int64_t it = 0; it < iters; ++it) {
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[i], b[j], acc[i][j], 0, 0, 0);
+  }
+  float total = 0.f;
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) total += acc[i][j][v];
+  if (clocks != nullptr && blockIdx.x == 0 && threadIdx.x == 0) {
+    clocks[0] = clock64() - c0;
+    clocks[1] = wall_clock64() - w0;
+  }
+  if (total == 12345.678f) sink[0] = total;   // keeps the products alive; practically never true
+}
+
 }  // namespace vrl

@@ -795,6 +795,23 @@ int vrl_stream_probe(const void* src, void* dst, int64_t n_rows, int64_t row_byt
   return launch_status();
 }
 
+int vrl_mfma_probe(int64_t n_workgroups, int64_t iters, int random_operands, float* sink, int64_t* clocks,
+                   int64_t* wall_clock_khz, void* stream) {
+  if (n_workgroups < 0 || iters < 0 || n_workgroups > kMaxGrid) return VRL_ERR_SHAPE;
+  if (wall_clock_khz != nullptr) {
+    int dev = 0, khz = 0;
+    if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&khz, hipDeviceAttributeWallClockRate, dev) != hipSuccess)
+      return launch_status() == VRL_OK ? VRL_ERR_HIP : VRL_ERR_HIP;  // the message, if any, is kept for vrl_last_hip_error
+    *wall_clock_khz = khz;
+  }
+  if (n_workgroups == 0) return VRL_OK;
+  if (sink == nullptr) return VRL_ERR_NULL;
+  if (!aligned(sink, 4) || !aligned(clocks, 8)) return VRL_ERR_ALIGN;
+  vrl::mfma_probe_kernel<<<dim3(static_cast<unsigned>(n_workgroups)), dim3(512), 0, static_cast<hipStream_t>(stream)>>>(
+      iters, random_operands != 0 ? 1 : 0, sink, clocks);
+  return launch_status();
+}
+
 const char* vrl_strerror(int status) {
   switch (status) {
     case VRL_OK: return "ok";
