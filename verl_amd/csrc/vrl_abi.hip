@@ -800,8 +800,10 @@ int vrl_mfma_probe(int64_t n_workgroups, int64_t iters, int random_operands, flo
   if (n_workgroups < 0 || iters < 0 || n_workgroups > kMaxGrid) return VRL_ERR_SHAPE;
   if (wall_clock_khz != nullptr) {
     int dev = 0, khz = 0;
-    if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&khz, hipDeviceAttributeWallClockRate, dev) != hipSuccess)
-      return launch_status() == VRL_OK ? VRL_ERR_HIP : VRL_ERR_HIP;  // the message, if any, is kept for vrl_last_hip_error
+    if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&khz, hipDeviceAttributeWallClockRate, dev) != hipSuccess) {
+      launch_status();   // keeps the runtime's message for vrl_last_hip_error
+      return VRL_ERR_HIP;
+    }
     *wall_clock_khz = khz;
   }
   if (n_workgroups == 0) return VRL_OK;
