@@ -532,13 +532,17 @@ def bench_ceilings(args, dev):
            "peak": HBM_PEAK_GBPS, "probes": []}
     sink = torch.zeros(1, dtype=torch.int32, device=dev)
     for name, rows, row_bytes in (("c3 micro-batch, 8192 x 151936 bf16", 8192, 151936 * 2),
-                                  ("c2, 65536 x 152064 bf16", 65536, 152064 * 2)):
+                                  ("c2, 65536 x 152064 bf16", 65536, 152064 * 2),
+                                  ("c1, 4096 x 32000 f32", 4096, 32000 * 4)):
         src = torch.empty(rows * row_bytes // 2, dtype=torch.int16, device=dev).fill_(5)
-        for mode, what, factor in ((0, "non-temporal read", 1), (1, "non-temporal copy", 2),
-                                   (2, "non-temporal copy, 512 workgroups walking the whole buffer", 2)):
-            if mode != 0 and rows * row_bytes > (8 << 30):
+        small = rows * row_bytes < (1 << 30)
+        modes = ((3, "non-temporal read, 32-bit row shape", 1),) if small else (
+            (0, "non-temporal read", 1), (1, "non-temporal copy", 2),
+            (2, "non-temporal copy, 512 workgroups walking the whole buffer", 2))
+        for mode, what, factor in modes:
+            if mode in (1, 2) and rows * row_bytes > (8 << 30):
                 continue
-            dst = torch.empty_like(src) if mode != 0 else None
+            dst = torch.empty_like(src) if mode in (1, 2) else None
 
             def run():
                 st = lib.vrl_stream_probe(src.data_ptr(), None if dst is None else dst.data_ptr(), rows, row_bytes, mode,
@@ -553,7 +557,7 @@ def bench_ceilings(args, dev):
                 b.record()
             torch.cuda.synchronize()
             ms = sum(a.elapsed_time(b) for a, b in evs) / len(evs)
-            if mode != 0 and not torch.equal(dst, src):
+            if dst is not None and not torch.equal(dst, src):
                 raise SystemExit("bench: the copy probe did not copy")
             out["probes"].append({"buffer": name, "probe": what, "kernel": "stream_probe_kernel", "avg_kernel_ms": ms,
                                   "bytes_per_launch": factor * rows * row_bytes,

@@ -384,6 +384,7 @@ int vrl_fused_score_verify(const void* logits, int dtype, int64_t n_rows, int64_
  *   mode 1: read src, write dst (n_rows * row_bytes each, not overlapping)                           -> backward ceiling
  *   mode 2: the same copy by 512 workgroups walking the buffer as a whole, 8 KiB per wavefront and trip (the fastest
  *           read+write stream found on MI355X; what no row-shaped read+write kernel can exceed)
+ *   mode 3: mode 0 with the workgroup shape the forward kernel uses for 32-bit logits (4 wavefronts, 4 loads in flight)
  * A measurement aid with no counterpart in the reference.
  */
 int vrl_stream_probe(const void* src, void* dst, int64_t n_rows, int64_t row_bytes, int mode, uint32_t* sink,

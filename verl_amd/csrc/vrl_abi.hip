@@ -773,10 +773,11 @@ int vrl_fused_score_verify(const void* logits, int dtype, int64_t n_rows, int64_
 
 int vrl_stream_probe(const void* src, void* dst, int64_t n_rows, int64_t row_bytes, int mode, uint32_t* sink,
                      void* stream) {
-  if (mode < 0 || mode > 2) return VRL_ERR_ARG;
+  if (mode < 0 || mode > 3) return VRL_ERR_ARG;
   if (n_rows < 0 || row_bytes < 0 || row_bytes % 16 != 0 || n_rows > kMaxGrid) return VRL_ERR_SHAPE;
   if (n_rows == 0 || row_bytes == 0) return VRL_OK;
-  if (src == nullptr || (mode != 0 && dst == nullptr) || (mode == 0 && sink == nullptr)) return VRL_ERR_NULL;
+  const bool reads_only = mode == 0 || mode == 3;
+  if (src == nullptr || (!reads_only && dst == nullptr) || (reads_only && sink == nullptr)) return VRL_ERR_NULL;
   if (!aligned(src, 16) || !aligned(dst, 16) || !aligned(sink, 4)) return VRL_ERR_ALIGN;
   const dim3 grid(static_cast<unsigned>(n_rows));
   hipStream_t s = static_cast<hipStream_t>(stream);
@@ -786,6 +787,10 @@ int vrl_stream_probe(const void* src, void* dst, int64_t n_rows, int64_t row_byt
     vrl::stream_probe_kernel<RowShape<VRL_BF16>::kWaves, RowShape<VRL_BF16>::kUnroll, false>
         <<<grid, dim3(RowShape<VRL_BF16>::kWaves * 64), 0, s>>>(static_cast<const vrl::u32x4*>(src), nullptr, vecs,
                                                                 0x9e3779b9u, sink);
+  else if (mode == 3)   // the forward kernel's workgroup shape for 32-bit logits
+    vrl::stream_probe_kernel<RowShape<VRL_F32>::kWaves, RowShape<VRL_F32>::kUnroll, false>
+        <<<grid, dim3(RowShape<VRL_F32>::kWaves * 64), 0, s>>>(static_cast<const vrl::u32x4*>(src), nullptr, vecs,
+                                                               0x9e3779b9u, sink);
   else if (mode == 1)
     vrl::stream_probe_kernel<kBackwardWaves, kBackwardUnroll, true><<<grid, dim3(kBackwardWaves * 64), 0, s>>>(
         static_cast<const vrl::u32x4*>(src), static_cast<vrl::u32x4*>(dst), vecs, 0u, nullptr);
