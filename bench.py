@@ -460,10 +460,11 @@ def bench_lm_head(args, dev):
                                   "note": "hand-written MFMA kernel, logits never written"},
         "matrix_core_ceiling": ceiling,
         "matrix_core_backward": {"forward_backward_ms": t_fb_m * 1e3,
-                                 "kernel": "library GEMM forward, lmhead_dlogits_kernel<bf16> (vrl_lmhead_dlogits) + two library "
-                                           "GEMMs backward",
+                                 "kernel": "library GEMM forward; backward lmhead_dlogits_kernel<bf16> (vrl_lmhead_dlogits), "
+                                           "lm_gemm_nt_kernel<bf16> (vrl_gemm_nt) for d hidden, a library GEMM for d W",
                                  "note": "the logits are formed again by the hand-written MFMA kernel and their gradient "
-                                         "is written from registers (no GEMM into the buffer, no pass over it)"},
+                                         "is written from registers (no GEMM into the buffer, no pass over it); d hidden "
+                                         "comes from the same main loop"},
         "weight_transpose": {"ms": t_tr * 1e3, "gbps": 2.0 * V * D * 2 / t_tr / 1e9, "kernel": "transpose_kernel<2>"},
         "parity_guard": {"rows": 256, "max_abs_err_logprob": e1, "max_abs_err_entropy": e2},
     }), flush=True)

@@ -225,6 +225,39 @@ def test_score_responses_backward_argument_errors(lib):
     assert call(n=0, x=None, out=None) == _lib.VRL_OK
 
 
+def test_gemm_nt_argument_errors(lib):
+    f = lib.vrl_gemm_nt
+    ok = dict(x=P, y=P, dt=_lib.VRL_BF16, NX=512, NY=256, K=256, xs=256, ys=256, out=P, os=512, acc=0, parts=1, ws=None)
+
+    def call(**kw):
+        a = {**ok, **kw}
+        return f(a["x"], a["y"], a["dt"], a["NX"], a["NY"], a["K"], a["xs"], a["ys"], a["out"], a["os"], a["acc"],
+                 a["parts"], a["ws"], None)
+
+    assert call(dt=_lib.VRL_F32) == _lib.VRL_ERR_DTYPE
+    assert call(NX=128) == _lib.VRL_ERR_SHAPE
+    assert call(NY=255) == _lib.VRL_ERR_SHAPE
+    assert call(NX=514, os=516) == _lib.VRL_ERR_SHAPE              # columns of out in quads
+    assert call(K=96) == _lib.VRL_ERR_SHAPE
+    assert call(K=64, xs=64, ys=64) == _lib.VRL_ERR_SHAPE          # the pipeline needs two steps
+    assert call(xs=128) == _lib.VRL_ERR_SHAPE
+    assert call(ys=260) == _lib.VRL_ERR_SHAPE
+    assert call(os=510) == _lib.VRL_ERR_SHAPE
+    assert call(parts=0) == _lib.VRL_ERR_ARG
+    assert call(parts=17) == _lib.VRL_ERR_ARG
+    assert call(parts=4) == _lib.VRL_ERR_ARG                        # ranges of fewer than two steps
+    assert call(x=None) == _lib.VRL_ERR_NULL
+    assert call(out=None) == _lib.VRL_ERR_NULL
+    assert call(K=512, xs=512, ys=512, parts=2) == _lib.VRL_ERR_NULL   # ranges need the workspace
+    assert call(x=P + 8) == _lib.VRL_ERR_ALIGN
+    assert call(out=P + 4) == _lib.VRL_ERR_ALIGN
+    need = ctypes.c_int64(-1)
+    parts = lib.vrl_gemm_nt_plan(_lib.VRL_BF16, 3584, 4096, 152064, ctypes.addressof(need))
+    assert 1 <= parts <= 16 and need.value == (parts * 3584 * 4096 if parts > 1 else 0)
+    assert lib.vrl_gemm_nt_plan(_lib.VRL_F32, 3584, 4096, 152064, None) == _lib.VRL_ERR_DTYPE
+    assert lib.vrl_gemm_nt_plan(_lib.VRL_BF16, 3584, 152064, 4096, ctypes.addressof(need)) == 1 and need.value == 0
+
+
 def test_mfma_probe_argument_errors(lib):
     f = lib.vrl_mfma_probe
     assert f(-1, 10, 1, P, None, None, None) == _lib.VRL_ERR_SHAPE

@@ -523,6 +523,153 @@ __global__ __launch_bounds__(kLmWaves * 64, 1) void lmhead_dlogits_kernel(
 }
 
 
+// ---- the two products of the backward on the same walk -----------------------------------------------------------
+// out[y][x] (+)= sum_k X[x][k] * Y[y][k] for X (NX, K) and Y (NY, K), both contiguous along k: d hidden = G . W with
+// X = W^T (hidden, vocab) and Y = G (tokens, vocab); d W = G^T . H with X = H^T (hidden, tokens) and Y = G^T (vocab,
+// tokens). X plays the walk's vocabulary side (a lane's accumulator quad is 4 consecutive x of one y, i.e. one 8-byte
+// store of out[y][x..x+3]), Y its token side.
+//
+// A work item is (y block of 256 rows, `tiles_per_item` x tiles, one of `k_parts` ranges of the contraction). Items
+// are dealt so that the workgroups resident on one XCD together form py x px patches of (y block, x split) pairs of
+// one contraction range and share their operand tiles through its L2; ids past the last patch leave at once.
+// MODE 0 stores the product in the operands' type, MODE 1 adds it to what `out` holds (one rounding, like a GEMM with
+// beta = 1), MODE 2 stores fp32 partial sums at partials[(kp * NY + y) * NX + x] for lm_gemm_reduce_kernel.
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+
+template <int DT>
+__device__ __forceinline__ void lm_unpack2(uint32_t w, float* x);   // two 16-bit elements of type DT -> fp32
+template <>
+__device__ __forceinline__ void lm_unpack2<1>(uint32_t w, float* x) {
+  x[0] = __uint_as_float(w << 16);
+  x[1] = __uint_as_float(w & 0xffff0000u);
+}
+template <>
+__device__ __forceinline__ void lm_unpack2<2>(uint32_t w, float* x) { Elem<2>::unpack2(w, x); }
+
+struct LmGemmShape {
+  int64_t NX, NY;          // rows of X / of Y = columns / rows of out
+  int64_t k_steps;         // contraction length / 64
+  int k_parts;             // ranges the contraction is cut into
+  int steps_per_part;      // ceil(k_steps / k_parts); the last range may be shorter
+  int tiles_per_item;      // x tiles one workgroup walks
+  int py, px;              // patch of (y blocks, x splits) per XCD
+};
+
+template <int DT, int MODE>
+__global__ __launch_bounds__(kLmWaves * 64, 1) void lm_gemm_nt_kernel(
+    const uint16_t* __restrict__ X, const uint16_t* __restrict__ Y, LmGemmShape g, int64_t x_stride, int64_t y_stride,
+    uint16_t* __restrict__ out, int64_t out_stride, float* __restrict__ partials) {
+  extern __shared__ __attribute__((aligned(1024))) char lds[];  // the operand ring
+  using O = ElemOut<DT>;
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wv = wave >> 1;
+  const int wt = wave & 1;
+
+  const int64_t nyb = (g.NY + kLmTokens - 1) / kLmTokens;
+  const int64_t nxt = (g.NX + kLmVocab - 1) / kLmVocab;
+  const int64_t nxs = (nxt + g.tiles_per_item - 1) / g.tiles_per_item;
+  const int64_t patches_y = nyb / g.py, patches_x = nxs / g.px;   // the host passes py | nyb and px | nxs
+  const int64_t per_part = patches_y * patches_x;
+  const int psize = g.py * g.px;
+  const int64_t id = blockIdx.x;
+  const int64_t local = id >> 3;
+  const int64_t patch = (local / psize) * 8 + (id & 7);
+  if (patch >= per_part * g.k_parts) return;   // the whole workgroup, before any barrier
+  const int within = (int)(local % psize);
+  const int kp = (int)(patch / per_part);
+  const int64_t r = patch % per_part;
+  const int64_t yb = (r % patches_y) * g.py + within % g.py;
+  const int64_t xsplit = (r / patches_y) * g.px + within / g.py;
+
+  LmWork work;
+  work.split = kp;
+  work.tok0 = yb * kLmTokens;
+  work.tok0_ld = work.tok0 + kLmTokens <= g.NY ? work.tok0 : g.NY - kLmTokens;
+  work.vt_begin = xsplit * g.tiles_per_item;
+  work.vt_end = work.vt_begin + g.tiles_per_item;
+  if (work.vt_end > nxt) work.vt_end = nxt;
+  const int64_t step0 = (int64_t)kp * g.steps_per_part;
+  int64_t nsteps = g.k_steps - step0;
+  if (nsteps > g.steps_per_part) nsteps = g.steps_per_part;
+
+  lm_walk_tiles<DT, true>(X + step0 * kLmK, Y + step0 * kLmK, g.NX, nsteps * kLmK, x_stride, y_stride, work, lds,
+                          [&](int64_t vt, lm_f32x16 (&acc)[2][4]) {
+    const bool edge = (vt + 1) * kLmVocab > g.NX;
+    const int64_t xrow0 = (edge ? g.NX - kLmVocab : vt * kLmVocab) + wv * 64 + 4 * (lane >> 5);
+    const int64_t xfirst = vt * kLmVocab;   // rows below belong to the tile before
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int64_t y = work.tok0_ld + wt * 128 + j * 32 + (lane & 31);
+      const bool y_mine = y >= work.tok0;
+#pragma unroll
+      for (int i = 0; i < 2; ++i) {
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          const int64_t x = xrow0 + i * 32 + 8 * q;   // first of 4 consecutive columns of out (a multiple of 4)
+          if (y_mine && x >= xfirst) {
+            float v[4];
+#pragma unroll
+            for (int e = 0; e < 4; ++e) v[e] = acc[i][j][q * 4 + e];
+            if constexpr (MODE == 2) {
+              f32x4 pk = {v[0], v[1], v[2], v[3]};
+              *reinterpret_cast<f32x4*>(partials + ((int64_t)kp * g.NY + y) * g.NX + x) = pk;
+            } else {
+              uint2* dst = reinterpret_cast<uint2*>(out + y * out_stride + x);
+              if constexpr (MODE == 1) {
+                const uint2 old = *dst;
+                float o[4];
+                lm_unpack2<DT>(old.x, o);
+                lm_unpack2<DT>(old.y, o + 2);
+#pragma unroll
+                for (int e = 0; e < 4; ++e) v[e] += o[e];
+              }
+              uint2 pk;
+              pk.x = O::pack2(v[0], v[1]);
+              pk.y = O::pack2(v[2], v[3]);
+              *dst = pk;
+            }
+          }
+        }
+        __builtin_amdgcn_sched_barrier(0);
+      }
+    }
+  });
+}
+
+// out[y][x] (+)= sum over the k_parts partial sums, added in range order (deterministic). One thread per 4 columns.
+template <int DT, bool ACCUMULATE>
+__global__ __launch_bounds__(256) void lm_gemm_reduce_kernel(const float* __restrict__ partials, int64_t NX, int64_t NY,
+                                                             int k_parts, uint16_t* __restrict__ out, int64_t out_stride) {
+  using O = ElemOut<DT>;
+  const int64_t quads_per_row = NX / 4;
+  const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (idx >= NY * quads_per_row) return;
+  const int64_t y = idx / quads_per_row;
+  const int64_t x = (idx % quads_per_row) * 4;
+  f32x4 s = *reinterpret_cast<const f32x4*>(partials + y * NX + x);
+  for (int p = 1; p < k_parts; ++p) {
+    const f32x4 v = __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(partials + ((int64_t)p * NY + y) * NX + x));
+    s += v;
+  }
+  uint2* dst = reinterpret_cast<uint2*>(out + y * out_stride + x);
+  if constexpr (ACCUMULATE) {
+    const uint2 old = *dst;
+    float o[4];
+    lm_unpack2<DT>(old.x, o);
+    lm_unpack2<DT>(old.y, o + 2);
+    s.x += o[0];
+    s.y += o[1];
+    s.z += o[2];
+    s.w += o[3];
+  }
+  uint2 pk;
+  pk.x = O::pack2(s.x, s.y);
+  pk.y = O::pack2(s.z, s.w);
+  *dst = pk;
+}
+
 // grid.x = ceil(T / 4), block = 256: wavefront w of a workgroup finishes token blockIdx.x * 4 + w.
 template <int DT>
 __global__ __launch_bounds__(256) void lmhead_finish_kernel(

@@ -337,6 +337,112 @@ int check_lmhead_shape(int dtype, int64_t n_tokens, int64_t vocab, int64_t hidde
   return VRL_OK;
 }
 
+
+// How vrl_gemm_nt cuts its work: enough (y block, x split, contraction range) items to fill the part's CUs in whole
+// rounds. One workgroup per CU runs at a time (the kernels take all of its LDS).
+struct GemmPlan {
+  vrl::LmGemmShape shape;
+  int64_t items;
+};
+
+int device_cus() {
+  static std::atomic<int> cus[kMaxDevices];
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return 256;
+  int n = cus[dev].load(std::memory_order_acquire);
+  if (n == 0) {
+    if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
+    cus[dev].store(n, std::memory_order_release);
+  }
+  return n;
+}
+
+int largest_divisor_up_to(int64_t n, int limit) {
+  for (int d = limit; d > 1; --d)
+    if (n % d == 0) return d;
+  return 1;
+}
+
+GemmPlan gemm_plan(int64_t NX, int64_t NY, int64_t K, int forced_parts) {
+  GemmPlan p;
+  vrl::LmGemmShape& g = p.shape;
+  g.NX = NX;
+  g.NY = NY;
+  g.k_steps = K / vrl::kLmK;
+  const int64_t nyb = (NY + vrl::kLmTokens - 1) / vrl::kLmTokens;
+  const int64_t nxt = (NX + vrl::kLmVocab - 1) / vrl::kLmVocab;
+  const int cus = device_cus();
+  // x tiles per workgroup: 2 when that still leaves 8 rounds of work (halves the share of pipeline fill and drain)
+  g.tiles_per_item = (nxt % 2 == 0 && nyb * (nxt / 2) >= 8LL * cus) ? 2 : 1;
+  const int64_t nxs = (nxt + g.tiles_per_item - 1) / g.tiles_per_item;
+  const int64_t base = nyb * nxs;
+  int best = 1;
+  if (forced_parts > 0) {
+    best = forced_parts;
+  } else if (base * 10 < 7LL * cus) {
+    // Too few output tiles for the CUs: cut the contraction until ~85 % of them have a workgroup. More than that does
+    // not pay: the part is power-bound on this loop, idle CUs raise the clock of the busy ones, and every cut costs a
+    // pass over fp32 partial sums (measured at 4096 x 152064 -> 3584: 224 workgroups 3.75 ms, 1792 in 8 ranges 3.82).
+    const int64_t want = (85LL * cus + 99) / 100;
+    int64_t parts = (want + base - 1) / base;
+    if (parts > 16) parts = 16;
+    while (parts > 1 && g.k_steps / parts < 32) --parts;
+    best = static_cast<int>(parts);
+  }
+  g.steps_per_part = static_cast<int>((g.k_steps + best - 1) / best);
+  g.k_parts = static_cast<int>((g.k_steps + g.steps_per_part - 1) / g.steps_per_part);   // no empty range
+  g.py = largest_divisor_up_to(nyb, 4);
+  g.px = largest_divisor_up_to(nxs, 8);
+  p.items = base * g.k_parts;
+  return p;
+}
+
+template <int DT>
+int launch_gemm_nt(const void* x, const void* y, const GemmPlan& plan, int64_t x_stride, int64_t y_stride, void* out,
+                   int64_t out_stride, int accumulate, float* workspace, hipStream_t s) {
+  const vrl::LmGemmShape& g = plan.shape;
+  const int psize = g.py * g.px;
+  const int64_t patches = plan.items / psize;
+  const int64_t grid = ((patches + 7) / 8) * 8 * psize;
+  if (grid > kMaxGrid) return VRL_ERR_SHAPE;
+  const dim3 gd(static_cast<unsigned>(grid)), bd(vrl::kLmWaves * 64);
+  const uint16_t* X = static_cast<const uint16_t*>(x);
+  const uint16_t* Y = static_cast<const uint16_t*>(y);
+  uint16_t* O = static_cast<uint16_t*>(out);
+#define VRL_GEMM_LAUNCH(MODE)                                                                                       \
+  {                                                                                                                 \
+    static std::atomic<bool> raised[kMaxDevices];                                                                   \
+    const int rs = raise_lds_limit(reinterpret_cast<const void*>(vrl::lm_gemm_nt_kernel<DT, MODE>), raised);        \
+    if (rs != VRL_OK) return rs;                                                                                    \
+    vrl::lm_gemm_nt_kernel<DT, MODE><<<gd, bd, vrl::kLmLdsBytes, s>>>(X, Y, g, x_stride, y_stride, O, out_stride,   \
+                                                                        workspace);                                 \
+  }
+  if (g.k_parts > 1) {
+    VRL_GEMM_LAUNCH(2)
+    const int64_t quads = g.NY * (g.NX / 4);
+    const dim3 rg(static_cast<unsigned>((quads + 255) / 256));
+    if (accumulate)
+      vrl::lm_gemm_reduce_kernel<DT, true><<<rg, dim3(256), 0, s>>>(workspace, g.NX, g.NY, g.k_parts, O, out_stride);
+    else
+      vrl::lm_gemm_reduce_kernel<DT, false><<<rg, dim3(256), 0, s>>>(workspace, g.NX, g.NY, g.k_parts, O, out_stride);
+  } else if (accumulate) {
+    VRL_GEMM_LAUNCH(1)
+  } else {
+    VRL_GEMM_LAUNCH(0)
+  }
+#undef VRL_GEMM_LAUNCH
+  return launch_status();
+}
+
+int check_gemm_nt(int dtype, int64_t NX, int64_t NY, int64_t K, int64_t x_stride, int64_t y_stride, int64_t out_stride) {
+  if (dtype != VRL_BF16 && dtype != VRL_F16) return VRL_ERR_DTYPE;
+  if (NX < vrl::kLmVocab || NY < vrl::kLmTokens || NX % 4 != 0 || K < 2 * vrl::kLmK || K % vrl::kLmK != 0 ||
+      x_stride < K || y_stride < K || x_stride % 8 != 0 || y_stride % 8 != 0 || out_stride < NX || out_stride % 4 != 0)
+    return VRL_ERR_SHAPE;
+  if (NY * (NX / 4) > kMaxGrid * 256LL) return VRL_ERR_SHAPE;
+  return VRL_OK;
+}
+
 }  // namespace
 
 extern "C" {
@@ -672,6 +778,30 @@ int vrl_lmhead_dlogits(const void* hidden, const void* weight, int dtype, int64_
                                            s);
   return launch_lmhead_dlogits<VRL_F16>(hidden, weight, n_tokens, vocab, hidden_size, h_stride, w_stride, labels,
                                         temperature, lse, entropy, g_logprob, g_entropy, n_splits, dlogits, d_stride, s);
+}
+
+int vrl_gemm_nt_plan(int dtype, int64_t NX, int64_t NY, int64_t K, int64_t* workspace_floats) {
+  const int st = check_gemm_nt(dtype, NX, NY, K, K, K, NX);
+  if (st != VRL_OK) return st;
+  const GemmPlan p = gemm_plan(NX, NY, K, 0);
+  if (workspace_floats != nullptr) *workspace_floats = p.shape.k_parts > 1 ? p.shape.k_parts * NX * NY : 0;
+  return p.shape.k_parts;
+}
+
+int vrl_gemm_nt(const void* x, const void* y, int dtype, int64_t NX, int64_t NY, int64_t K, int64_t x_stride,
+                int64_t y_stride, void* out, int64_t out_stride, int accumulate, int k_parts, float* workspace,
+                void* stream) {
+  const int st = check_gemm_nt(dtype, NX, NY, K, x_stride, y_stride, out_stride);
+  if (st != VRL_OK) return st;
+  if (k_parts < 1 || k_parts > 16 || K / vrl::kLmK / k_parts < 2) return VRL_ERR_ARG;
+  if (x == nullptr || y == nullptr || out == nullptr) return VRL_ERR_NULL;
+  const GemmPlan p = gemm_plan(NX, NY, K, k_parts);
+  if (p.shape.k_parts > 1 && workspace == nullptr) return VRL_ERR_NULL;
+  if (!aligned(x, 16) || !aligned(y, 16) || !aligned(out, 8) || !aligned(workspace, 16)) return VRL_ERR_ALIGN;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  if (dtype == VRL_BF16)
+    return launch_gemm_nt<VRL_BF16>(x, y, p, x_stride, y_stride, out, out_stride, accumulate, workspace, s);
+  return launch_gemm_nt<VRL_F16>(x, y, p, x_stride, y_stride, out, out_stride, accumulate, workspace, s);
 }
 
 int vrl_transpose(const void* src, int elem_size, int64_t rows, int64_t cols, int64_t src_stride,

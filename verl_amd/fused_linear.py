@@ -19,6 +19,7 @@ import torch
 
 from . import _lib
 from . import errors as _errors
+from . import gemm as _gemm
 from .layout import transpose_2d
 from .torch_functional import _DTYPE_CODES, _ptr
 
@@ -59,6 +60,16 @@ def _score_chunk(lib, logits, labels, temp, lp, h, lse, flag, stream):
                           labels.data_ptr(), _ptr(temp), lp.data_ptr(), h.data_ptr(), None, lse.data_ptr(),
                           flag.data_ptr(), stream)
     _lib.check("vrl_rowscore", st)
+
+
+def _d_hidden(grad_logits, weight, weight_t, out, own_kernel):
+    """out = grad_logits @ weight: this package's matrix-core kernel (``vrl_gemm_nt``) when asked for and the shapes
+    allow, the library otherwise (with the transposed copy of the weight when there is one: both operands contiguous
+    along the vocabulary)."""
+    if own_kernel and weight_t is not None and _gemm.gemm_nt_takes(weight_t, grad_logits) and out.stride(0) % 4 == 0:
+        _gemm.gemm_nt(weight_t, grad_logits, out=out)
+    else:
+        torch.matmul(grad_logits, weight if weight_t is None else weight_t.t(), out=out)
 
 
 class _FusedLinearForPPOFunction(torch.autograd.Function):
@@ -141,7 +152,7 @@ class _FusedLinearForPPOFunction(torch.autograd.Function):
                         logits.stride(0), stream)
                     _lib.check("vrl_lmhead_dlogits", st)
                     if need_dh:
-                        torch.matmul(logits, weight if weight_t is None else weight_t.t(), out=d_hidden[lo:hi])
+                        _d_hidden(logits, weight, weight_t, d_hidden[lo:hi], True)
                     if need_dw:
                         d_weight.addmm_(logits.t(), transpose_2d(hidden[lo:hi]).t() if half else hidden[lo:hi])
                     continue
@@ -165,7 +176,7 @@ class _FusedLinearForPPOFunction(torch.autograd.Function):
             if kept is not None:
                 # the gradient over all tokens' logits is in `kept`: one product each, nothing to accumulate
                 if need_dh:
-                    torch.matmul(kept, weight if weight_t is None else weight_t.t(), out=d_hidden)
+                    _d_hidden(kept, weight, weight_t, d_hidden, ctx.kernels == "mfma")
                 if need_dw:
                     torch.matmul(kept.t(), transpose_2d(hidden).t() if half else hidden, out=d_weight)
         return d_hidden, d_weight, None, None, None, None, None
@@ -187,8 +198,9 @@ def fused_linear_for_ppo(hidden_states: torch.Tensor, vocab_weights: torch.Tenso
     projecting again and forms ``d hidden`` and ``d W`` with one product each. Such a graph can be differentiated once.
 
     ``kernels`` chooses who forms the logits: ``"library"`` (a GEMM per chunk into the buffer) or ``"mfma"`` (this
-    package's matrix-core kernels: no buffer at all when no gradient is recorded, and a backward that writes the
-    gradient of the logits straight from registers); None takes ``DEFAULT_KERNELS``.
+    package's matrix-core kernels: no buffer at all when no gradient is recorded, a backward that writes the
+    gradient of the logits straight from registers and forms ``d hidden`` with ``vrl_gemm_nt``; ``d W`` stays a
+    library product); None takes ``DEFAULT_KERNELS``.
     """
     kernels = DEFAULT_KERNELS if kernels is None else kernels
     if kernels not in ("library", "mfma"):
@@ -231,8 +243,8 @@ def lm_head_score_mfma(hidden_states: torch.Tensor, vocab_weights: torch.Tensor,
     (verl/utils/kernel/kernels.py:531-756). bf16 or fp16 operands, at least 256 tokens and 256 vocabulary entries,
     hidden size a multiple of 64. ``temperature`` is a float or one value per token. The logits are kept in fp32
     (a GEMM that writes them rounds them to the operand type first), so results are slightly closer to the
-    all-fp32 value than ``fused_linear_for_ppo``'s. On MI355X it is slower than the library GEMM + row kernel that
-    ``fused_linear_for_ppo`` uses (9.3 ms against 6.4 ms at 8192 x 3584 -> 152064); it needs no logits buffer at all.
+    all-fp32 value than ``fused_linear_for_ppo``'s. On MI355X it is 3-5 % slower than the library GEMM + row kernel that
+    ``fused_linear_for_ppo`` uses (6.7 ms against 6.5 ms at 8192 x 3584 -> 152064); it needs no logits buffer at all.
     """
     if not hidden_states.is_cuda or not vocab_weights.is_cuda:
         raise RuntimeError("lm_head_score_mfma: tensors must be on the GPU; verl_amd has no CPU implementation")
