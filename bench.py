@@ -424,15 +424,22 @@ def bench_lm_head(args, dev):
         lp, h = fused_linear_for_ppo(hidden, weight, ids, temperature, chunk, False, "mfma")
         return torch.autograd.grad((lp, h), (hidden, weight), (g_lp, g_h))
 
-    # guard: the matrix-core backward against the library one
-    ga, gb = fwd_bwd(), fwd_bwd_mfma()
-    for x, y, what in ((ga[0], gb[0], "d hidden"), (ga[1], gb[1], "d weight")):
-        err = (x.float() - y.float()).abs().max().item()
-        if not err <= 3e-2 * max(x.float().abs().max().item(), 1e-6):
-            raise SystemExit(f"bench: matrix-core backward disagrees with the library path on {what} ({err})")
-    del ga, gb
+    def fwd_bwd_library():
+        lp, h = fused_linear_for_ppo(hidden, weight, ids, temperature, chunk, keep, "library")
+        return torch.autograd.grad((lp, h), (hidden, weight), (g_lp, g_h))
+
+    # guard: the paths with this package's matrix-core kernels against the all-library one
+    ga = fwd_bwd_library()
+    for gb, which in ((fwd_bwd(), "default"), (fwd_bwd_mfma(), "matrix-core")):
+        for x, y, what in ((ga[0], gb[0], "d hidden"), (ga[1], gb[1], "d weight")):
+            err = (x.float() - y.float()).abs().max().item()
+            if not err <= 3e-2 * max(x.float().abs().max().item(), 1e-6):
+                raise SystemExit(f"bench: the {which} backward disagrees with the library path on {what} ({err})")
+        del gb
+    del ga
     t_f = timed(fwd)
     t_fb = timed(fwd_bwd)
+    t_fb_lib = timed(fwd_bwd_library)
     t_m = timed(fwd_mfma)
     t_fb_m = timed(fwd_bwd_mfma)
     wt = torch.empty(D, V, dtype=weight.dtype, device=dev)
@@ -446,12 +453,14 @@ def bench_lm_head(args, dev):
         "data": "synthetic",
         "config": {"workload": "lm_head_8192x3584_v152064_bf16", "chunk_tokens": chunk, "keep_logits": keep,
                    "temperature": temperature,
-                   "step": "verl_amd.fused_linear_for_ppo forward + torch.autograd.grad for hidden and weight"},
+                   "step": "verl_amd.fused_linear_for_ppo forward + torch.autograd.grad for hidden and weight, default "
+                           "kernels (\"auto\": library GEMMs for the logits and d W, vrl_gemm_nt for d hidden)"},
         "forward_ms": t_f * 1e3,
         "forward_tokens_per_s": T / t_f,
         "roofline": {"bound": "mfma", "achieved": flops_fb / t_fb / 1e12, "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
                      "frac": flops_fb / t_fb / 1e12 / MFMA_BF16_PEAK_TFLOPS, "traffic": None,
-                     "kernel": "hipBLASLt bf16 GEMMs (library) + rowscore_kernel + rowscore_backward_kernel",
+                     "kernel": "hipBLASLt bf16 GEMMs (logits, d W) + lm_gemm_nt_kernel<bf16> (d hidden) + rowscore_kernel + "
+                               "rowscore_backward_kernel",
                      "forward_tflops": flops_f / t_f / 1e12},
         "single_kernel_forward": {"ms": t_m * 1e3, "tflops": flops_f / t_m / 1e12, "frac_of_mfma_peak": flops_f / t_m / 1e12 / MFMA_BF16_PEAK_TFLOPS,
                                   "kernel": "lmhead_partial_kernel<bf16> + lmhead_finish_kernel (vrl_lmhead_score)",
@@ -459,6 +468,7 @@ def bench_lm_head(args, dev):
                                   "frac_of_sustained_mfma_rate": flops_f / t_m / 1e12 / ceiling["tflops"],
                                   "note": "hand-written MFMA kernel, logits never written"},
         "matrix_core_ceiling": ceiling,
+        "all_library": {"forward_backward_ms": t_fb_lib * 1e3, "kernel": "torch.matmul for every product"},
         "matrix_core_backward": {"forward_backward_ms": t_fb_m * 1e3,
                                  "kernel": "library GEMM forward; backward lmhead_dlogits_kernel<bf16> (vrl_lmhead_dlogits), "
                                            "lm_gemm_nt_kernel<bf16> (vrl_gemm_nt) for d hidden, a library GEMM for d W",

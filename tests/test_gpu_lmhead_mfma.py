@@ -129,6 +129,36 @@ def test_dlogits_matches_fp64_autograd(dev, dtype, T, V, K, splits):
         assert bool((err <= rel * want.abs() + 2e-6).all()), err.max().item()
 
 
+@pytest.mark.parametrize("kernels", ["auto", "mfma"])
+def test_d_hidden_comes_from_the_matrix_core_product(dev, kernels):
+    """From 2048 tokens on the backward holds a transposed copy of the weight and, unless told "library", forms d hidden
+    with vrl_gemm_nt: same tolerances against torch autograd as the other paths, and the launch is counted."""
+    from verl_amd import gemm
+
+    g = torch.Generator(device=dev).manual_seed(78)
+    T, D, V = 2304, 512, 32256
+    hidden = torch.empty(T, D, device=dev).uniform_(-0.5, 0.5, generator=g).bfloat16().requires_grad_()
+    weight = torch.empty(V, D, device=dev).uniform_(-0.5, 0.5, generator=g).bfloat16().requires_grad_()
+    labels = torch.randint(0, V, (T,), generator=g, device=dev)
+    g_ent = torch.empty(T, device=dev).uniform_(-0.5, 0.5, generator=g)
+    g_lp = torch.empty(T, device=dev).uniform_(-1, 1, generator=g)
+    logits = torch.matmul(hidden.float(), weight.float().t()) / 1.5
+    ref_ent = torch.logsumexp(logits, -1) - (torch.softmax(logits, -1) * logits).sum(-1)
+    ref_lp = -torch.nn.functional.cross_entropy(logits, labels, reduction="none")
+    d_ref_h, d_ref_w = torch.autograd.grad((ref_ent, ref_lp), (hidden, weight), (g_ent, g_lp))
+    for chunk, keep in ((1024, False), (4096, False), (4096, True)):
+        before = gemm.counters["gemm_nt"]
+        lp, ent = fused_linear_for_ppo(hidden, weight, labels, 1.5, chunk_size=chunk, keep_logits=keep, kernels=kernels)
+        d_h, d_w = torch.autograd.grad((ent, lp), (hidden, weight), (g_ent, g_lp))
+        assert gemm.counters["gemm_nt"] > before
+        torch.testing.assert_close(d_ref_h.float(), d_h.float(), atol=1e-2, rtol=1e-2)
+        torch.testing.assert_close(d_ref_w.float(), d_w.float(), atol=1e-2, rtol=1e-2)
+    before = gemm.counters["gemm_nt"]
+    lp, ent = fused_linear_for_ppo(hidden, weight, labels, 1.5, kernels="library")
+    torch.autograd.grad((ent, lp), (hidden, weight), (g_ent, g_lp))
+    assert gemm.counters["gemm_nt"] == before
+
+
 def test_fused_linear_with_the_matrix_core_kernels(dev):
     """fused_linear_for_ppo(kernels="mfma"): forward from vrl_lmhead_score, backward through vrl_lmhead_dlogits and the
     two products, against torch autograd on the fp32 composition at the reference's tolerances

@@ -36,6 +36,7 @@ namespace vrl {
 #define VRL_GLOBAL_AS __attribute__((address_space(1)))
 
 typedef float lm_f32x16 __attribute__((ext_vector_type(16)));
+typedef float lm_f32x4 __attribute__((ext_vector_type(4)));
 
 constexpr int kLmTokens = 256;                    // tokens per workgroup tile
 constexpr int kLmVocab = 256;                     // vocabulary rows per tile
@@ -54,12 +55,18 @@ struct LmFrag<1> {
   __device__ static __forceinline__ lm_f32x16 mfma(type a, type b, lm_f32x16 c) {
     return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
   }
+  __device__ static __forceinline__ lm_f32x4 mfma16(type a, type b, lm_f32x4 c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0);
+  }
 };
 template <>
 struct LmFrag<2> {
   typedef _Float16 type __attribute__((ext_vector_type(8)));
   __device__ static __forceinline__ lm_f32x16 mfma(type a, type b, lm_f32x16 c) {
     return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
+  }
+  __device__ static __forceinline__ lm_f32x4 mfma16(type a, type b, lm_f32x4 c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, c, 0, 0, 0);
   }
 };
 
@@ -138,7 +145,7 @@ __device__ constexpr int lm_load_slot(int sb, int mm) {
 // then wait for them together).
 // EPILOGUE_STORES: on_tile writes to global memory. Stores count in vmcnt like loads but complete in their own order,
 // so the first barrier after on_tile waits for everything.
-template <int DT, bool EPILOGUE_STORES, class OnTile>
+template <int DT, int SHAPE, bool EPILOGUE_STORES, class OnTile>
 __device__ __forceinline__ void lm_walk_tiles(const uint16_t* __restrict__ W, const uint16_t* __restrict__ H, int64_t V,
                                               int64_t K, int64_t w_stride, int64_t h_stride, const LmWork& work,
                                               char* lds, OnTile&& on_tile) {
@@ -149,13 +156,6 @@ __device__ __forceinline__ void lm_walk_tiles(const uint16_t* __restrict__ W, co
   const int wv = wave >> 1;  // vocabulary quarter of the tile
   const int wt = wave & 1;   // token half of the tile
   const int ksteps = (int)(K / kLmK);
-
-  // fragment addressing: row (within its 32-row block) = lane&31, logical chunk = 2*sub + (lane>>5), sub in 0..3
-  int phys[4];
-#pragma unroll
-  for (int sb = 0; sb < 4; ++sb) phys[sb] = (((2 * sb + (lane >> 5)) ^ ((lane >> 1) & 7)) * 16);
-  const int fragoff_w = (wv * 64 + (lane & 31)) * kLmRowBytes;    // within a W slot
-  const int fragoff_h = (wt * 128 + (lane & 31)) * kLmRowBytes;   // within an H slot
 
   // One wave instruction moves 8 tile rows x 128 bytes into LDS (lane l lands at byte l*16 of the 1 KiB block): lane l
   // serves row r = l>>3 of the block and physical 16-byte slot p = l&7, and fetches the logical chunk that the swizzle
@@ -220,84 +220,179 @@ __device__ __forceinline__ void lm_walk_tiles(const uint16_t* __restrict__ W, co
     ++h_step;
   };
 
-  FragT a[2][2], b[2][4];
-  if (total_steps > 0) {
-    // W(0), H(0), W(1), H(1); the first two have to land before anything is read
+  if constexpr (SHAPE == 32) {
+    // fragment addressing: row (within its 32-row block) = lane&31, logical chunk = 2*sub + (lane>>5), sub in 0..3
+    int phys[4];
 #pragma unroll
-    for (int rep = 0; rep < 2; ++rep) {
-#pragma unroll
-      for (int i = 0; i < 4; ++i) load_w(i);
-      advance_w();
-#pragma unroll
-      for (int i = 0; i < 4; ++i) load_h(i);
-      advance_h();
-    }
-    asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
-    __builtin_amdgcn_s_barrier();
-#pragma unroll
-    for (int i = 0; i < 2; ++i) a[0][i] = *reinterpret_cast<const FragT*>(lds + fragoff_w + i * 32 * kLmRowBytes + phys[0]);
-#pragma unroll
-    for (int j = 0; j < 4; ++j) b[0][j] = *reinterpret_cast<const FragT*>(lds + kLmTileBytes + fragoff_h + j * 32 * kLmRowBytes + phys[0]);
-  }
+    for (int sb = 0; sb < 4; ++sb) phys[sb] = (((2 * sb + (lane >> 5)) ^ ((lane >> 1) & 7)) * 16);
+    const int fragoff_w = (wv * 64 + (lane & 31)) * kLmRowBytes;    // within a W slot
+    const int fragoff_h = (wt * 128 + (lane & 31)) * kLmRowBytes;   // within an H slot
 
-  int cw = 0, ch = 1;   // ring slots of the step being computed
-  bool after_epilogue = false;
-  for (int64_t vt = work.vt_begin; vt < work.vt_end; ++vt) {
-    lm_f32x16 acc[2][4];
+    FragT a[2][2], b[2][4];
+    if (total_steps > 0) {
+      // W(0), H(0), W(1), H(1); the first two have to land before anything is read
 #pragma unroll
-    for (int i = 0; i < 2; ++i)
+      for (int rep = 0; rep < 2; ++rep) {
 #pragma unroll
-      for (int j = 0; j < 4; ++j)
+        for (int i = 0; i < 4; ++i) load_w(i);
+        advance_w();
 #pragma unroll
-        for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
-
-    for (int ks = 0; ks < ksteps; ++ks) {
-      const int nw = next_slot(cw), nh = next_slot(ch);
-#pragma unroll
-      for (int sb = 0; sb < 4; ++sb) {
-        const int cu = sb & 1, nx = cu ^ 1;
-        if (sb == 3) {
-          if (EPILOGUE_STORES && after_epilogue) {
-            asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
-          } else {
-            asm volatile("s_waitcnt vmcnt(4) lgkmcnt(0)" ::: "memory");
-          }
-          __builtin_amdgcn_s_barrier();
-          after_epilogue = false;
-        }
-        // this quarter's matrix instructions run on fragment set `cu`; the reads fill set `nx` for the next quarter
-        // (of this step's tiles, or, in quarter 3, the first of the next step's)
-        const char* rw = lds + ((sb == 3) ? nw : cw) * kLmTileBytes + fragoff_w;
-        const char* rh = lds + ((sb == 3) ? nh : ch) * kLmTileBytes + fragoff_h;
-        const int rq = (sb + 1) & 3;
-#pragma unroll
-        for (int mm = 0; mm < 8; ++mm) {
-          const int i = mm >> 2, j = mm & 3;
-          acc[i][j] = LmFrag<DT>::mfma(a[cu][i], b[cu][j], acc[i][j]);
-          if (mm == 0) a[nx][0] = *reinterpret_cast<const FragT*>(rw + phys[rq]);
-          else if (mm < 5) b[nx][mm - 1] = *reinterpret_cast<const FragT*>(rh + (mm - 1) * 32 * kLmRowBytes + phys[rq]);
-          else if (mm == 5) a[nx][1] = *reinterpret_cast<const FragT*>(rw + 32 * kLmRowBytes + phys[rq]);
-          const int op = lm_load_slot(sb, mm);
-          if (op >= 5) load_h(op - 5);
-          else if (op >= 1) load_w(op - 1);
-        }
-#pragma unroll
-        for (int mm = 0; mm < 8; ++mm) {
-          __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                                   // one matrix instruction
-          if (mm < 6) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);                       // one LDS read
-          if (lm_load_slot(sb, mm) != 0) __builtin_amdgcn_sched_group_barrier(0x010, 1, 0);   // one load
-        }
-        __builtin_amdgcn_sched_barrier(0);
-        if (sb == 1) advance_w();
-        if (sb == 3) advance_h();
+        for (int i = 0; i < 4; ++i) load_h(i);
+        advance_h();
       }
-      cw = nw;
-      ch = nh;
+      asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
+      __builtin_amdgcn_s_barrier();
+#pragma unroll
+      for (int i = 0; i < 2; ++i) a[0][i] = *reinterpret_cast<const FragT*>(lds + fragoff_w + i * 32 * kLmRowBytes + phys[0]);
+#pragma unroll
+      for (int j = 0; j < 4; ++j) b[0][j] = *reinterpret_cast<const FragT*>(lds + kLmTileBytes + fragoff_h + j * 32 * kLmRowBytes + phys[0]);
     }
-    on_tile(vt, acc);
-    after_epilogue = true;
+
+    int cw = 0, ch = 1;   // ring slots of the step being computed
+    bool after_epilogue = false;
+    for (int64_t vt = work.vt_begin; vt < work.vt_end; ++vt) {
+      lm_f32x16 acc[2][4];
+#pragma unroll
+      for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+#pragma unroll
+          for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
+
+      for (int ks = 0; ks < ksteps; ++ks) {
+        const int nw = next_slot(cw), nh = next_slot(ch);
+#pragma unroll
+        for (int sb = 0; sb < 4; ++sb) {
+          const int cu = sb & 1, nx = cu ^ 1;
+          if (sb == 3) {
+            if (EPILOGUE_STORES && after_epilogue) {
+              asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+            } else {
+              asm volatile("s_waitcnt vmcnt(4) lgkmcnt(0)" ::: "memory");
+            }
+            __builtin_amdgcn_s_barrier();
+            after_epilogue = false;
+          }
+          // this quarter's matrix instructions run on fragment set `cu`; the reads fill set `nx` for the next quarter
+          // (of this step's tiles, or, in quarter 3, the first of the next step's)
+          const char* rw = lds + ((sb == 3) ? nw : cw) * kLmTileBytes + fragoff_w;
+          const char* rh = lds + ((sb == 3) ? nh : ch) * kLmTileBytes + fragoff_h;
+          const int rq = (sb + 1) & 3;
+#pragma unroll
+          for (int mm = 0; mm < 8; ++mm) {
+            const int i = mm >> 2, j = mm & 3;
+            acc[i][j] = LmFrag<DT>::mfma(a[cu][i], b[cu][j], acc[i][j]);
+            if (mm == 0) a[nx][0] = *reinterpret_cast<const FragT*>(rw + phys[rq]);
+            else if (mm < 5) b[nx][mm - 1] = *reinterpret_cast<const FragT*>(rh + (mm - 1) * 32 * kLmRowBytes + phys[rq]);
+            else if (mm == 5) a[nx][1] = *reinterpret_cast<const FragT*>(rw + 32 * kLmRowBytes + phys[rq]);
+            const int op = lm_load_slot(sb, mm);
+            if (op >= 5) load_h(op - 5);
+            else if (op >= 1) load_w(op - 1);
+          }
+#pragma unroll
+          for (int mm = 0; mm < 8; ++mm) {
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                                   // one matrix instruction
+            if (mm < 6) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);                       // one LDS read
+            if (lm_load_slot(sb, mm) != 0) __builtin_amdgcn_sched_group_barrier(0x010, 1, 0);   // one load
+          }
+          __builtin_amdgcn_sched_barrier(0);
+          if (sb == 1) advance_w();
+          if (sb == 3) advance_h();
+        }
+        cw = nw;
+        ch = nh;
+      }
+      on_tile(vt, acc);
+      after_epilogue = true;
+    }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // the last, redundant loads still target the ring
+  } else {
+    // row (within its 16-row block) = lane&15, logical chunk = 4*half + (lane>>4), half in 0..1
+    int phys[2];
+#pragma unroll
+    for (int hf = 0; hf < 2; ++hf) phys[hf] = (((4 * hf + (lane >> 4)) ^ ((lane >> 1) & 7)) * 16);
+    const int fragoff_w = (wv * 64 + (lane & 15)) * kLmRowBytes;    // within a W slot
+    const int fragoff_h = (wt * 128 + (lane & 15)) * kLmRowBytes;   // within an H slot
+
+    FragT a[4], b[8];
+    if (total_steps > 0) {
+#pragma unroll
+      for (int rep = 0; rep < 2; ++rep) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) load_w(i);
+        advance_w();
+#pragma unroll
+        for (int i = 0; i < 4; ++i) load_h(i);
+        advance_h();
+      }
+      asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
+      __builtin_amdgcn_s_barrier();
+#pragma unroll
+      for (int i = 0; i < 4; ++i) a[i] = *reinterpret_cast<const FragT*>(lds + fragoff_w + i * 16 * kLmRowBytes + phys[0]);
+#pragma unroll
+      for (int j = 0; j < 8; ++j) b[j] = *reinterpret_cast<const FragT*>(lds + kLmTileBytes + fragoff_h + j * 16 * kLmRowBytes + phys[0]);
+    }
+
+    int cw = 0, ch = 1;   // ring slots of the step being computed
+    bool after_epilogue = false;
+    for (int64_t vt = work.vt_begin; vt < work.vt_end; ++vt) {
+      lm_f32x4 acc[4][8];
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 8; ++j)
+#pragma unroll
+          for (int v = 0; v < 4; ++v) acc[i][j][v] = 0.f;
+
+      for (int ks = 0; ks < ksteps; ++ks) {
+        const int nw = next_slot(cw), nh = next_slot(ch);
+        // Two halves of 32 contraction elements, 32 matrix instructions each, with ONE set of fragments (4 of W, 8 of H):
+        // the products run column by column, an H fragment is dead after its 4 products and a W fragment after the last
+        // column, and each is refilled in place with the next half's as soon as it is dead - the second half's from this
+        // step's tiles during the first half, the next step's first half from the next tiles during the second. The
+        // step's barrier therefore sits between the halves: behind it W(s), H(s) are dead and W(s+1), H(s+1) must have
+        // landed. First half: the four loads of W(s+2) (into the slot H(s-1) left); second half: H(s+2) (slot of W(s)).
+#pragma unroll
+        for (int hf = 0; hf < 2; ++hf) {
+          if (hf == 1) {
+            if (EPILOGUE_STORES && after_epilogue) {
+              asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+            } else {
+              asm volatile("s_waitcnt vmcnt(4) lgkmcnt(0)" ::: "memory");
+            }
+            __builtin_amdgcn_s_barrier();
+            after_epilogue = false;
+          }
+          const char* rw = lds + ((hf == 1) ? nw : cw) * kLmTileBytes + fragoff_w + phys[hf ^ 1];
+          const char* rh = lds + ((hf == 1) ? nh : ch) * kLmTileBytes + fragoff_h + phys[hf ^ 1];
+#pragma unroll
+          for (int mm = 0; mm < 32; ++mm) {
+            const int j = mm >> 2, i = mm & 3;
+            acc[i][j] = LmFrag<DT>::mfma16(a[i], b[j], acc[i][j]);
+            if (i == 3) b[j] = *reinterpret_cast<const FragT*>(rh + j * 16 * kLmRowBytes);
+            if (j == 7) a[i] = *reinterpret_cast<const FragT*>(rw + i * 16 * kLmRowBytes);
+            if ((mm & 7) == 1) {
+              if (hf == 0) load_w(mm >> 3); else load_h(mm >> 3);
+            }
+          }
+#pragma unroll
+          for (int mm = 0; mm < 32; ++mm) {
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                                // one matrix instruction
+            if ((mm & 3) == 3) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);             // an H fragment
+            if ((mm >> 2) == 7) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);            // a W fragment
+            if ((mm & 7) == 1) __builtin_amdgcn_sched_group_barrier(0x010, 1, 0);             // one load
+          }
+          __builtin_amdgcn_sched_barrier(0);
+          if (hf == 0) advance_w(); else advance_h();
+        }
+        cw = nw;
+        ch = nh;
+      }
+      on_tile(vt, acc);
+      after_epilogue = true;
+    }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // the last, redundant loads still target the ring
   }
-  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // the last, redundant loads still target the ring
 }
 
 // grid.x = token blocks * n_splits, block = 512, dynamic LDS = kLmLdsBytes. Writes, per (token, split), the online-softmax
@@ -317,44 +412,40 @@ __global__ __launch_bounds__(kLmWaves * 64, 1) void lmhead_partial_kernel(
   const int wt = wave & 1;
   const LmWork work = lm_work(V, T, n_splits, tiles_per_split, xcd_map);
 
-  // per-lane softmax state for the 4 token columns this lane sees
-  float m[4], s[4], t[4], c[4];
+  // per-lane softmax state for the 8 token columns this lane sees (16 x 16 blocks: column = lane & 15)
+  float m[8], s[8], t[8], c[8];
 #pragma unroll
-  for (int j = 0; j < 4; ++j) {
+  for (int j = 0; j < 8; ++j) {
     m[j] = neg_inf();
     s[j] = 0.f;
     t[j] = 0.f;
-    const int64_t tok = work.tok0_ld + wt * 128 + j * 32 + (lane & 31);
+    const int64_t tok = work.tok0_ld + wt * 128 + j * 16 + (lane & 15);
     c[j] = make_scale<false>(temperature, tok).c;   // log2(e) / max(T, 1e-8), exactly what the finishing kernel uses
   }
 
-  lm_walk_tiles<DT, false>(W, H, V, K, w_stride, h_stride, work, lds, [&](int64_t vt, lm_f32x16 (&acc)[2][4]) {
-    // fold 64 logits per token column into the running state (two passes over the accumulators: maximum, then
-    // exponentials; nothing is buffered)
+  lm_walk_tiles<DT, 16, false>(W, H, V, K, w_stride, h_stride, work, lds, [&](int64_t vt, lm_f32x4 (&acc)[4][8]) {
+    // fold 16 logits per token column into the running state (maximum first, then the exponentials; nothing is
+    // buffered): acc[i][j][v] is vocabulary row tile_row0 + wv*64 + i*16 + 4*(lane>>4) + v of token column j
     const bool edge = (vt + 1) * kLmVocab > V;
-    const int64_t vrow0 = (edge ? V - kLmVocab : vt * kLmVocab) + wv * 64 + 4 * (lane >> 5);
+    const int64_t vrow0 = (edge ? V - kLmVocab : vt * kLmVocab) + wv * 64 + 4 * (lane >> 4);
     const int64_t vfirst = vt * kLmVocab;   // rows below belong to the tile before
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
+    for (int j = 0; j < 8; ++j) {
+      float x[16];
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int v = 0; v < 4; ++v) x[i * 4 + v] = acc[i][j][v];
+      if (edge) {
+#pragma unroll
+        for (int e = 0; e < 16; ++e) {
+          const int64_t vr = vrow0 + (e >> 2) * 16 + (e & 3);
+          x[e] = vr >= vfirst ? x[e] : neg_inf();
+        }
+      }
       float bm = neg_inf();
 #pragma unroll
-      for (int i = 0; i < 2; ++i) {
-        // one 32x32 block (16 accumulator registers) at a time; the scheduling barrier keeps the compiler from
-        // pulling the next blocks' accumulator copies forward
-        float x[16];
-#pragma unroll
-        for (int v = 0; v < 16; ++v) x[v] = acc[i][j][v];
-        if (edge) {
-#pragma unroll
-          for (int v = 0; v < 16; ++v) {
-            const int64_t vr = vrow0 + i * 32 + 8 * (v >> 2) + (v & 3);
-            x[v] = vr >= vfirst ? x[v] : neg_inf();
-          }
-        }
-#pragma unroll
-        for (int v = 0; v < 16; ++v) bm = __builtin_fmaxf(bm, x[v]);
-        __builtin_amdgcn_sched_barrier(0);
-      }
+      for (int e = 0; e < 16; ++e) bm = __builtin_fmaxf(bm, x[e]);
       bm *= c[j];   // c > 0: the maximum commutes with the scale
       if (bm > m[j]) {
         const float al = hw_exp2(m[j] - bm);  // m = -inf -> 0
@@ -366,50 +457,45 @@ __global__ __launch_bounds__(kLmWaves * 64, 1) void lmhead_partial_kernel(
       const float sub = (m[j] == neg_inf()) ? 0.f : m[j];
       float ps = 0.f, pt = 0.f;
 #pragma unroll
-      for (int i = 0; i < 2; ++i) {
-        float x[16];
-#pragma unroll
-        for (int v = 0; v < 16; ++v) x[v] = acc[i][j][v];
-        if (edge) {
-#pragma unroll
-          for (int v = 0; v < 16; ++v) {
-            const int64_t vr = vrow0 + i * 32 + 8 * (v >> 2) + (v & 3);
-            x[v] = vr >= vfirst ? x[v] : neg_inf();
-          }
-        }
-#pragma unroll
-        for (int v = 0; v < 16; ++v) {
-          const float d = __builtin_fmaf(x[v], c[j], -sub);
-          const float e = hw_exp2(d);
-          ps += e;
-          pt = __builtin_fmaf(e, (e == 0.f) ? 0.f : d, pt);
-        }
-        __builtin_amdgcn_sched_barrier(0);
+      for (int e = 0; e < 16; ++e) {
+        const float d = __builtin_fmaf(x[e], c[j], -sub);
+        const float ex = hw_exp2(d);
+        ps += ex;
+        pt = __builtin_fmaf(ex, (ex == 0.f) ? 0.f : d, pt);
       }
       s[j] += ps;
       t[j] += pt;
+      // one token column at a time: keeps the compiler from pulling the next columns' accumulator copies forward
+      __builtin_amdgcn_sched_barrier(0);
     }
   });
 
   __syncthreads();   // every wavefront has left the ring: its memory now serves the merge
-  // combine: lanes l and l^32 hold the same tokens (other vocabulary rows), then the four vocabulary-quarter
+  // combine: lanes l, l^16, l^32, l^48 hold the same tokens (other vocabulary rows), then the four vocabulary-quarter
   // wavefronts of a token half through LDS
 #pragma unroll
-  for (int j = 0; j < 4; ++j) {
-    const float om = __shfl_xor(m[j], 32);
-    const float os = __shfl_xor(s[j], 32);
-    const float ot = __shfl_xor(t[j], 32);
-    const float M = __builtin_fmaxf(m[j], om);
-    float S = 0.f, Tt = 0.f;
-    if (M != neg_inf()) {
-      const float a1 = hw_exp2(m[j] - M), a2 = hw_exp2(om - M);
-      const float d1 = (m[j] == neg_inf()) ? 0.f : m[j] - M;
-      const float d2 = (om == neg_inf()) ? 0.f : om - M;
-      S = a1 * s[j] + a2 * os;
-      Tt = a1 * (t[j] + d1 * s[j]) + a2 * (ot + d2 * os);
+  for (int j = 0; j < 8; ++j) {
+    float M = m[j], S = s[j], Tt = t[j];
+#pragma unroll
+    for (int sh = 16; sh <= 32; sh <<= 1) {
+      const float om = __shfl_xor(M, sh);
+      const float os = __shfl_xor(S, sh);
+      const float ot = __shfl_xor(Tt, sh);
+      const float N = __builtin_fmaxf(M, om);
+      float S2 = 0.f, T2 = 0.f;
+      if (N != neg_inf()) {
+        const float a1 = hw_exp2(M - N), a2 = hw_exp2(om - N);
+        const float d1 = (M == neg_inf()) ? 0.f : M - N;
+        const float d2 = (om == neg_inf()) ? 0.f : om - N;
+        S2 = a1 * S + a2 * os;
+        T2 = a1 * (Tt + d1 * S) + a2 * (ot + d2 * os);
+      }
+      M = N;
+      S = S2;
+      Tt = T2;
     }
-    if (lane < 32) {
-      const int col = wt * 128 + j * 32 + lane;
+    if (lane < 16) {
+      const int col = wt * 128 + j * 16 + lane;
       red[wv][col][0] = M;
       red[wv][col][1] = S;
       red[wv][col][2] = Tt;
@@ -492,7 +578,7 @@ __global__ __launch_bounds__(kLmWaves * 64, 1) void lmhead_dlogits_kernel(
     out[j] = dlogits + tok * d_stride;
   }
 
-  lm_walk_tiles<DT, true>(W, H, V, K, w_stride, h_stride, work, lds, [&](int64_t vt, lm_f32x16 (&acc)[2][4]) {
+  lm_walk_tiles<DT, 32, true>(W, H, V, K, w_stride, h_stride, work, lds, [&](int64_t vt, lm_f32x16 (&acc)[2][4]) {
     const bool edge = (vt + 1) * kLmVocab > V;
     const int vrow0 = (int)(edge ? V - kLmVocab : vt * kLmVocab) + wv * 64 + 4 * (lane >> 5);
     const int vfirst = (int)(vt * kLmVocab);   // rows below belong to the tile before
@@ -577,63 +663,72 @@ __global__ __launch_bounds__(kLmWaves * 64, 1) void lm_gemm_nt_kernel(
   const int64_t local = id >> 3;
   const int64_t patch = (local / psize) * 8 + (id & 7);
   if (patch >= per_part * g.k_parts) return;   // the whole workgroup, before any barrier
-  const int within = (int)(local % psize);
-  const int kp = (int)(patch / per_part);
-  const int64_t r = patch % per_part;
-  const int64_t yb = (r % patches_y) * g.py + within % g.py;
-  const int64_t xsplit = (r / patches_y) * g.px + within / g.py;
+  // (64-bit divisions run on the vector ALUs; readfirstlane brings their uniform results back to scalar registers)
+  const int within = __builtin_amdgcn_readfirstlane((int)(local % psize));
+  const int kp = __builtin_amdgcn_readfirstlane((int)(patch / per_part));
+  const int r = __builtin_amdgcn_readfirstlane((int)(patch % per_part));
+  const int yb = __builtin_amdgcn_readfirstlane((int)((r % patches_y) * g.py + within % g.py));
+  const int xsplit = __builtin_amdgcn_readfirstlane((int)((r / patches_y) * g.px + within / g.py));
 
   LmWork work;
   work.split = kp;
-  work.tok0 = yb * kLmTokens;
+  work.tok0 = (int64_t)yb * kLmTokens;
   work.tok0_ld = work.tok0 + kLmTokens <= g.NY ? work.tok0 : g.NY - kLmTokens;
-  work.vt_begin = xsplit * g.tiles_per_item;
+  work.vt_begin = (int64_t)xsplit * g.tiles_per_item;
   work.vt_end = work.vt_begin + g.tiles_per_item;
   if (work.vt_end > nxt) work.vt_end = nxt;
   const int64_t step0 = (int64_t)kp * g.steps_per_part;
   int64_t nsteps = g.k_steps - step0;
   if (nsteps > g.steps_per_part) nsteps = g.steps_per_part;
 
-  lm_walk_tiles<DT, true>(X + step0 * kLmK, Y + step0 * kLmK, g.NX, nsteps * kLmK, x_stride, y_stride, work, lds,
-                          [&](int64_t vt, lm_f32x16 (&acc)[2][4]) {
+  lm_walk_tiles<DT, 16, true>(X + step0 * kLmK, Y + step0 * kLmK, g.NX, nsteps * kLmK, x_stride, y_stride, work, lds,
+                              [&](int64_t vt, lm_f32x4 (&acc)[4][8]) {
+    // acc[i][j][0..3]: columns x0 .. x0+3 of out, x0 = tile_row0 + wv*64 + i*16 + 4*(lane>>4), of row
+    // y = tok0_ld + wt*128 + j*16 + (lane&15)
     const bool edge = (vt + 1) * kLmVocab > g.NX;
-    const int64_t xrow0 = (edge ? g.NX - kLmVocab : vt * kLmVocab) + wv * 64 + 4 * (lane >> 5);
-    const int64_t xfirst = vt * kLmVocab;   // rows below belong to the tile before
+    const int xrow0 = (int)(edge ? g.NX - kLmVocab : vt * kLmVocab) + wv * 64 + 4 * (lane >> 4);
+    const int xfirst = (int)(vt * kLmVocab);   // columns below belong to the tile before
+    // Row pointers are formed here, per tile, as "row of column block 0" + a uniform offset per block. The empty asm
+    // hides the lane's row from loop-invariant code motion, which would otherwise keep all 8 pointers (16 registers)
+    // alive through the main loop and spill.
+    int y_lane = lane & 15;
+    asm volatile("" : "+v"(y_lane));
+    const int64_t y0 = work.tok0_ld + wt * 128 + y_lane;
+    uint16_t* out_row0 = out + y0 * out_stride;
+    float* part_row0 = partials + ((int64_t)kp * g.NY + y0) * g.NX;
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      const int64_t y = work.tok0_ld + wt * 128 + j * 32 + (lane & 31);
-      const bool y_mine = y >= work.tok0;
+    for (int j = 0; j < 8; ++j) {
+      const bool y_mine = y0 + j * 16 >= work.tok0;
+      uint16_t* out_row = out_row0 + (int64_t)(j * 16) * out_stride;
+      float* part_row = part_row0 + (int64_t)(j * 16) * g.NX;
 #pragma unroll
-      for (int i = 0; i < 2; ++i) {
+      for (int i = 0; i < 4; ++i) {
+        const int x = xrow0 + i * 16;   // a multiple of 4
+        if (y_mine && x >= xfirst) {
+          float v[4];
 #pragma unroll
-        for (int q = 0; q < 4; ++q) {
-          const int64_t x = xrow0 + i * 32 + 8 * q;   // first of 4 consecutive columns of out (a multiple of 4)
-          if (y_mine && x >= xfirst) {
-            float v[4];
+          for (int e = 0; e < 4; ++e) v[e] = acc[i][j][e];
+          if constexpr (MODE == 2) {
+            f32x4 pk = {v[0], v[1], v[2], v[3]};
+            *reinterpret_cast<f32x4*>(part_row + x) = pk;
+          } else {
+            uint2* dst = reinterpret_cast<uint2*>(out_row + x);
+            if constexpr (MODE == 1) {
+              const uint2 old = *dst;
+              float o[4];
+              lm_unpack2<DT>(old.x, o);
+              lm_unpack2<DT>(old.y, o + 2);
 #pragma unroll
-            for (int e = 0; e < 4; ++e) v[e] = acc[i][j][q * 4 + e];
-            if constexpr (MODE == 2) {
-              f32x4 pk = {v[0], v[1], v[2], v[3]};
-              *reinterpret_cast<f32x4*>(partials + ((int64_t)kp * g.NY + y) * g.NX + x) = pk;
-            } else {
-              uint2* dst = reinterpret_cast<uint2*>(out + y * out_stride + x);
-              if constexpr (MODE == 1) {
-                const uint2 old = *dst;
-                float o[4];
-                lm_unpack2<DT>(old.x, o);
-                lm_unpack2<DT>(old.y, o + 2);
-#pragma unroll
-                for (int e = 0; e < 4; ++e) v[e] += o[e];
-              }
-              uint2 pk;
-              pk.x = O::pack2(v[0], v[1]);
-              pk.y = O::pack2(v[2], v[3]);
-              *dst = pk;
+              for (int e = 0; e < 4; ++e) v[e] += o[e];
             }
+            uint2 pk;
+            pk.x = O::pack2(v[0], v[1]);
+            pk.y = O::pack2(v[2], v[3]);
+            *dst = pk;
           }
         }
-        __builtin_amdgcn_sched_barrier(0);
       }
+      __builtin_amdgcn_sched_barrier(0);
     }
   });
 }

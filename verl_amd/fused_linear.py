@@ -30,13 +30,21 @@ __all__ = ["FusedLinearForPPO", "fused_linear_for_ppo", "linear_cross_entropy", 
 # projection reaches 1.4 PFLOP/s instead of 0.86 at 512, and the weight gradient is accumulated 8x less often.
 DEFAULT_CHUNK_TOKENS = 4096
 
-# Who forms the logits of a chunk. "library": torch.matmul (hipBLASLt) into the chunk buffer, then the row kernels over
-# it. "mfma": this package's own matrix-core kernels, which never round the logits to the operand type: forward
-# vrl_lmhead_score (no buffer at all, only when no gradient is recorded), backward vrl_lmhead_dlogits (logits formed
-# again on the matrix cores and turned into their gradient in registers; the buffer receives the gradient directly).
-# The default is what is faster on MI355X today (the library GEMM by ~10 %); VERL_AMD_LMHEAD_KERNELS or the
-# ``kernels`` argument select the other. Shapes the matrix-core kernels do not take always go to the library.
-DEFAULT_KERNELS = os.environ.get("VERL_AMD_LMHEAD_KERNELS", "library")
+# Which matrix products are this package's own kernels.
+#   "library": every product is torch.matmul (hipBLASLt); the row kernels run over the chunk buffer.
+#   "mfma":    every step that has a hand-written matrix-core kernel uses it: the forward without gradients is one
+#              kernel that never writes logits (vrl_lmhead_score), the backward forms the logits again and writes their
+#              gradient from registers (vrl_lmhead_dlogits) and forms d hidden with vrl_gemm_nt; d W stays a library
+#              product (the hand-written one needs a transposed copy of the gradient buffer).
+#   "auto":    each step by what is measured fastest on MI355X at 8192 x 3584 -> 152064 bf16, as long as the forward is the
+#              same arithmetic with and without gradients: library GEMM + row kernels for the logits (forward and
+#              backward), vrl_gemm_nt for d hidden (3.36 against 3.73 ms), library for d W. The single forward kernel is
+#              as fast as the library GEMM + row kernel (6.52 against 6.53 ms) and needs no buffer, but it keeps the
+#              logits in fp32 where the GEMM rounds them to the operand type: old log-probs from it (no gradients)
+#              and new ones from the GEMM (gradients) would differ by that rounding, a policy ratio other than 1 before
+#              any update. "mfma" accepts that; "auto" does not.
+# The environment variable and the ``kernels`` argument select; shapes a hand-written kernel does not take go to the library.
+DEFAULT_KERNELS = os.environ.get("VERL_AMD_LMHEAD_KERNELS", "auto")
 
 
 def _mfma_takes(hidden: torch.Tensor, weight: torch.Tensor, n_tokens: int) -> bool:
@@ -170,13 +178,13 @@ class _FusedLinearForPPOFunction(torch.autograd.Function):
                 if kept is not None:
                     continue
                 if need_dh:
-                    torch.matmul(logits, weight if weight_t is None else weight_t.t(), out=d_hidden[lo:hi])
+                    _d_hidden(logits, weight, weight_t, d_hidden[lo:hi], ctx.kernels != "library")
                 if need_dw:
                     d_weight.addmm_(logits.t(), transpose_2d(hidden[lo:hi]).t() if half else hidden[lo:hi])
             if kept is not None:
                 # the gradient over all tokens' logits is in `kept`: one product each, nothing to accumulate
                 if need_dh:
-                    _d_hidden(kept, weight, weight_t, d_hidden, ctx.kernels == "mfma")
+                    _d_hidden(kept, weight, weight_t, d_hidden, ctx.kernels != "library")
                 if need_dw:
                     torch.matmul(kept.t(), transpose_2d(hidden).t() if half else hidden, out=d_weight)
         return d_hidden, d_weight, None, None, None, None, None
@@ -197,14 +205,16 @@ def fused_linear_for_ppo(hidden_states: torch.Tensor, vocab_weights: torch.Tenso
     ``tokens x vocab`` logits (2.5 GB for 8192 x 152064 bf16), the backward writes their gradient over them instead of
     projecting again and forms ``d hidden`` and ``d W`` with one product each. Such a graph can be differentiated once.
 
-    ``kernels`` chooses who forms the logits: ``"library"`` (a GEMM per chunk into the buffer) or ``"mfma"`` (this
-    package's matrix-core kernels: no buffer at all when no gradient is recorded, a backward that writes the
-    gradient of the logits straight from registers and forms ``d hidden`` with ``vrl_gemm_nt``; ``d W`` stays a
-    library product); None takes ``DEFAULT_KERNELS``.
+    ``kernels`` chooses which matrix products are this package's own kernels: ``"library"`` (none: torch.matmul
+    throughout), ``"mfma"`` (all that exist: no buffer at all when no gradient is recorded, a backward that forms the
+    logits again and writes their gradient straight from registers, ``d hidden`` from ``vrl_gemm_nt``; ``d W`` stays a
+    library product) or ``"auto"`` (each step by what measures fastest on MI355X while log-probs computed with and
+    without gradients stay bit-identical: library products for the logits, ``vrl_gemm_nt`` for ``d hidden``); None takes ``DEFAULT_KERNELS`` ("auto" unless ``VERL_AMD_LMHEAD_KERNELS`` says
+    otherwise).
     """
     kernels = DEFAULT_KERNELS if kernels is None else kernels
-    if kernels not in ("library", "mfma"):
-        raise ValueError(f"kernels must be 'library' or 'mfma', got {kernels!r}")
+    if kernels not in ("auto", "library", "mfma"):
+        raise ValueError(f"kernels must be 'auto', 'library' or 'mfma', got {kernels!r}")
     if not hidden_states.is_cuda or not vocab_weights.is_cuda:
         raise RuntimeError("fused_linear_for_ppo: tensors must be on the GPU; verl_amd has no CPU implementation")
     if hidden_states.dtype != vocab_weights.dtype or hidden_states.dtype not in _DTYPE_CODES:
@@ -243,8 +253,9 @@ def lm_head_score_mfma(hidden_states: torch.Tensor, vocab_weights: torch.Tensor,
     (verl/utils/kernel/kernels.py:531-756). bf16 or fp16 operands, at least 256 tokens and 256 vocabulary entries,
     hidden size a multiple of 64. ``temperature`` is a float or one value per token. The logits are kept in fp32
     (a GEMM that writes them rounds them to the operand type first), so results are slightly closer to the
-    all-fp32 value than ``fused_linear_for_ppo``'s. On MI355X it is 3-5 % slower than the library GEMM + row kernel that
-    ``fused_linear_for_ppo`` uses (6.7 ms against 6.5 ms at 8192 x 3584 -> 152064); it needs no logits buffer at all.
+    all-fp32 value than a path that writes them. On MI355X it takes as long as the library GEMM + row kernel (6.5 ms at
+    8192 x 3584 -> 152064) and needs no logits buffer at all; ``fused_linear_for_ppo(kernels="mfma")`` uses it when no
+    gradient is recorded.
     """
     if not hidden_states.is_cuda or not vocab_weights.is_cuda:
         raise RuntimeError("lm_head_score_mfma: tensors must be on the GPU; verl_amd has no CPU implementation")

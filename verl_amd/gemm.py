@@ -7,6 +7,7 @@ module instead when ``kernels="mfma"``.
 
 from __future__ import annotations
 
+import ctypes
 from typing import Optional
 
 import torch
@@ -14,6 +15,9 @@ import torch
 from . import _lib
 
 _DTYPE_CODES = {torch.bfloat16: _lib.VRL_BF16, torch.float16: _lib.VRL_F16}
+
+# vrl_gemm_nt launches from this module since import (what a caller can count to see which products were its own)
+counters = {"gemm_nt": 0}
 
 
 def gemm_nt_takes(x: torch.Tensor, y: torch.Tensor) -> bool:
@@ -49,8 +53,6 @@ def gemm_nt(x: torch.Tensor, y: torch.Tensor, out: Optional[torch.Tensor] = None
         raise ValueError(f"gemm_nt: out must be ({NY}, {NX}) {x.dtype} on {dev}, contiguous along its last axis")
     lib = _lib.load()
     code = _DTYPE_CODES[x.dtype]
-    import ctypes
-
     need = ctypes.c_int64(0)
     planned = lib.vrl_gemm_nt_plan(code, NX, NY, K, ctypes.addressof(need))
     if planned < 0:
@@ -62,4 +64,5 @@ def gemm_nt(x: torch.Tensor, y: torch.Tensor, out: Optional[torch.Tensor] = None
                              out.stride(0), 1 if accumulate else 0, parts, None if work is None else work.data_ptr(),
                              _lib.stream_ptr(dev))
     _lib.check("vrl_gemm_nt", st)
+    counters["gemm_nt"] += 1
     return out
