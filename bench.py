@@ -454,13 +454,14 @@ def bench_lm_head(args, dev):
         "config": {"workload": "lm_head_8192x3584_v152064_bf16", "chunk_tokens": chunk, "keep_logits": keep,
                    "temperature": temperature,
                    "step": "verl_amd.fused_linear_for_ppo forward + torch.autograd.grad for hidden and weight, default "
-                           "kernels (\"auto\": library GEMMs for the logits and d W, vrl_gemm_nt for d hidden)"},
+                           "kernels (\"auto\": library GEMM + row kernel forward; backward vrl_lmhead_dlogits, vrl_gemm_nt for d hidden, a "
+                           "library GEMM for d W)"},
         "forward_ms": t_f * 1e3,
         "forward_tokens_per_s": T / t_f,
         "roofline": {"bound": "mfma", "achieved": flops_fb / t_fb / 1e12, "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
                      "frac": flops_fb / t_fb / 1e12 / MFMA_BF16_PEAK_TFLOPS, "traffic": None,
-                     "kernel": "hipBLASLt bf16 GEMMs (logits, d W) + lm_gemm_nt_kernel<bf16> (d hidden) + rowscore_kernel + "
-                               "rowscore_backward_kernel",
+                     "kernel": "hipBLASLt bf16 GEMMs (forward logits, d W) + rowscore_kernel + lmhead_dlogits_kernel<bf16> + "
+                               "lm_gemm_nt_kernel<bf16> (d hidden)",
                      "forward_tflops": flops_f / t_f / 1e12},
         "single_kernel_forward": {"ms": t_m * 1e3, "tflops": flops_f / t_m / 1e12, "frac_of_mfma_peak": flops_f / t_m / 1e12 / MFMA_BF16_PEAK_TFLOPS,
                                   "kernel": "lmhead_partial_kernel<bf16> + lmhead_finish_kernel (vrl_lmhead_score)",
@@ -470,8 +471,8 @@ def bench_lm_head(args, dev):
         "matrix_core_ceiling": ceiling,
         "all_library": {"forward_backward_ms": t_fb_lib * 1e3, "kernel": "torch.matmul for every product"},
         "matrix_core_backward": {"forward_backward_ms": t_fb_m * 1e3,
-                                 "kernel": "library GEMM forward; backward lmhead_dlogits_kernel<bf16> (vrl_lmhead_dlogits), "
-                                           "lm_gemm_nt_kernel<bf16> (vrl_gemm_nt) for d hidden, a library GEMM for d W",
+                                 "kernel": "kernels=\"mfma\": the default's backward; without gradients the forward is the single "
+                                           "kernel",
                                  "note": "the logits are formed again by the hand-written MFMA kernel and their gradient "
                                          "is written from registers (no GEMM into the buffer, no pass over it); d hidden "
                                          "comes from the same main loop"},

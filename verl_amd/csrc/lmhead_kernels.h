@@ -532,8 +532,8 @@ __global__ __launch_bounds__(kLmWaves * 64, 1) void lmhead_partial_kernel(
 // Backward: dlogits[tok, v] = (g_logprob[tok] * (1[v == label[tok]] - p) - g_entropy[tok] * p * (log p + entropy[tok])) / T[tok]
 // with p = exp(z - lse[tok]), z = logits / T, for all tokens and the vocabulary tiles of each split, written in the
 // operands' type to dlogits[tok * d_stride + v] (d_stride, V multiples of 8; 16-byte aligned base). Same grid and LDS as
-// lmhead_partial_kernel. A lane holds 4 consecutive vocabulary entries of one token per accumulator quad, i.e. one
-// 8-byte store; lanes l and l+32 complete 16 contiguous bytes, the four quads of a block 64.
+// lmhead_partial_kernel. A lane holds 4 consecutive vocabulary entries of one token per 16 x 16 block, i.e. one 8-byte
+// store; lanes l, l+16, l+32, l+48 complete 32 contiguous bytes of the token's row.
 template <int DT>
 __global__ __launch_bounds__(kLmWaves * 64, 1) void lmhead_dlogits_kernel(
     const uint16_t* __restrict__ W, const uint16_t* __restrict__ H, int64_t V, int64_t T, int64_t K, int64_t w_stride,
@@ -550,15 +550,13 @@ __global__ __launch_bounds__(kLmWaves * 64, 1) void lmhead_dlogits_kernel(
   const int wt = wave & 1;
   const LmWork work = lm_work(V, T, n_splits, tiles_per_split, xcd_map);
 
-  // the row constants of the 4 token columns this lane sees
-  RowGrad f[4];
-  int label[4];       // -1: no label term
-  bool tok_mine[4];   // false for the rows an edge block shares with the block before
-  uint16_t* out[4];
+  // the row constants of the 8 token columns this lane sees (16 x 16 blocks: column = lane & 15)
+  RowGrad f[8];
+  int label[8];       // -1: no label term
+  const int64_t tok_lane0 = work.tok0_ld + wt * 128 + (lane & 15);
 #pragma unroll
-  for (int j = 0; j < 4; ++j) {
-    const int64_t tok = work.tok0_ld + wt * 128 + j * 32 + (lane & 31);
-    tok_mine[j] = tok >= work.tok0;
+  for (int j = 0; j < 8; ++j) {
+    const int64_t tok = tok_lane0 + j * 16;
     float Tm = 1.f;
     if (temperature != nullptr) {
       Tm = temperature[tok];
@@ -575,35 +573,39 @@ __global__ __launch_bounds__(kLmWaves * 64, 1) void lmhead_dlogits_kernel(
     f[j].lab = gl * rT;
     const int64_t lab = (g_logprob != nullptr) ? labels[tok] : -1;
     label[j] = (lab >= 0 && lab < V) ? (int)lab : -1;   // an out-of-range label was reported by the forward pass
-    out[j] = dlogits + tok * d_stride;
   }
 
-  lm_walk_tiles<DT, 32, true>(W, H, V, K, w_stride, h_stride, work, lds, [&](int64_t vt, lm_f32x16 (&acc)[2][4]) {
+  lm_walk_tiles<DT, 16, true>(W, H, V, K, w_stride, h_stride, work, lds, [&](int64_t vt, lm_f32x4 (&acc)[4][8]) {
+    // acc[i][j][0..3]: vocabulary entries vr .. vr+3, vr = tile_row0 + wv*64 + i*16 + 4*(lane>>4), of token column j
     const bool edge = (vt + 1) * kLmVocab > V;
-    const int vrow0 = (int)(edge ? V - kLmVocab : vt * kLmVocab) + wv * 64 + 4 * (lane >> 5);
+    const int vrow0 = (int)(edge ? V - kLmVocab : vt * kLmVocab) + wv * 64 + 4 * (lane >> 4);
     const int vfirst = (int)(vt * kLmVocab);   // rows below belong to the tile before
+    // The row pointers are formed per tile from the first column's (the empty asm keeps loop-invariant code motion from
+    // holding all 8 of them in registers through the main loop).
+    int64_t tok0v = tok_lane0;
+    asm volatile("" : "+v"(tok0v));
+    uint16_t* out0 = dlogits + tok0v * d_stride;
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
+    for (int j = 0; j < 8; ++j) {
+      const bool tok_mine = tok0v + j * 16 >= work.tok0;   // false for the rows an edge block shares with the block before
+      uint16_t* out = out0 + (int64_t)(j * 16) * d_stride;
 #pragma unroll
-      for (int i = 0; i < 2; ++i) {
+      for (int i = 0; i < 4; ++i) {
+        const int vr = vrow0 + i * 16;   // first of 4 consecutive vocabulary entries (a multiple of 4)
+        float y[4];
 #pragma unroll
-        for (int q = 0; q < 4; ++q) {
-          const int vr = vrow0 + i * 32 + 8 * q;   // first of 4 consecutive vocabulary entries (a multiple of 4)
-          float y[4];
-#pragma unroll
-          for (int e = 0; e < 4; ++e) {
-            y[e] = f[j](acc[i][j][q * 4 + e]);
-            if (vr + e == label[j]) y[e] += f[j].lab;
-          }
-          if (tok_mine[j] && vr >= vfirst) {
-            uint2 pk;
-            pk.x = O::pack2(y[0], y[1]);
-            pk.y = O::pack2(y[2], y[3]);
-            *reinterpret_cast<uint2*>(out[j] + vr) = pk;
-          }
+        for (int e = 0; e < 4; ++e) {
+          y[e] = f[j](acc[i][j][e]);
+          if (vr + e == label[j]) y[e] += f[j].lab;
         }
-        __builtin_amdgcn_sched_barrier(0);
+        if (tok_mine && vr >= vfirst) {
+          uint2 pk;
+          pk.x = O::pack2(y[0], y[1]);
+          pk.y = O::pack2(y[2], y[3]);
+          *reinterpret_cast<uint2*>(out + vr) = pk;
+        }
       }
+      __builtin_amdgcn_sched_barrier(0);
     }
   });
 }

@@ -37,8 +37,9 @@ DEFAULT_CHUNK_TOKENS = 4096
 #              gradient from registers (vrl_lmhead_dlogits) and forms d hidden with vrl_gemm_nt; d W stays a library
 #              product (the hand-written one needs a transposed copy of the gradient buffer).
 #   "auto":    each step by what is measured fastest on MI355X at 8192 x 3584 -> 152064 bf16, as long as the forward is the
-#              same arithmetic with and without gradients: library GEMM + row kernels for the logits (forward and
-#              backward), vrl_gemm_nt for d hidden (3.36 against 3.73 ms), library for d W. The single forward kernel is
+#              same arithmetic with and without gradients: library GEMM + row kernel for the forward; in the backward
+#              vrl_lmhead_dlogits (3.46 ms per 4096 tokens against 3.53 ms for the library GEMM + row backward) and
+#              vrl_gemm_nt for d hidden (3.36 against 3.73 ms), library for d W. The single forward kernel is
 #              as fast as the library GEMM + row kernel (6.52 against 6.53 ms) and needs no buffer, but it keeps the
 #              logits in fp32 where the GEMM rounds them to the operand type: old log-probs from it (no gradients)
 #              and new ones from the GEMM (gradients) would differ by that rounding, a policy ratio other than 1 before
@@ -149,7 +150,7 @@ class _FusedLinearForPPOFunction(torch.autograd.Function):
             for lo in range(0, T, chunk):
                 hi = min(lo + chunk, T)
                 n = hi - lo
-                if kept is None and ctx.kernels == "mfma" and _mfma_takes(hidden[lo:hi], weight, n) and V % 8 == 0:
+                if kept is None and ctx.kernels != "library" and _mfma_takes(hidden[lo:hi], weight, n) and V % 8 == 0:
                     # logits formed again on the matrix cores, their gradient written straight into the buffer
                     logits = buf[:n]
                     st = lib.vrl_lmhead_dlogits(
@@ -209,7 +210,8 @@ def fused_linear_for_ppo(hidden_states: torch.Tensor, vocab_weights: torch.Tenso
     throughout), ``"mfma"`` (all that exist: no buffer at all when no gradient is recorded, a backward that forms the
     logits again and writes their gradient straight from registers, ``d hidden`` from ``vrl_gemm_nt``; ``d W`` stays a
     library product) or ``"auto"`` (each step by what measures fastest on MI355X while log-probs computed with and
-    without gradients stay bit-identical: library products for the logits, ``vrl_gemm_nt`` for ``d hidden``); None takes ``DEFAULT_KERNELS`` ("auto" unless ``VERL_AMD_LMHEAD_KERNELS`` says
+    without gradients stay bit-identical: a library product for the forward's logits, this package's kernels for the
+    backward's gradient of the logits and ``d hidden``); None takes ``DEFAULT_KERNELS`` ("auto" unless ``VERL_AMD_LMHEAD_KERNELS`` says
     otherwise).
     """
     kernels = DEFAULT_KERNELS if kernels is None else kernels
