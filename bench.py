@@ -583,22 +583,23 @@ def bench_ceilings(args, dev):
 
 
 def mfma_ceiling(dev, steps):
-    """What the part sustains on bf16 32x32x16 matrix instructions alone (vrl_mfma_probe: one workgroup of 8 wavefronts
-    per CU, register operands, no memory traffic), with the shader clock it ran at: once on pseudo-random operands (what
-    the LM-head kernels' matrix time is measured against: the part holds a lower clock when the operand bits toggle),
-    once on small constants (the nominal rate). Returns the record of the random-operand run with the other inside."""
+    """What the part sustains on bf16 matrix instructions alone (vrl_mfma_probe: one workgroup of 8 wavefronts per CU,
+    register operands, no memory traffic), with the shader clock it ran at: on pseudo-random operands with the
+    instruction of the LM-head kernels (16x16x32; what their matrix time is measured against: the part holds a lower
+    clock when the operand bits toggle), the same with 32x32x16, and on small constants (the nominal rate). Returns the
+    first record with the others inside."""
     lib = _lib.load()
     stream = torch.cuda.current_stream(dev).cuda_stream
     n_wg = torch.cuda.get_device_properties(dev).multi_processor_count
-    iters = 20000   # 8 products per round: about as many per wavefront as the LM-head kernel issues at 8192 tokens
+    iters = 20000   # 64 x 128 x 16 wavefront tiles: about as many as the LM-head kernel forms per wavefront at 8192 tokens
     sink = torch.zeros(1, dtype=torch.float32, device=dev)
     clocks = torch.zeros(2, dtype=torch.int64, device=dev)
     khz = ctypes.c_int64(0)
     records = []
-    for random_operands in (1, 0):
+    for instruction, random_operands in ((16, 1), (32, 1), (32, 0)):
         def run():
-            st = lib.vrl_mfma_probe(n_wg, iters, random_operands, sink.data_ptr(), clocks.data_ptr(), ctypes.addressof(khz),
-                                    stream)
+            st = lib.vrl_mfma_probe(n_wg, iters, instruction, random_operands, sink.data_ptr(), clocks.data_ptr(),
+                                    ctypes.addressof(khz), stream)
             _lib.check("vrl_mfma_probe", st)
 
         spin_up(run)
@@ -609,16 +610,18 @@ def mfma_ceiling(dev, steps):
             b.record()
         torch.cuda.synchronize()
         ms = sum(a.elapsed_time(b) for a, b in evs) / len(evs)
-        flops = n_wg * 8 * iters * 8 * 2.0 * 32 * 32 * 16
+        flops = n_wg * 8 * iters * 2.0 * 64 * 128 * 16
         cyc, ticks = clocks.tolist()
-        records.append({"operands": "pseudo-random bf16 in (-1, 1)" if random_operands else "small constants",
+        records.append({"instruction": "v_mfma_f32_16x16x32_bf16" if instruction == 16 else "v_mfma_f32_32x32x16_bf16",
+                        "operands": "pseudo-random bf16 in (-1, 1)" if random_operands else "small constants",
                         "avg_kernel_ms": ms, "tflops": flops / (ms * 1e-3) / 1e12,
                         "frac_of_peak": flops / (ms * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS,
                         "shader_clock_ghz": (cyc / ticks) * khz.value * 1e-6 if ticks else None})
-    out = {"probe": "v_mfma_f32_32x32x16_bf16 on register operands, 8 wavefronts per CU, nothing else",
+    out = {"probe": "bf16 matrix instructions on register operands, 8 wavefronts per CU, nothing else",
            "kernel": "mfma_probe_kernel", "workgroups": n_wg}
     out.update(records[0])
-    out["with_constant_operands"] = records[1]
+    out["same_operands_32x32x16"] = records[1]
+    out["with_constant_operands"] = records[2]
     return out
 
 

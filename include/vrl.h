@@ -413,16 +413,16 @@ int vrl_stream_probe(const void* src, void* dst, int64_t n_rows, int64_t row_byt
 
 /*
  * vrl_mfma_probe — the matrix-core counterpart of vrl_stream_probe: n_workgroups workgroups of 8 wavefronts each issue
- * `iters` rounds of the 8 v_mfma_f32_32x32x16_bf16 of a 64 x 128 wavefront tile on register operands (2 * 32*32*16 flops
- * per product and wavefront), nothing else. random_operands != 0: pseudo-random bf16 operands in (-1, 1), otherwise small
- * constants; the part is power-managed and holds a lower clock when the operand bits toggle, so the first is the ceiling
- * the LM-head kernels are measured against and the second shows the nominal rate. clocks (optional, device, 2 x int64):
- * shader clocks and constant-rate wall-clock ticks that wavefront 0 of workgroup 0 spent in its loop; wall_clock_khz
- * (optional, HOST pointer): the rate of that wall clock. sink (device, 1 float) is practically never written.
- * No counterpart in the reference: a measurement aid.
+ * the products of `iters` 64 x 128 x 16 wavefront tiles (2 * 64 * 128 * 16 flops each) on register operands, nothing else.
+ * instruction: 32 = v_mfma_f32_32x32x16_bf16, 16 = v_mfma_f32_16x16x32_bf16 (what the LM-head kernels issue; iters even).
+ * random_operands != 0: pseudo-random bf16 operands in (-1, 1), otherwise small constants; the part is power-managed and
+ * holds a lower clock when the operand bits toggle, so the first is the ceiling the LM-head kernels are measured against
+ * and the second shows the nominal rate. clocks (optional, device, 2 x int64): shader clocks and constant-rate wall-clock
+ * ticks that wavefront 0 of workgroup 0 spent in its loop; wall_clock_khz (optional, HOST pointer): the rate of that wall
+ * clock. sink (device, 1 float) is practically never written. No counterpart in the reference: a measurement aid.
  */
-int vrl_mfma_probe(int64_t n_workgroups, int64_t iters, int random_operands, float* sink, int64_t* clocks,
-                   int64_t* wall_clock_khz, void* stream);
+int vrl_mfma_probe(int64_t n_workgroups, int64_t iters, int instruction, int random_operands, float* sink,
+                   int64_t* clocks, int64_t* wall_clock_khz, void* stream);
 
 /* Text for a VRL_* status code; never NULL. */
 const char* vrl_strerror(int status);

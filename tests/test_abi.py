@@ -260,12 +260,13 @@ def test_gemm_nt_argument_errors(lib):
 
 def test_mfma_probe_argument_errors(lib):
     f = lib.vrl_mfma_probe
-    assert f(-1, 10, 1, P, None, None, None) == _lib.VRL_ERR_SHAPE
-    assert f(4, -1, 1, P, None, None, None) == _lib.VRL_ERR_SHAPE
-    assert f(4, 10, 1, None, None, None, None) == _lib.VRL_ERR_NULL
-    assert f(4, 10, 0, P + 2, None, None, None) == _lib.VRL_ERR_ALIGN
-    assert f(4, 10, 0, P, P + 4, None, None) == _lib.VRL_ERR_ALIGN
-    assert f(0, 10, 1, None, None, None, None) == _lib.VRL_OK
+    assert f(-1, 10, 32, 1, P, None, None, None) == _lib.VRL_ERR_SHAPE
+    assert f(4, -1, 16, 1, P, None, None, None) == _lib.VRL_ERR_SHAPE
+    assert f(4, 10, 8, 1, P, None, None, None) == _lib.VRL_ERR_ARG
+    assert f(4, 10, 32, 1, None, None, None, None) == _lib.VRL_ERR_NULL
+    assert f(4, 10, 16, 0, P + 2, None, None, None) == _lib.VRL_ERR_ALIGN
+    assert f(4, 10, 32, 0, P, P + 4, None, None) == _lib.VRL_ERR_ALIGN
+    assert f(0, 10, 16, 1, None, None, None, None) == _lib.VRL_OK
 
 
 def test_lmhead_dlogits_argument_errors(lib):

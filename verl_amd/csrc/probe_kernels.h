@@ -77,9 +77,9 @@ __global__ __launch_bounds__(256) void stream_probe_flat_copy_kernel(const u32x4
   }
 }
 
-// Matrix-core probe: what the part sustains on v_mfma_f32_32x32x16_bf16 with nothing else in the way. 512 threads per
-// workgroup (two wavefronts per SIMD, like the LM-head kernels), every wavefront issues `iters` rounds of the 8 products
-// of a 64 x 128 wavefront tile (2 A fragments x 4 B fragments) on register operands. `random_operands` fills the
+// Matrix-core probe: what the part sustains on bf16 matrix instructions with nothing else in the way. 512 threads per
+// workgroup (two wavefronts per SIMD, like the LM-head kernels), every wavefront issues `iters` rounds of the products
+// of a 64 x 128 wavefront tile over 16 contraction elements on register operands. `random_operands` fills the
 // fragments with pseudo-random bf16 values in (-1, 1) (what real activations and weights look like to the multipliers);
 // otherwise every element is a small integer multiple of 1/8, the same in all products. The part is power-managed: the
 // clock it holds, and with it the rate, depends on how much the operand bits toggle. Thread 0 of workgroup 0 reports how
@@ -96,39 +96,71 @@ __device__ __forceinline__ float probe_uniform(uint32_t x) {   // (-1, 1), from 
   return static_cast<float>(static_cast<int32_t>(x)) * (1.0f / 2147483648.0f);
 }
 
+typedef float probe_f32x4 __attribute__((ext_vector_type(4)));
+
+// SHAPE 32: v_mfma_f32_32x32x16_bf16, 2 x 4 blocks per round; SHAPE 16: v_mfma_f32_16x16x32_bf16, 4 x 8 blocks per round
+// (the instruction of the LM-head kernels). `iters` counts 64 x 128 x 16 wavefront tiles (2 * 64 * 128 * 16 flops); a
+// SHAPE 16 round covers 32 contraction elements, so it runs iters / 2 rounds.
+template <int SHAPE>
 __global__ __launch_bounds__(512, 1) void mfma_probe_kernel(int64_t iters, int random_operands, float* __restrict__ sink,
                                                             int64_t* __restrict__ clocks) {
-  probe_bf16x8 a[2], b[4];
+  constexpr int NA = SHAPE == 32 ? 2 : 4, NB = SHAPE == 32 ? 4 : 8;
+  probe_bf16x8 a[NA], b[NB];
   const uint32_t me = blockIdx.x * 512u + threadIdx.x;
 #pragma unroll
-  for (int f = 0; f < 6; ++f)
+  for (int f = 0; f < NA + NB; ++f)
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
-      const float v = random_operands ? probe_uniform(me * 48u + f * 8u + i) : 0.125f * static_cast<float>((threadIdx.x + i) & 7);
-      if (f < 2) a[f][i] = static_cast<__bf16>(v); else b[f - 2][i] = static_cast<__bf16>(v);
+      const float v = random_operands ? probe_uniform(me * 96u + f * 8u + i) : 0.125f * static_cast<float>((threadIdx.x + i) & 7);
+      if (f < NA) a[f][i] = static_cast<__bf16>(v); else b[f - NA][i] = static_cast<__bf16>(v);
     }
-  probe_f32x16 acc[2][4];
-#pragma unroll
-  for (int i = 0; i < 2; ++i)
-#pragma unroll
-    for (int j = 0; j < 4; ++j)
-#pragma unroll
-      for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
-  const long long c0 = clock64();
-  const long long w0 = wall_clock64();
-  for (int64_t it = 0; it < iters; ++it) {
+  float total = 0.f;
+  long long c0, w0;
+  if constexpr (SHAPE == 32) {
+    probe_f32x16 acc[2][4];
 #pragma unroll
     for (int i = 0; i < 2; ++i)
 #pragma unroll
-      for (int j = 0; j < 4; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[i], b[j], acc[i][j], 0, 0, 0);
+      for (int j = 0; j < 4; ++j)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
+    c0 = clock64();
+    w0 = wall_clock64();
+    for (int64_t it = 0; it < iters; ++it) {
+#pragma unroll
+      for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[i], b[j], acc[i][j], 0, 0, 0);
+    }
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) total += acc[i][j][v];
+  } else {
+    probe_f32x4 acc[4][8];
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+      for (int j = 0; j < 8; ++j)
+#pragma unroll
+        for (int v = 0; v < 4; ++v) acc[i][j][v] = 0.f;
+    c0 = clock64();
+    w0 = wall_clock64();
+    for (int64_t it = 0; it < iters / 2; ++it) {
+#pragma unroll
+      for (int j = 0; j < 8; ++j)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[i], b[j], acc[i][j], 0, 0, 0);
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+      for (int j = 0; j < 8; ++j)
+#pragma unroll
+        for (int v = 0; v < 4; ++v) total += acc[i][j][v];
   }
-  float total = 0.f;
-#pragma unroll
-  for (int i = 0; i < 2; ++i)
-#pragma unroll
-    for (int j = 0; j < 4; ++j)
-#pragma unroll
-      for (int v = 0; v < 16; ++v) total += acc[i][j][v];
   if (clocks != nullptr && blockIdx.x == 0 && threadIdx.x == 0) {
     clocks[0] = clock64() - c0;
     clocks[1] = wall_clock64() - w0;

@@ -930,9 +930,10 @@ int vrl_stream_probe(const void* src, void* dst, int64_t n_rows, int64_t row_byt
   return launch_status();
 }
 
-int vrl_mfma_probe(int64_t n_workgroups, int64_t iters, int random_operands, float* sink, int64_t* clocks,
-                   int64_t* wall_clock_khz, void* stream) {
+int vrl_mfma_probe(int64_t n_workgroups, int64_t iters, int instruction, int random_operands, float* sink,
+                   int64_t* clocks, int64_t* wall_clock_khz, void* stream) {
   if (n_workgroups < 0 || iters < 0 || n_workgroups > kMaxGrid) return VRL_ERR_SHAPE;
+  if (instruction != 16 && instruction != 32) return VRL_ERR_ARG;
   if (wall_clock_khz != nullptr) {
     int dev = 0, khz = 0;
     if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&khz, hipDeviceAttributeWallClockRate, dev) != hipSuccess) {
@@ -944,8 +945,12 @@ int vrl_mfma_probe(int64_t n_workgroups, int64_t iters, int random_operands, flo
   if (n_workgroups == 0) return VRL_OK;
   if (sink == nullptr) return VRL_ERR_NULL;
   if (!aligned(sink, 4) || !aligned(clocks, 8)) return VRL_ERR_ALIGN;
-  vrl::mfma_probe_kernel<<<dim3(static_cast<unsigned>(n_workgroups)), dim3(512), 0, static_cast<hipStream_t>(stream)>>>(
-      iters, random_operands != 0 ? 1 : 0, sink, clocks);
+  const dim3 grid(static_cast<unsigned>(n_workgroups));
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  if (instruction == 16)
+    vrl::mfma_probe_kernel<16><<<grid, dim3(512), 0, s>>>(iters, random_operands != 0 ? 1 : 0, sink, clocks);
+  else
+    vrl::mfma_probe_kernel<32><<<grid, dim3(512), 0, s>>>(iters, random_operands != 0 ? 1 : 0, sink, clocks);
   return launch_status();
 }
 
