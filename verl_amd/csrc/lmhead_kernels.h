@@ -2,21 +2,23 @@
 // and folded straight into the online-softmax partial (m, s, t) of their token; they never reach HBM.
 //
 // lmhead_partial_kernel: one workgroup of 8 wavefronts (two per SIMD) owns 256 tokens and walks a range of 256-row
-// vocabulary tiles (its "split"); per tile it runs the full contraction in steps of 64 (v_mfma_f32_32x32x16 on
-// bf16 / fp16, fp32 accumulators). A wavefront owns a 64 (vocabulary) x 128 (tokens) part of the tile: 8 blocks of
-// 32x32 = 128 accumulator registers, so two wavefronts fit a SIMD and one's matrix instructions cover the other's
-// waits. Operands go global -> LDS directly (128-bit loads) into a ring of five 32 KiB operand tiles (all 160 KiB of a
-// CU's LDS, one workgroup per CU), swizzled so that the 128-bit fragment reads are free of bank conflicts (measured:
-// SQ_LDS_BANK_CONFLICT = 0). A step is four quarter steps of 16 contraction elements with one workgroup barrier, placed
-// before the LAST quarter's matrix instructions; the loads of the tiles two steps ahead are spread over the step
-// (lm_walk_tiles).
-// The MFMA is issued with the vocabulary on its row side so that a lane's 16 results of a block belong to ONE
-// token: the softmax state needs no cross-lane traffic until the very end.
+// vocabulary tiles (its "split"); per tile it runs the full contraction in steps of 64 (v_mfma_f32_16x16x32 on
+// bf16 / fp16, fp32 accumulators: with operands whose bits toggle like real data the power-managed part sustains a
+// higher clock on this instruction than on 32x32x16). A wavefront owns a 64 (vocabulary) x 128 (tokens) part of the
+// tile: 4 x 8 blocks of 16x16 = 128 accumulator registers, so two wavefronts fit a SIMD and one's matrix instructions
+// cover the other's waits. Operands go global -> LDS directly (128-bit loads) into a ring of five 32 KiB operand tiles
+// (all 160 KiB of a CU's LDS, one workgroup per CU), swizzled so that the 128-bit fragment reads are free of bank
+// conflicts (measured: SQ_LDS_BANK_CONFLICT = 0). A step is two halves of 32 contraction elements with one workgroup
+// barrier between them; the loads of the tiles two steps ahead are spread over the step (lm_walk_tiles).
+// The MFMA is issued with the vocabulary on its row side so that a lane's 4 results of a block are 4 consecutive
+// vocabulary entries of ONE token: the softmax state needs no cross-lane traffic until the very end, and a gradient
+// or product block is one 8-byte store.
 //
 // lmhead_dlogits_kernel: the same walk over (token block, vocabulary tiles) for the backward pass. The logits tile is
 // recomputed on the matrix cores and turned, in registers, into the gradient with respect to the logits
-// (the row-backward arithmetic of backward_kernels.h), which is stored in the operands' type; the two products that
-// follow (d hidden, d W) are plain GEMMs over that buffer.
+// (the row-backward arithmetic of backward_kernels.h), which is stored in the operands' type.
+//
+// lm_gemm_nt_kernel: out (+)= Y . X^T on the same walk, for the two products that follow (d hidden, d W).
 //
 // lmhead_finish_kernel: one wavefront per token forms the label's logit as a dot product in fp32, merges the
 // token's partials over the splits and writes log-prob, entropy and logsumexp (same finish as the row kernel).
@@ -35,7 +37,6 @@ namespace vrl {
 #define VRL_LDS_AS __attribute__((address_space(3)))
 #define VRL_GLOBAL_AS __attribute__((address_space(1)))
 
-typedef float lm_f32x16 __attribute__((ext_vector_type(16)));
 typedef float lm_f32x4 __attribute__((ext_vector_type(4)));
 
 constexpr int kLmTokens = 256;                    // tokens per workgroup tile
@@ -52,9 +53,6 @@ struct LmFrag;
 template <>
 struct LmFrag<1> {
   typedef __bf16 type __attribute__((ext_vector_type(8)));
-  __device__ static __forceinline__ lm_f32x16 mfma(type a, type b, lm_f32x16 c) {
-    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
-  }
   __device__ static __forceinline__ lm_f32x4 mfma16(type a, type b, lm_f32x4 c) {
     return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0);
   }
@@ -62,9 +60,6 @@ struct LmFrag<1> {
 template <>
 struct LmFrag<2> {
   typedef _Float16 type __attribute__((ext_vector_type(8)));
-  __device__ static __forceinline__ lm_f32x16 mfma(type a, type b, lm_f32x16 c) {
-    return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
-  }
   __device__ static __forceinline__ lm_f32x4 mfma16(type a, type b, lm_f32x4 c) {
     return __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, c, 0, 0, 0);
   }
@@ -113,39 +108,32 @@ __device__ __forceinline__ LmWork lm_work(int64_t V, int64_t T, int n_splits, in
   return w;
 }
 
-// Which load a wavefront issues behind matrix instruction `mm` (0..7) of quarter step `sb` (0..3) of a step:
-// 0 none, 1..4 part 0..3 of the W tile two steps ahead, 5..8 part 0..3 of the H tile two steps ahead.
-__device__ constexpr int lm_load_slot(int sb, int mm) {
-  if (sb == 3) return (mm & 1) ? 5 + (mm >> 1) : 0;
-  if (sb == 0) return mm == 1 ? 1 : mm == 5 ? 2 : 0;
-  if (sb == 1) return mm == 1 ? 3 : mm == 5 ? 4 : 0;
-  return 0;
-}
-
 // The matrix-core walk shared by the forward and backward kernels. All 512 threads call it. For every vocabulary
 // tile of `work` it forms the 256 x 256 block of logits of tokens [tok0_ld, tok0_ld + 256) and hands this wavefront's
-// 64 (vocabulary) x 128 (tokens) part to on_tile(vt, acc): acc[i][j][v] is the logit of
-//   vocabulary row  tile_row0 + wv*64 + i*32 + 8*(v>>2) + 4*(lane>>5) + (v&3)
-//   token           tok0_ld + wt*128 + j*32 + (lane&31)
+// 64 (vocabulary) x 128 (tokens) part to on_tile(vt, acc): acc[i][j][v] (i < 4, j < 8, v < 4) is the logit of
+//   vocabulary row  tile_row0 + wv*64 + i*16 + 4*(lane>>4) + v
+//   token           tok0_ld + wt*128 + j*16 + (lane&15)
 // with wv = wave>>1, wt = wave&1 and tile_row0 = vt*256 (V-256 for an edge tile, whose rows below vt*256 repeat the
 // tile before). `lds` is kLmLdsBytes (160 KiB), 1 KiB aligned. On return no load is in flight; callers that reuse
 // `lds` afterwards put a workgroup barrier first.
 //
 // LDS is a ring of five 32 KiB operand tiles. Item 2s is the W tile of global step s (a step = 64 contraction elements
-// of one vocabulary tile), item 2s+1 its H tile; item n lives in slot n mod 5. During step s:
-//   quarters 0, 1   request W(s+2) into the slot H(s-1) left (two loads per quarter and wavefront)
-//   quarter 2       no loads; its end is the step's only workgroup barrier: every wavefront holds the fragments of
-//                   quarter 3 in registers, so W(s) and H(s) are dead, and W(s+1), H(s+1) have landed (vmcnt(4): only
-//                   the four W(s+2) loads may still be in flight)
-//   quarter 3       requests H(s+2) into the slot W(s) left, reads the first fragments of step s+1
-// so the 64 loads a step needs are spread over it instead of arriving at the address unit in one burst, a W tile (the
-// operand that comes from HBM) has five quarters to land and an H tile (L2 / infinity cache) three. Within a quarter
-// every matrix instruction is followed by at most one fragment read and one load; the scheduling-group barriers pin
-// that interleave (left alone, the compiler gathers the reads in front of the barrier, where all eight wavefronts
-// then wait for them together).
+// of one vocabulary tile), item 2s+1 its H tile; item n lives in slot n mod 5. A step is two halves of 32 contraction
+// elements, 32 matrix instructions each, with ONE set of fragments (4 of W, 8 of H): the products run column by column,
+// an H fragment is dead after its 4 products and a W fragment after the last column, and each is refilled in place with
+// the next half's as soon as it is dead - the second half's from this step's tiles during the first half, the next
+// step's first half from the next tiles during the second. During step s:
+//   first half    requests W(s+2) into the slot H(s-1) left (four loads per wavefront)
+//   barrier       the step's only one: every wavefront holds the second half's fragments, so W(s) and H(s) are dead,
+//                 and W(s+1), H(s+1) have landed (vmcnt(4): only the four W(s+2) loads may still be in flight)
+//   second half   requests H(s+2) into the slot W(s) left
+// so the 64 loads a step needs are spread over it instead of arriving at the address unit in one burst, and the W tile
+// (the operand that comes from HBM) has a step and a half to land. Every matrix instruction is followed by at most one
+// fragment read and one load; the scheduling-group barriers pin that interleave (left alone, the compiler gathers the
+// reads in front of the barrier, where all eight wavefronts then wait for them together).
 // EPILOGUE_STORES: on_tile writes to global memory. Stores count in vmcnt like loads but complete in their own order,
 // so the first barrier after on_tile waits for everything.
-template <int DT, int SHAPE, bool EPILOGUE_STORES, class OnTile>
+template <int DT, bool EPILOGUE_STORES, class OnTile>
 __device__ __forceinline__ void lm_walk_tiles(const uint16_t* __restrict__ W, const uint16_t* __restrict__ H, int64_t V,
                                               int64_t K, int64_t w_stride, int64_t h_stride, const LmWork& work,
                                               char* lds, OnTile&& on_tile) {
@@ -220,179 +208,91 @@ __device__ __forceinline__ void lm_walk_tiles(const uint16_t* __restrict__ W, co
     ++h_step;
   };
 
-  if constexpr (SHAPE == 32) {
-    // fragment addressing: row (within its 32-row block) = lane&31, logical chunk = 2*sub + (lane>>5), sub in 0..3
-    int phys[4];
+  // row (within its 16-row block) = lane&15, logical chunk = 4*half + (lane>>4), half in 0..1
+  int phys[2];
 #pragma unroll
-    for (int sb = 0; sb < 4; ++sb) phys[sb] = (((2 * sb + (lane >> 5)) ^ ((lane >> 1) & 7)) * 16);
-    const int fragoff_w = (wv * 64 + (lane & 31)) * kLmRowBytes;    // within a W slot
-    const int fragoff_h = (wt * 128 + (lane & 31)) * kLmRowBytes;   // within an H slot
+  for (int hf = 0; hf < 2; ++hf) phys[hf] = (((4 * hf + (lane >> 4)) ^ ((lane >> 1) & 7)) * 16);
+  const int fragoff_w = (wv * 64 + (lane & 15)) * kLmRowBytes;    // within a W slot
+  const int fragoff_h = (wt * 128 + (lane & 15)) * kLmRowBytes;   // within an H slot
 
-    FragT a[2][2], b[2][4];
-    if (total_steps > 0) {
-      // W(0), H(0), W(1), H(1); the first two have to land before anything is read
+  FragT a[4], b[8];
+  if (total_steps > 0) {
 #pragma unroll
-      for (int rep = 0; rep < 2; ++rep) {
+    for (int rep = 0; rep < 2; ++rep) {
 #pragma unroll
-        for (int i = 0; i < 4; ++i) load_w(i);
-        advance_w();
+      for (int i = 0; i < 4; ++i) load_w(i);
+      advance_w();
 #pragma unroll
-        for (int i = 0; i < 4; ++i) load_h(i);
-        advance_h();
-      }
-      asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
-      __builtin_amdgcn_s_barrier();
-#pragma unroll
-      for (int i = 0; i < 2; ++i) a[0][i] = *reinterpret_cast<const FragT*>(lds + fragoff_w + i * 32 * kLmRowBytes + phys[0]);
-#pragma unroll
-      for (int j = 0; j < 4; ++j) b[0][j] = *reinterpret_cast<const FragT*>(lds + kLmTileBytes + fragoff_h + j * 32 * kLmRowBytes + phys[0]);
+      for (int i = 0; i < 4; ++i) load_h(i);
+      advance_h();
     }
-
-    int cw = 0, ch = 1;   // ring slots of the step being computed
-    bool after_epilogue = false;
-    for (int64_t vt = work.vt_begin; vt < work.vt_end; ++vt) {
-      lm_f32x16 acc[2][4];
+    asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
+    __builtin_amdgcn_s_barrier();
 #pragma unroll
-      for (int i = 0; i < 2; ++i)
+    for (int i = 0; i < 4; ++i) a[i] = *reinterpret_cast<const FragT*>(lds + fragoff_w + i * 16 * kLmRowBytes + phys[0]);
 #pragma unroll
-        for (int j = 0; j < 4; ++j)
-#pragma unroll
-          for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
-
-      for (int ks = 0; ks < ksteps; ++ks) {
-        const int nw = next_slot(cw), nh = next_slot(ch);
-#pragma unroll
-        for (int sb = 0; sb < 4; ++sb) {
-          const int cu = sb & 1, nx = cu ^ 1;
-          if (sb == 3) {
-            if (EPILOGUE_STORES && after_epilogue) {
-              asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
-            } else {
-              asm volatile("s_waitcnt vmcnt(4) lgkmcnt(0)" ::: "memory");
-            }
-            __builtin_amdgcn_s_barrier();
-            after_epilogue = false;
-          }
-          // this quarter's matrix instructions run on fragment set `cu`; the reads fill set `nx` for the next quarter
-          // (of this step's tiles, or, in quarter 3, the first of the next step's)
-          const char* rw = lds + ((sb == 3) ? nw : cw) * kLmTileBytes + fragoff_w;
-          const char* rh = lds + ((sb == 3) ? nh : ch) * kLmTileBytes + fragoff_h;
-          const int rq = (sb + 1) & 3;
-#pragma unroll
-          for (int mm = 0; mm < 8; ++mm) {
-            const int i = mm >> 2, j = mm & 3;
-            acc[i][j] = LmFrag<DT>::mfma(a[cu][i], b[cu][j], acc[i][j]);
-            if (mm == 0) a[nx][0] = *reinterpret_cast<const FragT*>(rw + phys[rq]);
-            else if (mm < 5) b[nx][mm - 1] = *reinterpret_cast<const FragT*>(rh + (mm - 1) * 32 * kLmRowBytes + phys[rq]);
-            else if (mm == 5) a[nx][1] = *reinterpret_cast<const FragT*>(rw + 32 * kLmRowBytes + phys[rq]);
-            const int op = lm_load_slot(sb, mm);
-            if (op >= 5) load_h(op - 5);
-            else if (op >= 1) load_w(op - 1);
-          }
-#pragma unroll
-          for (int mm = 0; mm < 8; ++mm) {
-            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                                   // one matrix instruction
-            if (mm < 6) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);                       // one LDS read
-            if (lm_load_slot(sb, mm) != 0) __builtin_amdgcn_sched_group_barrier(0x010, 1, 0);   // one load
-          }
-          __builtin_amdgcn_sched_barrier(0);
-          if (sb == 1) advance_w();
-          if (sb == 3) advance_h();
-        }
-        cw = nw;
-        ch = nh;
-      }
-      on_tile(vt, acc);
-      after_epilogue = true;
-    }
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // the last, redundant loads still target the ring
-  } else {
-    // row (within its 16-row block) = lane&15, logical chunk = 4*half + (lane>>4), half in 0..1
-    int phys[2];
-#pragma unroll
-    for (int hf = 0; hf < 2; ++hf) phys[hf] = (((4 * hf + (lane >> 4)) ^ ((lane >> 1) & 7)) * 16);
-    const int fragoff_w = (wv * 64 + (lane & 15)) * kLmRowBytes;    // within a W slot
-    const int fragoff_h = (wt * 128 + (lane & 15)) * kLmRowBytes;   // within an H slot
-
-    FragT a[4], b[8];
-    if (total_steps > 0) {
-#pragma unroll
-      for (int rep = 0; rep < 2; ++rep) {
-#pragma unroll
-        for (int i = 0; i < 4; ++i) load_w(i);
-        advance_w();
-#pragma unroll
-        for (int i = 0; i < 4; ++i) load_h(i);
-        advance_h();
-      }
-      asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
-      __builtin_amdgcn_s_barrier();
-#pragma unroll
-      for (int i = 0; i < 4; ++i) a[i] = *reinterpret_cast<const FragT*>(lds + fragoff_w + i * 16 * kLmRowBytes + phys[0]);
-#pragma unroll
-      for (int j = 0; j < 8; ++j) b[j] = *reinterpret_cast<const FragT*>(lds + kLmTileBytes + fragoff_h + j * 16 * kLmRowBytes + phys[0]);
-    }
-
-    int cw = 0, ch = 1;   // ring slots of the step being computed
-    bool after_epilogue = false;
-    for (int64_t vt = work.vt_begin; vt < work.vt_end; ++vt) {
-      lm_f32x4 acc[4][8];
-#pragma unroll
-      for (int i = 0; i < 4; ++i)
-#pragma unroll
-        for (int j = 0; j < 8; ++j)
-#pragma unroll
-          for (int v = 0; v < 4; ++v) acc[i][j][v] = 0.f;
-
-      for (int ks = 0; ks < ksteps; ++ks) {
-        const int nw = next_slot(cw), nh = next_slot(ch);
-        // Two halves of 32 contraction elements, 32 matrix instructions each, with ONE set of fragments (4 of W, 8 of H):
-        // the products run column by column, an H fragment is dead after its 4 products and a W fragment after the last
-        // column, and each is refilled in place with the next half's as soon as it is dead - the second half's from this
-        // step's tiles during the first half, the next step's first half from the next tiles during the second. The
-        // step's barrier therefore sits between the halves: behind it W(s), H(s) are dead and W(s+1), H(s+1) must have
-        // landed. First half: the four loads of W(s+2) (into the slot H(s-1) left); second half: H(s+2) (slot of W(s)).
-#pragma unroll
-        for (int hf = 0; hf < 2; ++hf) {
-          if (hf == 1) {
-            if (EPILOGUE_STORES && after_epilogue) {
-              asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
-            } else {
-              asm volatile("s_waitcnt vmcnt(4) lgkmcnt(0)" ::: "memory");
-            }
-            __builtin_amdgcn_s_barrier();
-            after_epilogue = false;
-          }
-          const char* rw = lds + ((hf == 1) ? nw : cw) * kLmTileBytes + fragoff_w + phys[hf ^ 1];
-          const char* rh = lds + ((hf == 1) ? nh : ch) * kLmTileBytes + fragoff_h + phys[hf ^ 1];
-#pragma unroll
-          for (int mm = 0; mm < 32; ++mm) {
-            const int j = mm >> 2, i = mm & 3;
-            acc[i][j] = LmFrag<DT>::mfma16(a[i], b[j], acc[i][j]);
-            if (i == 3) b[j] = *reinterpret_cast<const FragT*>(rh + j * 16 * kLmRowBytes);
-            if (j == 7) a[i] = *reinterpret_cast<const FragT*>(rw + i * 16 * kLmRowBytes);
-            if ((mm & 7) == 1) {
-              if (hf == 0) load_w(mm >> 3); else load_h(mm >> 3);
-            }
-          }
-#pragma unroll
-          for (int mm = 0; mm < 32; ++mm) {
-            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                                // one matrix instruction
-            if ((mm & 3) == 3) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);             // an H fragment
-            if ((mm >> 2) == 7) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);            // a W fragment
-            if ((mm & 7) == 1) __builtin_amdgcn_sched_group_barrier(0x010, 1, 0);             // one load
-          }
-          __builtin_amdgcn_sched_barrier(0);
-          if (hf == 0) advance_w(); else advance_h();
-        }
-        cw = nw;
-        ch = nh;
-      }
-      on_tile(vt, acc);
-      after_epilogue = true;
-    }
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // the last, redundant loads still target the ring
+    for (int j = 0; j < 8; ++j) b[j] = *reinterpret_cast<const FragT*>(lds + kLmTileBytes + fragoff_h + j * 16 * kLmRowBytes + phys[0]);
   }
+
+  int cw = 0, ch = 1;   // ring slots of the step being computed
+  bool after_epilogue = false;
+  for (int64_t vt = work.vt_begin; vt < work.vt_end; ++vt) {
+    lm_f32x4 acc[4][8];
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+      for (int j = 0; j < 8; ++j)
+#pragma unroll
+        for (int v = 0; v < 4; ++v) acc[i][j][v] = 0.f;
+
+    for (int ks = 0; ks < ksteps; ++ks) {
+      const int nw = next_slot(cw), nh = next_slot(ch);
+      // Two halves of 32 contraction elements, 32 matrix instructions each, with ONE set of fragments (4 of W, 8 of H):
+      // the products run column by column, an H fragment is dead after its 4 products and a W fragment after the last
+      // column, and each is refilled in place with the next half's as soon as it is dead - the second half's from this
+      // step's tiles during the first half, the next step's first half from the next tiles during the second. The
+      // step's barrier therefore sits between the halves: behind it W(s), H(s) are dead and W(s+1), H(s+1) must have
+      // landed. First half: the four loads of W(s+2) (into the slot H(s-1) left); second half: H(s+2) (slot of W(s)).
+#pragma unroll
+      for (int hf = 0; hf < 2; ++hf) {
+        if (hf == 1) {
+          if (EPILOGUE_STORES && after_epilogue) {
+            asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+          } else {
+            asm volatile("s_waitcnt vmcnt(4) lgkmcnt(0)" ::: "memory");
+          }
+          __builtin_amdgcn_s_barrier();
+          after_epilogue = false;
+        }
+        const char* rw = lds + ((hf == 1) ? nw : cw) * kLmTileBytes + fragoff_w + phys[hf ^ 1];
+        const char* rh = lds + ((hf == 1) ? nh : ch) * kLmTileBytes + fragoff_h + phys[hf ^ 1];
+#pragma unroll
+        for (int mm = 0; mm < 32; ++mm) {
+          const int j = mm >> 2, i = mm & 3;
+          acc[i][j] = LmFrag<DT>::mfma16(a[i], b[j], acc[i][j]);
+          if (i == 3) b[j] = *reinterpret_cast<const FragT*>(rh + j * 16 * kLmRowBytes);
+          if (j == 7) a[i] = *reinterpret_cast<const FragT*>(rw + i * 16 * kLmRowBytes);
+          if ((mm & 7) == 1) {
+            if (hf == 0) load_w(mm >> 3); else load_h(mm >> 3);
+          }
+        }
+#pragma unroll
+        for (int mm = 0; mm < 32; ++mm) {
+          __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                                // one matrix instruction
+          if ((mm & 3) == 3) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);             // an H fragment
+          if ((mm >> 2) == 7) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);            // a W fragment
+          if ((mm & 7) == 1) __builtin_amdgcn_sched_group_barrier(0x010, 1, 0);             // one load
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        if (hf == 0) advance_w(); else advance_h();
+      }
+      cw = nw;
+      ch = nh;
+    }
+    on_tile(vt, acc);
+    after_epilogue = true;
+  }
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // the last, redundant loads still target the ring
 }
 
 // grid.x = token blocks * n_splits, block = 512, dynamic LDS = kLmLdsBytes. Writes, per (token, split), the online-softmax
@@ -423,7 +323,7 @@ __global__ __launch_bounds__(kLmWaves * 64, 1) void lmhead_partial_kernel(
     c[j] = make_scale<false>(temperature, tok).c;   // log2(e) / max(T, 1e-8), exactly what the finishing kernel uses
   }
 
-  lm_walk_tiles<DT, 16, false>(W, H, V, K, w_stride, h_stride, work, lds, [&](int64_t vt, lm_f32x4 (&acc)[4][8]) {
+  lm_walk_tiles<DT, false>(W, H, V, K, w_stride, h_stride, work, lds, [&](int64_t vt, lm_f32x4 (&acc)[4][8]) {
     // fold 16 logits per token column into the running state (maximum first, then the exponentials; nothing is
     // buffered): acc[i][j][v] is vocabulary row tile_row0 + wv*64 + i*16 + 4*(lane>>4) + v of token column j
     const bool edge = (vt + 1) * kLmVocab > V;
@@ -575,7 +475,7 @@ __global__ __launch_bounds__(kLmWaves * 64, 1) void lmhead_dlogits_kernel(
     label[j] = (lab >= 0 && lab < V) ? (int)lab : -1;   // an out-of-range label was reported by the forward pass
   }
 
-  lm_walk_tiles<DT, 16, true>(W, H, V, K, w_stride, h_stride, work, lds, [&](int64_t vt, lm_f32x4 (&acc)[4][8]) {
+  lm_walk_tiles<DT, true>(W, H, V, K, w_stride, h_stride, work, lds, [&](int64_t vt, lm_f32x4 (&acc)[4][8]) {
     // acc[i][j][0..3]: vocabulary entries vr .. vr+3, vr = tile_row0 + wv*64 + i*16 + 4*(lane>>4), of token column j
     const bool edge = (vt + 1) * kLmVocab > V;
     const int vrow0 = (int)(edge ? V - kLmVocab : vt * kLmVocab) + wv * 64 + 4 * (lane >> 4);
@@ -683,7 +583,7 @@ __global__ __launch_bounds__(kLmWaves * 64, 1) void lm_gemm_nt_kernel(
   int64_t nsteps = g.k_steps - step0;
   if (nsteps > g.steps_per_part) nsteps = g.steps_per_part;
 
-  lm_walk_tiles<DT, 16, true>(X + step0 * kLmK, Y + step0 * kLmK, g.NX, nsteps * kLmK, x_stride, y_stride, work, lds,
+  lm_walk_tiles<DT, true>(X + step0 * kLmK, Y + step0 * kLmK, g.NX, nsteps * kLmK, x_stride, y_stride, work, lds,
                               [&](int64_t vt, lm_f32x4 (&acc)[4][8]) {
     // acc[i][j][0..3]: columns x0 .. x0+3 of out, x0 = tile_row0 + wv*64 + i*16 + 4*(lane>>4), of row
     // y = tok0_ld + wt*128 + j*16 + (lane&15)
