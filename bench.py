@@ -383,12 +383,16 @@ def bench_lm_head(args, dev):
         with torch.no_grad():
             return fused_linear_for_ppo(hidden, weight, ids, temperature, chunk)
 
+    def fwd_library():
+        with torch.no_grad():
+            return fused_linear_for_ppo(hidden, weight, ids, temperature, chunk, False, "library")
+
     def fwd_bwd():
         lp, h = fused_linear_for_ppo(hidden, weight, ids, temperature, chunk, keep)
         return torch.autograd.grad((lp, h), (hidden, weight), (g_lp, g_h))
 
-    # guard: first tokens against torch in fp32 on the bf16 logits the same GEMM produces
-    lp, h = fwd()
+    # guard: first tokens of the library forward against torch in fp32 on the bf16 logits the same GEMM produces
+    lp, h = fwd_library()
     z = torch.matmul(hidden[:256].detach(), weight.detach().t()).float() / temperature
     e1 = (lp[:256] - torch.log_softmax(z, -1).gather(-1, ids[:256, None]).squeeze(-1)).abs().max().item()
     e2 = (h[:256] - (torch.logsumexp(z, -1) - (torch.softmax(z, -1) * z).sum(-1))).abs().max().item()
@@ -438,6 +442,7 @@ def bench_lm_head(args, dev):
         del gb
     del ga
     t_f = timed(fwd)
+    t_f_lib = timed(fwd_library)
     t_fb = timed(fwd_bwd)
     t_fb_lib = timed(fwd_bwd_library)
     t_m = timed(fwd_mfma)
@@ -454,14 +459,14 @@ def bench_lm_head(args, dev):
         "config": {"workload": "lm_head_8192x3584_v152064_bf16", "chunk_tokens": chunk, "keep_logits": keep,
                    "temperature": temperature,
                    "step": "verl_amd.fused_linear_for_ppo forward + torch.autograd.grad for hidden and weight, default "
-                           "kernels (\"auto\": library GEMM + row kernel forward; backward vrl_lmhead_dlogits, vrl_gemm_nt for d hidden, a "
-                           "library GEMM for d W)"},
+                           "kernels (\"auto\": vrl_lmhead_score forward; backward vrl_lmhead_dlogits, vrl_gemm_nt for d hidden, a library "
+                           "GEMM for d W)"},
         "forward_ms": t_f * 1e3,
         "forward_tokens_per_s": T / t_f,
         "roofline": {"bound": "mfma", "achieved": flops_fb / t_fb / 1e12, "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
                      "frac": flops_fb / t_fb / 1e12 / MFMA_BF16_PEAK_TFLOPS, "traffic": None,
-                     "kernel": "hipBLASLt bf16 GEMMs (forward logits, d W) + rowscore_kernel + lmhead_dlogits_kernel<bf16> + "
-                               "lm_gemm_nt_kernel<bf16> (d hidden)",
+                     "kernel": "lmhead_partial_kernel<bf16> + lmhead_finish_kernel, lmhead_dlogits_kernel<bf16>, "
+                               "lm_gemm_nt_kernel<bf16> (d hidden), hipBLASLt bf16 GEMM (d W)",
                      "forward_tflops": flops_f / t_f / 1e12},
         "single_kernel_forward": {"ms": t_m * 1e3, "tflops": flops_f / t_m / 1e12, "frac_of_mfma_peak": flops_f / t_m / 1e12 / MFMA_BF16_PEAK_TFLOPS,
                                   "kernel": "lmhead_partial_kernel<bf16> + lmhead_finish_kernel (vrl_lmhead_score)",
@@ -469,10 +474,10 @@ def bench_lm_head(args, dev):
                                   "frac_of_sustained_mfma_rate": flops_f / t_m / 1e12 / ceiling["tflops"],
                                   "note": "hand-written MFMA kernel, logits never written"},
         "matrix_core_ceiling": ceiling,
-        "all_library": {"forward_backward_ms": t_fb_lib * 1e3, "kernel": "torch.matmul for every product"},
+        "all_library": {"forward_ms": t_f_lib * 1e3, "forward_backward_ms": t_fb_lib * 1e3,
+                        "kernel": "torch.matmul for every product (kernels=\"library\")"},
         "matrix_core_backward": {"forward_backward_ms": t_fb_m * 1e3,
-                                 "kernel": "kernels=\"mfma\": the default's backward; without gradients the forward is the single "
-                                           "kernel",
+                                 "kernel": "kernels=\"mfma\": the same kernels as the default today",
                                  "note": "the logits are formed again by the hand-written MFMA kernel and their gradient "
                                          "is written from registers (no GEMM into the buffer, no pass over it); d hidden "
                                          "comes from the same main loop"},

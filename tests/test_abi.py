@@ -322,7 +322,6 @@ def test_lmhead_argument_errors(lib):
     assert call(T=255) == _lib.VRL_ERR_SHAPE and call(V=100) == _lib.VRL_ERR_SHAPE
     assert call(K=96) == _lib.VRL_ERR_SHAPE and call(hs=64) == _lib.VRL_ERR_SHAPE and call(ws=132) == _lib.VRL_ERR_SHAPE
     assert call(S=0) == _lib.VRL_ERR_SHAPE and call(S=65) == _lib.VRL_ERR_SHAPE
-    assert call(V=1 << 25, K=64, hs=64, ws=64) == _lib.VRL_ERR_SHAPE          # weight of 4 GiB: 32-bit offsets
     assert call(lp=None, ent=None) == _lib.VRL_ERR_ARG
     assert call(h=None) == _lib.VRL_ERR_NULL and call(part=None) == _lib.VRL_ERR_NULL
     assert call(lab=None) == _lib.VRL_ERR_NULL and call(flag=None) == _lib.VRL_ERR_NULL

@@ -53,7 +53,11 @@ def test_bf16_module_3d_inputs(dev):
     hidden = torch.empty(B, S, D, device=dev).uniform_(-0.5, 0.5, generator=g).bfloat16().requires_grad_()
     weight = torch.empty(V, D, device=dev).uniform_(-0.5, 0.5, generator=g).bfloat16().requires_grad_()
     labels = torch.randint(0, V, (B, S), generator=g, device=dev)
-    mod = FusedLinearForPPO(chunk_size=64)
+    # the default forward keeps the logits in fp32: it sits on the all-fp32 reference
+    d_lp, d_ent = FusedLinearForPPO(chunk_size=64)(hidden, weight, labels, temperature=1.5)
+    f_lp, f_ent = _torch_reference(hidden.detach().view(-1, D), weight.detach(), labels.view(-1), 1.5)
+    assert (d_lp.view(-1) - f_lp).abs().max().item() <= 1e-4 and (d_ent.view(-1) - f_ent).abs().max().item() <= 1e-4
+    mod = FusedLinearForPPO(chunk_size=64, kernels="library")
     lp, ent = mod(hidden, weight, labels, temperature=1.5)
     assert lp.shape == (B, S) and ent.shape == (B, S)
     # the kernels' share, exactly: fp32 math on the bf16 logits the library GEMM produced

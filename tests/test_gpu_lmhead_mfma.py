@@ -196,16 +196,51 @@ def test_fused_linear_with_the_matrix_core_kernels(dev):
 
 def test_close_to_the_library_path_and_3d_inputs(dev):
     g = torch.Generator(device=dev).manual_seed(4)
-    B, S, K, V = 2, 260, 256, 5003
+    B, S, K, V = 2, 260, 256, 5008
     h = torch.empty(B, S, K, device=dev).uniform_(-0.5, 0.5, generator=g).bfloat16()
     w = torch.empty(V, K, device=dev).uniform_(-0.5, 0.5, generator=g).bfloat16()
     ids = torch.randint(0, V, (B, S), generator=g, device=dev)
     lp, ent = lm_head_score_mfma(h, w, ids, 1.5)
     with torch.no_grad():
-        lp2, ent2 = fused_linear_for_ppo(h, w, ids, 1.5)
+        lp2, ent2 = fused_linear_for_ppo(h, w, ids, 1.5, kernels="library")
+        lp3, ent3 = fused_linear_for_ppo(h, w, ids, 1.5)
     assert lp.shape == (B, S)
-    # the other path rounds |logit| ~ 3 to bf16 (2^-8 relative) before the softmax
+    # the library path rounds |logit| ~ 3 to bf16 (2^-8 relative) before the softmax
     assert (lp - lp2).abs().max().item() <= 3e-2 and (ent - ent2).abs().max().item() <= 3e-2
+    # the default forward IS this kernel
+    assert torch.equal(lp3, lp) and torch.equal(ent3, ent)
+
+
+def test_default_forward_is_the_same_with_and_without_gradients_and_for_any_token_count(dev):
+    """A trainer compares old log-probs (no gradients, its own micro-batching) with new ones (gradients, other
+    micro-batches) of the same weights: the default forward must give the same bits for a token whatever the call
+    looks like. Fewer than 256 tokens are padded to one block."""
+    g = torch.Generator(device=dev).manual_seed(14)
+    T, K, V = 700, 128, 3000
+    h = torch.empty(T, K, device=dev).uniform_(-0.5, 0.5, generator=g).bfloat16()
+    w = torch.empty(V, K, device=dev).uniform_(-0.5, 0.5, generator=g).bfloat16()
+    ids = torch.randint(0, V, (T,), generator=g, device=dev)
+    with torch.no_grad():
+        lp_all, ent_all = fused_linear_for_ppo(h, w, ids, 0.8)
+    hg, wg = h.clone().requires_grad_(), w.clone().requires_grad_()
+    lp_g, ent_g = fused_linear_for_ppo(hg, wg, ids, 0.8, chunk_size=256)
+    assert torch.equal(lp_g.detach(), lp_all) and torch.equal(ent_g.detach(), ent_all)
+    for lo, hi in ((0, 100), (100, 356), (356, 700), (699, 700)):
+        with torch.no_grad():
+            lp_p, ent_p = fused_linear_for_ppo(h[lo:hi], w, ids[lo:hi], 0.8)
+        assert torch.equal(lp_p, lp_all[lo:hi]) and torch.equal(ent_p, ent_all[lo:hi]), (lo, hi)
+        lp_q, ent_q = fused_linear_for_ppo(hg[lo:hi], wg, ids[lo:hi], 0.8)
+        assert torch.equal(lp_q.detach(), lp_all[lo:hi]), (lo, hi)
+    # gradients through the padded call
+    lp_q, ent_q = fused_linear_for_ppo(hg[:100], wg, ids[:100], 0.8)
+    d_h, d_w = torch.autograd.grad((lp_q.sum() + 0.1 * ent_q.sum(),), (hg, wg))
+    hf, wf = h.float().requires_grad_(), w.float().requires_grad_()
+    z = (hf[:100] @ wf.t()) / 0.8
+    ref = torch.log_softmax(z, -1).gather(-1, ids[:100, None]).sum() + 0.1 * (torch.logsumexp(z, -1) - (torch.softmax(z, -1) * z).sum(-1)).sum()
+    r_h, r_w = torch.autograd.grad(ref, (hf, wf))
+    torch.testing.assert_close(r_h, d_h.float(), atol=2e-2, rtol=4e-2)
+    torch.testing.assert_close(r_w, d_w.float(), atol=2e-2, rtol=4e-2)
+    assert not d_h[100:].any()
 
 
 def test_special_values_and_errors(dev):
@@ -218,8 +253,11 @@ def test_special_values_and_errors(dev):
     bad[7] = V
     with pytest.raises(IndexError):
         lm_head_score_mfma(h, w, bad)
+    short = lm_head_score_mfma(h[:100], w, ids[:100])               # fewer than 256 tokens: padded to one block
+    full = lm_head_score_mfma(h, w, ids)
+    assert torch.equal(short[0], full[0][:100]) and torch.equal(short[1], full[1][:100])
     with pytest.raises(ValueError):
-        lm_head_score_mfma(h[:100], w, ids[:100])                  # fewer than 256 tokens
+        lm_head_score_mfma(h, w[:200], ids.clamp(max=199))         # fewer than 256 vocabulary entries
     with pytest.raises(ValueError):
         lm_head_score_mfma(h[:, :32], w[:, :32], ids)              # hidden size not a multiple of 64
     with pytest.raises(TypeError):

@@ -330,8 +330,6 @@ int check_lmhead_shape(int dtype, int64_t n_tokens, int64_t vocab, int64_t hidde
       h_stride < hidden_size || w_stride < hidden_size || h_stride % 8 != 0 || w_stride % 8 != 0 ||
       n_splits < 1 || n_splits > vrl::kLmMaxSplits)
     return VRL_ERR_SHAPE;
-  // 32-bit byte offsets inside each operand; grid size
-  if (vocab * w_stride * 2 >= (1LL << 32) || n_tokens * h_stride * 2 >= (1LL << 32)) return VRL_ERR_SHAPE;
   if (((n_tokens + vrl::kLmTokens - 1) / vrl::kLmTokens) * n_splits > kMaxGrid || (n_tokens + 3) / 4 > kMaxGrid)
     return VRL_ERR_SHAPE;
   return VRL_OK;

@@ -1,13 +1,19 @@
 """LM head + scoring without ever holding the full ``(tokens, vocab)`` logits.
 
 Same call as the reference's ``FusedLinearForPPO`` (verl/utils/experimental/torch_functional.py:211-231):
-``(hidden_states, vocab_weights, input_ids, temperature) -> (log_probs fp32, entropy)``, chunked over
-tokens. Per chunk the projection ``hidden @ W^T`` is one library GEMM (torch.matmul, i.e. hipBLASLt)
-into a reusable ``(chunk, vocab)`` buffer, and everything after it is the HIP row kernel: forward
-``vrl_rowscore`` (one pass over the chunk's logits), backward ``vrl_rowscore_backward`` writing the
-gradient over the recomputed logits in place, followed by the two GEMMs for ``d hidden`` and ``d W``.
-The reference does the post-GEMM part with ~10 torch ops per chunk (softmax, logsumexp, log_softmax,
-gather, scatter, ...; :27-79); peak extra memory here is one ``(chunk, vocab)`` buffer.
+``(hidden_states, vocab_weights, input_ids, temperature) -> (log_probs fp32, entropy)``.
+
+Default path (bf16 / fp16 models): the forward is one hand-written matrix-core kernel that folds the logits into the
+softmax state as it forms them and never writes them (``vrl_lmhead_score``); the backward walks the tokens in chunks, forms
+each chunk's logits again on the matrix cores and writes their gradient into a reusable ``(chunk, vocab)`` buffer
+(``vrl_lmhead_dlogits``), then forms ``d hidden`` with ``vrl_gemm_nt`` and ``d W`` with a library GEMM. Peak extra memory
+is that one buffer, in the backward only.
+
+Library path (``kernels="library"``, fp32 models, ``keep_logits=True``): per chunk the projection ``hidden @ W^T`` is one
+library GEMM (torch.matmul, i.e. hipBLASLt) into the buffer, and everything after it is the HIP row kernel: forward
+``vrl_rowscore`` (one pass over the chunk's logits), backward ``vrl_rowscore_backward`` writing the gradient over the
+recomputed logits in place, followed by the two GEMMs. The reference does the post-GEMM part with ~10 torch ops per chunk
+(softmax, logsumexp, log_softmax, gather, scatter, ...; :27-79).
 """
 
 from __future__ import annotations
@@ -32,30 +38,40 @@ DEFAULT_CHUNK_TOKENS = 4096
 
 # Which matrix products are this package's own kernels.
 #   "library": every product is torch.matmul (hipBLASLt); the row kernels run over the chunk buffer.
-#   "mfma":    every step that has a hand-written matrix-core kernel uses it: the forward without gradients is one
-#              kernel that never writes logits (vrl_lmhead_score), the backward forms the logits again and writes their
-#              gradient from registers (vrl_lmhead_dlogits) and forms d hidden with vrl_gemm_nt; d W stays a library
-#              product (the hand-written one needs a transposed copy of the gradient buffer).
-#   "auto":    each step by what is measured fastest on MI355X at 8192 x 3584 -> 152064 bf16, as long as the forward is the
-#              same arithmetic with and without gradients: library GEMM + row kernel for the forward; in the backward
-#              vrl_lmhead_dlogits (3.46 ms per 4096 tokens against 3.53 ms for the library GEMM + row backward) and
-#              vrl_gemm_nt for d hidden (3.36 against 3.73 ms), library for d W. The single forward kernel is
-#              as fast as the library GEMM + row kernel (6.52 against 6.53 ms) and needs no buffer, but it keeps the
-#              logits in fp32 where the GEMM rounds them to the operand type: old log-probs from it (no gradients)
-#              and new ones from the GEMM (gradients) would differ by that rounding, a policy ratio other than 1 before
-#              any update. "mfma" accepts that; "auto" does not.
-# The environment variable and the ``kernels`` argument select; shapes a hand-written kernel does not take go to the library.
+#   "auto" (default) and "mfma" (the same today): every step that has a hand-written matrix-core kernel which is at least
+#              as fast as the library uses it. The forward is one kernel that never writes logits (vrl_lmhead_score: as fast
+#              as the library GEMM + row kernel at 8192 x 3584 -> 152064 bf16, 6.5 ms, no (chunk, vocab) buffer, logits kept
+#              in fp32), with and without gradients and whatever the number of tokens, so that old (no-grad) and new
+#              (grad) log-probs of the same weights are bit-identical; the backward forms the logits again and writes
+#              their gradient from registers (vrl_lmhead_dlogits, 3.46 ms per 4096 tokens against 3.53 ms for the library
+#              GEMM + row backward) and forms d hidden with vrl_gemm_nt (3.36 against 3.73 ms); d W stays a library product
+#              (the hand-written one needs a transposed copy of the gradient buffer). keep_logits=True needs the logits
+#              in memory and therefore takes the library forward, also without gradients.
+# The environment variable and the ``kernels`` argument select; models the kernels do not take (fp32, a hidden size that is
+# not a multiple of 64, fewer than 256 vocabulary entries) go to the library.
 DEFAULT_KERNELS = os.environ.get("VERL_AMD_LMHEAD_KERNELS", "auto")
 
 
-def _mfma_takes(hidden: torch.Tensor, weight: torch.Tensor, n_tokens: int) -> bool:
-    """Shape rules of vrl_lmhead_score / vrl_lmhead_dlogits (include/vrl.h)."""
+def _mfma_takes_model(hidden: torch.Tensor, weight: torch.Tensor) -> bool:
+    """Whether the matrix-core LM-head kernels take this model (element type, hidden size, vocabulary): everything
+    about their shape rules (include/vrl.h) that does not depend on how many tokens a call brings."""
     V, K = weight.shape
-    return (hidden.dtype in (torch.bfloat16, torch.float16) and n_tokens >= 256 and V >= 256 and V % 8 == 0
-            and K % 64 == 0 and hidden.stride(-1) == 1 and weight.stride(-1) == 1
+    return (hidden.dtype in (torch.bfloat16, torch.float16) and V >= 256 and V % 8 == 0 and K % 64 == 0
+            and hidden.stride(-1) == 1 and weight.stride(-1) == 1
             and hidden.stride(0) % 8 == 0 and weight.stride(0) % 8 == 0
-            and V * weight.stride(0) * 2 < (1 << 32) and n_tokens * hidden.stride(0) * 2 < (1 << 32)
             and hidden.data_ptr() % 16 == 0 and weight.data_ptr() % 16 == 0)
+
+
+def _mfma_takes(hidden: torch.Tensor, weight: torch.Tensor, n_tokens: int) -> bool:
+    """Shape rules of vrl_lmhead_score / vrl_lmhead_dlogits (include/vrl.h) for a call with ``n_tokens`` rows."""
+    return n_tokens >= 256 and _mfma_takes_model(hidden, weight)
+
+
+def _own_forward_in_use(kernels: str, keep_logits: bool, hidden: torch.Tensor, weight: torch.Tensor) -> bool:
+    """Whether the forward is vrl_lmhead_score. Decided by the caller's options and by the model only, never by the number
+    of tokens or by whether gradients are recorded: a trainer's old (no-grad) and new (grad) log-probs of the same
+    weights then come from the same arithmetic whatever the micro-batch sizes are."""
+    return kernels != "library" and not keep_logits and _mfma_takes_model(hidden, weight)
 
 
 # From this many tokens on, one transposed copy of the weight per backward (0.44 ms for 152064 x 3584 bf16) is
@@ -94,6 +110,14 @@ class _FusedLinearForPPOFunction(torch.autograd.Function):
         h = torch.empty(T, **f32)
         lse = torch.empty(T, **f32)
         flag = torch.zeros(1, dtype=torch.int32, device=dev)
+        if _own_forward_in_use(kernels, keep_logits, hidden, weight):
+            temp_all = None if temperature == 1.0 else torch.full((T,), float(temperature), **f32)
+            lp, h, lse = _own_forward(hidden, weight, input_ids, temp_all, None, "fused_linear_for_ppo")
+            ctx.save_for_backward(hidden, weight, input_ids, lse, h)
+            ctx.temperature = float(temperature)
+            ctx.chunk_size = int(chunk_size)
+            ctx.kept_logits = None
+            return lp.clone(), h.clone()
         temp = None if temperature == 1.0 else torch.full((min(chunk_size, max(T, 1)),), float(temperature), **f32)
         lib = _lib.load()
         keep = bool(keep_logits) and T > 0 and (ctx.needs_input_grad[0] or ctx.needs_input_grad[1])
@@ -207,12 +231,12 @@ def fused_linear_for_ppo(hidden_states: torch.Tensor, vocab_weights: torch.Tenso
     projecting again and forms ``d hidden`` and ``d W`` with one product each. Such a graph can be differentiated once.
 
     ``kernels`` chooses which matrix products are this package's own kernels: ``"library"`` (none: torch.matmul
-    throughout), ``"mfma"`` (all that exist: no buffer at all when no gradient is recorded, a backward that forms the
-    logits again and writes their gradient straight from registers, ``d hidden`` from ``vrl_gemm_nt``; ``d W`` stays a
-    library product) or ``"auto"`` (each step by what measures fastest on MI355X while log-probs computed with and
-    without gradients stay bit-identical: a library product for the forward's logits, this package's kernels for the
-    backward's gradient of the logits and ``d hidden``); None takes ``DEFAULT_KERNELS`` ("auto" unless ``VERL_AMD_LMHEAD_KERNELS`` says
-    otherwise).
+    throughout) or ``"auto"`` / ``"mfma"`` (all that are at least as fast: a forward that is one kernel and never
+    writes logits, a backward that forms the logits again, writes their gradient straight from registers and forms
+    ``d hidden`` with ``vrl_gemm_nt``; ``d W`` stays a library product). Which forward runs depends on this option, on
+    ``keep_logits`` and on the model, never on the number of tokens or on whether gradients are recorded, so log-probs
+    computed with and without gradients are bit-identical. None takes ``DEFAULT_KERNELS`` ("auto" unless
+    ``VERL_AMD_LMHEAD_KERNELS`` says otherwise).
     """
     kernels = DEFAULT_KERNELS if kernels is None else kernels
     if kernels not in ("auto", "library", "mfma"):
@@ -240,24 +264,62 @@ def fused_linear_for_ppo(hidden_states: torch.Tensor, vocab_weights: torch.Tenso
     ids = input_ids.reshape(-1).to(device=h2.device, dtype=torch.int64).contiguous()
     w2 = vocab_weights.contiguous()
     needs_grad = torch.is_grad_enabled() and (h2.requires_grad or w2.requires_grad)
-    if kernels == "mfma" and not needs_grad and _mfma_takes(h2, w2, h2.shape[0]):
-        lp, ent = lm_head_score_mfma(h2, w2, ids, float(temperature))
+    if not needs_grad and _own_forward_in_use(kernels, keep_logits, h2, w2):
+        temp = None if float(temperature) == 1.0 else torch.full((h2.shape[0],), float(temperature), dtype=torch.float32,
+                                                                  device=h2.device)
+        with torch.no_grad():
+            lp, ent, _ = _own_forward(h2, w2, ids, temp, None, "fused_linear_for_ppo")
         return lp.reshape(lead), ent.reshape(lead)
     lp, ent = _FusedLinearForPPOFunction.apply(h2, w2, ids, float(temperature), int(chunk_size), bool(keep_logits),
                                                kernels)
     return lp.reshape(lead), ent.reshape(lead)
 
 
+def _own_forward(h, w, ids, temp, n_splits, what):
+    """(log-prob, entropy, logsumexp), fp32, of the rows of ``h`` from vrl_lmhead_score. ``temp`` is None or one value per
+    token. The kernels work on blocks of 256 tokens: a shorter input is copied into a zero-padded block first."""
+    T, K = h.shape
+    V = w.shape[0]
+    dev = h.device
+    f32 = dict(dtype=torch.float32, device=dev)
+    if T == 0:
+        return torch.empty(0, **f32), torch.empty(0, **f32), torch.empty(0, **f32)
+    n = max(T, 256)
+    if n != T:
+        hp = torch.zeros((n, K), dtype=h.dtype, device=dev)
+        hp[:T] = h
+        ip = torch.zeros(n, dtype=torch.int64, device=dev)
+        ip[:T] = ids
+        tp = None
+        if temp is not None:
+            tp = torch.ones(n, **f32)
+            tp[:T] = temp
+        h, ids, temp = hp, ip, tp
+    lib = _lib.load()
+    splits = lib.vrl_lmhead_plan(n, V) if n_splits is None else int(n_splits)
+    partials = torch.empty(n * splits * 4, **f32)
+    lp = torch.empty(n, **f32)
+    ent = torch.empty(n, **f32)
+    lse = torch.empty(n, **f32)
+    flag = torch.zeros(1, dtype=torch.int32, device=dev)
+    with torch.cuda.device(dev):
+        st = lib.vrl_lmhead_score(h.data_ptr(), w.data_ptr(), _DTYPE_CODES[h.dtype], n, V, K, h.stride(0), w.stride(0),
+                                  ids.data_ptr(), _ptr(temp), splits, partials.data_ptr(), lp.data_ptr(), ent.data_ptr(),
+                                  lse.data_ptr(), flag.data_ptr(), _lib.stream_ptr(dev))
+    _lib.check("vrl_lmhead_score", st)
+    _errors.report(flag, {_lib.VRL_FLAG_LABEL_OOB: (IndexError, f"{what}: an input id is outside [0, {V})")})
+    return lp[:T], ent[:T], lse[:T]
+
+
 def lm_head_score_mfma(hidden_states: torch.Tensor, vocab_weights: torch.Tensor, input_ids: torch.Tensor,
                        temperature=1.0, n_splits: Optional[int] = None):
     """Forward-only (log_probs, entropy), fp32, from one hand-written matrix-core kernel that never writes logits
     (``vrl_lmhead_score``): the counterpart of the reference's Triton ``efficient_entropy_forward``
-    (verl/utils/kernel/kernels.py:531-756). bf16 or fp16 operands, at least 256 tokens and 256 vocabulary entries,
-    hidden size a multiple of 64. ``temperature`` is a float or one value per token. The logits are kept in fp32
+    (verl/utils/kernel/kernels.py:531-756). bf16 or fp16 operands, at least 256 vocabulary entries, hidden size a
+    multiple of 64 (fewer than 256 tokens are padded to 256 rows for the call). ``temperature`` is a float or one value per token. The logits are kept in fp32
     (a GEMM that writes them rounds them to the operand type first), so results are slightly closer to the
     all-fp32 value than a path that writes them. On MI355X it takes as long as the library GEMM + row kernel (6.5 ms at
-    8192 x 3584 -> 152064) and needs no logits buffer at all; ``fused_linear_for_ppo(kernels="mfma")`` uses it when no
-    gradient is recorded.
+    8192 x 3584 -> 152064) and needs no logits buffer at all; it is ``fused_linear_for_ppo``'s default forward.
     """
     if not hidden_states.is_cuda or not vocab_weights.is_cuda:
         raise RuntimeError("lm_head_score_mfma: tensors must be on the GPU; verl_amd has no CPU implementation")
@@ -277,9 +339,9 @@ def lm_head_score_mfma(hidden_states: torch.Tensor, vocab_weights: torch.Tensor,
     w = vocab_weights.detach().contiguous()
     T, K = h.shape
     V = w.shape[0]
-    if T < 256 or V < 256 or K % 64 != 0:
-        raise ValueError(f"lm_head_score_mfma needs >= 256 tokens, >= 256 vocabulary entries and a hidden size that is "
-                         f"a multiple of 64; got {T}, {V}, {K}")
+    if V < 256 or K % 64 != 0:
+        raise ValueError(f"lm_head_score_mfma needs >= 256 vocabulary entries and a hidden size that is a multiple of "
+                         f"64; got {V}, {K}")
     dev = h.device
     ids = input_ids.reshape(-1).to(device=dev, dtype=torch.int64).contiguous()
     temp = None
@@ -290,19 +352,7 @@ def lm_head_score_mfma(hidden_states: torch.Tensor, vocab_weights: torch.Tensor,
             raise ValueError(f"temperature has {temp.numel()} entries, expected one per token ({T})")
     elif float(temperature) != 1.0:
         temp = torch.full((T,), float(temperature), dtype=torch.float32, device=dev)
-    lib = _lib.load()
-    splits = lib.vrl_lmhead_plan(T, V) if n_splits is None else int(n_splits)
-    f32 = dict(dtype=torch.float32, device=dev)
-    partials = torch.empty(T * splits * 4, **f32)
-    lp = torch.empty(T, **f32)
-    ent = torch.empty(T, **f32)
-    flag = torch.zeros(1, dtype=torch.int32, device=dev)
-    with torch.cuda.device(dev):
-        st = lib.vrl_lmhead_score(h.data_ptr(), w.data_ptr(), _DTYPE_CODES[h.dtype], T, V, K, h.stride(0), w.stride(0),
-                                  ids.data_ptr(), _ptr(temp), splits, partials.data_ptr(), lp.data_ptr(), ent.data_ptr(),
-                                  None, flag.data_ptr(), _lib.stream_ptr(dev))
-    _lib.check("vrl_lmhead_score", st)
-    _errors.report(flag, {_lib.VRL_FLAG_LABEL_OOB: (IndexError, f"lm_head_score_mfma: an input id is outside [0, {V})")})
+    lp, ent, _ = _own_forward(h, w, ids, temp, n_splits, "lm_head_score_mfma")
     return lp.reshape(lead), ent.reshape(lead)
 
 
