@@ -62,11 +62,6 @@ def _mfma_takes_model(hidden: torch.Tensor, weight: torch.Tensor) -> bool:
             and hidden.data_ptr() % 16 == 0 and weight.data_ptr() % 16 == 0)
 
 
-def _mfma_takes(hidden: torch.Tensor, weight: torch.Tensor, n_tokens: int) -> bool:
-    """Shape rules of vrl_lmhead_score / vrl_lmhead_dlogits (include/vrl.h) for a call with ``n_tokens`` rows."""
-    return n_tokens >= 256 and _mfma_takes_model(hidden, weight)
-
-
 def _own_forward_in_use(kernels: str, keep_logits: bool, hidden: torch.Tensor, weight: torch.Tensor) -> bool:
     """Whether the forward is vrl_lmhead_score. Decided by the caller's options and by the model only, never by the number
     of tokens or by whether gradients are recorded: a trainer's old (no-grad) and new (grad) log-probs of the same
@@ -85,6 +80,13 @@ def _score_chunk(lib, logits, labels, temp, lp, h, lse, flag, stream):
                           labels.data_ptr(), _ptr(temp), lp.data_ptr(), h.data_ptr(), None, lse.data_ptr(),
                           flag.data_ptr(), stream)
     _lib.check("vrl_rowscore", st)
+
+
+def _padded(x: torch.Tensor, rows: int) -> torch.Tensor:
+    """``x`` with zero rows appended up to ``rows``."""
+    out = torch.zeros((rows,) + tuple(x.shape[1:]), dtype=x.dtype, device=x.device)
+    out[: x.shape[0]] = x
+    return out
 
 
 def _d_hidden(grad_logits, weight, weight_t, out, own_kernel):
@@ -163,7 +165,22 @@ class _FusedLinearForPPOFunction(torch.autograd.Function):
         d_hidden = torch.empty_like(hidden) if need_dh else None
         d_weight = (torch.empty_like(weight) if kept is not None else torch.zeros_like(weight)) if need_dw else None
         lib = _lib.load()
-        buf = kept if kept is not None else torch.empty((min(chunk, max(T, 1)), V), dtype=hidden.dtype, device=dev)
+        # With this package's own kernels every chunk is at least one block of 256 tokens: a smaller chunk size is raised
+        # to 256, a short tail joins the chunk before it, and a call with fewer than 256 tokens is padded to one block
+        # (zero hidden states and zero incoming gradients give zero rows), so the backward never falls back to logits
+        # that a library GEMM rounded differently from the forward's.
+        own = kept is None and ctx.kernels != "library" and V % 8 == 0 and _mfma_takes_model(hidden, weight)
+        step = max(chunk, 256) if own else chunk
+        starts = list(range(0, T, step))
+        if own and len(starts) > 1 and T - starts[-1] < 256:
+            starts.pop()
+        bounds = [(lo, starts[i + 1] if i + 1 < len(starts) else T) for i, lo in enumerate(starts)]
+        rows = max([hi - lo for lo, hi in bounds] + [1])
+        if own:
+            rows = max(rows, 256)
+        if temp is not None and temp.numel() < rows:
+            temp = torch.full((rows,), ctx.temperature, **f32)
+        buf = kept if kept is not None else torch.empty((rows, V), dtype=hidden.dtype, device=dev)
         dt = _DTYPE_CODES[hidden.dtype]
         # For 16-bit operands the library GEMM is 25-35 % faster when both operands are contiguous along the
         # contraction axis (vocab for `d hidden`, tokens for `d W`); fp32 runs at the fp32 matrix peak either way.
@@ -171,18 +188,27 @@ class _FusedLinearForPPOFunction(torch.autograd.Function):
         weight_t = transpose_2d(weight) if (half and need_dh and T >= _WEIGHT_TRANSPOSE_MIN_TOKENS) else None
         with torch.cuda.device(dev):
             stream = _lib.stream_ptr(dev)
-            for lo in range(0, T, chunk):
-                hi = min(lo + chunk, T)
+            for lo, hi in bounds:
                 n = hi - lo
-                if kept is None and ctx.kernels != "library" and _mfma_takes(hidden[lo:hi], weight, n) and V % 8 == 0:
+                if own:
                     # logits formed again on the matrix cores, their gradient written straight into the buffer
                     logits = buf[:n]
+                    c_h, c_ids, c_lse, c_ent = hidden[lo:hi], input_ids[lo:hi], lse[lo:hi], h[lo:hi]
+                    c_gl = None if gl is None else gl[lo:hi]
+                    c_gh = None if gh is None else gh[lo:hi]
+                    m = n
+                    if n < 256:
+                        m = 256
+                        c_h = _padded(c_h, m)
+                        c_ids, c_lse, c_ent = _padded(c_ids, m), _padded(c_lse, m), _padded(c_ent, m)
+                        c_gl = None if c_gl is None else _padded(c_gl, m)
+                        c_gh = None if c_gh is None else _padded(c_gh, m)
                     st = lib.vrl_lmhead_dlogits(
-                        hidden[lo:hi].data_ptr(), weight.data_ptr(), dt, n, V, D, hidden.stride(0), weight.stride(0),
-                        input_ids[lo:hi].data_ptr(), None if temp is None else temp.data_ptr(), lse[lo:hi].data_ptr(),
-                        h[lo:hi].data_ptr(), None if gl is None else gl[lo:hi].data_ptr(),
-                        None if gh is None else gh[lo:hi].data_ptr(), lib.vrl_lmhead_plan(n, V), logits.data_ptr(),
-                        logits.stride(0), stream)
+                        c_h.data_ptr(), weight.data_ptr(), dt, m, V, D, c_h.stride(0), weight.stride(0),
+                        c_ids.data_ptr(), None if temp is None else temp.data_ptr(), c_lse.data_ptr(),
+                        c_ent.data_ptr(), None if c_gl is None else c_gl.data_ptr(),
+                        None if c_gh is None else c_gh.data_ptr(), lib.vrl_lmhead_plan(m, V), buf.data_ptr(),
+                        buf.stride(0), stream)
                     _lib.check("vrl_lmhead_dlogits", st)
                     if need_dh:
                         _d_hidden(logits, weight, weight_t, d_hidden[lo:hi], True)
