@@ -459,14 +459,14 @@ def bench_lm_head(args, dev):
         "config": {"workload": "lm_head_8192x3584_v152064_bf16", "chunk_tokens": chunk, "keep_logits": keep,
                    "temperature": temperature,
                    "step": "verl_amd.fused_linear_for_ppo forward + torch.autograd.grad for hidden and weight, default "
-                           "kernels (\"auto\": vrl_lmhead_score forward; backward vrl_lmhead_dlogits, vrl_gemm_nt for d hidden, a library "
-                           "GEMM for d W)"},
+                           "kernels (\"auto\": vrl_lmhead_score forward; backward vrl_lmhead_dlogits, vrl_gemm for d hidden and "
+                           "d W, operands read in place; no library GEMM)"},
         "forward_ms": t_f * 1e3,
         "forward_tokens_per_s": T / t_f,
         "roofline": {"bound": "mfma", "achieved": flops_fb / t_fb / 1e12, "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
                      "frac": flops_fb / t_fb / 1e12 / MFMA_BF16_PEAK_TFLOPS, "traffic": None,
                      "kernel": "lmhead_partial_kernel<bf16> + lmhead_finish_kernel, lmhead_dlogits_kernel<bf16>, "
-                               "lm_gemm_nt_kernel<bf16> (d hidden), hipBLASLt bf16 GEMM (d W)",
+                               "lm_gemm_kernel<bf16> (d hidden, d W)",
                      "forward_tflops": flops_f / t_f / 1e12},
         "single_kernel_forward": {"ms": t_m * 1e3, "tflops": flops_f / t_m / 1e12, "frac_of_mfma_peak": flops_f / t_m / 1e12 / MFMA_BF16_PEAK_TFLOPS,
                                   "kernel": "lmhead_partial_kernel<bf16> + lmhead_finish_kernel (vrl_lmhead_score)",
@@ -480,8 +480,10 @@ def bench_lm_head(args, dev):
                                  "kernel": "kernels=\"mfma\": the same kernels as the default today",
                                  "note": "the logits are formed again by the hand-written MFMA kernel and their gradient "
                                          "is written from registers (no GEMM into the buffer, no pass over it); d hidden "
-                                         "comes from the same main loop"},
-        "weight_transpose": {"ms": t_tr * 1e3, "gbps": 2.0 * V * D * 2 / t_tr / 1e9, "kernel": "transpose_kernel<2>"},
+                                         "and d W come from the same main loop, which reads W, the hidden states and the "
+                                         "gradient buffer as they lie (transposing LDS reads)"},
+        "weight_transpose": {"ms": t_tr * 1e3, "gbps": 2.0 * V * D * 2 / t_tr / 1e9, "kernel": "transpose_kernel<2>",
+                             "note": "the copy the all-library backward makes once per call; the default path needs none"},
         "parity_guard": {"rows": 256, "max_abs_err_logprob": e1, "max_abs_err_entropy": e2},
     }), flush=True)
 

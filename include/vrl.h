@@ -286,22 +286,28 @@ int vrl_lmhead_dlogits(const void* hidden, const void* weight, int dtype, int64_
                        const float* g_entropy, int n_splits, void* dlogits, int64_t d_stride, void* stream);
 
 /*
- * vrl_gemm_nt — out[y][x] (+)= sum_k x[x][k] * y[y][k] on the matrix cores, with the main loop of the LM-head kernels:
- * the two products that follow vrl_lmhead_dlogits in the backward,
- *   d hidden (tokens, hidden) = G . W      : x = W^T (hidden, vocab), y = G (tokens, vocab)
- *   d W      (vocab, hidden) += G^T . H    : x = H^T (hidden, tokens), y = G^T (vocab, tokens), accumulate = 1
- * (the transposed copies come from vrl_transpose). x is (NX, K), y is (NY, K), both contiguous along k with row strides
- * x_stride / y_stride (elements, multiples of 8, 16-byte aligned bases); out is (NY, NX) in the operands' type (VRL_BF16 or
- * VRL_F16) with row stride out_stride (a multiple of 4, 8-byte aligned base); fp32 accumulation, one rounding. NX, NY >=
- * 256, NX a multiple of 4, K a multiple of 64. accumulate != 0 adds the product to what out holds.
+ * vrl_gemm — out[y][x] (+)= sum_k X[x][k] * Y[y][k] on the matrix cores, with the main loop of the LM-head kernels: the
+ * two products that follow vrl_lmhead_dlogits in the backward, read from the tensors as they lie,
+ *   d hidden (tokens, hidden) = G . W      : x = W (vocab, hidden), contraction-major; y = G (tokens, vocab), row-major
+ *   d W      (vocab, hidden) += G^T . H    : x = H (tokens, hidden) and y = G (tokens, vocab), both contraction-major,
+ *                                            accumulate = 1 from the second chunk of tokens on.
+ * A row-major operand is (N, K), contiguous along the contraction, with row stride >= K; a contraction-major one
+ * (x_contraction_major / y_contraction_major != 0) is (K, N), contiguous along its N rows, with row stride >= N and N a
+ * multiple of 8. Strides are in elements and multiples of 8, bases 16-byte aligned. out is (NY, NX) in the operands' type
+ * (VRL_BF16 or VRL_F16) with row stride out_stride (a multiple of 4, 8-byte aligned base); fp32 accumulation, one
+ * rounding; the result does not depend on the operands' layouts. NX, NY >= 256, NX a multiple of 4, K a multiple of 64
+ * and >= 128. accumulate != 0 adds the product to what out holds.
  * k_parts (1..16, normally what vrl_gemm_nt_plan returns) cuts the contraction into ranges that are summed in a fixed
  * order through `workspace` (k_parts * NX * NY floats, 16-byte aligned; may be NULL when k_parts == 1): that is how a
  * product with few output tiles still fills the CUs. vrl_gemm_nt_plan returns the number of ranges it would use for a
- * shape (or a negative status) and stores the workspace it needs.
+ * shape (or a negative status) and stores the workspace it needs. vrl_gemm_nt is vrl_gemm for two row-major operands.
  *
  * Replaces the two torch.matmul calls of the reference's backward (verl/utils/kernel/kernels.py:1710-1720).
  */
 int vrl_gemm_nt_plan(int dtype, int64_t NX, int64_t NY, int64_t K, int64_t* workspace_floats);
+int vrl_gemm(const void* x, const void* y, int dtype, int64_t NX, int64_t NY, int64_t K, int64_t x_stride,
+             int64_t y_stride, int x_contraction_major, int y_contraction_major, void* out, int64_t out_stride,
+             int accumulate, int k_parts, float* workspace, void* stream);
 int vrl_gemm_nt(const void* x, const void* y, int dtype, int64_t NX, int64_t NY, int64_t K, int64_t x_stride,
                 int64_t y_stride, void* out, int64_t out_stride, int accumulate, int k_parts, float* workspace,
                 void* stream);

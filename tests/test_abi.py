@@ -258,6 +258,28 @@ def test_gemm_nt_argument_errors(lib):
     assert lib.vrl_gemm_nt_plan(_lib.VRL_BF16, 3584, 152064, 4096, ctypes.addressof(need)) == 1 and need.value == 0
 
 
+def test_gemm_layout_argument_errors(lib):
+    f = lib.vrl_gemm
+    ok = dict(x=P, y=P, dt=_lib.VRL_BF16, NX=512, NY=256, K=256, xs=512, ys=256, xt=1, yt=0, out=P, os=512, acc=0, parts=1,
+              ws=None)
+
+    def call(**kw):
+        a = {**ok, **kw}
+        return f(a["x"], a["y"], a["dt"], a["NX"], a["NY"], a["K"], a["xs"], a["ys"], a["xt"], a["yt"], a["out"], a["os"],
+                 a["acc"], a["parts"], a["ws"], None)
+
+    assert call(dt=_lib.VRL_F32) == _lib.VRL_ERR_DTYPE
+    assert call(xs=256) == _lib.VRL_ERR_SHAPE                       # contraction-major x: stride counts its rows (512)
+    assert call(NX=516, xs=520, os=516) == _lib.VRL_ERR_SHAPE      # ... which come in groups of 8
+    assert call(yt=1, NY=260, ys=264) == _lib.VRL_ERR_SHAPE
+    assert call(yt=1, NY=512, ys=256) == _lib.VRL_ERR_SHAPE
+    assert call(xt=0, xs=128) == _lib.VRL_ERR_SHAPE                # row-major x: stride counts the contraction (256)
+    assert call(K=96) == _lib.VRL_ERR_SHAPE
+    assert call(parts=0) == _lib.VRL_ERR_ARG
+    assert call(y=None) == _lib.VRL_ERR_NULL
+    assert call(x=P + 8) == _lib.VRL_ERR_ALIGN
+
+
 def test_mfma_probe_argument_errors(lib):
     f = lib.vrl_mfma_probe
     assert f(-1, 10, 32, 1, P, None, None, None) == _lib.VRL_ERR_SHAPE

@@ -130,9 +130,10 @@ def test_dlogits_matches_fp64_autograd(dev, dtype, T, V, K, splits):
 
 
 @pytest.mark.parametrize("kernels", ["auto", "mfma"])
-def test_d_hidden_comes_from_the_matrix_core_product(dev, kernels):
-    """From 2048 tokens on the backward holds a transposed copy of the weight and, unless told "library", forms d hidden
-    with vrl_gemm_nt: same tolerances against torch autograd as the other paths, and the launch is counted."""
+def test_backward_products_come_from_the_matrix_core_kernel(dev, kernels):
+    """Unless told "library", the backward forms d hidden and d W with vrl_gemm, reading the weight, the hidden states and
+    the gradient buffer in place: same tolerances against torch autograd as the other paths, and the launches are
+    counted (two per chunk)."""
     from verl_amd import gemm
 
     g = torch.Generator(device=dev).manual_seed(78)
@@ -146,17 +147,17 @@ def test_d_hidden_comes_from_the_matrix_core_product(dev, kernels):
     ref_ent = torch.logsumexp(logits, -1) - (torch.softmax(logits, -1) * logits).sum(-1)
     ref_lp = -torch.nn.functional.cross_entropy(logits, labels, reduction="none")
     d_ref_h, d_ref_w = torch.autograd.grad((ref_ent, ref_lp), (hidden, weight), (g_ent, g_lp))
-    for chunk, keep in ((1024, False), (4096, False), (4096, True)):
-        before = gemm.counters["gemm_nt"]
+    for chunk, keep, launches in ((1024, False, 6), (4096, False, 2), (4096, True, 2)):
+        before = gemm.counters["gemm"]
         lp, ent = fused_linear_for_ppo(hidden, weight, labels, 1.5, chunk_size=chunk, keep_logits=keep, kernels=kernels)
         d_h, d_w = torch.autograd.grad((ent, lp), (hidden, weight), (g_ent, g_lp))
-        assert gemm.counters["gemm_nt"] > before
+        assert gemm.counters["gemm"] == before + launches
         torch.testing.assert_close(d_ref_h.float(), d_h.float(), atol=1e-2, rtol=1e-2)
         torch.testing.assert_close(d_ref_w.float(), d_w.float(), atol=1e-2, rtol=1e-2)
-    before = gemm.counters["gemm_nt"]
+    before = gemm.counters["gemm"]
     lp, ent = fused_linear_for_ppo(hidden, weight, labels, 1.5, kernels="library")
     torch.autograd.grad((ent, lp), (hidden, weight), (g_ent, g_lp))
-    assert gemm.counters["gemm_nt"] == before
+    assert gemm.counters["gemm"] == before
 
 
 def test_fused_linear_with_the_matrix_core_kernels(dev):

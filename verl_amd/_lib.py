@@ -57,6 +57,7 @@ SIGNATURES = {
     "vrl_lmhead_dlogits": (_INT, [_P, _P, _INT, _I64, _I64, _I64, _I64, _I64, _P, _P, _P, _P, _P, _P, _INT, _P, _I64, _P]),
     "vrl_gemm_nt_plan": (_INT, [_INT, _I64, _I64, _I64, _P]),
     "vrl_gemm_nt": (_INT, [_P, _P, _INT, _I64, _I64, _I64, _I64, _I64, _P, _I64, _INT, _INT, _P, _P]),
+    "vrl_gemm": (_INT, [_P, _P, _INT, _I64, _I64, _I64, _I64, _I64, _INT, _INT, _P, _I64, _INT, _INT, _P, _P]),
     "vrl_lmhead_plan": (_INT, [_I64, _I64]),
     "vrl_transpose": (_INT, [_P, _INT, _I64, _I64, _I64, _P, _I64, _P]),
     "vrl_rollout_corr": (

@@ -18,7 +18,7 @@
 // recomputed on the matrix cores and turned, in registers, into the gradient with respect to the logits
 // (the row-backward arithmetic of backward_kernels.h), which is stored in the operands' type.
 //
-// lm_gemm_nt_kernel: out (+)= Y . X^T on the same walk, for the two products that follow (d hidden, d W).
+// lm_gemm_kernel: out (+)= Y . X^T on the same walk, for the two products that follow (d hidden, d W).
 //
 // lmhead_finish_kernel: one wavefront per token forms the label's logit as a dot product in fp32, merges the
 // token's partials over the splits and writes log-prob, entropy and logsumexp (same finish as the row kernel).
@@ -28,6 +28,8 @@
 
 #include <hip/hip_runtime.h>
 #include <stdint.h>
+
+#include <type_traits>
 
 #include "backward_kernels.h"
 #include "rowscore_kernels.h"
@@ -133,7 +135,14 @@ __device__ __forceinline__ LmWork lm_work(int64_t V, int64_t T, int n_splits, in
 // reads in front of the barrier, where all eight wavefronts then wait for them together).
 // EPILOGUE_STORES: on_tile writes to global memory. Stores count in vmcnt like loads but complete in their own order,
 // so the first barrier after on_tile waits for everything.
-template <int DT, bool EPILOGUE_STORES, class OnTile>
+//
+// W_CM / H_CM: that operand is stored contraction-major, M[k][row] with `stride` elements between consecutive k (the
+// layout of the other factor of a product whose contraction runs over the operands' rows, e.g. W itself in G . W).
+// A tile is then 64 rows of k x 512 bytes; one wave instruction still moves 8 memory rows x 128 bytes (8 k x 64 rows).
+// In LDS the tile is [k>>3][16-row block][k&7 (^4 for odd k>>3)][16 rows]: a fragment is two transposing reads
+// (ds_read_b64_tr_b16: 16 lanes read 4 k x 16 rows and each receives the 4 k of its row), the 8 k-rows a half
+// wavefront reads fall on distinct banks, and the row block enters the address as a plain offset of 256 bytes.
+template <int DT, bool EPILOGUE_STORES, bool W_CM = false, bool H_CM = false, class OnTile>
 __device__ __forceinline__ void lm_walk_tiles(const uint16_t* __restrict__ W, const uint16_t* __restrict__ H, int64_t V,
                                               int64_t K, int64_t w_stride, int64_t h_stride, const LmWork& work,
                                               char* lds, OnTile&& on_tile) {
@@ -152,15 +161,31 @@ __device__ __forceinline__ void lm_walk_tiles(const uint16_t* __restrict__ W, co
   // 8 rows alternate in the swizzle's row bits, hence two lane offsets.
   const int lr = lane >> 3;
   const int lc_e = (lane & 7) ^ (lr >> 1), lc_o = (lane & 7) ^ (4 + (lr >> 1));
-  const uint32_t w_lane_e = (uint32_t)((lr * w_stride + lc_e * 8) * 2), w_lane_o = (uint32_t)((lr * w_stride + lc_o * 8) * 2);
-  const uint32_t h_lane_e = (uint32_t)((lr * h_stride + lc_e * 8) * 2), h_lane_o = (uint32_t)((lr * h_stride + lc_o * 8) * 2);
-  const uint64_t w_blk = (uint64_t)(8 * w_stride * 2), h_blk = (uint64_t)(8 * h_stride * 2);   // 8 rows in bytes
+  // contraction-major: lane l lands in (block l>>4 of the instruction's four, k&7 slot (l&15)>>1, 16-byte half l&1) and
+  // fetches memory row (slot ^ 4*(wave&1)) of the wavefront's eight, bytes 32*(l>>4) + 16*(l&1) of the 128
+  const int cm_row = ((lane & 15) >> 1) ^ ((wave & 1) << 2);
+  const int cm_byte = (lane >> 4) * 32 + (lane & 1) * 16;
+  const uint32_t w_lane_e = W_CM ? (uint32_t)(cm_row * w_stride * 2 + cm_byte) : (uint32_t)((lr * w_stride + lc_e * 8) * 2);
+  const uint32_t w_lane_o = W_CM ? w_lane_e : (uint32_t)((lr * w_stride + lc_o * 8) * 2);
+  const uint32_t h_lane_e = H_CM ? (uint32_t)(cm_row * h_stride * 2 + cm_byte) : (uint32_t)((lr * h_stride + lc_e * 8) * 2);
+  const uint32_t h_lane_o = H_CM ? h_lane_e : (uint32_t)((lr * h_stride + lc_o * 8) * 2);
+  // bytes from one of a wavefront's four instructions to the next (8 rows / 64 rows of the tile further on), from one
+  // step to the next (64 contraction elements), and from tile row 0 to the wavefront's first memory row
+  const uint64_t w_blk = W_CM ? (uint64_t)128 : (uint64_t)(8 * w_stride * 2);
+  const uint64_t h_blk = H_CM ? (uint64_t)128 : (uint64_t)(8 * h_stride * 2);
+  const uint64_t w_adv = W_CM ? (uint64_t)(kLmK * w_stride * 2) : (uint64_t)kLmRowBytes;
+  const uint64_t h_adv = H_CM ? (uint64_t)(kLmK * h_stride * 2) : (uint64_t)kLmRowBytes;
+  const uint64_t w_row = W_CM ? (uint64_t)2 : (uint64_t)(w_stride * 2);   // bytes per tile row
+  const uint64_t h_row = H_CM ? (uint64_t)2 : (uint64_t)(h_stride * 2);
+  const uint64_t w_first = W_CM ? (uint64_t)(wave * 8 * w_stride * 2) : (uint64_t)wave * 4 * w_blk;
+  const uint64_t h_first = H_CM ? (uint64_t)(wave * 8 * h_stride * 2) : (uint64_t)wave * 4 * h_blk;
 
   // Two load cursors, one per operand: uniform byte pointers to this wavefront's first row (it brings rows
-  // [32*wave, 32*wave + 32) of a tile with four instructions) of the W / H tile to request next, and the ring slot it
-  // goes to. A step advances a pointer by 128 bytes; at the end of a vocabulary tile W jumps to the next tile's rows
-  // and H returns to k = 0. Past the last step the pointers stay put: the last tiles are requested again into slots
-  // nobody reads any more (in bounds, harmless), so the main loop needs no "is there more" branch around its loads.
+  // [32*wave, 32*wave + 32) of a tile, or contraction rows [8*wave, 8*wave + 8) of a contraction-major one, with four
+  // instructions) of the W / H tile to request next, and the ring slot it goes to. A step advances a pointer by 64
+  // contraction elements; at the end of a vocabulary tile W jumps to the next tile's rows and H returns to k = 0. Past
+  // the last step the pointers stay put: the last tiles are requested again into slots nobody reads any more (in
+  // bounds, harmless), so the main loop needs no "is there more" branch around its loads.
   const int64_t total_steps = (work.vt_end > work.vt_begin ? (work.vt_end - work.vt_begin) : 0) * ksteps;
   auto uniform64 = [](uint64_t v) {
     const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)v);
@@ -168,8 +193,8 @@ __device__ __forceinline__ void lm_walk_tiles(const uint16_t* __restrict__ W, co
     return ((uint64_t)hi << 32) | lo;
   };
   auto vrow_of = [&](int64_t vt) { return (vt + 1) * kLmVocab <= V ? vt * kLmVocab : V - kLmVocab; };
-  uint64_t wp = uniform64(reinterpret_cast<uint64_t>(W) + (uint64_t)(vrow_of(work.vt_begin) * w_stride * 2) + wave * 4 * w_blk);
-  uint64_t hp = uniform64(reinterpret_cast<uint64_t>(H) + (uint64_t)(work.tok0_ld * h_stride * 2) + wave * 4 * h_blk);
+  uint64_t wp = uniform64(reinterpret_cast<uint64_t>(W) + (uint64_t)vrow_of(work.vt_begin) * w_row + w_first);
+  uint64_t hp = uniform64(reinterpret_cast<uint64_t>(H) + (uint64_t)work.tok0_ld * h_row + h_first);
   int64_t w_step = 0, w_vt = work.vt_begin, h_step = 0;
   int w_ks = 0, h_ks = 0;
   int w_slot = 0, h_slot = 1;
@@ -192,8 +217,8 @@ __device__ __forceinline__ void lm_walk_tiles(const uint16_t* __restrict__ W, co
     const bool more = w_step + 1 < total_steps;
     const bool tile_end = w_ks + 1 == ksteps;
     const int64_t dv = vrow_of(w_vt + 1) - vrow_of(w_vt);
-    const uint64_t jump = (uint64_t)(dv * w_stride * 2) - (uint64_t)(ksteps - 1) * kLmRowBytes;
-    wp += more ? (tile_end ? jump : (uint64_t)kLmRowBytes) : (uint64_t)0;
+    const uint64_t jump = (uint64_t)dv * w_row - (uint64_t)(ksteps - 1) * w_adv;
+    wp += more ? (tile_end ? jump : w_adv) : (uint64_t)0;
     w_vt += (more && tile_end) ? 1 : 0;
     w_ks = more ? (tile_end ? 0 : w_ks + 1) : w_ks;
     ++w_step;
@@ -202,18 +227,50 @@ __device__ __forceinline__ void lm_walk_tiles(const uint16_t* __restrict__ W, co
     h_slot = next_slot(h_slot);
     const bool more = h_step + 1 < total_steps;
     const bool tile_end = h_ks + 1 == ksteps;
-    const uint64_t back = (uint64_t)0 - (uint64_t)(ksteps - 1) * kLmRowBytes;
-    hp += more ? (tile_end ? back : (uint64_t)kLmRowBytes) : (uint64_t)0;
+    const uint64_t back = (uint64_t)0 - (uint64_t)(ksteps - 1) * h_adv;
+    hp += more ? (tile_end ? back : h_adv) : (uint64_t)0;
     h_ks = more ? (tile_end ? 0 : h_ks + 1) : h_ks;
     ++h_step;
   };
 
-  // row (within its 16-row block) = lane&15, logical chunk = 4*half + (lane>>4), half in 0..1
-  int phys[2];
+  // Fragment addresses. Row-major tile: row (within its 16-row block) = lane&15, logical chunk = 4*half + (lane>>4).
+  // Contraction-major tile: the lane's group g = lane>>4 owns k = 32*half + 8*g .. +7 and fetches them with two
+  // transposing reads (k .. k+3 and k+4 .. k+7); in each, lane s = lane&15 of the group supplies the address of
+  // k-row s>>2, rows 4*(s&3) .. +3 of the block.
+  int phys[2], cm_q[2];
 #pragma unroll
-  for (int hf = 0; hf < 2; ++hf) phys[hf] = (((4 * hf + (lane >> 4)) ^ ((lane >> 1) & 7)) * 16);
-  const int fragoff_w = (wv * 64 + (lane & 15)) * kLmRowBytes;    // within a W slot
-  const int fragoff_h = (wt * 128 + (lane & 15)) * kLmRowBytes;   // within an H slot
+  for (int hf = 0; hf < 2; ++hf) {
+    phys[hf] = (((4 * hf + (lane >> 4)) ^ ((lane >> 1) & 7)) * 16);
+    cm_q[hf] = (lane >> 4) * 4096 + (4 * (hf ^ ((lane >> 4) & 1)) + ((lane & 15) >> 2)) * 32 + (lane & 3) * 8;
+  }
+  constexpr int kWBlock = W_CM ? 256 : 16 * kLmRowBytes;   // from one 16-row block of a tile to the next
+  constexpr int kHBlock = H_CM ? 256 : 16 * kLmRowBytes;
+  constexpr int kCmHalf = 4 * 4096;                         // second half of a contraction-major tile
+  const int fragoff_w = W_CM ? wv * 4 * 256 : (wv * 64 + (lane & 15)) * kLmRowBytes;    // within a W slot
+  const int fragoff_h = H_CM ? wt * 8 * 256 : (wt * 128 + (lane & 15)) * kLmRowBytes;   // within an H slot
+  typedef short s16x4 __attribute__((ext_vector_type(4)));
+  typedef short s16x8 __attribute__((ext_vector_type(8)));
+  auto read_cm = [](const char* p0, const char* p1) {
+    const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((VRL_LDS_AS s16x4*)p0);
+    const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((VRL_LDS_AS s16x4*)p1);
+    const s16x8 v = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+    return __builtin_bit_cast(FragT, v);
+  };
+  // p0 (and p1 for a contraction-major tile) point at block 0 of the wanted half of a slot
+  auto read_w = [&](const char* p0, const char* p1, int i) {
+    if constexpr (W_CM) return read_cm(p0 + i * kWBlock, p1 + i * kWBlock);
+    else return *reinterpret_cast<const FragT*>(p0 + i * kWBlock);
+  };
+  auto read_h = [&](const char* p0, const char* p1, int j) {
+    if constexpr (H_CM) return read_cm(p0 + j * kHBlock, p1 + j * kHBlock);
+    else return *reinterpret_cast<const FragT*>(p0 + j * kHBlock);
+  };
+  auto w_ptr = [&](int slot, int hf, int q) {
+    return lds + slot * kLmTileBytes + fragoff_w + (W_CM ? cm_q[q] + hf * kCmHalf : phys[hf]);
+  };
+  auto h_ptr = [&](int slot, int hf, int q) {
+    return lds + slot * kLmTileBytes + fragoff_h + (H_CM ? cm_q[q] + hf * kCmHalf : phys[hf]);
+  };
 
   FragT a[4], b[8];
   if (total_steps > 0) {
@@ -229,9 +286,9 @@ __device__ __forceinline__ void lm_walk_tiles(const uint16_t* __restrict__ W, co
     asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
     __builtin_amdgcn_s_barrier();
 #pragma unroll
-    for (int i = 0; i < 4; ++i) a[i] = *reinterpret_cast<const FragT*>(lds + fragoff_w + i * 16 * kLmRowBytes + phys[0]);
+    for (int i = 0; i < 4; ++i) a[i] = read_w(w_ptr(0, 0, 0), w_ptr(0, 0, 1), i);
 #pragma unroll
-    for (int j = 0; j < 8; ++j) b[j] = *reinterpret_cast<const FragT*>(lds + kLmTileBytes + fragoff_h + j * 16 * kLmRowBytes + phys[0]);
+    for (int j = 0; j < 8; ++j) b[j] = read_h(h_ptr(1, 0, 0), h_ptr(1, 0, 1), j);
   }
 
   int cw = 0, ch = 1;   // ring slots of the step being computed
@@ -264,14 +321,16 @@ __device__ __forceinline__ void lm_walk_tiles(const uint16_t* __restrict__ W, co
           __builtin_amdgcn_s_barrier();
           after_epilogue = false;
         }
-        const char* rw = lds + ((hf == 1) ? nw : cw) * kLmTileBytes + fragoff_w + phys[hf ^ 1];
-        const char* rh = lds + ((hf == 1) ? nh : ch) * kLmTileBytes + fragoff_h + phys[hf ^ 1];
+        const char* rw0 = w_ptr((hf == 1) ? nw : cw, hf ^ 1, 0);
+        const char* rw1 = W_CM ? w_ptr((hf == 1) ? nw : cw, hf ^ 1, 1) : rw0;
+        const char* rh0 = h_ptr((hf == 1) ? nh : ch, hf ^ 1, 0);
+        const char* rh1 = H_CM ? h_ptr((hf == 1) ? nh : ch, hf ^ 1, 1) : rh0;
 #pragma unroll
         for (int mm = 0; mm < 32; ++mm) {
           const int j = mm >> 2, i = mm & 3;
           acc[i][j] = LmFrag<DT>::mfma16(a[i], b[j], acc[i][j]);
-          if (i == 3) b[j] = *reinterpret_cast<const FragT*>(rh + j * 16 * kLmRowBytes);
-          if (j == 7) a[i] = *reinterpret_cast<const FragT*>(rw + i * 16 * kLmRowBytes);
+          if (i == 3) b[j] = read_h(rh0, rh1, j);
+          if (j == 7) a[i] = read_w(rw0, rw1, i);
           if ((mm & 7) == 1) {
             if (hf == 0) load_w(mm >> 3); else load_h(mm >> 3);
           }
@@ -279,8 +338,8 @@ __device__ __forceinline__ void lm_walk_tiles(const uint16_t* __restrict__ W, co
 #pragma unroll
         for (int mm = 0; mm < 32; ++mm) {
           __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                                // one matrix instruction
-          if ((mm & 3) == 3) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);             // an H fragment
-          if ((mm >> 2) == 7) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);            // a W fragment
+          if ((mm & 3) == 3) __builtin_amdgcn_sched_group_barrier(0x100, H_CM ? 2 : 1, 0);  // an H fragment
+          if ((mm >> 2) == 7) __builtin_amdgcn_sched_group_barrier(0x100, W_CM ? 2 : 1, 0); // a W fragment
           if ((mm & 7) == 1) __builtin_amdgcn_sched_group_barrier(0x010, 1, 0);             // one load
         }
         __builtin_amdgcn_sched_barrier(0);
@@ -512,9 +571,11 @@ __global__ __launch_bounds__(kLmWaves * 64, 1) void lmhead_dlogits_kernel(
 
 
 // ---- the two products of the backward on the same walk -----------------------------------------------------------
-// out[y][x] (+)= sum_k X[x][k] * Y[y][k] for X (NX, K) and Y (NY, K), both contiguous along k: d hidden = G . W with
-// X = W^T (hidden, vocab) and Y = G (tokens, vocab); d W = G^T . H with X = H^T (hidden, tokens) and Y = G^T (vocab,
-// tokens). X plays the walk's vocabulary side (a lane's accumulator quad is 4 consecutive x of one y, i.e. one 8-byte
+// out[y][x] (+)= sum_k X[x][k] * Y[y][k]. An operand is either row-major, (rows, K) contiguous along k, or
+// contraction-major (X_CM / Y_CM), (K, rows) contiguous along its rows, so neither product needs a transposed copy:
+//   d hidden = G . W   : X = W (vocab, hidden) contraction-major, Y = G (tokens, vocab) row-major
+//   d W      = G^T . H : X = H (tokens, hidden) and Y = G (tokens, vocab), both contraction-major.
+// X plays the walk's vocabulary side (a lane's accumulator quad is 4 consecutive x of one y, i.e. one 8-byte
 // store of out[y][x..x+3]), Y its token side.
 //
 // A work item is (y block of 256 rows, `tiles_per_item` x tiles, one of `k_parts` ranges of the contraction). Items
@@ -543,8 +604,8 @@ struct LmGemmShape {
   int py, px;              // patch of (y blocks, x splits) per XCD
 };
 
-template <int DT, int MODE>
-__global__ __launch_bounds__(kLmWaves * 64, 1) void lm_gemm_nt_kernel(
+template <int DT, int MODE, bool X_CM, bool Y_CM>
+__global__ __launch_bounds__(kLmWaves * 64, 1) void lm_gemm_kernel(
     const uint16_t* __restrict__ X, const uint16_t* __restrict__ Y, LmGemmShape g, int64_t x_stride, int64_t y_stride,
     uint16_t* __restrict__ out, int64_t out_stride, float* __restrict__ partials) {
   extern __shared__ __attribute__((aligned(1024))) char lds[];  // the operand ring
@@ -583,8 +644,10 @@ __global__ __launch_bounds__(kLmWaves * 64, 1) void lm_gemm_nt_kernel(
   int64_t nsteps = g.k_steps - step0;
   if (nsteps > g.steps_per_part) nsteps = g.steps_per_part;
 
-  lm_walk_tiles<DT, true>(X + step0 * kLmK, Y + step0 * kLmK, g.NX, nsteps * kLmK, x_stride, y_stride, work, lds,
-                              [&](int64_t vt, lm_f32x4 (&acc)[4][8]) {
+  const uint16_t* x0 = X + step0 * kLmK * (X_CM ? x_stride : 1);
+  const uint16_t* y0p = Y + step0 * kLmK * (Y_CM ? y_stride : 1);
+  lm_walk_tiles<DT, true, X_CM, Y_CM>(x0, y0p, g.NX, nsteps * kLmK, x_stride, y_stride, work, lds,
+                                      [&](int64_t vt, lm_f32x4 (&acc)[4][8]) {
     // acc[i][j][0..3]: columns x0 .. x0+3 of out, x0 = tile_row0 + wv*64 + i*16 + 4*(lane>>4), of row
     // y = tok0_ld + wt*128 + j*16 + (lane&15)
     const bool edge = (vt + 1) * kLmVocab > g.NX;
@@ -598,40 +661,53 @@ __global__ __launch_bounds__(kLmWaves * 64, 1) void lm_gemm_nt_kernel(
     const int64_t y0 = work.tok0_ld + wt * 128 + y_lane;
     uint16_t* out_row0 = out + y0 * out_stride;
     float* part_row0 = partials + ((int64_t)kp * g.NY + y0) * g.NX;
+    // Interior tiles (all 256 x 256 results are this item's own) store without conditions: straight-line code, whose
+    // loads (MODE 1) and stores the compiler can keep in flight together. Edge tiles, which repeat rows or columns of
+    // the tile before, check each quad.
+    auto write_tile = [&](auto guard_tag) {
+      constexpr bool GUARD = decltype(guard_tag)::value;
 #pragma unroll
-    for (int j = 0; j < 8; ++j) {
-      const bool y_mine = y0 + j * 16 >= work.tok0;
-      uint16_t* out_row = out_row0 + (int64_t)(j * 16) * out_stride;
-      float* part_row = part_row0 + (int64_t)(j * 16) * g.NX;
+      for (int j = 0; j < 8; ++j) {
+        const bool y_mine = !GUARD || y0 + j * 16 >= work.tok0;
+        uint16_t* out_row = out_row0 + (int64_t)(j * 16) * out_stride;
+        float* part_row = part_row0 + (int64_t)(j * 16) * g.NX;
+        // MODE 1: what out holds at this column's four quads, requested together (a row or column that belongs to the
+        // tile before is a valid address all the same; only its store is skipped)
+        uint2 old[4];
+        if constexpr (MODE == 1) {
 #pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        const int x = xrow0 + i * 16;   // a multiple of 4
-        if (y_mine && x >= xfirst) {
+          for (int i = 0; i < 4; ++i) old[i] = *reinterpret_cast<const uint2*>(out_row + xrow0 + i * 16);
+        }
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const int x = xrow0 + i * 16;   // a multiple of 4
           float v[4];
 #pragma unroll
           for (int e = 0; e < 4; ++e) v[e] = acc[i][j][e];
-          if constexpr (MODE == 2) {
-            f32x4 pk = {v[0], v[1], v[2], v[3]};
-            *reinterpret_cast<f32x4*>(part_row + x) = pk;
-          } else {
-            uint2* dst = reinterpret_cast<uint2*>(out_row + x);
-            if constexpr (MODE == 1) {
-              const uint2 old = *dst;
-              float o[4];
-              lm_unpack2<DT>(old.x, o);
-              lm_unpack2<DT>(old.y, o + 2);
+          if constexpr (MODE == 1) {
+            float o[4];
+            lm_unpack2<DT>(old[i].x, o);
+            lm_unpack2<DT>(old[i].y, o + 2);
 #pragma unroll
-              for (int e = 0; e < 4; ++e) v[e] += o[e];
+            for (int e = 0; e < 4; ++e) v[e] += o[e];
+          }
+          if (!GUARD || (y_mine && x >= xfirst)) {
+            if constexpr (MODE == 2) {
+              f32x4 pk = {v[0], v[1], v[2], v[3]};
+              *reinterpret_cast<f32x4*>(part_row + x) = pk;
+            } else {
+              uint2 pk;
+              pk.x = O::pack2(v[0], v[1]);
+              pk.y = O::pack2(v[2], v[3]);
+              *reinterpret_cast<uint2*>(out_row + x) = pk;
             }
-            uint2 pk;
-            pk.x = O::pack2(v[0], v[1]);
-            pk.y = O::pack2(v[2], v[3]);
-            *dst = pk;
           }
         }
+        __builtin_amdgcn_sched_barrier(0);
       }
-      __builtin_amdgcn_sched_barrier(0);
-    }
+    };
+    if (edge || work.tok0_ld != work.tok0) write_tile(std::true_type{});
+    else write_tile(std::false_type{});
   });
 }
 

@@ -336,7 +336,7 @@ int check_lmhead_shape(int dtype, int64_t n_tokens, int64_t vocab, int64_t hidde
 }
 
 
-// How vrl_gemm_nt cuts its work: enough (y block, x split, contraction range) items to fill the part's CUs in whole
+// How vrl_gemm cuts its work: enough (y block, x split, contraction range) items to fill the part's CUs in whole
 // rounds. One workgroup per CU runs at a time (the kernels take all of its LDS).
 struct GemmPlan {
   vrl::LmGemmShape shape;
@@ -395,9 +395,9 @@ GemmPlan gemm_plan(int64_t NX, int64_t NY, int64_t K, int forced_parts) {
   return p;
 }
 
-template <int DT>
-int launch_gemm_nt(const void* x, const void* y, const GemmPlan& plan, int64_t x_stride, int64_t y_stride, void* out,
-                   int64_t out_stride, int accumulate, float* workspace, hipStream_t s) {
+template <int DT, bool X_CM, bool Y_CM>
+int launch_gemm(const void* x, const void* y, const GemmPlan& plan, int64_t x_stride, int64_t y_stride, void* out,
+                int64_t out_stride, int accumulate, float* workspace, hipStream_t s) {
   const vrl::LmGemmShape& g = plan.shape;
   const int psize = g.py * g.px;
   const int64_t patches = plan.items / psize;
@@ -410,10 +410,11 @@ int launch_gemm_nt(const void* x, const void* y, const GemmPlan& plan, int64_t x
 #define VRL_GEMM_LAUNCH(MODE)                                                                                       \
   {                                                                                                                 \
     static std::atomic<bool> raised[kMaxDevices];                                                                   \
-    const int rs = raise_lds_limit(reinterpret_cast<const void*>(vrl::lm_gemm_nt_kernel<DT, MODE>), raised);        \
+    const int rs =                                                                                                  \
+        raise_lds_limit(reinterpret_cast<const void*>(vrl::lm_gemm_kernel<DT, MODE, X_CM, Y_CM>), raised);          \
     if (rs != VRL_OK) return rs;                                                                                    \
-    vrl::lm_gemm_nt_kernel<DT, MODE><<<gd, bd, vrl::kLmLdsBytes, s>>>(X, Y, g, x_stride, y_stride, O, out_stride,   \
-                                                                        workspace);                                 \
+    vrl::lm_gemm_kernel<DT, MODE, X_CM, Y_CM><<<gd, bd, vrl::kLmLdsBytes, s>>>(X, Y, g, x_stride, y_stride, O,      \
+                                                                               out_stride, workspace);              \
   }
   if (g.k_parts > 1) {
     VRL_GEMM_LAUNCH(2)
@@ -432,10 +433,27 @@ int launch_gemm_nt(const void* x, const void* y, const GemmPlan& plan, int64_t x
   return launch_status();
 }
 
-int check_gemm_nt(int dtype, int64_t NX, int64_t NY, int64_t K, int64_t x_stride, int64_t y_stride, int64_t out_stride) {
+template <int DT>
+int launch_gemm_layout(int x_cm, int y_cm, const void* x, const void* y, const GemmPlan& plan, int64_t x_stride,
+                       int64_t y_stride, void* out, int64_t out_stride, int accumulate, float* workspace,
+                       hipStream_t s) {
+  if (x_cm && y_cm)
+    return launch_gemm<DT, true, true>(x, y, plan, x_stride, y_stride, out, out_stride, accumulate, workspace, s);
+  if (x_cm)
+    return launch_gemm<DT, true, false>(x, y, plan, x_stride, y_stride, out, out_stride, accumulate, workspace, s);
+  if (y_cm)
+    return launch_gemm<DT, false, true>(x, y, plan, x_stride, y_stride, out, out_stride, accumulate, workspace, s);
+  return launch_gemm<DT, false, false>(x, y, plan, x_stride, y_stride, out, out_stride, accumulate, workspace, s);
+}
+
+// A row-major operand is (N, K) with stride >= K; a contraction-major one is (K, N) with stride >= N and whole 16-byte
+// groups of rows (N a multiple of 8).
+int check_gemm(int dtype, int64_t NX, int64_t NY, int64_t K, int64_t x_stride, int64_t y_stride, int x_cm, int y_cm,
+               int64_t out_stride) {
   if (dtype != VRL_BF16 && dtype != VRL_F16) return VRL_ERR_DTYPE;
   if (NX < vrl::kLmVocab || NY < vrl::kLmTokens || NX % 4 != 0 || K < 2 * vrl::kLmK || K % vrl::kLmK != 0 ||
-      x_stride < K || y_stride < K || x_stride % 8 != 0 || y_stride % 8 != 0 || out_stride < NX || out_stride % 4 != 0)
+      x_stride < (x_cm ? NX : K) || y_stride < (y_cm ? NY : K) || x_stride % 8 != 0 || y_stride % 8 != 0 ||
+      (x_cm && NX % 8 != 0) || (y_cm && NY % 8 != 0) || out_stride < NX || out_stride % 4 != 0)
     return VRL_ERR_SHAPE;
   if (NY * (NX / 4) > kMaxGrid * 256LL) return VRL_ERR_SHAPE;
   return VRL_OK;
@@ -779,17 +797,18 @@ int vrl_lmhead_dlogits(const void* hidden, const void* weight, int dtype, int64_
 }
 
 int vrl_gemm_nt_plan(int dtype, int64_t NX, int64_t NY, int64_t K, int64_t* workspace_floats) {
-  const int st = check_gemm_nt(dtype, NX, NY, K, K, K, NX);
+  const int st = check_gemm(dtype, NX, NY, K, K, K, 0, 0, NX);
   if (st != VRL_OK) return st;
   const GemmPlan p = gemm_plan(NX, NY, K, 0);
   if (workspace_floats != nullptr) *workspace_floats = p.shape.k_parts > 1 ? p.shape.k_parts * NX * NY : 0;
   return p.shape.k_parts;
 }
 
-int vrl_gemm_nt(const void* x, const void* y, int dtype, int64_t NX, int64_t NY, int64_t K, int64_t x_stride,
-                int64_t y_stride, void* out, int64_t out_stride, int accumulate, int k_parts, float* workspace,
-                void* stream) {
-  const int st = check_gemm_nt(dtype, NX, NY, K, x_stride, y_stride, out_stride);
+int vrl_gemm(const void* x, const void* y, int dtype, int64_t NX, int64_t NY, int64_t K, int64_t x_stride,
+             int64_t y_stride, int x_contraction_major, int y_contraction_major, void* out, int64_t out_stride,
+             int accumulate, int k_parts, float* workspace, void* stream) {
+  const int x_cm = x_contraction_major != 0, y_cm = y_contraction_major != 0;
+  const int st = check_gemm(dtype, NX, NY, K, x_stride, y_stride, x_cm, y_cm, out_stride);
   if (st != VRL_OK) return st;
   if (k_parts < 1 || k_parts > 16 || K / vrl::kLmK / k_parts < 2) return VRL_ERR_ARG;
   if (x == nullptr || y == nullptr || out == nullptr) return VRL_ERR_NULL;
@@ -798,8 +817,16 @@ int vrl_gemm_nt(const void* x, const void* y, int dtype, int64_t NX, int64_t NY,
   if (!aligned(x, 16) || !aligned(y, 16) || !aligned(out, 8) || !aligned(workspace, 16)) return VRL_ERR_ALIGN;
   hipStream_t s = static_cast<hipStream_t>(stream);
   if (dtype == VRL_BF16)
-    return launch_gemm_nt<VRL_BF16>(x, y, p, x_stride, y_stride, out, out_stride, accumulate, workspace, s);
-  return launch_gemm_nt<VRL_F16>(x, y, p, x_stride, y_stride, out, out_stride, accumulate, workspace, s);
+    return launch_gemm_layout<VRL_BF16>(x_cm, y_cm, x, y, p, x_stride, y_stride, out, out_stride, accumulate, workspace,
+                                        s);
+  return launch_gemm_layout<VRL_F16>(x_cm, y_cm, x, y, p, x_stride, y_stride, out, out_stride, accumulate, workspace, s);
+}
+
+int vrl_gemm_nt(const void* x, const void* y, int dtype, int64_t NX, int64_t NY, int64_t K, int64_t x_stride,
+                int64_t y_stride, void* out, int64_t out_stride, int accumulate, int k_parts, float* workspace,
+                void* stream) {
+  return vrl_gemm(x, y, dtype, NX, NY, K, x_stride, y_stride, 0, 0, out, out_stride, accumulate, k_parts, workspace,
+                  stream);
 }
 
 int vrl_transpose(const void* src, int elem_size, int64_t rows, int64_t cols, int64_t src_stride,

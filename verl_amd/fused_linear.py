@@ -6,8 +6,9 @@ Same call as the reference's ``FusedLinearForPPO`` (verl/utils/experimental/torc
 Default path (bf16 / fp16 models): the forward is one hand-written matrix-core kernel that folds the logits into the
 softmax state as it forms them and never writes them (``vrl_lmhead_score``); the backward walks the tokens in chunks, forms
 each chunk's logits again on the matrix cores and writes their gradient into a reusable ``(chunk, vocab)`` buffer
-(``vrl_lmhead_dlogits``), then forms ``d hidden`` with ``vrl_gemm_nt`` and ``d W`` with a library GEMM. Peak extra memory
-is that one buffer, in the backward only.
+(``vrl_lmhead_dlogits``), then forms ``d hidden`` and ``d W`` with ``vrl_gemm``, which reads the weight, the hidden states
+and the gradient buffer as they lie (no transposed copies). No library GEMM runs. Peak extra memory is that one buffer, in
+the backward only.
 
 Library path (``kernels="library"``, fp32 models, ``keep_logits=True``): per chunk the projection ``hidden @ W^T`` is one
 library GEMM (torch.matmul, i.e. hipBLASLt) into the buffer, and everything after it is the HIP row kernel: forward
@@ -44,8 +45,10 @@ DEFAULT_CHUNK_TOKENS = 4096
 #              in fp32), with and without gradients and whatever the number of tokens, so that old (no-grad) and new
 #              (grad) log-probs of the same weights are bit-identical; the backward forms the logits again and writes
 #              their gradient from registers (vrl_lmhead_dlogits, 3.46 ms per 4096 tokens against 3.53 ms for the library
-#              GEMM + row backward) and forms d hidden with vrl_gemm_nt (3.36 against 3.73 ms); d W stays a library product
-#              (the hand-written one needs a transposed copy of the gradient buffer). keep_logits=True needs the logits
+#              GEMM + row backward) and forms d hidden and d W with vrl_gemm (3.25 against 3.73 ms, and 3.62 / 3.85 ms
+#              storing / accumulating against 3.80 / 4.04 ms for the library on the same box), which reads W, the hidden
+#              states and the gradient buffer in place: the contraction of either product runs over rows of its operands,
+#              and the kernel takes such operands through transposing LDS reads. keep_logits=True needs the logits
 #              in memory and therefore takes the library forward, also without gradients.
 # The environment variable and the ``kernels`` argument select; models the kernels do not take (fp32, a hidden size that is
 # not a multiple of 64, fewer than 256 vocabulary entries) go to the library.
@@ -90,13 +93,17 @@ def _padded(x: torch.Tensor, rows: int) -> torch.Tensor:
 
 
 def _d_hidden(grad_logits, weight, weight_t, out, own_kernel):
-    """out = grad_logits @ weight: this package's matrix-core kernel (``vrl_gemm_nt``) when asked for and the shapes
-    allow, the library otherwise (with the transposed copy of the weight when there is one: both operands contiguous
-    along the vocabulary)."""
-    if own_kernel and weight_t is not None and _gemm.gemm_nt_takes(weight_t, grad_logits) and out.stride(0) % 4 == 0:
-        _gemm.gemm_nt(weight_t, grad_logits, out=out)
+    """out = grad_logits @ weight: this package's matrix-core kernel (``vrl_gemm``, the weight read as it lies) when
+    asked for and the shapes allow, the library otherwise (with the transposed copy of the weight when there is one:
+    both operands contiguous along the vocabulary)."""
+    if own_kernel and _own_d_hidden_takes(grad_logits, weight, out):
+        _gemm.gemm(weight, grad_logits, x_t=True, out=out)
     else:
         torch.matmul(grad_logits, weight if weight_t is None else weight_t.t(), out=out)
+
+
+def _own_d_hidden_takes(grad_logits, weight, out) -> bool:
+    return _gemm.gemm_takes(weight, grad_logits, True, False) and out.stride(0) % 4 == 0 and out.stride(1) == 1
 
 
 class _FusedLinearForPPOFunction(torch.autograd.Function):
@@ -163,12 +170,14 @@ class _FusedLinearForPPOFunction(torch.autograd.Function):
         temp = None if ctx.temperature == 1.0 else torch.full((min(chunk, max(T, 1)),), ctx.temperature, **f32)
         need_dh, need_dw = ctx.needs_input_grad[0], ctx.needs_input_grad[1]
         d_hidden = torch.empty_like(hidden) if need_dh else None
-        d_weight = (torch.empty_like(weight) if kept is not None else torch.zeros_like(weight)) if need_dw else None
+        d_weight = torch.empty_like(weight) if need_dw else None
+        dw_started = False     # whether d_weight holds a partial sum yet
         lib = _lib.load()
         # With this package's own kernels every chunk is at least one block of 256 tokens: a smaller chunk size is raised
         # to 256, a short tail joins the chunk before it, and a call with fewer than 256 tokens is padded to one block
         # (zero hidden states and zero incoming gradients give zero rows), so the backward never falls back to logits
-        # that a library GEMM rounded differently from the forward's.
+        # that a library GEMM rounded differently from the forward's. A chunk is also padded to a multiple of 64 tokens,
+        # the step of the contraction of d W.
         own = kept is None and ctx.kernels != "library" and V % 8 == 0 and _mfma_takes_model(hidden, weight)
         step = max(chunk, 256) if own else chunk
         starts = list(range(0, T, step))
@@ -177,7 +186,7 @@ class _FusedLinearForPPOFunction(torch.autograd.Function):
         bounds = [(lo, starts[i + 1] if i + 1 < len(starts) else T) for i, lo in enumerate(starts)]
         rows = max([hi - lo for lo, hi in bounds] + [1])
         if own:
-            rows = max(rows, 256)
+            rows = max((rows + 63) // 64 * 64, 256)
         if temp is not None and temp.numel() < rows:
             temp = torch.full((rows,), ctx.temperature, **f32)
         buf = kept if kept is not None else torch.empty((rows, V), dtype=hidden.dtype, device=dev)
@@ -185,7 +194,9 @@ class _FusedLinearForPPOFunction(torch.autograd.Function):
         # For 16-bit operands the library GEMM is 25-35 % faster when both operands are contiguous along the
         # contraction axis (vocab for `d hidden`, tokens for `d W`); fp32 runs at the fp32 matrix peak either way.
         half = hidden.element_size() == 2
-        weight_t = transpose_2d(weight) if (half and need_dh and T >= _WEIGHT_TRANSPOSE_MIN_TOKENS) else None
+        own_dh = own and ctx.kernels != "library" and need_dh and _own_d_hidden_takes(buf[:256], weight, d_hidden)
+        weight_t = (transpose_2d(weight)
+                    if (half and need_dh and not own_dh and T >= _WEIGHT_TRANSPOSE_MIN_TOKENS) else None)
         with torch.cuda.device(dev):
             stream = _lib.stream_ptr(dev)
             for lo, hi in bounds:
@@ -196,9 +207,8 @@ class _FusedLinearForPPOFunction(torch.autograd.Function):
                     c_h, c_ids, c_lse, c_ent = hidden[lo:hi], input_ids[lo:hi], lse[lo:hi], h[lo:hi]
                     c_gl = None if gl is None else gl[lo:hi]
                     c_gh = None if gh is None else gh[lo:hi]
-                    m = n
-                    if n < 256:
-                        m = 256
+                    m = max((n + 63) // 64 * 64, 256)
+                    if m != n:
                         c_h = _padded(c_h, m)
                         c_ids, c_lse, c_ent = _padded(c_ids, m), _padded(c_lse, m), _padded(c_ent, m)
                         c_gl = None if c_gl is None else _padded(c_gl, m)
@@ -213,7 +223,14 @@ class _FusedLinearForPPOFunction(torch.autograd.Function):
                     if need_dh:
                         _d_hidden(logits, weight, weight_t, d_hidden[lo:hi], True)
                     if need_dw:
-                        d_weight.addmm_(logits.t(), transpose_2d(hidden[lo:hi]).t() if half else hidden[lo:hi])
+                        # d W (+)= G^T . H over the padded chunk (its extra rows are zero in both), read in place
+                        if _gemm.gemm_takes(c_h, buf[:m], True, True):
+                            _gemm.gemm(c_h, buf[:m], x_t=True, y_t=True, out=d_weight, accumulate=dw_started)
+                        else:
+                            if not dw_started:
+                                d_weight.zero_()
+                            d_weight.addmm_(logits.t(), transpose_2d(hidden[lo:hi]).t())
+                        dw_started = True
                     continue
                 if kept is not None:
                     logits = buf[lo:hi]
@@ -231,13 +248,22 @@ class _FusedLinearForPPOFunction(torch.autograd.Function):
                 if need_dh:
                     _d_hidden(logits, weight, weight_t, d_hidden[lo:hi], ctx.kernels != "library")
                 if need_dw:
+                    if not dw_started:
+                        d_weight.zero_()
+                        dw_started = True
                     d_weight.addmm_(logits.t(), transpose_2d(hidden[lo:hi]).t() if half else hidden[lo:hi])
             if kept is not None:
                 # the gradient over all tokens' logits is in `kept`: one product each, nothing to accumulate
                 if need_dh:
                     _d_hidden(kept, weight, weight_t, d_hidden, ctx.kernels != "library")
                 if need_dw:
-                    torch.matmul(kept.t(), transpose_2d(hidden).t() if half else hidden, out=d_weight)
+                    if ctx.kernels != "library" and _gemm.gemm_takes(hidden, kept, True, True):
+                        _gemm.gemm(hidden, kept, x_t=True, y_t=True, out=d_weight)
+                    else:
+                        torch.matmul(kept.t(), transpose_2d(hidden).t() if half else hidden, out=d_weight)
+                    dw_started = True
+            if need_dw and not dw_started:
+                d_weight.zero_()          # no tokens
         return d_hidden, d_weight, None, None, None, None, None
 
 
@@ -259,7 +285,7 @@ def fused_linear_for_ppo(hidden_states: torch.Tensor, vocab_weights: torch.Tenso
     ``kernels`` chooses which matrix products are this package's own kernels: ``"library"`` (none: torch.matmul
     throughout) or ``"auto"`` / ``"mfma"`` (all that are at least as fast: a forward that is one kernel and never
     writes logits, a backward that forms the logits again, writes their gradient straight from registers and forms
-    ``d hidden`` with ``vrl_gemm_nt``; ``d W`` stays a library product). Which forward runs depends on this option, on
+    ``d hidden`` and ``d W`` with ``vrl_gemm``: no library GEMM is called). Which forward runs depends on this option, on
     ``keep_logits`` and on the model, never on the number of tokens or on whether gradients are recorded, so log-probs
     computed with and without gradients are bit-identical. None takes ``DEFAULT_KERNELS`` ("auto" unless
     ``VERL_AMD_LMHEAD_KERNELS`` says otherwise).
