@@ -252,7 +252,7 @@ int vrl_transpose(const void* src, int elem_size, int64_t rows, int64_t cols, in
  * NOT rounded to the operand type on the way, unlike a GEMM that writes them out). Forward only.
  * `partials` is caller-owned scratch of n_tokens * n_splits * 4 floats; vrl_lmhead_plan gives n_splits.
  * Requirements checked on the host: n_tokens >= 256, vocab >= 256, hidden_size a multiple of 64, pitches multiples
- * of 8 elements, 16-byte aligned operands, each operand below 4 GiB, 1 <= n_splits <= 64. out_logprob (with labels
+ * of 8 elements and at most 2^28, n_tokens and vocab at most 2^30, 16-byte aligned operands, 1 <= n_splits <= 64. out_logprob (with labels
  * and err_flag), out_entropy, out_lse: any may be NULL, not all.
  *
  * Replaces the reference's fused linear + cross-entropy forward:
@@ -296,7 +296,7 @@ int vrl_lmhead_dlogits(const void* hidden, const void* weight, int dtype, int64_
  * multiple of 8. Strides are in elements and multiples of 8, bases 16-byte aligned. out is (NY, NX) in the operands' type
  * (VRL_BF16 or VRL_F16) with row stride out_stride (a multiple of 4, 8-byte aligned base); fp32 accumulation, one
  * rounding; the result does not depend on the operands' layouts. NX, NY >= 256, NX a multiple of 4, K a multiple of 64
- * and >= 128. accumulate != 0 adds the product to what out holds.
+ * and >= 128; strides at most 2^28 elements, NX, NY and K at most 2^30. accumulate != 0 adds the product to what out holds.
  * k_parts (1..16, normally what vrl_gemm_nt_plan returns) cuts the contraction into ranges that are summed in a fixed
  * order through `workspace` (k_parts * NX * NY floats, 16-byte aligned; may be NULL when k_parts == 1): that is how a
  * product with few output tiles still fills the CUs. vrl_gemm_nt_plan returns the number of ranges it would use for a

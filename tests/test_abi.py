@@ -275,6 +275,7 @@ def test_gemm_layout_argument_errors(lib):
     assert call(yt=1, NY=512, ys=256) == _lib.VRL_ERR_SHAPE
     assert call(xt=0, xs=128) == _lib.VRL_ERR_SHAPE                # row-major x: stride counts the contraction (256)
     assert call(K=96) == _lib.VRL_ERR_SHAPE
+    assert call(xs=(1 << 28) + 8) == _lib.VRL_ERR_SHAPE            # lane offsets are 32-bit
     assert call(parts=0) == _lib.VRL_ERR_ARG
     assert call(y=None) == _lib.VRL_ERR_NULL
     assert call(x=P + 8) == _lib.VRL_ERR_ALIGN

@@ -323,9 +323,16 @@ int launch_lmhead_dlogits(const void* hidden, const void* weight, int64_t T, int
 }
 
 // Shape rules the matrix-core kernels share.
+// The matrix-core walk adds a lane's share of a load address (up to 7 rows + 128 bytes) as a 32-bit offset, and keeps
+// row and column indices in 32-bit registers.
+constexpr int64_t kLmMaxStride = int64_t(1) << 28;
+constexpr int64_t kLmMaxRows = int64_t(1) << 30;
+
 int check_lmhead_shape(int dtype, int64_t n_tokens, int64_t vocab, int64_t hidden_size, int64_t h_stride,
                        int64_t w_stride, int n_splits) {
   if (dtype != VRL_BF16 && dtype != VRL_F16) return VRL_ERR_DTYPE;
+  if (h_stride > kLmMaxStride || w_stride > kLmMaxStride || vocab > kLmMaxRows || n_tokens > kLmMaxRows)
+    return VRL_ERR_SHAPE;
   if (n_tokens < vrl::kLmTokens || vocab < vrl::kLmVocab || hidden_size <= 0 || hidden_size % vrl::kLmK != 0 ||
       h_stride < hidden_size || w_stride < hidden_size || h_stride % 8 != 0 || w_stride % 8 != 0 ||
       n_splits < 1 || n_splits > vrl::kLmMaxSplits)
@@ -451,6 +458,8 @@ int launch_gemm_layout(int x_cm, int y_cm, const void* x, const void* y, const G
 int check_gemm(int dtype, int64_t NX, int64_t NY, int64_t K, int64_t x_stride, int64_t y_stride, int x_cm, int y_cm,
                int64_t out_stride) {
   if (dtype != VRL_BF16 && dtype != VRL_F16) return VRL_ERR_DTYPE;
+  if (x_stride > kLmMaxStride || y_stride > kLmMaxStride || NX > kLmMaxRows || NY > kLmMaxRows || K > kLmMaxRows)
+    return VRL_ERR_SHAPE;
   if (NX < vrl::kLmVocab || NY < vrl::kLmTokens || NX % 4 != 0 || K < 2 * vrl::kLmK || K % vrl::kLmK != 0 ||
       x_stride < (x_cm ? NX : K) || y_stride < (y_cm ? NY : K) || x_stride % 8 != 0 || y_stride % 8 != 0 ||
       (x_cm && NX % 8 != 0) || (y_cm && NY % 8 != 0) || out_stride < NX || out_stride % 4 != 0)
