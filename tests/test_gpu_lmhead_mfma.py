@@ -160,6 +160,49 @@ def test_backward_products_come_from_the_matrix_core_kernel(dev, kernels):
     assert gemm.counters["gemm"] == before
 
 
+def test_benchmark_shape_backward_against_fp64(dev):
+    """8192 tokens x 3584 -> 152064 bf16, chunks of 4096 (what bench.py --lm-head times): d hidden and d W of the default
+    path (vrl_lmhead_dlogits + vrl_gemm, two chunks, the second accumulated) against the closed-form gradient in fp64,
+    formed 1024 tokens at a time; the all-library path is measured against the same reference beside it. Bar: 2^-7 +
+    2^-10 of the largest reference element: a row of either gradient is dominated by its label term, whose factor from
+    the gradient buffer is rounded to bf16 once (up to 2^-8 relative) before the product is rounded to bf16 again (2^-8);
+    both paths round that factor alike, so their errors agree to three digits (6.5e-3 and 6.2e-3)."""
+    T, K, V = 8192, 3584, 152064
+    temp = 1.5
+    g = torch.Generator(device=dev).manual_seed(4001)
+    h = torch.empty(T, K, device=dev).uniform_(-0.5, 0.5, generator=g).bfloat16().requires_grad_()
+    w = (torch.empty(V, K, device=dev).uniform_(-0.5, 0.5, generator=g) * 0.05).bfloat16().requires_grad_()
+    ids = torch.randint(0, V, (T,), generator=g, device=dev)
+    g_lp = torch.empty(T, device=dev).uniform_(-1, 1, generator=g)
+    g_ent = torch.empty(T, device=dev).uniform_(-0.5, 0.5, generator=g)
+    got = {}
+    for kernels in ("auto", "library"):
+        lp, ent = fused_linear_for_ppo(h, w, ids, temp, chunk_size=4096, kernels=kernels)
+        got[kernels] = torch.autograd.grad((lp, ent), (h, w), (g_lp, g_ent))
+        del lp, ent
+    w64 = w.detach().double()
+    ref_dw = torch.zeros(V, K, dtype=torch.float64, device=dev)
+    ref_dh = torch.empty(T, K, dtype=torch.float64, device=dev)
+    for lo in range(0, T, 1024):
+        h64 = h.detach()[lo:lo + 1024].double()
+        z = (h64 @ w64.t()) / temp
+        logp = torch.log_softmax(z, -1)
+        p = logp.exp()
+        ent64 = -(p * logp).sum(-1)
+        G = -(g_ent[lo:lo + 1024].double()[:, None]) * p * (logp + ent64[:, None]) - g_lp[lo:lo + 1024].double()[:, None] * p
+        G[torch.arange(G.shape[0], device=dev), ids[lo:lo + 1024]] += g_lp[lo:lo + 1024].double()
+        G /= temp
+        ref_dh[lo:lo + 1024] = G @ w64
+        ref_dw += G.t() @ h64
+        del z, logp, p, G
+    for kernels, (dh, dw) in got.items():
+        e_h = (dh.double() - ref_dh).abs().max().item() / ref_dh.abs().max().item()
+        e_w = (dw.double() - ref_dw).abs().max().item() / ref_dw.abs().max().item()
+        print(f"[lmhead backward 8192x3584->152064, kernels={kernels}] max err / max |ref|: d hidden {e_h:.2e}, d W {e_w:.2e}",
+              flush=True)
+        assert e_h <= 2.0 ** -7 + 2.0 ** -10 and e_w <= 2.0 ** -7 + 2.0 ** -10, (kernels, e_h, e_w)
+
+
 def test_fused_linear_with_the_matrix_core_kernels(dev):
     """fused_linear_for_ppo(kernels="mfma"): forward from vrl_lmhead_score, backward through vrl_lmhead_dlogits and the
     two products, against torch autograd on the fp32 composition at the reference's tolerances
