@@ -449,6 +449,29 @@ def bench_lm_head(args, dev):
     t_fb_m = timed(fwd_bwd_mfma)
     wt = torch.empty(D, V, dtype=weight.dtype, device=dev)
     t_tr = timed(lambda: transpose_2d(weight.detach(), wt))
+    # the two products of the backward on one chunk's worth of tokens, own kernel against the library on operands laid
+    # out as the library likes them best (transposed copies made beforehand and not timed)
+    from verl_amd import gemm as own_gemm
+    n_c = min(chunk, T)
+    with torch.no_grad():
+        G = (torch.randn(n_c, V, generator=g, device=dev) * 0.01).bfloat16()
+        Hc = hidden.detach()[:n_c]
+        Ht = transpose_2d(Hc)
+        d_h = torch.empty(n_c, D, dtype=torch.bfloat16, device=dev)
+        d_w = torch.zeros(V, D, dtype=torch.bfloat16, device=dev)
+        Wd = weight.detach()
+        products = {
+            "tokens": n_c,
+            "d_hidden": {"own_ms": timed(lambda: own_gemm.gemm(Wd, G, x_t=True, out=d_h)) * 1e3,
+                         "library_ms": timed(lambda: torch.matmul(G, wt.t(), out=d_h)) * 1e3},
+            "d_weight_stored": {"own_ms": timed(lambda: own_gemm.gemm(Hc, G, x_t=True, y_t=True, out=d_w)) * 1e3,
+                                "library_ms": timed(lambda: torch.matmul(G.t(), Ht.t(), out=d_w)) * 1e3},
+            "d_weight_accumulated": {"own_ms": timed(lambda: own_gemm.gemm(Hc, G, x_t=True, y_t=True, out=d_w, accumulate=True)) * 1e3,
+                                     "library_ms": timed(lambda: d_w.addmm_(G.t(), Ht.t())) * 1e3},
+            "note": "own: vrl_gemm on W, the hidden states and the gradient buffer as they lie; library: torch.matmul / "
+                    "addmm_ on the transposed copies of W and of the hidden chunk (made beforehand, not timed)",
+        }
+        del G, Ht, d_h, d_w
     flops_f, flops_fb = 2.0 * T * D * V, 6.0 * T * D * V
     ceiling = mfma_ceiling(dev, args.steps)
     print(json.dumps({
@@ -482,6 +505,7 @@ def bench_lm_head(args, dev):
                                          "is written from registers (no GEMM into the buffer, no pass over it); d hidden "
                                          "and d W come from the same main loop, which reads W, the hidden states and the "
                                          "gradient buffer as they lie (transposing LDS reads)"},
+        "backward_products": products,
         "weight_transpose": {"ms": t_tr * 1e3, "gbps": 2.0 * V * D * 2 / t_tr / 1e9, "kernel": "transpose_kernel<2>",
                              "note": "the copy the all-library backward makes once per call; the default path needs none"},
         "parity_guard": {"rows": 256, "max_abs_err_logprob": e1, "max_abs_err_entropy": e2},

@@ -133,7 +133,7 @@ def test_dlogits_matches_fp64_autograd(dev, dtype, T, V, K, splits):
 def test_backward_products_come_from_the_matrix_core_kernel(dev, kernels):
     """Unless told "library", the backward forms d hidden and d W with vrl_gemm, reading the weight, the hidden states and
     the gradient buffer in place: same tolerances against torch autograd as the other paths, and the launches are
-    counted (two per chunk)."""
+    counted (two per chunk; with kept logits d hidden only, the single d W product over all tokens is the library's)."""
     from verl_amd import gemm
 
     g = torch.Generator(device=dev).manual_seed(78)
@@ -147,7 +147,7 @@ def test_backward_products_come_from_the_matrix_core_kernel(dev, kernels):
     ref_ent = torch.logsumexp(logits, -1) - (torch.softmax(logits, -1) * logits).sum(-1)
     ref_lp = -torch.nn.functional.cross_entropy(logits, labels, reduction="none")
     d_ref_h, d_ref_w = torch.autograd.grad((ref_ent, ref_lp), (hidden, weight), (g_ent, g_lp))
-    for chunk, keep, launches in ((1024, False, 6), (4096, False, 2), (4096, True, 2)):
+    for chunk, keep, launches in ((1024, False, 6), (4096, False, 2), (4096, True, 1)):
         before = gemm.counters["gemm"]
         lp, ent = fused_linear_for_ppo(hidden, weight, labels, 1.5, chunk_size=chunk, keep_logits=keep, kernels=kernels)
         d_h, d_w = torch.autograd.grad((ent, lp), (hidden, weight), (g_ent, g_lp))

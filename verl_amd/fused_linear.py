@@ -257,10 +257,8 @@ class _FusedLinearForPPOFunction(torch.autograd.Function):
                 if need_dh:
                     _d_hidden(kept, weight, weight_t, d_hidden, ctx.kernels != "library")
                 if need_dw:
-                    if ctx.kernels != "library" and _gemm.gemm_takes(hidden, kept, True, True):
-                        _gemm.gemm(hidden, kept, x_t=True, y_t=True, out=d_weight)
-                    else:
-                        torch.matmul(kept.t(), transpose_2d(hidden).t() if half else hidden, out=d_weight)
+                    # one product over all tokens: here the library is the faster one (6.7 against 7.2 ms at 8192 tokens)
+                    torch.matmul(kept.t(), transpose_2d(hidden).t() if half else hidden, out=d_weight)
                     dw_started = True
             if need_dw and not dw_started:
                 d_weight.zero_()          # no tokens
