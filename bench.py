@@ -205,6 +205,8 @@ class Step:
 
 # HBM bytes per launch of rowscore_backward_kernel from rocprofv3 --pmc (FETCH_SIZE, WRITE_SIZE; same scaling as above).
 MEASURED_BACKWARD_TRAFFIC_BYTES = {"c3": 4981794581}   # profiles/rowscore_backward_kernel_hbm_counters_c3.md
+# profiles/score_responses_kernel_hbm_counters_c3_packed.md (forward, backward), for the packed micro-batch bench_score_responses builds
+MEASURED_SCORE_RESPONSES_TRAFFIC_BYTES = (1676672404, 4168192835)
 
 
 def bench_backward(args, dev, workload=None):
@@ -855,8 +857,11 @@ def bench_score_responses(args, dev, steps, warmup):
     torch.cuda.synchronize()
     bwd_ms = sum(a.elapsed_time(b) for a, b in evs) / len(evs)
     bwd_bytes = n_resp * (w.V * 2 + 8 + 16) + n * w.V * 2 + (B + 1) * 8 + B * 8
+    # the counters were read at this very micro-batch (5515 response rows of 8192); another one has no measured traffic
+    measured = MEASURED_SCORE_RESPONSES_TRAFFIC_BYTES if (n, n_resp, B) == (8192, 5515, 4) else (None, None)
     backward = {"avg_kernel_ms": bwd_ms, "kernel": "score_responses_backward_kernel",
                 "algorithmic_bytes_per_launch": bwd_bytes, "achieved_gbps": bwd_bytes / (bwd_ms * 1e-3) / 1e9,
+                "traffic": measured[1],
                 "all_rows_backward_bytes": n * (w.V * 4 + 8 + 16),
                 "parity_guard": "bit-equal to vrl_rowscore_backward with per-token gradients"}
     return {
@@ -866,7 +871,10 @@ def bench_score_responses(args, dev, steps, warmup):
                    "response_rows_per_step": n_resp, "sequences": B, "padded_response_len": T,
                    "step": "vrl_score_responses through the C ABI (labels rolled in-kernel, prompt rows not read)"},
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                     "frac": achieved / HBM_PEAK_GBPS, "traffic": None, "kernel": "score_responses_kernel",
+                     "frac": achieved / HBM_PEAK_GBPS, "traffic": measured[0],
+                     "traffic_source": "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of this kernel at this micro-batch, "
+                                       "profiles/score_responses_kernel_hbm_counters_c3_packed.md",
+                     "kernel": "score_responses_kernel",
                      "avg_kernel_ms": avg_ms, "algorithmic_bytes_per_launch": bytes_launch},
         "all_rows_equivalent_tokens_per_s": n * steps / wall,
         "backward": backward,
@@ -926,6 +934,8 @@ def main():
         bench_ceilings(args, dev)
         return
     if args.score_responses:
+        if args.copy_calibration:
+            copy_calibration(dev)
         print(json.dumps(bench_score_responses(args, dev, args.steps, args.warmup)), flush=True)
         return
     if args.backward:
