@@ -37,7 +37,7 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0
 # HBM bytes per row-kernel launch measured with rocprofv3 (--pmc FETCH_SIZE and --pmc WRITE_SIZE, one run each,
 # both scaled by what the same counter reads for a plain 1 GiB device copy: x1.999956 and x1.0). The workload
 # shapes are fixed, so the figure is a property of (kernel, shape); the counter summary is kept under profiles/.
-MEASURED_TRAFFIC_BYTES = {"c2": 19943644231, "c3": 2490946810, "c4": 67292547122}
+MEASURED_TRAFFIC_BYTES = {"c1": 525600443, "c2": 19943644231, "c3": 2490946810, "c4": 67292547122}
 METRIC = "verified tokens/sec + achieved HBM GB/s (% of peak), vocab 152k bf16, 1 GPU"
 
 
@@ -739,7 +739,8 @@ def bench_forward(args, dev, workload, steps, warmup, with_cpu_baseline):
             "frac": achieved / HBM_PEAK_GBPS,
             "traffic": None if resized else MEASURED_TRAFFIC_BYTES.get(workload),
             "traffic_source": None if resized or workload not in MEASURED_TRAFFIC_BYTES else
-            "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of this kernel at this shape, profiles/rowscore_kernel_hbm_counters_c2_c3_c4.md",
+            "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of this kernel at this shape, profiles/rowscore_kernel_hbm_counters_" +
+            ("c1.md" if workload == "c1" else "c2_c3_c4.md"),
             "kernel": "rowscore_kernel",
             "avg_kernel_ms": avg_kern_ms,
             "algorithmic_bytes_per_launch": bytes_score,
