@@ -103,6 +103,44 @@ def test_contraction_major_operands_with_row_strides(dev):
     _check(got, xt.t().contiguous(), yt.t().contiguous())
 
 
+def test_random_shapes_strides_and_layouts(dev):
+    """Seeded random shapes (edge tiles on both sides, odd tile counts, contraction ranges), operands as views into wider
+    buffers, every layout pair, stored and accumulated: bit-equal to the row-major product of contiguous copies, which is
+    itself checked against fp64."""
+    import random
+
+    rng = random.Random(20240607)
+    g = torch.Generator(device=dev).manual_seed(17)
+    for case in range(12):
+        NX = rng.randrange(256, 1100, 8)
+        NY = rng.randrange(256, 1100, 8)
+        K = rng.randrange(128, 1100, 64)
+        dtype = (torch.bfloat16, torch.float16)[case % 2]
+        parts = rng.choice([None, 1, 2]) if K >= 256 else None
+        x = (torch.randn(NX, K, generator=g, device=dev) * 0.5).to(dtype)
+        y = (torch.randn(NY, K, generator=g, device=dev) * 0.5).to(dtype)
+        base = torch.randn(NY, NX, generator=g, device=dev).to(dtype)
+        want = gemm.gemm_nt(x, y, k_parts=parts)
+        _check(want, x, y)
+        want_acc = base.clone()
+        gemm.gemm_nt(x, y, out=want_acc, accumulate=True, k_parts=parts)
+
+        def widened(t, pad):                      # the same values as a view into a buffer with a longer row
+            buf = torch.full((t.shape[0], t.shape[1] + pad), 3.0, dtype=t.dtype, device=dev)
+            buf[:, :t.shape[1]] = t
+            return buf[:, :t.shape[1]]
+
+        px, py = 8 * rng.randrange(0, 4), 8 * rng.randrange(0, 4)
+        for x_t, y_t in ((False, False), (True, False), (False, True), (True, True)):
+            xo = widened(x.t().contiguous() if x_t else x, px)
+            yo = widened(y.t().contiguous() if y_t else y, py)
+            got = gemm.gemm(xo, yo, x_t, y_t, k_parts=parts)
+            assert torch.equal(got, want), (case, NX, NY, K, x_t, y_t, parts)
+            acc = base.clone()
+            gemm.gemm(xo, yo, x_t, y_t, out=acc, accumulate=True, k_parts=parts)
+            assert torch.equal(acc, want_acc), (case, NX, NY, K, x_t, y_t, parts)
+
+
 def test_backward_products_of_the_lm_head_read_in_place(dev):
     """d hidden = G @ W and d W (+)= G.T @ H from G (tokens, vocab), W (vocab, hidden) and H (tokens, hidden) as they
     lie, against the same products through transposed copies (bit-equal) and against fp32 (tolerance)."""
