@@ -194,7 +194,8 @@ class _FusedLinearForPPOFunction(torch.autograd.Function):
         # For 16-bit operands the library GEMM is 25-35 % faster when both operands are contiguous along the
         # contraction axis (vocab for `d hidden`, tokens for `d W`); fp32 runs at the fp32 matrix peak either way.
         half = hidden.element_size() == 2
-        own_dh = own and ctx.kernels != "library" and need_dh and _own_d_hidden_takes(buf[:256], weight, d_hidden)
+        # (only a library `d hidden` wants the transposed weight; the package's own product reads W as it lies)
+        own_dh = ctx.kernels != "library" and need_dh and _own_d_hidden_takes(buf[:256], weight, d_hidden)
         weight_t = (transpose_2d(weight)
                     if (half and need_dh and not own_dh and T >= _WEIGHT_TRANSPOSE_MIN_TOKENS) else None)
         with torch.cuda.device(dev):
