@@ -288,6 +288,42 @@ def test_default_forward_is_the_same_with_and_without_gradients_and_for_any_toke
     assert not d_h[100:].any()
 
 
+def test_token_results_do_not_depend_on_the_call_when_the_vocabulary_is_cut_alike(dev):
+    """A token's partial softmax states are summed in the order of the vocabulary ranges. Calls of 8192 tokens or more all
+    use 8 ranges: the same token gives the same bits in a call of 8192 and in one of 16640 tokens. Smaller calls are cut
+    finer (here 64 and 32 ranges): a few ulps apart, and bit-identical again once `forward_splits` pins the number."""
+    g = torch.Generator(device=dev).manual_seed(15)
+    K, V = 64, 16384                                     # 64 vocabulary tiles
+    T = 16640
+    h = torch.empty(T, K, device=dev).uniform_(-1.0, 1.0, generator=g).bfloat16()
+    w = torch.empty(V, K, device=dev).uniform_(-1.0, 1.0, generator=g).bfloat16()
+    ids = torch.randint(0, V, (T,), generator=g, device=dev)
+    lib = _lib.load()
+    assert lib.vrl_lmhead_plan(T, V) == 8 and lib.vrl_lmhead_plan(8192, V) == 8 and lib.vrl_lmhead_plan(10 ** 6, V) == 8
+    assert lib.vrl_lmhead_plan(256, V) == 64 and lib.vrl_lmhead_plan(2048, V) == 32
+    with torch.no_grad():
+        lp_all, ent_all = fused_linear_for_ppo(h, w, ids, 0.9)
+        lp_a, ent_a = fused_linear_for_ppo(h[:8192], w, ids[:8192], 0.9)
+        assert torch.equal(lp_a, lp_all[:8192]) and torch.equal(ent_a, ent_all[:8192])
+        lp_b, ent_b = fused_linear_for_ppo(h[8192:], w, ids[8192:], 0.9)          # 8448 tokens
+        assert torch.equal(lp_b, lp_all[8192:]) and torch.equal(ent_b, ent_all[8192:])
+        # smaller calls, planned: 64 and 32 ranges
+        lp_s, ent_s = fused_linear_for_ppo(h[:256], w, ids[:256], 0.9)
+        lp_m, ent_m = fused_linear_for_ppo(h[:2048], w, ids[:2048], 0.9)
+        for got_lp, got_ent, n in ((lp_s, ent_s, 256), (lp_m, ent_m, 2048)):
+            assert (got_lp - lp_all[:n]).abs().max().item() <= 4e-6 and (got_ent - ent_all[:n]).abs().max().item() <= 4e-6
+        # pinned: the same bits whatever the size of the call
+        pin_all = fused_linear_for_ppo(h, w, ids, 0.9, forward_splits=16)
+        for lo, hi in ((0, 256), (300, 2348), (8000, 16640), (5, 6)):
+            lp_p, ent_p = fused_linear_for_ppo(h[lo:hi], w, ids[lo:hi], 0.9, forward_splits=16)
+            assert torch.equal(lp_p, pin_all[0][lo:hi]) and torch.equal(ent_p, pin_all[1][lo:hi]), (lo, hi)
+    hg = h[:300].clone().requires_grad_()
+    lp_g, _ = fused_linear_for_ppo(hg, w, ids[:300], 0.9, forward_splits=16)        # and with gradients
+    assert torch.equal(lp_g.detach(), pin_all[0][:300])
+    with pytest.raises(ValueError):
+        fused_linear_for_ppo(h[:256], w, ids[:256], 0.9, forward_splits=65)
+
+
 def test_special_values_and_errors(dev):
     g = torch.Generator(device=dev).manual_seed(6)
     T, V, K = 256, 512, 64

@@ -753,6 +753,10 @@ int vrl_lmhead_plan(int64_t n_tokens, int64_t vocab) {
   const int64_t vtiles = (vocab + vrl::kLmVocab - 1) / vrl::kLmVocab;
   int64_t s = (256 + tblocks - 1) / tblocks;  // one workgroup per CU
   s = ((s + 3) / 4) * 4;                       // groups of 4 splits share an XCD with 8 token blocks
+  // Never fewer than 8: every call of 8192 tokens or more then cuts the vocabulary alike and sums a token's partial
+  // softmax states in the same order, so its results do not depend on how many tokens came with it (more workgroups
+  // than CUs cost nothing: they run in rounds).
+  if (s < 8) s = 8;
   if (s > vrl::kLmMaxSplits) s = vrl::kLmMaxSplits;
   if (s > vtiles) s = vtiles;
   if (s < 1) s = 1;

@@ -43,7 +43,8 @@ DEFAULT_CHUNK_TOKENS = 4096
 #              as fast as the library uses it. The forward is one kernel that never writes logits (vrl_lmhead_score: as fast
 #              as the library GEMM + row kernel at 8192 x 3584 -> 152064 bf16, 6.5 ms, no (chunk, vocab) buffer, logits kept
 #              in fp32), with and without gradients and whatever the number of tokens, so that old (no-grad) and new
-#              (grad) log-probs of the same weights are bit-identical; the backward forms the logits again and writes
+#              (grad) log-probs of the same weights are bit-identical when both calls cut the vocabulary alike (see
+#              DEFAULT_FORWARD_SPLITS) and a few ulps apart otherwise; the backward forms the logits again and writes
 #              their gradient from registers (vrl_lmhead_dlogits, 3.46 ms per 4096 tokens against 3.53 ms for the library
 #              GEMM + row backward) and forms d hidden and d W with vrl_gemm (3.25 against 3.73 ms, and 3.62 / 3.85 ms
 #              storing / accumulating against 3.80 / 4.04 ms for the library on the same box), which reads W, the hidden
@@ -53,6 +54,14 @@ DEFAULT_CHUNK_TOKENS = 4096
 # The environment variable and the ``kernels`` argument select; models the kernels do not take (fp32, a hidden size that is
 # not a multiple of 64, fewer than 256 vocabulary entries) go to the library.
 DEFAULT_KERNELS = os.environ.get("VERL_AMD_LMHEAD_KERNELS", "auto")
+
+# Into how many ranges the single forward kernel cuts the vocabulary. None lets the library plan per call: 8 for every call
+# of 8192 tokens or more, more for fewer tokens so that the CUs stay busy. A token's partial softmax states are summed in
+# range order, so two calls give the same bits for a token exactly when they use the same number of ranges: always for
+# calls of >= 8192 tokens, and for any mix of sizes when this is pinned (1..64; `forward_splits` argument, or the
+# environment variable VERL_AMD_LMHEAD_SPLITS). Differently cut calls agree to a few fp32 ulps of the logsumexp.
+_env_splits = os.environ.get("VERL_AMD_LMHEAD_SPLITS", "")
+DEFAULT_FORWARD_SPLITS = int(_env_splits) if _env_splits.strip() else None
 
 
 def _mfma_takes_model(hidden: torch.Tensor, weight: torch.Tensor) -> bool:
@@ -68,7 +77,8 @@ def _mfma_takes_model(hidden: torch.Tensor, weight: torch.Tensor) -> bool:
 def _own_forward_in_use(kernels: str, keep_logits: bool, hidden: torch.Tensor, weight: torch.Tensor) -> bool:
     """Whether the forward is vrl_lmhead_score. Decided by the caller's options and by the model only, never by the number
     of tokens or by whether gradients are recorded: a trainer's old (no-grad) and new (grad) log-probs of the same
-    weights then come from the same arithmetic whatever the micro-batch sizes are."""
+    weights then come from the same kernel whatever the micro-batch sizes are (and from the same summation order when
+    the calls use the same number of vocabulary ranges, see DEFAULT_FORWARD_SPLITS)."""
     return kernels != "library" and not keep_logits and _mfma_takes_model(hidden, weight)
 
 
@@ -108,7 +118,7 @@ def _own_d_hidden_takes(grad_logits, weight, out) -> bool:
 
 class _FusedLinearForPPOFunction(torch.autograd.Function):
     @staticmethod
-    def forward(ctx, hidden, weight, input_ids, temperature, chunk_size, keep_logits, kernels):
+    def forward(ctx, hidden, weight, input_ids, temperature, chunk_size, keep_logits, kernels, forward_splits=None):
         ctx.set_materialize_grads(False)
         ctx.kernels = kernels
         T, D = hidden.shape
@@ -121,7 +131,7 @@ class _FusedLinearForPPOFunction(torch.autograd.Function):
         flag = torch.zeros(1, dtype=torch.int32, device=dev)
         if _own_forward_in_use(kernels, keep_logits, hidden, weight):
             temp_all = None if temperature == 1.0 else torch.full((T,), float(temperature), **f32)
-            lp, h, lse = _own_forward(hidden, weight, input_ids, temp_all, None, "fused_linear_for_ppo")
+            lp, h, lse = _own_forward(hidden, weight, input_ids, temp_all, forward_splits, "fused_linear_for_ppo")
             ctx.save_for_backward(hidden, weight, input_ids, lse, h)
             ctx.temperature = float(temperature)
             ctx.chunk_size = int(chunk_size)
@@ -152,7 +162,7 @@ class _FusedLinearForPPOFunction(torch.autograd.Function):
     def backward(ctx, g_lp: Optional[torch.Tensor], g_h: Optional[torch.Tensor]):
         hidden, weight, input_ids, lse, h = ctx.saved_tensors
         if g_lp is None and g_h is None:
-            return None, None, None, None, None, None, None
+            return None, None, None, None, None, None, None, None
         kept = ctx.kept_logits
         if kept is not None:
             ctx.kept_logits = None        # the gradient is written over them: they serve one backward
@@ -263,12 +273,12 @@ class _FusedLinearForPPOFunction(torch.autograd.Function):
                     dw_started = True
             if need_dw and not dw_started:
                 d_weight.zero_()          # no tokens
-        return d_hidden, d_weight, None, None, None, None, None
+        return d_hidden, d_weight, None, None, None, None, None, None
 
 
 def fused_linear_for_ppo(hidden_states: torch.Tensor, vocab_weights: torch.Tensor, input_ids: torch.Tensor,
                          temperature: float = 1.0, chunk_size: int = DEFAULT_CHUNK_TOKENS, keep_logits: bool = False,
-                         kernels: Optional[str] = None):
+                         kernels: Optional[str] = None, forward_splits: Optional[int] = None):
     """(log_probs fp32, entropy fp32) of ``softmax((hidden_states @ vocab_weights.T) / temperature)`` at ``input_ids``.
 
     ``hidden_states`` is ``(tokens, hidden)`` or ``(batch, seq, hidden)`` with ``input_ids`` of the matching leading
@@ -288,10 +298,18 @@ def fused_linear_for_ppo(hidden_states: torch.Tensor, vocab_weights: torch.Tenso
     ``keep_logits`` and on the model, never on the number of tokens or on whether gradients are recorded, so log-probs
     computed with and without gradients are bit-identical. None takes ``DEFAULT_KERNELS`` ("auto" unless
     ``VERL_AMD_LMHEAD_KERNELS`` says otherwise).
+
+    ``forward_splits`` pins the number of vocabulary ranges of that forward (1..64; None: planned per call, 8 for every
+    call of 8192 tokens or more, ``DEFAULT_FORWARD_SPLITS`` / ``VERL_AMD_LMHEAD_SPLITS`` override). Calls with the same
+    number of ranges give a token the same bits whatever else is in the call; a trainer whose micro-batches can be
+    smaller than 8192 tokens and that wants old and new log-probs of unchanged weights to be bit-identical pins it.
     """
     kernels = DEFAULT_KERNELS if kernels is None else kernels
     if kernels not in ("auto", "library", "mfma"):
         raise ValueError(f"kernels must be 'auto', 'library' or 'mfma', got {kernels!r}")
+    forward_splits = DEFAULT_FORWARD_SPLITS if forward_splits is None else forward_splits
+    if forward_splits is not None and not 1 <= int(forward_splits) <= 64:
+        raise ValueError(f"forward_splits must be in 1..64, got {forward_splits}")
     if not hidden_states.is_cuda or not vocab_weights.is_cuda:
         raise RuntimeError("fused_linear_for_ppo: tensors must be on the GPU; verl_amd has no CPU implementation")
     if hidden_states.dtype != vocab_weights.dtype or hidden_states.dtype not in _DTYPE_CODES:
@@ -319,10 +337,10 @@ def fused_linear_for_ppo(hidden_states: torch.Tensor, vocab_weights: torch.Tenso
         temp = None if float(temperature) == 1.0 else torch.full((h2.shape[0],), float(temperature), dtype=torch.float32,
                                                                   device=h2.device)
         with torch.no_grad():
-            lp, ent, _ = _own_forward(h2, w2, ids, temp, None, "fused_linear_for_ppo")
+            lp, ent, _ = _own_forward(h2, w2, ids, temp, forward_splits, "fused_linear_for_ppo")
         return lp.reshape(lead), ent.reshape(lead)
     lp, ent = _FusedLinearForPPOFunction.apply(h2, w2, ids, float(temperature), int(chunk_size), bool(keep_logits),
-                                               kernels)
+                                               kernels, None if forward_splits is None else int(forward_splits))
     return lp.reshape(lead), ent.reshape(lead)
 
 
@@ -347,7 +365,7 @@ def _own_forward(h, w, ids, temp, n_splits, what):
             tp[:T] = temp
         h, ids, temp = hp, ip, tp
     lib = _lib.load()
-    splits = lib.vrl_lmhead_plan(n, V) if n_splits is None else int(n_splits)
+    splits = lib.vrl_lmhead_plan(n, V) if n_splits is None else min(int(n_splits), (V + 255) // 256)
     partials = torch.empty(n * splits * 4, **f32)
     lp = torch.empty(n, **f32)
     ent = torch.empty(n, **f32)
@@ -434,12 +452,14 @@ def linear_cross_entropy(hidden: torch.Tensor, weight: torch.Tensor, labels: tor
 class FusedLinearForPPO(torch.nn.Module):
     """Module form, constructed and called like verl's (verl/utils/experimental/torch_functional.py:211-231)."""
 
-    def __init__(self, chunk_size: int = DEFAULT_CHUNK_TOKENS, keep_logits: bool = False, kernels: Optional[str] = None):
+    def __init__(self, chunk_size: int = DEFAULT_CHUNK_TOKENS, keep_logits: bool = False, kernels: Optional[str] = None,
+                 forward_splits: Optional[int] = None):
         super().__init__()
         self.chunk_size = chunk_size
         self.keep_logits = keep_logits
         self.kernels = kernels
+        self.forward_splits = forward_splits
 
     def forward(self, hidden_states, vocab_weights, input_ids, temperature: float = 1.0):
         return fused_linear_for_ppo(hidden_states, vocab_weights, input_ids, temperature, self.chunk_size,
-                                    self.keep_logits, self.kernels)
+                                    self.keep_logits, self.kernels, self.forward_splits)
