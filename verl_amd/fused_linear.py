@@ -46,11 +46,14 @@ DEFAULT_CHUNK_TOKENS = 4096
 #              (grad) log-probs of the same weights are bit-identical when both calls cut the vocabulary alike (see
 #              DEFAULT_FORWARD_SPLITS) and a few ulps apart otherwise; the backward forms the logits again and writes
 #              their gradient from registers (vrl_lmhead_dlogits, 3.46 ms per 4096 tokens against 3.53 ms for the library
-#              GEMM + row backward) and forms d hidden and d W with vrl_gemm (3.25 against 3.73 ms, and 3.62 / 3.85 ms
-#              storing / accumulating against 3.80 / 4.04 ms for the library on the same box), which reads W, the hidden
-#              states and the gradient buffer in place: the contraction of either product runs over rows of its operands,
-#              and the kernel takes such operands through transposing LDS reads. keep_logits=True needs the logits
-#              in memory and therefore takes the library forward, also without gradients.
+#              GEMM + row backward) and forms d hidden and d W with vrl_gemm, which reads W, the hidden states and the
+#              gradient buffer in place: the contraction of either product runs over rows of its operands, and the kernel
+#              takes such operands through transposing LDS reads. Per 4096-token chunk d hidden takes 3.4 ms against 3.8 ms
+#              for the library (which also wants a transposed copy of W); d W 3.7 / 4.0 ms stored / accumulated against
+#              3.5 / 3.6 ms for the library on transposed copies: timed alone the library's d W is the faster one, within a
+#              step the two ways tie (the library's needs the copies and a zero fill of d W), so the path stays free of
+#              library calls. keep_logits=True needs the logits in memory and therefore takes the library forward, also
+#              without gradients, and the library's single d W product over all tokens.
 # The environment variable and the ``kernels`` argument select; models the kernels do not take (fp32, a hidden size that is
 # not a multiple of 64, fewer than 256 vocabulary entries) go to the library.
 DEFAULT_KERNELS = os.environ.get("VERL_AMD_LMHEAD_KERNELS", "auto")
