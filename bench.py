@@ -443,12 +443,17 @@ def bench_lm_head(args, dev):
                 raise SystemExit(f"bench: the {which} backward disagrees with the library path on {what} ({err})")
         del gb
     del ga
-    t_f = timed(fwd)
-    t_f_lib = timed(fwd_library)
-    t_fb = timed(fwd_bwd)
-    t_fb_lib = timed(fwd_bwd_library)
-    t_m = timed(fwd_mfma)
-    t_fb_m = timed(fwd_bwd_mfma)
+    # The part is power-managed and drifts by a few per cent within seconds: the paths that are compared are timed
+    # alternately, twice, and each keeps its better time.
+    def timed_pairwise(*fns):
+        best = [float("inf")] * len(fns)
+        for _ in range(2):
+            for i, fn in enumerate(fns):
+                best[i] = min(best[i], timed(fn))
+        return best
+
+    t_f, t_f_lib, t_m = timed_pairwise(fwd, fwd_library, fwd_mfma)
+    t_fb, t_fb_lib, t_fb_m = timed_pairwise(fwd_bwd, fwd_bwd_library, fwd_bwd_mfma)
     wt = torch.empty(D, V, dtype=weight.dtype, device=dev)
     t_tr = timed(lambda: transpose_2d(weight.detach(), wt))
     # the two products of the backward on one chunk's worth of tokens, own kernel against the library on operands laid
@@ -476,7 +481,7 @@ def bench_lm_head(args, dev):
         del G, Ht, d_h, d_w
     flops_f, flops_fb = 2.0 * T * D * V, 6.0 * T * D * V
     ceiling = mfma_ceiling(dev, args.steps)
-    print(json.dumps({
+    return {
         "metric": "tokens/sec of LM head + scoring, forward + backward, never holding more than one chunk of logits",
         "value": T / t_fb, "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": t_fb * 1e3, "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16",
@@ -511,7 +516,7 @@ def bench_lm_head(args, dev):
         "weight_transpose": {"ms": t_tr * 1e3, "gbps": 2.0 * V * D * 2 / t_tr / 1e9, "kernel": "transpose_kernel<2>",
                              "note": "the copy the all-library backward makes once per call; the default path needs none"},
         "parity_guard": {"rows": 256, "max_abs_err_logprob": e1, "max_abs_err_entropy": e2},
-    }), flush=True)
+    }
 
 
 def cpu_baseline(step: Step, budget_s: float = 12.0, runs: int = 4):
@@ -929,7 +934,7 @@ def main():
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
     if args.lm_head:
-        bench_lm_head(args, dev)
+        print(json.dumps(bench_lm_head(args, dev)), flush=True)
         return
     if args.ceilings:
         bench_ceilings(args, dev)
@@ -966,6 +971,16 @@ def main():
     others.append(compact(bench_backward(few, dev, "c3")))
     torch.cuda.empty_cache()
     others.append(compact(bench_score_responses(few, dev, few.steps, few.warmup)))
+    # the LM head fused with the scoring (matrix-core bound, its own roofline): the short form of `--lm-head`
+    torch.cuda.empty_cache()
+    lm = argparse.Namespace(**vars(args))
+    lm.steps, lm.warmup = min(args.steps, 5), min(args.warmup, 2)
+    rec = bench_lm_head(lm, dev)
+    short = compact(rec)
+    short.update({k: rec[k] for k in ("forward_ms", "all_library", "backward_products")})
+    short["single_kernel_forward"] = {k: rec["single_kernel_forward"][k] for k in ("ms", "tflops", "frac_of_mfma_peak",
+                                                                                 "frac_of_sustained_mfma_rate")}
+    others.append(short)
     out["workloads"] = others
     print(json.dumps(out), flush=True)
 
