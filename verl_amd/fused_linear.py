@@ -39,9 +39,9 @@ DEFAULT_CHUNK_TOKENS = 4096
 
 # Which matrix products are this package's own kernels.
 #   "library": every product is torch.matmul (hipBLASLt); the row kernels run over the chunk buffer.
-#   "auto" (default) and "mfma" (the same today): every step that has a hand-written matrix-core kernel which is at least
-#              as fast as the library uses it. The forward is one kernel that never writes logits (vrl_lmhead_score: as fast
-#              as the library GEMM + row kernel at 8192 x 3584 -> 152064 bf16, 6.5 ms, no (chunk, vocab) buffer, logits kept
+#   "auto" (default) and "mfma" (the same today): every step runs this package's own matrix-core kernel.
+#              The forward is one kernel that never writes logits (vrl_lmhead_score: within 1-3 % of
+#              the library GEMM + row kernel at 8192 x 3584 -> 152064 bf16, 6.5-6.8 ms, no (chunk, vocab) buffer, logits kept
 #              in fp32), with and without gradients and whatever the number of tokens, so that old (no-grad) and new
 #              (grad) log-probs of the same weights are bit-identical when both calls cut the vocabulary alike (see
 #              DEFAULT_FORWARD_SPLITS) and a few ulps apart otherwise; the backward forms the logits again and writes
@@ -295,7 +295,7 @@ def fused_linear_for_ppo(hidden_states: torch.Tensor, vocab_weights: torch.Tenso
     projecting again and forms ``d hidden`` and ``d W`` with one product each. Such a graph can be differentiated once.
 
     ``kernels`` chooses which matrix products are this package's own kernels: ``"library"`` (none: torch.matmul
-    throughout) or ``"auto"`` / ``"mfma"`` (all that are at least as fast: a forward that is one kernel and never
+    throughout) or ``"auto"`` / ``"mfma"`` (all of them: a forward that is one kernel and never
     writes logits, a backward that forms the logits again, writes their gradient straight from registers and forms
     ``d hidden`` and ``d W`` with ``vrl_gemm``: no library GEMM is called). Which forward runs depends on this option, on
     ``keep_logits`` and on the model, never on the number of tokens or on whether gradients are recorded, so log-probs
