@@ -4,12 +4,15 @@
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c2|c3|c4|c1|c5]
     python bench.py --backward [--workload ...]          (the row op's backward kernel)
     python bench.py --lm-head [--chunk N] [--keep-logits]  (LM head + scoring without the full logits)
+    python bench.py --score-responses                     (packed logits -> (B, T) blocks in one launch, and its backward)
+    python bench.py --ceilings                            (plain read / copy of the same buffers, matrix-core probe)
 
 One step = one pass of vrl_fused_score_verify (row kernel + verify kernel, through
 the C ABI, outputs preallocated) over the whole synthetic batch, logits resident
 in HBM. Prints one JSON line: whole-job verified tokens/s, the HBM roofline of
 the row kernel (algorithmic bytes / average kernel time from HIP events on the
 launch stream), and the same computation in torch on the host cores (bounded sample).
+With no workload option the line also carries short records of every other workload under "workloads".
 """
 
 from __future__ import annotations
