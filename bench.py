@@ -913,6 +913,9 @@ def main():
     ap.add_argument("--seqs", type=int, default=0, help="... with another number of sequences")
     ap.add_argument("--dtype", choices=["bf16", "f32"], default=None, help="... with another logits element type")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-lm-head", action="store_true",
+                    help="default run: leave out the short LM-head record (its library path launches the row kernels too, "
+                         "which mixes their averages in a kernel trace)")
     ap.add_argument("--backward", action="store_true",
                     help="time vrl_rowscore_backward on the workload instead of the fused forward step")
     ap.add_argument("--score-responses", action="store_true",
@@ -975,15 +978,16 @@ def main():
     torch.cuda.empty_cache()
     others.append(compact(bench_score_responses(few, dev, few.steps, few.warmup)))
     # the LM head fused with the scoring (matrix-core bound, its own roofline): the short form of `--lm-head`
-    torch.cuda.empty_cache()
-    lm = argparse.Namespace(**vars(args))
-    lm.steps, lm.warmup = min(args.steps, 5), min(args.warmup, 2)
-    rec = bench_lm_head(lm, dev)
-    short = compact(rec)
-    short.update({k: rec[k] for k in ("forward_ms", "all_library", "backward_products")})
-    short["single_kernel_forward"] = {k: rec["single_kernel_forward"][k] for k in ("ms", "tflops", "frac_of_mfma_peak",
-                                                                                 "frac_of_sustained_mfma_rate")}
-    others.append(short)
+    if not args.no_lm_head:
+        torch.cuda.empty_cache()
+        lm = argparse.Namespace(**vars(args))
+        lm.steps, lm.warmup = min(args.steps, 5), min(args.warmup, 2)
+        rec = bench_lm_head(lm, dev)
+        short = compact(rec)
+        short.update({k: rec[k] for k in ("forward_ms", "all_library", "backward_products")})
+        short["single_kernel_forward"] = {k: rec["single_kernel_forward"][k] for k in ("ms", "tflops", "frac_of_mfma_peak",
+                                                                                     "frac_of_sustained_mfma_rate")}
+        others.append(short)
     out["workloads"] = others
     print(json.dumps(out), flush=True)
 
