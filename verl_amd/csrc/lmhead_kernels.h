@@ -125,14 +125,20 @@ __device__ __forceinline__ LmWork lm_work(int64_t V, int64_t T, int n_splits, in
 // an H fragment is dead after its 4 products and a W fragment after the last column, and each is refilled in place with
 // the next half's as soon as it is dead - the second half's from this step's tiles during the first half, the next
 // step's first half from the next tiles during the second. During step s:
-//   first half    requests W(s+2) into the slot H(s-1) left (four loads per wavefront)
+//   first half    requests W(s+2) into the slot H(s-1) left (eight loads per loading wavefront)
 //   barrier       the step's only one: every wavefront holds the second half's fragments, so W(s) and H(s) are dead,
-//                 and W(s+1), H(s+1) have landed (vmcnt(4): only the four W(s+2) loads may still be in flight)
+//                 and W(s+1), H(s+1) have landed (vmcnt(8): only the eight W(s+2) loads may still be in flight)
 //   second half   requests H(s+2) into the slot W(s) left
 // so the 64 loads a step needs are spread over it instead of arriving at the address unit in one burst, and the W tile
 // (the operand that comes from HBM) has a step and a half to land. Every matrix instruction is followed by at most one
 // fragment read and one load; the scheduling-group barriers pin that interleave (left alone, the compiler gathers the
 // reads in front of the barrier, where all eight wavefronts then wait for them together).
+// Only wavefronts 0-3 load (LOADER), one per SIMD: a load instruction holds its wavefront in issue for tens of cycles
+// while the address unit takes it, and when both wavefronts of a SIMD carry loads at the same places of the same
+// instruction stream they are held at the same time and the SIMD's matrix pipe idles. With one loading and one purely
+// computing wavefront per SIMD the pipe always has a wavefront to issue from: 6.11 against 6.49 ms for the forward at
+// 8192 x 3584 -> 152064 bf16 in one process, with the very same results. The two roles are two instantiations of the
+// walk, chosen by a wave-uniform branch, so each stays straight-line code.
 // EPILOGUE_STORES: on_tile writes to global memory. Stores count in vmcnt like loads but complete in their own order,
 // so the first barrier after on_tile waits for everything.
 //
@@ -142,10 +148,10 @@ __device__ __forceinline__ LmWork lm_work(int64_t V, int64_t T, int n_splits, in
 // In LDS the tile is [k>>3][16-row block][k&7 (^4 for odd k>>3)][16 rows]: a fragment is two transposing reads
 // (ds_read_b64_tr_b16: 16 lanes read 4 k x 16 rows and each receives the 4 k of its row), the 8 k-rows a half
 // wavefront reads fall on distinct banks, and the row block enters the address as a plain offset of 256 bytes.
-template <int DT, bool EPILOGUE_STORES, bool W_CM = false, bool H_CM = false, class OnTile>
-__device__ __forceinline__ void lm_walk_tiles(const uint16_t* __restrict__ W, const uint16_t* __restrict__ H, int64_t V,
-                                              int64_t K, int64_t w_stride, int64_t h_stride, const LmWork& work,
-                                              char* lds, OnTile&& on_tile) {
+template <int DT, bool EPILOGUE_STORES, bool W_CM, bool H_CM, bool LOADER, class OnTile>
+__device__ __forceinline__ void lm_walk_tiles_as(const uint16_t* __restrict__ W, const uint16_t* __restrict__ H, int64_t V,
+                                                 int64_t K, int64_t w_stride, int64_t h_stride, const LmWork& work,
+                                                 char* lds, OnTile&& on_tile) {
   using FragT = typename LmFrag<DT>::type;
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -154,6 +160,8 @@ __device__ __forceinline__ void lm_walk_tiles(const uint16_t* __restrict__ W, co
   const int wt = wave & 1;   // token half of the tile
   const int ksteps = (int)(K / kLmK);
 
+  // Loading wavefront p = wave & 3 brings rows [64p, 64p + 64) of a tile (contraction rows [16p, 16p + 16) of a
+  // contraction-major one) with eight instructions.
   // One wave instruction moves 8 tile rows x 128 bytes into LDS (lane l lands at byte l*16 of the 1 KiB block): lane l
   // serves row r = l>>3 of the block and physical 16-byte slot p = l&7, and fetches the logical chunk that the swizzle
   // assigns to that slot. Physical slot p of tile row R holds logical chunk p ^ ((R >> 1) & 7): 16 consecutive rows
@@ -162,27 +170,28 @@ __device__ __forceinline__ void lm_walk_tiles(const uint16_t* __restrict__ W, co
   const int lr = lane >> 3;
   const int lc_e = (lane & 7) ^ (lr >> 1), lc_o = (lane & 7) ^ (4 + (lr >> 1));
   // contraction-major: lane l lands in (block l>>4 of the instruction's four, k&7 slot (l&15)>>1, 16-byte half l&1) and
-  // fetches memory row (slot ^ 4*(wave&1)) of the wavefront's eight, bytes 32*(l>>4) + 16*(l&1) of the 128
-  const int cm_row = ((lane & 15) >> 1) ^ ((wave & 1) << 2);
+  // fetches memory row (slot, ^4 in an odd group of 8 contraction rows) of the group's eight, bytes 32*(l>>4) + 16*(l&1)
+  // of the 128. A loading wavefront's instructions 0-3 serve its even group, 4-7 its odd one.
+  const int cm_slot = (lane & 15) >> 1;
   const int cm_byte = (lane >> 4) * 32 + (lane & 1) * 16;
-  const uint32_t w_lane_e = W_CM ? (uint32_t)(cm_row * w_stride * 2 + cm_byte) : (uint32_t)((lr * w_stride + lc_e * 8) * 2);
-  const uint32_t w_lane_o = W_CM ? w_lane_e : (uint32_t)((lr * w_stride + lc_o * 8) * 2);
-  const uint32_t h_lane_e = H_CM ? (uint32_t)(cm_row * h_stride * 2 + cm_byte) : (uint32_t)((lr * h_stride + lc_e * 8) * 2);
-  const uint32_t h_lane_o = H_CM ? h_lane_e : (uint32_t)((lr * h_stride + lc_o * 8) * 2);
-  // bytes from one of a wavefront's four instructions to the next (8 rows / 64 rows of the tile further on), from one
-  // step to the next (64 contraction elements), and from tile row 0 to the wavefront's first memory row
-  const uint64_t w_blk = W_CM ? (uint64_t)128 : (uint64_t)(8 * w_stride * 2);
-  const uint64_t h_blk = H_CM ? (uint64_t)128 : (uint64_t)(8 * h_stride * 2);
+  const uint32_t w_lane_e = W_CM ? (uint32_t)(cm_slot * w_stride * 2 + cm_byte) : (uint32_t)((lr * w_stride + lc_e * 8) * 2);
+  const uint32_t w_lane_o = W_CM ? (uint32_t)((cm_slot ^ 4) * w_stride * 2 + cm_byte) : (uint32_t)((lr * w_stride + lc_o * 8) * 2);
+  const uint32_t h_lane_e = H_CM ? (uint32_t)(cm_slot * h_stride * 2 + cm_byte) : (uint32_t)((lr * h_stride + lc_e * 8) * 2);
+  const uint32_t h_lane_o = H_CM ? (uint32_t)((cm_slot ^ 4) * h_stride * 2 + cm_byte) : (uint32_t)((lr * h_stride + lc_o * 8) * 2);
+  // bytes of 8 memory rows, from one step to the next (64 contraction elements), and from tile row 0 to the
+  // wavefront's first memory row
+  const uint64_t w_blk = (uint64_t)(8 * w_stride * 2);
+  const uint64_t h_blk = (uint64_t)(8 * h_stride * 2);
   const uint64_t w_adv = W_CM ? (uint64_t)(kLmK * w_stride * 2) : (uint64_t)kLmRowBytes;
   const uint64_t h_adv = H_CM ? (uint64_t)(kLmK * h_stride * 2) : (uint64_t)kLmRowBytes;
   const uint64_t w_row = W_CM ? (uint64_t)2 : (uint64_t)(w_stride * 2);   // bytes per tile row
   const uint64_t h_row = H_CM ? (uint64_t)2 : (uint64_t)(h_stride * 2);
-  const uint64_t w_first = W_CM ? (uint64_t)(wave * 8 * w_stride * 2) : (uint64_t)wave * 4 * w_blk;
-  const uint64_t h_first = H_CM ? (uint64_t)(wave * 8 * h_stride * 2) : (uint64_t)wave * 4 * h_blk;
+  const int pw = wave & 3;
+  const uint64_t w_first = (uint64_t)pw * (W_CM ? 2 : 8) * w_blk;
+  const uint64_t h_first = (uint64_t)pw * (H_CM ? 2 : 8) * h_blk;
 
-  // Two load cursors, one per operand: uniform byte pointers to this wavefront's first row (it brings rows
-  // [32*wave, 32*wave + 32) of a tile, or contraction rows [8*wave, 8*wave + 8) of a contraction-major one, with four
-  // instructions) of the W / H tile to request next, and the ring slot it goes to. A step advances a pointer by 64
+  // Two load cursors, one per operand: uniform byte pointers to this wavefront's first row of the W / H tile to
+  // request next, and the ring slot it goes to. A step advances a pointer by 64
   // contraction elements; at the end of a vocabulary tile W jumps to the next tile's rows and H returns to k = 0. Past
   // the last step the pointers stay put: the last tiles are requested again into slots nobody reads any more (in
   // bounds, harmless), so the main loop needs no "is there more" branch around its loads.
@@ -198,15 +207,19 @@ __device__ __forceinline__ void lm_walk_tiles(const uint16_t* __restrict__ W, co
   int64_t w_step = 0, w_vt = work.vt_begin, h_step = 0;
   int w_ks = 0, h_ks = 0;
   int w_slot = 0, h_slot = 1;
-  const int wave_rows = wave * 32 * kLmRowBytes;
+  const int wave_rows = pw * 64 * kLmRowBytes;
+  // instruction i of eight: rows 8i .. 8i+7 of the wavefront's 64; contraction-major: group i>>2 of its two groups of
+  // 8 contraction rows, rows 64*(i&3) .. +63 of the tile (128 bytes of each memory row)
   auto load_w = [&](int i) {
-    const char* src = reinterpret_cast<const char*>(wp + i * w_blk);
-    __builtin_amdgcn_global_load_lds((const VRL_GLOBAL_AS void*)(src + ((i & 1) ? w_lane_o : w_lane_e)),
+    const char* src = reinterpret_cast<const char*>(wp + (W_CM ? (i >> 2) * w_blk + (i & 3) * 128 : i * w_blk));
+    const bool odd = W_CM ? ((i >> 2) & 1) : (i & 1);
+    __builtin_amdgcn_global_load_lds((const VRL_GLOBAL_AS void*)(src + (odd ? w_lane_o : w_lane_e)),
                                      (VRL_LDS_AS void*)(lds + w_slot * kLmTileBytes + wave_rows + i * 8 * kLmRowBytes), 16, 0, 0);
   };
   auto load_h = [&](int i) {
-    const char* src = reinterpret_cast<const char*>(hp + i * h_blk);
-    __builtin_amdgcn_global_load_lds((const VRL_GLOBAL_AS void*)(src + ((i & 1) ? h_lane_o : h_lane_e)),
+    const char* src = reinterpret_cast<const char*>(hp + (H_CM ? (i >> 2) * h_blk + (i & 3) * 128 : i * h_blk));
+    const bool odd = H_CM ? ((i >> 2) & 1) : (i & 1);
+    __builtin_amdgcn_global_load_lds((const VRL_GLOBAL_AS void*)(src + (odd ? h_lane_o : h_lane_e)),
                                      (VRL_LDS_AS void*)(lds + h_slot * kLmTileBytes + wave_rows + i * 8 * kLmRowBytes), 16, 0, 0);
   };
   auto next_slot = [](int slot) { return slot + 2 >= kLmRingSlots ? slot + 2 - kLmRingSlots : slot + 2; };
@@ -276,14 +289,18 @@ __device__ __forceinline__ void lm_walk_tiles(const uint16_t* __restrict__ W, co
   if (total_steps > 0) {
 #pragma unroll
     for (int rep = 0; rep < 2; ++rep) {
+      if constexpr (LOADER) {
 #pragma unroll
-      for (int i = 0; i < 4; ++i) load_w(i);
+        for (int i = 0; i < 8; ++i) load_w(i);
+      }
       advance_w();
+      if constexpr (LOADER) {
 #pragma unroll
-      for (int i = 0; i < 4; ++i) load_h(i);
+        for (int i = 0; i < 8; ++i) load_h(i);
+      }
       advance_h();
     }
-    asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
+    if constexpr (LOADER) asm volatile("s_waitcnt vmcnt(16)" ::: "memory");
     __builtin_amdgcn_s_barrier();
 #pragma unroll
     for (int i = 0; i < 4; ++i) a[i] = read_w(w_ptr(0, 0, 0), w_ptr(0, 0, 1), i);
@@ -315,8 +332,10 @@ __device__ __forceinline__ void lm_walk_tiles(const uint16_t* __restrict__ W, co
         if (hf == 1) {
           if (EPILOGUE_STORES && after_epilogue) {
             asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+          } else if (LOADER) {
+            asm volatile("s_waitcnt vmcnt(8) lgkmcnt(0)" ::: "memory");
           } else {
-            asm volatile("s_waitcnt vmcnt(4) lgkmcnt(0)" ::: "memory");
+            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
           }
           __builtin_amdgcn_s_barrier();
           after_epilogue = false;
@@ -331,8 +350,8 @@ __device__ __forceinline__ void lm_walk_tiles(const uint16_t* __restrict__ W, co
           acc[i][j] = LmFrag<DT>::mfma16(a[i], b[j], acc[i][j]);
           if (i == 3) b[j] = read_h(rh0, rh1, j);
           if (j == 7) a[i] = read_w(rw0, rw1, i);
-          if ((mm & 7) == 1) {
-            if (hf == 0) load_w(mm >> 3); else load_h(mm >> 3);
+          if (LOADER && (mm & 3) == 1) {
+            if (hf == 0) load_w(mm >> 2); else load_h(mm >> 2);
           }
         }
 #pragma unroll
@@ -340,7 +359,7 @@ __device__ __forceinline__ void lm_walk_tiles(const uint16_t* __restrict__ W, co
           __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                                // one matrix instruction
           if ((mm & 3) == 3) __builtin_amdgcn_sched_group_barrier(0x100, H_CM ? 2 : 1, 0);  // an H fragment
           if ((mm >> 2) == 7) __builtin_amdgcn_sched_group_barrier(0x100, W_CM ? 2 : 1, 0); // a W fragment
-          if ((mm & 7) == 1) __builtin_amdgcn_sched_group_barrier(0x010, 1, 0);             // one load
+          if (LOADER && (mm & 3) == 1) __builtin_amdgcn_sched_group_barrier(0x010, 1, 0);   // one load
         }
         __builtin_amdgcn_sched_barrier(0);
         if (hf == 0) advance_w(); else advance_h();
@@ -352,6 +371,17 @@ __device__ __forceinline__ void lm_walk_tiles(const uint16_t* __restrict__ W, co
     after_epilogue = true;
   }
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // the last, redundant loads still target the ring
+}
+
+template <int DT, bool EPILOGUE_STORES, bool W_CM = false, bool H_CM = false, class OnTile>
+__device__ __forceinline__ void lm_walk_tiles(const uint16_t* __restrict__ W, const uint16_t* __restrict__ H, int64_t V,
+                                              int64_t K, int64_t w_stride, int64_t h_stride, const LmWork& work,
+                                              char* lds, OnTile&& on_tile) {
+  const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+  if (wave < 4)
+    lm_walk_tiles_as<DT, EPILOGUE_STORES, W_CM, H_CM, true>(W, H, V, K, w_stride, h_stride, work, lds, on_tile);
+  else
+    lm_walk_tiles_as<DT, EPILOGUE_STORES, W_CM, H_CM, false>(W, H, V, K, w_stride, h_stride, work, lds, on_tile);
 }
 
 // grid.x = token blocks * n_splits, block = 512, dynamic LDS = kLmLdsBytes. Writes, per (token, split), the online-softmax
