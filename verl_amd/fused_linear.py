@@ -40,19 +40,17 @@ DEFAULT_CHUNK_TOKENS = 4096
 # Which matrix products are this package's own kernels.
 #   "library": every product is torch.matmul (hipBLASLt); the row kernels run over the chunk buffer.
 #   "auto" (default) and "mfma" (the same today): every step runs this package's own matrix-core kernel.
-#              The forward is one kernel that never writes logits (vrl_lmhead_score: within 1-3 % of
-#              the library GEMM + row kernel at 8192 x 3584 -> 152064 bf16, 6.5-6.8 ms, no (chunk, vocab) buffer, logits kept
+#              The forward is one kernel that never writes logits (vrl_lmhead_score: 6.1-6.25 ms at 8192 x 3584 ->
+#              152064 bf16 against 6.5 ms for the library GEMM + row kernel, no (chunk, vocab) buffer, logits kept
 #              in fp32), with and without gradients and whatever the number of tokens, so that old (no-grad) and new
 #              (grad) log-probs of the same weights are bit-identical when both calls cut the vocabulary alike (see
 #              DEFAULT_FORWARD_SPLITS) and a few ulps apart otherwise; the backward forms the logits again and writes
-#              their gradient from registers (vrl_lmhead_dlogits, 3.46 ms per 4096 tokens against 3.53 ms for the library
+#              their gradient from registers (vrl_lmhead_dlogits, 3.33 ms per 4096 tokens against 3.53 ms for the library
 #              GEMM + row backward) and forms d hidden and d W with vrl_gemm, which reads W, the hidden states and the
 #              gradient buffer in place: the contraction of either product runs over rows of its operands, and the kernel
-#              takes such operands through transposing LDS reads. Per 4096-token chunk d hidden takes 3.4 ms against 3.8 ms
-#              for the library (which also wants a transposed copy of W); d W 3.7 / 4.0 ms stored / accumulated against
-#              3.5 / 3.6 ms for the library on transposed copies: timed alone the library's d W is the faster one, within a
-#              step the two ways tie (the library's needs the copies and a zero fill of d W), so the path stays free of
-#              library calls. keep_logits=True needs the logits in memory and therefore takes the library forward, also
+#              takes such operands through transposing LDS reads. Per 4096-token chunk d hidden takes 3.3 ms against 3.75 ms
+#              for the library (which also wants a transposed copy of W); d W 3.44 / 3.7 ms stored / accumulated against
+#              3.4 / 3.5 ms for the library on transposed copies (which also needs the copies and a zero fill of d W). keep_logits=True needs the logits in memory and therefore takes the library forward, also
 #              without gradients, and the library's single d W product over all tokens.
 # The environment variable and the ``kernels`` argument select; models the kernels do not take (fp32, a hidden size that is
 # not a multiple of 64, fewer than 256 vocabulary entries) go to the library.
