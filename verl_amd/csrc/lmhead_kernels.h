@@ -148,7 +148,8 @@ __device__ __forceinline__ LmWork lm_work(int64_t V, int64_t T, int n_splits, in
 // In LDS the tile is [k>>3][16-row block][k&7 (^4 for odd k>>3)][16 rows]: a fragment is two transposing reads
 // (ds_read_b64_tr_b16: 16 lanes read 4 k x 16 rows and each receives the 4 k of its row), the 8 k-rows a half
 // wavefront reads fall on distinct banks, and the row block enters the address as a plain offset of 256 bytes.
-template <int DT, bool EPILOGUE_STORES, bool W_CM, bool H_CM, int LOAD_GROUP, int LOAD_PHASE, bool LOADER, class OnTile>
+template <int DT, bool EPILOGUE_STORES, bool W_CM, bool H_CM, int LOAD_GROUP, int LOAD_PHASE, int H_DELAY, bool LOADER,
+          class OnTile>
 __device__ __forceinline__ void lm_walk_tiles_as(const uint16_t* __restrict__ W, const uint16_t* __restrict__ H, int64_t V,
                                                  int64_t K, int64_t w_stride, int64_t h_stride, const LmWork& work,
                                                  char* lds, OnTile&& on_tile) {
@@ -285,6 +286,7 @@ __device__ __forceinline__ void lm_walk_tiles_as(const uint16_t* __restrict__ W,
     return lds + slot * kLmTileBytes + fragoff_h + (H_CM ? cm_q[q] + hf * kCmHalf : phys[hf]);
   };
 
+  constexpr int HD = LOADER ? H_DELAY : 0;   // a loading wavefront refills an H fragment this many instructions later
   FragT a[4], b[8];
   if (total_steps > 0) {
 #pragma unroll
@@ -348,7 +350,11 @@ __device__ __forceinline__ void lm_walk_tiles_as(const uint16_t* __restrict__ W,
         for (int mm = 0; mm < 32; ++mm) {
           const int j = mm >> 2, i = mm & 3;
           acc[i][j] = LmFrag<DT>::mfma16(a[i], b[j], acc[i][j]);
-          if (i == 3) b[j] = read_h(rh0, rh1, j);
+#pragma unroll
+          for (int jj = 0; jj < 8; ++jj) {
+            const int at = 4 * jj + 3 + HD < 31 ? 4 * jj + 3 + HD : 31;
+            if (at == mm) b[jj] = read_h(rh0, rh1, jj);
+          }
           if (j == 7) a[i] = read_w(rw0, rw1, i);
           if (LOADER && ((mm + 1 + LOAD_PHASE) % (4 * LOAD_GROUP)) == 0) {
 #pragma unroll
@@ -361,7 +367,11 @@ __device__ __forceinline__ void lm_walk_tiles_as(const uint16_t* __restrict__ W,
 #pragma unroll
         for (int mm = 0; mm < 32; ++mm) {
           __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                                // one matrix instruction
-          if ((mm & 3) == 3) __builtin_amdgcn_sched_group_barrier(0x100, H_CM ? 2 : 1, 0);  // an H fragment
+#pragma unroll
+          for (int jj = 0; jj < 8; ++jj) {
+            const int at = 4 * jj + 3 + HD < 31 ? 4 * jj + 3 + HD : 31;
+            if (at == mm) __builtin_amdgcn_sched_group_barrier(0x100, H_CM ? 2 : 1, 0);  // an H fragment
+          }
           if ((mm >> 2) == 7) __builtin_amdgcn_sched_group_barrier(0x100, W_CM ? 2 : 1, 0); // a W fragment
           if (LOADER && ((mm + 1 + LOAD_PHASE) % (4 * LOAD_GROUP)) == 0) __builtin_amdgcn_sched_group_barrier(0x010, LOAD_GROUP, 0);
         }
@@ -381,18 +391,20 @@ __device__ __forceinline__ void lm_walk_tiles_as(const uint16_t* __restrict__ W,
 // behind every 4 * LOAD_GROUP matrix instructions, LOAD_PHASE instructions before the end of such a run (0 = behind the
 // last product of a column, where the H fragment is refilled too). The kernels differ by 1-3 % in which placement suits
 // them (a sweep per kernel at 8192 / 4096 x 3584 <-> 152064 bf16): the forward takes pairs at phase 0, the two products
-// single loads one instruction earlier, the gradient kernel single loads three instructions earlier.
-template <int DT, bool EPILOGUE_STORES, bool W_CM, bool H_CM, int LOAD_GROUP, int LOAD_PHASE, class OnTile>
+// single loads one instruction earlier, the gradient kernel single loads three instructions earlier. H_DELAY moves the
+// loading wavefronts' refills of the H fragments that many instructions back, away from the computing wavefronts' (which
+// stay right behind a column's last product): worth 3 % to the d hidden product, nothing or less to the others.
+template <int DT, bool EPILOGUE_STORES, bool W_CM, bool H_CM, int LOAD_GROUP, int LOAD_PHASE, int H_DELAY, class OnTile>
 __device__ __forceinline__ void lm_walk_tiles(const uint16_t* __restrict__ W, const uint16_t* __restrict__ H, int64_t V,
                                               int64_t K, int64_t w_stride, int64_t h_stride, const LmWork& work,
                                               char* lds, OnTile&& on_tile) {
   const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
   if (wave < 4)
-    lm_walk_tiles_as<DT, EPILOGUE_STORES, W_CM, H_CM, LOAD_GROUP, LOAD_PHASE, true>(W, H, V, K, w_stride, h_stride, work,
-                                                                                 lds, on_tile);
+    lm_walk_tiles_as<DT, EPILOGUE_STORES, W_CM, H_CM, LOAD_GROUP, LOAD_PHASE, H_DELAY, true>(W, H, V, K, w_stride, h_stride,
+                                                                                          work, lds, on_tile);
   else
-    lm_walk_tiles_as<DT, EPILOGUE_STORES, W_CM, H_CM, LOAD_GROUP, LOAD_PHASE, false>(W, H, V, K, w_stride, h_stride, work,
-                                                                                  lds, on_tile);
+    lm_walk_tiles_as<DT, EPILOGUE_STORES, W_CM, H_CM, LOAD_GROUP, LOAD_PHASE, H_DELAY, false>(W, H, V, K, w_stride, h_stride,
+                                                                                           work, lds, on_tile);
 }
 
 // grid.x = token blocks * n_splits, block = 512, dynamic LDS = kLmLdsBytes. Writes, per (token, split), the online-softmax
@@ -423,7 +435,7 @@ __global__ __launch_bounds__(kLmWaves * 64, 1) void lmhead_partial_kernel(
     c[j] = make_scale<false>(temperature, tok).c;   // log2(e) / max(T, 1e-8), exactly what the finishing kernel uses
   }
 
-  lm_walk_tiles<DT, false, false, false, 2, 0>(W, H, V, K, w_stride, h_stride, work, lds, [&](int64_t vt, lm_f32x4 (&acc)[4][8]) {
+  lm_walk_tiles<DT, false, false, false, 2, 0, 0>(W, H, V, K, w_stride, h_stride, work, lds, [&](int64_t vt, lm_f32x4 (&acc)[4][8]) {
     // fold 16 logits per token column into the running state (maximum first, then the exponentials; nothing is
     // buffered): acc[i][j][v] is vocabulary row tile_row0 + wv*64 + i*16 + 4*(lane>>4) + v of token column j
     const bool edge = (vt + 1) * kLmVocab > V;
@@ -575,7 +587,7 @@ __global__ __launch_bounds__(kLmWaves * 64, 1) void lmhead_dlogits_kernel(
     label[j] = (lab >= 0 && lab < V) ? (int)lab : -1;   // an out-of-range label was reported by the forward pass
   }
 
-  lm_walk_tiles<DT, true, false, false, 1, 3>(W, H, V, K, w_stride, h_stride, work, lds, [&](int64_t vt, lm_f32x4 (&acc)[4][8]) {
+  lm_walk_tiles<DT, true, false, false, 1, 3, 0>(W, H, V, K, w_stride, h_stride, work, lds, [&](int64_t vt, lm_f32x4 (&acc)[4][8]) {
     // acc[i][j][0..3]: vocabulary entries vr .. vr+3, vr = tile_row0 + wv*64 + i*16 + 4*(lane>>4), of token column j
     const bool edge = (vt + 1) * kLmVocab > V;
     const int vrow0 = (int)(edge ? V - kLmVocab : vt * kLmVocab) + wv * 64 + 4 * (lane >> 4);
@@ -687,7 +699,7 @@ __global__ __launch_bounds__(kLmWaves * 64, 1) void lm_gemm_kernel(
 
   const uint16_t* x0 = X + step0 * kLmK * (X_CM ? x_stride : 1);
   const uint16_t* y0p = Y + step0 * kLmK * (Y_CM ? y_stride : 1);
-  lm_walk_tiles<DT, true, X_CM, Y_CM, 1, 1>(x0, y0p, g.NX, nsteps * kLmK, x_stride, y_stride, work, lds,
+  lm_walk_tiles<DT, true, X_CM, Y_CM, 1, 1, (X_CM && !Y_CM) ? 1 : 0>(x0, y0p, g.NX, nsteps * kLmK, x_stride, y_stride, work, lds,
                                       [&](int64_t vt, lm_f32x4 (&acc)[4][8]) {
     // acc[i][j][0..3]: columns x0 .. x0+3 of out, x0 = tile_row0 + wv*64 + i*16 + 4*(lane>>4), of row
     // y = tok0_ld + wt*128 + j*16 + (lane&15)
