@@ -9,7 +9,8 @@
 // cover the other's waits. Operands go global -> LDS directly (128-bit loads) into a ring of five 32 KiB operand tiles
 // (all 160 KiB of a CU's LDS, one workgroup per CU), swizzled so that the 128-bit fragment reads are free of bank
 // conflicts (measured: SQ_LDS_BANK_CONFLICT = 0). A step is two halves of 32 contraction elements with one workgroup
-// barrier between them; the loads of the tiles two steps ahead are spread over the step (lm_walk_tiles).
+// barrier between them; the loads of the tiles two steps ahead are spread over the step and issued by one wavefront of
+// each SIMD only, so that its partner always has matrix instructions to issue (lm_walk_tiles).
 // The MFMA is issued with the vocabulary on its row side so that a lane's 4 results of a block are 4 consecutive
 // vocabulary entries of ONE token: the softmax state needs no cross-lane traffic until the very end, and a gradient
 // or product block is one 8-byte store.
