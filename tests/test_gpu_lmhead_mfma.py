@@ -324,6 +324,70 @@ def test_token_results_do_not_depend_on_the_call_when_the_vocabulary_is_cut_alik
         fused_linear_for_ppo(h[:256], w, ids[:256], 0.9, forward_splits=65)
 
 
+def test_matrix_core_entry_points_replay_from_a_graph(dev):
+    """vrl_lmhead_score, vrl_lmhead_dlogits and vrl_gemm (d hidden stored, d W accumulated) only enqueue kernels: captured
+    once into a graph and replayed three times with new inputs in the same buffers, every replay equals the eager
+    result bit for bit."""
+    lib = _lib.load()
+    T, K, V = 512, 256, 1024
+    BF = _lib.VRL_BF16
+    gd = torch.Generator(device=dev).manual_seed(21)
+    h = torch.empty(T, K, dtype=torch.bfloat16, device=dev)
+    w = torch.empty(V, K, dtype=torch.bfloat16, device=dev)
+    ids = torch.empty(T, dtype=torch.int64, device=dev)
+    g_lp = torch.empty(T, device=dev)
+    g_ent = torch.empty(T, device=dev)
+    splits = lib.vrl_lmhead_plan(T, V)
+    partials = torch.empty(T * splits * 4, device=dev)
+    lp = torch.empty(T, device=dev); ent = torch.empty(T, device=dev); lse = torch.empty(T, device=dev)
+    flag = torch.zeros(1, dtype=torch.int32, device=dev)
+    G = torch.empty(T, V, dtype=torch.bfloat16, device=dev)
+    d_h = torch.empty(T, K, dtype=torch.bfloat16, device=dev)
+    d_w = torch.empty(V, K, dtype=torch.bfloat16, device=dev)
+    d_w0 = torch.empty(V, K, dtype=torch.bfloat16, device=dev)
+
+    def fill():
+        h.copy_(torch.empty(T, K, device=dev).uniform_(-0.5, 0.5, generator=gd))
+        w.copy_(torch.empty(V, K, device=dev).uniform_(-0.5, 0.5, generator=gd))
+        ids.copy_(torch.randint(0, V, (T,), generator=gd, device=dev))
+        g_lp.copy_(torch.empty(T, device=dev).uniform_(-1, 1, generator=gd))
+        g_ent.copy_(torch.empty(T, device=dev).uniform_(-0.5, 0.5, generator=gd))
+        d_w0.copy_(torch.empty(V, K, device=dev).uniform_(-1, 1, generator=gd))
+
+    def call(stream):
+        assert lib.vrl_lmhead_score(h.data_ptr(), w.data_ptr(), BF, T, V, K, K, K, ids.data_ptr(), None, splits,
+                                    partials.data_ptr(), lp.data_ptr(), ent.data_ptr(), lse.data_ptr(), flag.data_ptr(),
+                                    stream) == 0
+        assert lib.vrl_lmhead_dlogits(h.data_ptr(), w.data_ptr(), BF, T, V, K, K, K, ids.data_ptr(), None, lse.data_ptr(),
+                                      ent.data_ptr(), g_lp.data_ptr(), g_ent.data_ptr(), lib.vrl_lmhead_plan(T, V),
+                                      G.data_ptr(), V, stream) == 0
+        # d hidden = G . W (W contraction-major), d W = d W0 + G^T . H (both contraction-major, accumulated)
+        assert lib.vrl_gemm(w.data_ptr(), G.data_ptr(), BF, K, T, V, K, V, 1, 0, d_h.data_ptr(), K, 0, 1, None, stream) == 0
+        d_w.copy_(d_w0)
+        assert lib.vrl_gemm(h.data_ptr(), G.data_ptr(), BF, K, V, T, K, V, 1, 1, d_w.data_ptr(), K, 1, 1, None, stream) == 0
+
+    outs = (lp, ent, lse, G, d_h, d_w)
+    fill()
+    call(torch.cuda.current_stream(dev).cuda_stream)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        call(torch.cuda.current_stream(dev).cuda_stream)
+    for _ in range(3):
+        fill()
+        call(torch.cuda.current_stream(dev).cuda_stream)
+        torch.cuda.synchronize()
+        eager = [t.clone() for t in outs]
+        for t in outs:
+            t.fill_(float("nan"))
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        for a, b in zip(eager, outs):
+            assert torch.equal(a, b)
+        assert torch.isfinite(d_w.float()).all() and int(flag.item()) == 0
+
+
 def test_special_values_and_errors(dev):
     g = torch.Generator(device=dev).manual_seed(6)
     T, V, K = 256, 512, 64
