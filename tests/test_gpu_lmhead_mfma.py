@@ -239,6 +239,32 @@ def test_fused_linear_with_the_matrix_core_kernels(dev):
         fused_linear_for_ppo(hidden, weight, labels, 1.5, kernels="cublas")
 
 
+def test_fused_linear_fp16_model(dev):
+    """The same default path on an fp16 model (v_mfma_f32_16x16x32_f16): forward at the fp32 tolerance, gradients at the
+    reference's tolerances, two chunks with a padded tail."""
+    g = torch.Generator(device=dev).manual_seed(79)
+    T, D, V = 600, 256, 4096
+    hidden = torch.empty(T, D, device=dev).uniform_(-0.5, 0.5, generator=g).half().requires_grad_()
+    weight = torch.empty(V, D, device=dev).uniform_(-0.5, 0.5, generator=g).half().requires_grad_()
+    labels = torch.randint(0, V, (T,), generator=g, device=dev)
+    g_ent = torch.empty(T, device=dev).uniform_(-0.5, 0.5, generator=g)
+    g_lp = torch.empty(T, device=dev).uniform_(-1, 1, generator=g)
+    logits = torch.matmul(hidden.float(), weight.float().t()) / 0.7
+    ref_ent = torch.logsumexp(logits, -1) - (torch.softmax(logits, -1) * logits).sum(-1)
+    ref_lp = -torch.nn.functional.cross_entropy(logits, labels, reduction="none")
+    d_ref_h, d_ref_w = torch.autograd.grad((ref_ent, ref_lp), (hidden, weight), (g_ent, g_lp))
+    from verl_amd import gemm
+    before = gemm.counters["gemm"]
+    lp, ent = fused_linear_for_ppo(hidden, weight, labels, 0.7, chunk_size=256)
+    torch.testing.assert_close(ref_lp, lp, atol=1e-4, rtol=1e-4)
+    torch.testing.assert_close(ref_ent, ent, atol=1e-4, rtol=1e-4)
+    d_h, d_w = torch.autograd.grad((ent, lp), (hidden, weight), (g_ent, g_lp))
+    assert gemm.counters["gemm"] == before + 4          # chunks [0, 256) and [256, 600), two products each
+    assert d_h.dtype == torch.float16 and d_w.dtype == torch.float16
+    torch.testing.assert_close(d_ref_h.float(), d_h.float(), atol=2e-3, rtol=1e-2)
+    torch.testing.assert_close(d_ref_w.float(), d_w.float(), atol=2e-3, rtol=1e-2)
+
+
 def test_close_to_the_library_path_and_3d_inputs(dev):
     g = torch.Generator(device=dev).manual_seed(4)
     B, S, K, V = 2, 260, 256, 5008
