@@ -311,7 +311,9 @@ int vrl_gemm(const void* x, const void* y, int dtype, int64_t NX, int64_t NY, in
 int vrl_gemm_nt(const void* x, const void* y, int dtype, int64_t NX, int64_t NY, int64_t K, int64_t x_stride,
                 int64_t y_stride, void* out, int64_t out_stride, int accumulate, int k_parts, float* workspace,
                 void* stream);
-/* Vocabulary splits per 256-token block that fill the part (about one workgroup per CU) for this shape. */
+/* Vocabulary splits per 256-token block for this shape: enough to give every CU a workgroup, never fewer than 8 (so that
+ * every call of 8192 tokens or more cuts the vocabulary alike and gives a token the same bits whatever the call's size),
+ * at most 64 and at most one per 256-row vocabulary tile. */
 int vrl_lmhead_plan(int64_t n_tokens, int64_t vocab);
 
 /*
