@@ -282,48 +282,110 @@ def bench_backward(args, dev, workload=None):
     }
 
 
+VERIFY_RING_BYTES = 3 * (256 << 20)   # three times the 256 MB last-level cache
+
+
 class VerifyOnlyStep:
     """c5: 512 sequences with log-uniform lengths in [32, 16384], packed; only the verify kernel is timed
-    (its logits would be 408 GB, scored in 8192-token micro-batches like c3)."""
+    (its logits would be 408 GB, scored in 8192-token micro-batches like c3). One set of per-token arrays is 30 bytes
+    per token (44 MB), which the 256 MB last-level cache would hold from one launch to the next, so the launches walk a
+    ring of identical sets that is three times that cache: every launch finds its inputs in HBM."""
 
-    def __init__(self, w: synthetic.Workload, dev, seed: int):
+    def __init__(self, w: synthetic.Workload, dev, seed: int, two_pass=None, lengths=None):
         self.w, self.dev = w, dev
-        lengths = synthetic.draw_lengths(w, seed + 2)
+        lengths = synthetic.draw_lengths(w, seed + 2) if lengths is None else torch.tensor(lengths)
         self.cu = synthetic.pack_by_lengths(lengths).to(dev)
         self.B = lengths.numel()
         self.n = int(lengths.sum())
         self.n_valid = self.n
         self.layout = f"packed {self.B} sequences, {self.n} tokens (verify only)"
         g = torch.Generator(device=dev).manual_seed(seed + 1)
-        self.lp = -torch.rand(self.n, generator=g, device=dev) * 6
-        self.lp_old = synthetic.drift_old_logprobs(self.lp, w, seed).contiguous()
-        self.log_u = torch.log(torch.rand(self.n, generator=g, device=dev))
-        self.ids = torch.randint(0, w.V, (self.n,), generator=g, device=dev)
+        lp = -torch.rand(self.n, generator=g, device=dev) * 6
+        lp_old = synthetic.drift_old_logprobs(lp, w, seed).contiguous()
+        log_u = torch.log(torch.rand(self.n, generator=g, device=dev))
+        ids = torch.randint(0, w.V, (self.n,), generator=g, device=dev)
         self.off = sv.thresh_offset_from_lenience(w.lenience)
-        self.accept = torch.empty(self.n, dtype=torch.uint8, device=dev)
+        self.bytes_per_set = self.n * (4 + 4 + 4 + 8 + 1 + 8 + 1)
+        copies = min(32, max(2, -(-VERIFY_RING_BYTES // self.bytes_per_set)))
+        self.ring = []
+        for i in range(copies):
+            # (copies made by an elementwise kernel: a device-to-device memcpy does not survive counter collection)
+            src = (lp, lp_old, log_u, ids) if i == 0 else tuple(t.add(0) for t in (lp, lp_old, log_u, ids))
+            self.ring.append(src + (torch.empty(self.n, dtype=torch.uint8, device=dev), torch.empty_like(ids),
+                                    torch.empty(self.n, dtype=torch.uint8, device=dev)))
+        self.lp, self.lp_old, self.log_u, self.ids, self.accept, self.out_ids, self.out_mask = self.ring[0]
+        self.turn = 0
         self.first = torch.empty(self.B, dtype=torch.int32, device=dev)
         self.prefix = torch.empty(self.B, dtype=torch.int32, device=dev)
         self.near = torch.empty(self.B, dtype=torch.int32, device=dev)
-        self.out_ids = torch.empty_like(self.ids)
-        self.out_mask = torch.empty(self.n, dtype=torch.uint8, device=dev)
         self.flag = torch.zeros(1, dtype=torch.int32, device=dev)
         self.lib = _lib.load()
         self.stream = torch.cuda.current_stream(dev).cuda_stream
+        # the form the library plans for this shape: two flat passes with half a byte per token of scratch
+        self.two_pass = bool(self.lib.vrl_spec_verify_plan(1, self.B, 0, self.n)) if two_pass is None else bool(two_pass)
+        self.work = (torch.empty(int(self.lib.vrl_spec_verify_workspace(self.n)), dtype=torch.uint8, device=dev)
+                     if self.two_pass else None)
 
     def verify(self):
+        lp, lp_old, log_u, ids, accept, out_ids, out_mask = self.ring[self.turn]
+        self.turn = (self.turn + 1) % len(self.ring)
         st = self.lib.vrl_spec_verify(
-            self.lp.data_ptr(), self.lp_old.data_ptr(), self.log_u.data_ptr(), None, self.cu.data_ptr(), self.B, 0,
-            self.n, self.off, 1e-6, self.accept.data_ptr(), self.first.data_ptr(), self.prefix.data_ptr(),
-            self.near.data_ptr(), self.ids.data_ptr(), 0, self.out_ids.data_ptr(), self.out_mask.data_ptr(),
-            self.flag.data_ptr(), self.stream)
+            lp.data_ptr(), lp_old.data_ptr(), log_u.data_ptr(), None, self.cu.data_ptr(), self.B, 0,
+            self.n, self.off, 1e-6, accept.data_ptr(), self.first.data_ptr(), self.prefix.data_ptr(),
+            self.near.data_ptr(), ids.data_ptr(), 0, out_ids.data_ptr(), out_mask.data_ptr(),
+            self.flag.data_ptr(), None if self.work is None else self.work.data_ptr(),
+            0 if self.work is None else self.work.numel(), self.stream)
         _lib.check("vrl_spec_verify", st)
 
 
+# HBM bytes per call of the two verify kernels at c5 from rocprofv3 --pmc (FETCH_SIZE, WRITE_SIZE; same scaling as above),
+# profiles/verify_two_pass_kernels_c5_trace_and_hbm_counters.md: 17.63 + 2.23 MB (verify_tokens_kernel) and 1.24 + 13.13 MB
+# (verify_finish_kernel); the 0.73 MB of ballot words are written once and read once on top of the algorithmic bytes.
+MEASURED_VERIFY_TRAFFIC_BYTES = {"two-pass": 34229825}
+
+
+def batch_time_ms(fn, launches: int, batches: int = 5):
+    """Average time of one call of `fn` in ms: `launches` calls back to back between one pair of HIP events on the
+    launch stream, the median over `batches` such batches. For kernels of a few microseconds an event pair per launch
+    measures the events."""
+    times = []
+    for _ in range(batches):
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        a.record()
+        for _ in range(launches):
+            fn()
+        b.record()
+        torch.cuda.synchronize()
+        times.append(a.elapsed_time(b) / launches)
+    return statistics.median(times)
+
+
 def bench_verify_only(args, dev, with_cpu_baseline=True):
-    """tokens/s of vrl_spec_verify alone on the c5 workload; 4+4+4 in, 1 out per token, plus the truncated draft
-    (8 in, 8+1 out) = 30 B/token with the draft, 14 B/token (13 + per-sequence outputs) without."""
+    """tokens/s of vrl_spec_verify alone on the c5 workload. Algorithmic bytes per token: 4+4+4 in (new and old
+    log-probs, log u), 1 out (accept), and for the truncated draft 8+1 out = 22 B/token, plus 8 in for every token
+    before its sequence's cut (a draft id is only read where it is kept) and 20 B per sequence."""
     w = synthetic.WORKLOADS["c5"]
-    step = VerifyOnlyStep(w, dev, seed=5000)
+    def note(msg):
+        print(f"[bench c5] {msg}", file=sys.stderr, flush=True)
+
+    step = VerifyOnlyStep(w, dev, seed=5000, two_pass={"auto": None, "two-pass": True, "per-sequence": False}[args.verify_form])
+    note(f"{len(step.ring)} array sets built")
+    # guard: the first set's results against the vectorised statement of the rule, bit for bit
+    step.verify()
+    torch.cuda.synchronize()
+    from oracle import verify as overify  # checker / baseline only
+
+    if not args.no_guard:
+        ref = overify.verify(step.lp.cpu(), step.lp_old.cpu(), step.log_u.cpu(), None, step.off, cu_seqlens=step.cu.cpu(),
+                             draft_ids=step.ids.cpu())
+        same = (torch.equal(step.accept.cpu(), ref["accept"].to(torch.uint8)) and
+                torch.equal(step.first.cpu(), ref["first_reject"].to(torch.int32)) and
+                torch.equal(step.prefix.cpu(), ref["prefix_len"].to(torch.int32)) and
+                torch.equal(step.out_ids.cpu(), ref["out_ids"]) and
+                torch.equal(step.out_mask.cpu(), ref["out_mask"].to(torch.uint8)))
+        if not same or int(step.flag.item()) != 0:
+            raise SystemExit("bench: vrl_spec_verify disagrees with the oracle on c5")
+    note("guard done")
     spin_up(step.verify)
     for _ in range(args.warmup):
         step.verify()
@@ -333,28 +395,41 @@ def bench_verify_only(args, dev, with_cpu_baseline=True):
         step.verify()
     torch.cuda.synchronize()
     wall = time.perf_counter() - t0
-    evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(args.steps)]
-    for a, b in evs:
-        a.record()
-        step.verify()
-        b.record()
-    torch.cuda.synchronize()
-    avg_ms = sum(a.elapsed_time(b) for a, b in evs) / len(evs)
-    bytes_launch = step.n * (4 + 4 + 4 + 1 + 8 + 8 + 1) + step.B * (12 + 8)
+    launches = max(args.steps, len(step.ring) * 4)
+    avg_ms = batch_time_ms(step.verify, launches)
+    note("timed")
+    if args.copy_calibration:
+        copy_calibration(dev)
+        note("copy calibration done")
+    # what the same call costs when it moves next to nothing (8 packed sequences of 512 tokens): the launches themselves
+    tiny = VerifyOnlyStep(w.scaled(name="c5_tiny", B=8, T=512), dev, seed=5100, two_pass=step.two_pass, lengths=[512] * 8)
+    spin_up(tiny.verify, 30.0)
+    floor_ms = batch_time_ms(tiny.verify, launches)
+    kept = int(step.first.sum().item())   # no mask here: the tokens before a sequence's first rejection are the kept ones
+    bytes_launch = step.n * (4 + 4 + 4 + 1 + 8 + 1) + kept * 8 + step.B * (12 + 8)
     achieved = bytes_launch / (avg_ms * 1e-3) / 1e9
     out = {
         "metric": METRIC, "value": step.n * args.steps / wall, "unit": "tokens/s", "n_gpus": 1, "steps": args.steps,
         "warmup": args.warmup, "ms_per_step": wall * 1e3 / args.steps, "higher_is_better": True, "scaling": "weak",
         "vs_baseline": None, "dtype": "f32", "data": "synthetic",
         "config": {"workload": w.name, "layout": step.layout, "launches_per_step": 1, "tokens_per_step": step.n,
-                   "lenience": w.lenience, "step": "vrl_spec_verify with truncated draft, through the C ABI"},
+                   "lenience": w.lenience, "array_sets_rotated": len(step.ring),
+                   "launches_per_call": 2 if step.two_pass else 1,
+                   "step": "vrl_spec_verify with truncated draft, through the C ABI"},
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                     "frac": achieved / HBM_PEAK_GBPS, "traffic": None, "kernel": "spec_verify_kernel",
-                     "avg_kernel_ms": avg_ms, "algorithmic_bytes_per_launch": bytes_launch},
+                     "frac": achieved / HBM_PEAK_GBPS,
+                     "traffic": MEASURED_VERIFY_TRAFFIC_BYTES.get("two-pass" if step.two_pass else "per-sequence"),
+                     "kernel": "verify_tokens_kernel + verify_finish_kernel" if step.two_pass else "spec_verify_kernel",
+                     "avg_kernel_ms": avg_ms, "algorithmic_bytes_per_launch": bytes_launch,
+                     "timing": f"{launches} launches back to back between one HIP event pair, median of 5 batches",
+                     "launch_floor_ms": floor_ms,
+                     "achieved_net_of_launch_floor": bytes_launch / max((avg_ms - floor_ms) * 1e-3, 1e-9) / 1e9,
+                     "launch_floor": "the same call on 8 packed sequences of 512 tokens (0.1 MB): what the launches cost "
+                                     "before any byte moves"},
+        "parity_guard": "skipped (--no-guard)" if args.no_guard else
+                        "accept, first_reject, prefix_len and the truncated draft equal to the oracle, bit for bit",
     }
     if with_cpu_baseline:
-        from oracle import verify as overify  # baseline only
-
         ln, lo, lu, ids, cu = step.lp.cpu(), step.lp_old.cpu(), step.log_u.cpu(), step.ids.cpu(), step.cu.cpu()
         times = []
         for _ in range(3):
@@ -926,6 +1001,11 @@ def main():
     ap.add_argument("--keep-logits", action="store_true", help="--lm-head: keep the logits for the backward")
     ap.add_argument("--ceilings", action="store_true",
                     help="time plain non-temporal read / copy probes with the row kernels' access pattern")
+    ap.add_argument("--verify-form", choices=["auto", "two-pass", "per-sequence"], default="auto",
+                    help="--workload c5: which form of vrl_spec_verify to time (auto: what vrl_spec_verify_plan says)")
+    ap.add_argument("--no-guard", action="store_true",
+                    help="--workload c5: leave out the comparison with the oracle on the host (a counter-collecting "
+                         "profiler does not survive the large device-to-host copies it needs)")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run a plain device copy of known size (for scaling rocprofv3 byte counters)")
     args = ap.parse_args()

@@ -36,7 +36,7 @@
 extern "C" {
 #endif
 
-#define VRL_ABI_VERSION 2
+#define VRL_ABI_VERSION 3
 
 /* status codes */
 #define VRL_OK 0
@@ -354,8 +354,19 @@ int vrl_rollout_corr_num_stats(void);
  *   near_count[b]   = number of valid tokens with |d - tau| < near_eps
  * Optional truncated draft (all three or none): for positions >= first_reject
  *   out_ids = pad_id, out_mask = 0; below it they copy draft_ids / mask.
- * err_flag is required for the packed layout (VRL_FLAG_SEQ_RANGE; tokens that no
- * in-range span covers are not written) and may be NULL for the padded one.
+ * err_flag is required for the packed layout (VRL_FLAG_SEQ_RANGE) and may be NULL for the padded one.
+ *
+ * Two forms, chosen by `workspace`:
+ *   workspace == NULL (workspace_bytes 0): one launch, one workgroup per sequence. Right for batches of sequences of
+ *     similar, moderate length. Tokens that no in-range span covers are not written (packed layout, bad offsets).
+ *   workspace != NULL: two launches that walk the token arrays in tiles of 1024 tokens whatever sequence a token
+ *     belongs to, so that no CU is left with a long sequence's bytes (512 packed sequences of 32 ... 16384 tokens:
+ *     the per-sequence form takes as long as its longest sequences' CUs). What a sequence needs from its other tiles
+ *     travels through `workspace` as four bits per token: caller-owned device scratch of at least
+ *     vrl_spec_verify_workspace(n_tokens) bytes (0.5 bytes per token), 8-byte aligned, contents meaningless before
+ *     and after. accept is written for every token of the arrays. Same integers as the other form.
+ * vrl_spec_verify_plan returns 1 when the library would take the second form for a shape (packed != 0: cu_seqlens
+ * given), so a caller can size the scratch before the call; passing a workspace is what selects it.
  *
  * No function in the reference computes this (its recipe/ submodule is not
  * vendored: .gitmodules:1-3). Layout, mask and sign conventions follow
@@ -367,7 +378,10 @@ int vrl_spec_verify(const float* logp_new, const float* logp_old, const float* l
                     const uint8_t* mask, const int64_t* cu_seqlens, int64_t B, int64_t T, int64_t n_tokens,
                     float thresh_offset, float near_eps, uint8_t* accept, int32_t* first_reject,
                     int32_t* prefix_len, int32_t* near_count, const int64_t* draft_ids,
-                    int64_t pad_id, int64_t* out_ids, uint8_t* out_mask, int32_t* err_flag, void* stream);
+                    int64_t pad_id, int64_t* out_ids, uint8_t* out_mask, int32_t* err_flag, void* workspace,
+                    int64_t workspace_bytes, void* stream);
+int64_t vrl_spec_verify_workspace(int64_t n_tokens);
+int vrl_spec_verify_plan(int packed, int64_t B, int64_t T, int64_t n_tokens);
 
 /*
  * vrl_truncate_draft — apply an already known first_reject[b] to a draft:
@@ -387,7 +401,8 @@ int vrl_truncate_draft(const int64_t* draft_ids, const uint8_t* mask, const int6
  * checks n_rows == B*T (padded); the verify kernel holds the packed offsets to
  * n_rows and reports VRL_FLAG_SEQ_RANGE through the same err_flag.
  *
- * Two launches on `stream`: the row kernel, then the verify kernel. (Doing the
+ * Two launches on `stream`: the row kernel, then the verify kernel in its one-workgroup-per-sequence form (a caller
+ * with widely differing sequence lengths calls vrl_rowscore and vrl_spec_verify with a workspace instead). (Doing the
  * verification inside the row kernel, by the last workgroup of each sequence,
  * was measured and is slower on MI355X: the agent-scope release each workgroup
  * needs costs more than the second launch.)

@@ -16,7 +16,7 @@ def _declarations():
     text = open(HEADER).read()
     text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
     decls = {}
-    for m in re.finditer(r"\b(?:int|const char\*)\s+(vrl_\w+)\s*\(([^)]*)\)\s*;", text):
+    for m in re.finditer(r"\b(?:int|int64_t|const char\*)\s+(vrl_\w+)\s*\(([^)]*)\)\s*;", text):
         args = m.group(2).strip()
         n = 0 if args in ("", "void") else len(args.split(","))
         decls[m.group(1)] = n
@@ -396,8 +396,9 @@ def test_verify_argument_errors(lib):
     f = lib.vrl_spec_verify
 
     def call(ln=P, lo=P, lu=P, mask=None, cu=None, B=2, T=8, n=16, accept=P, first=P, prefix=P, near=P, ids=None,
-             out_ids=None, out_mask=None, flag=None):
-        return f(ln, lo, lu, mask, cu, B, T, n, 0.0, 1e-6, accept, first, prefix, near, ids, 0, out_ids, out_mask, flag, None)
+             out_ids=None, out_mask=None, flag=None, work=None, work_bytes=0):
+        return f(ln, lo, lu, mask, cu, B, T, n, 0.0, 1e-6, accept, first, prefix, near, ids, 0, out_ids, out_mask, flag,
+                 work, work_bytes, None)
 
     assert call(n=15) == _lib.VRL_ERR_SHAPE                       # padded: the arrays hold exactly B*T tokens
     assert call(n=-1) == _lib.VRL_ERR_SHAPE
@@ -415,6 +416,16 @@ def test_verify_argument_errors(lib):
     assert call(lo=P + 2) == _lib.VRL_ERR_ALIGN
     assert call(cu=P + 4, flag=P) == _lib.VRL_ERR_ALIGN
     assert call(B=0, n=0, ln=None, lo=None, lu=None, accept=None, first=None, prefix=None, near=None) == _lib.VRL_OK
+    # the scratch of the two-pass form: half a byte per token in whole tiles of 1024 tokens, plus 4 bytes per tile
+    need = lib.vrl_spec_verify_workspace
+    assert need(0) == 0 and need(1) == 16 * 4 * 8 + 4 and need(1024) == 516 and need(1025) == 2 * 516
+    assert call(work=P, work_bytes=need(16) - 1) == _lib.VRL_ERR_SHAPE
+    assert call(work=None, work_bytes=8) == _lib.VRL_ERR_ARG
+    assert call(work=P, work_bytes=-1) == _lib.VRL_ERR_ARG
+    assert call(work=P + 4, work_bytes=need(16)) == _lib.VRL_ERR_ALIGN
+    plan = lib.vrl_spec_verify_plan
+    assert plan(1, 512, 0, 1 << 20) == 1 and plan(1, 6, 0, 8192) == 0 and plan(1, 0, 0, 0) == 0
+    assert plan(0, 16, 8192, 16 * 8192) == 1 and plan(0, 64, 1024, 65536) == 0 and plan(0, 4096, 256, 1 << 20) == 0
 
 
 def test_truncate_and_fused_argument_errors(lib):

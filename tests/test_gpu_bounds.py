@@ -42,13 +42,29 @@ def test_verify_and_truncate_hold_bad_offsets_to_the_arrays(dev, case):
         s = _lib.stream_ptr(dev)
         st = lib.vrl_spec_verify(ln.data_ptr(), lo.data_ptr(), lu.data_ptr(), mask.data_ptr(), cu.data_ptr(), B, 0, N, 0.0,
                                  1e-6, accept.data_ptr(), first.data_ptr(), prefix.data_ptr(), near.data_ptr(),
-                                 ids.data_ptr(), -1, out_ids.data_ptr(), out_mask.data_ptr(), flag.data_ptr(), s)
+                                 ids.data_ptr(), -1, out_ids.data_ptr(), out_mask.data_ptr(), flag.data_ptr(), None, 0, s)
         assert st == _lib.VRL_OK
         torch.cuda.synchronize(dev)
         assert int(flag.item()) & _lib.VRL_FLAG_SEQ_RANGE
         assert ar.guards_intact()
         # per-sequence results are those of the spans cut to [0, N]
         cuts = np.clip(np.array(BAD_OFFSETS[case], dtype=np.int64), 0, N)
+        for b in range(B):
+            length = max(int(cuts[b + 1]) - int(cuts[b]), 0)
+            assert 0 <= int(first[b]) <= length and 0 <= int(prefix[b]) <= length
+        # the two-pass form (its scratch between guards too): same guarantees
+        flag.zero_()
+        nbytes = lib.vrl_spec_verify_workspace(N)
+        work = ar.make(nbytes, torch.uint8)
+        print(f"[bounds] two-pass verify with cu_seqlens={BAD_OFFSETS[case]} over {N} tokens", flush=True)
+        st = lib.vrl_spec_verify(ln.data_ptr(), lo.data_ptr(), lu.data_ptr(), mask.data_ptr(), cu.data_ptr(), B, 0, N, 0.0,
+                                 1e-6, accept.data_ptr(), first.data_ptr(), prefix.data_ptr(), near.data_ptr(),
+                                 ids.data_ptr(), -1, out_ids.data_ptr(), out_mask.data_ptr(), flag.data_ptr(),
+                                 work.data_ptr(), nbytes, s)
+        assert st == _lib.VRL_OK
+        torch.cuda.synchronize(dev)
+        assert int(flag.item()) & _lib.VRL_FLAG_SEQ_RANGE
+        assert ar.guards_intact()
         for b in range(B):
             length = max(int(cuts[b + 1]) - int(cuts[b]), 0)
             assert 0 <= int(first[b]) <= length and 0 <= int(prefix[b]) <= length

@@ -147,9 +147,11 @@ def test_one_row_longer_than_two_gibibytes(dev, dtype, V):
     assert abs(g.double().sum().item()) <= 1e-3   # the gradient of a log-prob sums to zero over the row
 
 
-def test_very_long_sequences_verify(dev):
+@pytest.mark.parametrize("two_pass", [False, True])
+def test_very_long_sequences_verify(dev, two_pass):
     """Two padded sequences of five million tokens: positions beyond any 16-bit or LDS-sized assumption; first
-    rejections placed by hand near the end and in the middle, the rest accepts by construction (d = 0.5 >= log u)."""
+    rejections placed by hand near the end and in the middle, the rest accepts by construction (d = 0.5 >= log u).
+    In the two-pass form a tile near the end learns from thousands of tiles back that no rejection is pending."""
     T = 5_000_011
     ln = torch.zeros(2, T, device=dev)
     lo = torch.full((2, T), -0.5, device=dev)
@@ -162,7 +164,7 @@ def test_very_long_sequences_verify(dev):
     log_u[0, T - 3] = -1.0
     log_u[1, 2_345_678] = -1.0
     ids = torch.arange(2 * T, device=dev).view(2, T)
-    res = sv.spec_verify(ln, lo, mask, log_u=log_u, thresh_offset=0.0, draft_ids=ids, pad_id=-1)
+    res = sv.spec_verify(ln, lo, mask, log_u=log_u, thresh_offset=0.0, draft_ids=ids, pad_id=-1, two_pass=two_pass)
     assert res.first_reject.tolist() == [T - 3, 2_345_678] and res.prefix_len.tolist() == [T - 3, 2_345_678]
     assert int(res.accept[0].sum()) == T - 1 and int(res.accept[1].sum()) == T - 1000 - 1
     assert bool((res.out_ids[0, :T - 3] == ids[0, :T - 3]).all()) and bool((res.out_ids[0, T - 3:] == -1).all())

@@ -32,7 +32,7 @@ VRL_FLAG_LABEL_OOB = 1
 VRL_FLAG_SLICE_RANGE = 2
 VRL_FLAG_SEQ_RANGE = 4
 
-ABI_VERSION = 2
+ABI_VERSION = 3
 
 _c = ctypes
 _P = _c.c_void_p
@@ -67,8 +67,10 @@ SIGNATURES = {
     "vrl_rollout_corr_num_stats": (_INT, []),
     "vrl_spec_verify": (
         _INT,
-        [_P, _P, _P, _P, _P, _I64, _I64, _I64, _F32, _F32, _P, _P, _P, _P, _P, _I64, _P, _P, _P, _P],
+        [_P, _P, _P, _P, _P, _I64, _I64, _I64, _F32, _F32, _P, _P, _P, _P, _P, _I64, _P, _P, _P, _P, _I64, _P],
     ),
+    "vrl_spec_verify_workspace": (_I64, [_I64]),
+    "vrl_spec_verify_plan": (_INT, [_INT, _I64, _I64, _I64]),
     "vrl_truncate_draft": (_INT, [_P, _P, _P, _I64, _I64, _I64, _P, _I64, _P, _P, _P, _P]),
     "vrl_fused_score_verify": (
         _INT,

@@ -16,6 +16,7 @@
 #include "rollout_corr_kernels.h"
 #include "rowscore_kernels.h"
 #include "transpose_kernels.h"
+#include "verify_flat_kernels.h"
 #include "verify_kernels.h"
 
 namespace {
@@ -248,6 +249,11 @@ int check_verify(const float* logp_new, const float* logp_old, const float* log_
     return VRL_ERR_ALIGN;
   return VRL_OK;
 }
+
+// From this many tokens on vrl_spec_verify_plan recommends the two flat passes (packed layout; padded: with at least
+// kFlatMinPaddedT tokens per sequence and fewer than two sequences per CU as well).
+constexpr int64_t kFlatMinTokens = 131072;
+constexpr int64_t kFlatMinPaddedT = 4096;
 
 // Wavefronts per sequence for the verify/truncate kernels. A workgroup handles 4 * 64 * waves tokens per
 // memory round trip; long sequences want many wavefronts, a batch of many short ones wants few (idle
@@ -874,23 +880,63 @@ int vrl_transpose(const void* src, int elem_size, int64_t rows, int64_t cols, in
   return launch_status();
 }
 
+int64_t vrl_spec_verify_workspace(int64_t n_tokens) {
+  return n_tokens > 0 ? vrl::flat_workspace_bytes(n_tokens) : 0;
+}
+
+int vrl_spec_verify_plan(int packed, int64_t B, int64_t T, int64_t n_tokens) {
+  if (B <= 0 || n_tokens < kFlatMinTokens) return 0;
+  // Packed lengths live on the device: from this many tokens on, one long sequence among them would cost a workgroup
+  // per sequence more than the second launch costs. Padded: few long sequences leave most CUs without a workgroup.
+  if (packed) return 1;
+  return (T >= kFlatMinPaddedT && B < 2 * device_cus()) ? 1 : 0;
+}
+
 int vrl_spec_verify(const float* logp_new, const float* logp_old, const float* log_u,
                     const uint8_t* mask, const int64_t* cu_seqlens, int64_t B, int64_t T, int64_t n_tokens,
                     float thresh_offset, float near_eps, uint8_t* accept, int32_t* first_reject,
                     int32_t* prefix_len, int32_t* near_count, const int64_t* draft_ids,
-                    int64_t pad_id, int64_t* out_ids, uint8_t* out_mask, int32_t* err_flag, void* stream) {
+                    int64_t pad_id, int64_t* out_ids, uint8_t* out_mask, int32_t* err_flag, void* workspace,
+                    int64_t workspace_bytes, void* stream) {
   const int st = check_verify(logp_new, logp_old, log_u, mask, cu_seqlens, B, T, n_tokens, err_flag, accept,
                               first_reject, prefix_len, near_count, draft_ids, out_ids, out_mask);
   if (st != VRL_OK || B == 0) return st;
+  if (workspace_bytes < 0 || (workspace == nullptr && workspace_bytes != 0)) return VRL_ERR_ARG;
+  if (workspace != nullptr && workspace_bytes < vrl_spec_verify_workspace(n_tokens)) return VRL_ERR_SHAPE;
+  if (!aligned(workspace, 8)) return VRL_ERR_ALIGN;
   const vrl::VerifyArgs v{logp_new, logp_old, log_u, mask, cu_seqlens, B, T, n_tokens, err_flag, thresh_offset,
                           near_eps, accept, first_reject, prefix_len, near_count, draft_ids, pad_id, out_ids,
                           out_mask};
-  const dim3 grid(static_cast<unsigned>(B));
   hipStream_t s = static_cast<hipStream_t>(stream);
-  switch (verify_waves(cu_seqlens, B, T)) {
-    case 1: vrl::spec_verify_kernel<1><<<grid, dim3(64), 0, s>>>(v); break;
-    case 4: vrl::spec_verify_kernel<4><<<grid, dim3(256), 0, s>>>(v); break;
-    default: vrl::spec_verify_kernel<16><<<grid, dim3(1024), 0, s>>>(v); break;
+  if (workspace != nullptr && n_tokens > 0) {
+    // two flat passes over the tokens (verify_flat_kernels.h): a workspace is the caller's request for them
+    const vrl::FlatWork ws = vrl::flat_work(workspace, n_tokens);
+    const int64_t draft_tiles = out_ids != nullptr ? ws.n_tiles : 0;
+    const int64_t finish_grid = draft_tiles + (B + 3) / 4;
+    if (ws.n_tiles > kMaxGrid || finish_grid > kMaxGrid) return VRL_ERR_SHAPE;
+    vrl::verify_tokens_kernel<<<dim3(static_cast<unsigned>(ws.n_tiles)), dim3(vrl::kFlatThreads), 0, s>>>(v, ws);
+    vrl::verify_finish_kernel<<<dim3(static_cast<unsigned>(finish_grid)), dim3(vrl::kFlatThreads), 0, s>>>(v, ws,
+                                                                                                         draft_tiles);
+    return launch_status();
+  }
+  const dim3 grid(static_cast<unsigned>(B));
+  // 16-byte accesses when every array allows them (what an allocator hands out does; a view that starts at an odd
+  // element may not): same results, fewer and wider memory instructions.
+  const bool vec = aligned(logp_new, 16) && aligned(logp_old, 16) && aligned(log_u, 16) && aligned(mask, 4) &&
+                   aligned(accept, 4) && aligned(draft_ids, 16) && aligned(out_ids, 16) && aligned(out_mask, 4);
+  const int waves = verify_waves(cu_seqlens, B, T);
+  if (vec) {
+    switch (waves) {
+      case 1: vrl::spec_verify_vec_kernel<1><<<grid, dim3(64), 0, s>>>(v); break;
+      case 4: vrl::spec_verify_vec_kernel<4><<<grid, dim3(256), 0, s>>>(v); break;
+      default: vrl::spec_verify_vec_kernel<16><<<grid, dim3(1024), 0, s>>>(v); break;
+    }
+  } else {
+    switch (waves) {
+      case 1: vrl::spec_verify_kernel<1><<<grid, dim3(64), 0, s>>>(v); break;
+      case 4: vrl::spec_verify_kernel<4><<<grid, dim3(256), 0, s>>>(v); break;
+      default: vrl::spec_verify_kernel<16><<<grid, dim3(1024), 0, s>>>(v); break;
+    }
   }
   return launch_status();
 }
@@ -936,7 +982,7 @@ int vrl_fused_score_verify(const void* logits, int dtype, int64_t n_rows, int64_
   if (st != VRL_OK) return st;
   return vrl_spec_verify(out_logprob, logp_old, log_u, mask, cu_seqlens, B, T, n_rows, thresh_offset, near_eps,
                          accept, first_reject, prefix_len, near_count, draft_ids, pad_id, out_ids,
-                         out_mask, err_flag, stream);
+                         out_mask, err_flag, nullptr, 0, stream);
 }
 
 int vrl_stream_probe(const void* src, void* dst, int64_t n_rows, int64_t row_bytes, int mode, uint32_t* sink,

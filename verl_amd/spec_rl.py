@@ -165,6 +165,7 @@ def spec_verify(
     draft_ids: Optional[torch.Tensor] = None,
     pad_id: int = 0,
     check=None,
+    two_pass: Optional[bool] = None,
 ) -> VerifyResult:
     """Verify a draft against new log-probs; see the module docstring for the rule.
 
@@ -172,6 +173,11 @@ def spec_verify(
     ``cu_seqlens`` (``B+1`` row offsets that partition the tokens; anything else raises
     ValueError, when and how is ``check``'s business as in verl_amd.errors). With
     ``draft_ids`` the truncated draft and mask come back too.
+
+    ``two_pass`` picks the kernel form: False is one workgroup per sequence, True two flat passes over the tokens whose
+    work does not depend on how the tokens are cut into sequences (a scratch tensor of half a byte per token is
+    allocated for them); None lets the library choose by shape (``vrl_spec_verify_plan``: large packed batches, and
+    padded ones with few long sequences). The results are the same integers.
     """
     _errors.poll()
     if not logp_new.is_cuda:
@@ -197,12 +203,18 @@ def spec_verify(
             thresh_offset=off, out_ids=out_ids, out_mask=None if out_mask is None else out_mask.view(torch.bool),
         )
     lib = _lib.load()
+    if two_pass is None:
+        two_pass = bool(lib.vrl_spec_verify_plan(int(cu is not None), B, T, ln.numel()))
+    work = None
+    if two_pass and B > 0:
+        work = torch.empty(int(lib.vrl_spec_verify_workspace(ln.numel())), dtype=torch.uint8, device=dev)
     with torch.cuda.device(dev):
         stream = _lib.stream_ptr(dev)
         st = lib.vrl_spec_verify(
             ln.data_ptr(), lo.data_ptr(), lu.data_ptr(), _ptr(m8), _ptr(cu), B, T, ln.numel(), off, float(near_eps),
             accept.data_ptr(), first.data_ptr(), prefix.data_ptr(), near.data_ptr(),
-            _ptr(ids), int(pad_id), _ptr(out_ids), _ptr(out_mask), _ptr(flag), stream,
+            _ptr(ids), int(pad_id), _ptr(out_ids), _ptr(out_mask), _ptr(flag), _ptr(work),
+            0 if work is None else work.numel(), stream,
         )
     _lib.check("vrl_spec_verify", st)
     if flag is not None and B > 0:
