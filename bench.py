@@ -10,8 +10,8 @@
 One step = one pass of vrl_fused_score_verify (row kernel + verify kernel, through
 the C ABI, outputs preallocated) over the whole synthetic batch, logits resident
 in HBM. Prints one JSON line: whole-job verified tokens/s, the HBM roofline of
-the row kernel (algorithmic bytes / average kernel time from HIP events on the
-launch stream), and the same computation in torch on the host cores (bounded sample).
+the row kernel (algorithmic bytes / average kernel time: launches back to back
+between one HIP event pair on the launch stream), and the same computation in torch on the host cores (bounded sample).
 With no workload option the line also carries short records of every other workload under "workloads".
 """
 
@@ -31,6 +31,7 @@ REPO = os.path.dirname(os.path.abspath(__file__))
 if REPO not in sys.path:
     sys.path.insert(0, REPO)
 
+import bench_probes  # noqa: E402  (measurement aids only: the read / copy / matrix-core ceilings)
 from verl_amd import _lib, synthetic  # noqa: E402
 from verl_amd import spec_rl as sv  # noqa: E402
 from verl_amd import torch_functional as vf  # noqa: E402
@@ -58,6 +59,22 @@ def spin_up(fn, ms: float = SPINUP_MS):
         for _ in range(8):
             fn()
         torch.cuda.synchronize()
+
+
+def batch_time_ms(fn, launches: int, batches: int = 5):
+    """Average time of one call of `fn` in ms: `launches` calls back to back between one pair of HIP events on the
+    launch stream, the median over `batches` such batches. For kernels of a few microseconds an event pair per launch
+    measures the events."""
+    times = []
+    for _ in range(batches):
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        a.record()
+        for _ in range(launches):
+            fn()
+        b.record()
+        torch.cuda.synchronize()
+        times.append(a.elapsed_time(b) / launches)
+    return statistics.median(times)
 
 
 def algorithmic_bytes_per_token(V: int, esize: int, with_temperature: bool, with_verify: bool) -> int:
@@ -258,13 +275,7 @@ def bench_backward(args, dev, workload=None):
         run()
     torch.cuda.synchronize()
     wall = time.perf_counter() - t0
-    evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(args.steps)]
-    for a, b in evs:
-        a.record()
-        run()
-        b.record()
-    torch.cuda.synchronize()
-    avg_ms = sum(a.elapsed_time(b) for a, b in evs) / len(evs)
+    avg_ms = batch_time_ms(run, args.steps, 3)
     esize = 2 if w.dtype == torch.bfloat16 else 4
     bytes_launch = step.n * (2 * w.V * esize + 8 + 4 + 4 + 4 + 4 + (4 if step.temp is not None else 0))
     achieved = bytes_launch / (avg_ms * 1e-3) / 1e9
@@ -342,22 +353,6 @@ class VerifyOnlyStep:
 # profiles/verify_two_pass_kernels_c5_trace_and_hbm_counters.md: 17.63 + 2.23 MB (verify_tokens_kernel) and 1.24 + 13.13 MB
 # (verify_finish_kernel); the 0.73 MB of ballot words are written once and read once on top of the algorithmic bytes.
 MEASURED_VERIFY_TRAFFIC_BYTES = {"two-pass": 34229825}
-
-
-def batch_time_ms(fn, launches: int, batches: int = 5):
-    """Average time of one call of `fn` in ms: `launches` calls back to back between one pair of HIP events on the
-    launch stream, the median over `batches` such batches. For kernels of a few microseconds an event pair per launch
-    measures the events."""
-    times = []
-    for _ in range(batches):
-        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        a.record()
-        for _ in range(launches):
-            fn()
-        b.record()
-        torch.cuda.synchronize()
-        times.append(a.elapsed_time(b) / launches)
-    return statistics.median(times)
 
 
 def bench_verify_only(args, dev, with_cpu_baseline=True):
@@ -654,7 +649,7 @@ def copy_calibration(dev):
 def bench_ceilings(args, dev):
     """The memory system's own ceilings for the row kernels' access pattern (vrl_stream_probe): a non-temporal read
     of c3's rows (forward kernel) and a non-temporal copy of them (backward kernel), plus torch's device copy."""
-    lib = _lib.load()
+    lib = bench_probes.load()
     stream = torch.cuda.current_stream(dev).cuda_stream
     out = {"metric": "HBM GB/s delivered to the row kernels' access pattern without arithmetic", "unit": "GB/s",
            "peak": HBM_PEAK_GBPS, "probes": []}
@@ -704,7 +699,7 @@ def mfma_ceiling(dev, steps):
     instruction of the LM-head kernels (16x16x32; what their matrix time is measured against: the part holds a lower
     clock when the operand bits toggle), the same with 32x32x16, and on small constants (the nominal rate). Returns the
     first record with the others inside."""
-    lib = _lib.load()
+    lib = bench_probes.load()
     stream = torch.cuda.current_stream(dev).cuda_stream
     n_wg = torch.cuda.get_device_properties(dev).multi_processor_count
     iters = 20000   # 64 x 128 x 16 wavefront tiles: about as many as the LM-head kernel forms per wavefront at 8192 tokens
@@ -772,15 +767,8 @@ def bench_forward(args, dev, workload, steps, warmup, with_cpu_baseline):
     ms_per_step = wall * 1e3 / steps
     tokens_per_s = step.n_valid * steps / wall
 
-    # Row kernel alone, one HIP event pair per launch on the launch stream.
-    evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(steps)]
-    for a, b in evs:
-        a.record()
-        step.score()
-        b.record()
-    torch.cuda.synchronize()
-    kern_ms = [a.elapsed_time(b) for a, b in evs]
-    avg_kern_ms = sum(kern_ms) / len(kern_ms)
+    # Row kernel alone: `steps` launches back to back between one HIP event pair on the launch stream, median of 3 batches.
+    avg_kern_ms = batch_time_ms(step.score, steps, 3)
     esize = 2 if w.dtype == torch.bfloat16 else 4
     bytes_score = algorithmic_bytes_per_token(w.V, esize, step.temp is not None, False) * step.n
     achieved = bytes_score / (avg_kern_ms * 1e-3) / 1e9
@@ -884,15 +872,12 @@ def bench_score_responses(args, dev, steps, warmup):
     for _ in range(warmup):
         run()
     torch.cuda.synchronize()
-    evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(steps)]
     t0 = time.perf_counter()
-    for a, b in evs:
-        a.record()
+    for _ in range(steps):
         run()
-        b.record()
     torch.cuda.synchronize()
     wall = time.perf_counter() - t0
-    avg_ms = sum(a.elapsed_time(b) for a, b in evs) / len(evs)
+    avg_ms = batch_time_ms(run, steps, 3)
     n_resp = int(resp.sum())
     bytes_launch = n_resp * (w.V * 2 + 8 + 4 + 4) + (B + 1) * 8 + B * 8 + B * T * 8 - n_resp * 8
     achieved = bytes_launch / (avg_ms * 1e-3) / 1e9
@@ -933,13 +918,7 @@ def bench_score_responses(args, dev, steps, warmup):
     for _ in range(warmup):
         run_backward()
     torch.cuda.synchronize()
-    evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(steps)]
-    for a, b in evs:
-        a.record()
-        run_backward()
-        b.record()
-    torch.cuda.synchronize()
-    bwd_ms = sum(a.elapsed_time(b) for a, b in evs) / len(evs)
+    bwd_ms = batch_time_ms(run_backward, steps, 3)
     bwd_bytes = n_resp * (w.V * 2 + 8 + 16) + n * w.V * 2 + (B + 1) * 8 + B * 8
     # the counters were read at this very micro-batch (5515 response rows of 8192); another one has no measured traffic
     measured = MEASURED_SCORE_RESPONSES_TRAFFIC_BYTES if (n, n_resp, B) == (8192, 5515, 4) else (None, None)

@@ -281,17 +281,6 @@ def test_gemm_layout_argument_errors(lib):
     assert call(x=P + 8) == _lib.VRL_ERR_ALIGN
 
 
-def test_mfma_probe_argument_errors(lib):
-    f = lib.vrl_mfma_probe
-    assert f(-1, 10, 32, 1, P, None, None, None) == _lib.VRL_ERR_SHAPE
-    assert f(4, -1, 16, 1, P, None, None, None) == _lib.VRL_ERR_SHAPE
-    assert f(4, 10, 8, 1, P, None, None, None) == _lib.VRL_ERR_ARG
-    assert f(4, 10, 32, 1, None, None, None, None) == _lib.VRL_ERR_NULL
-    assert f(4, 10, 16, 0, P + 2, None, None, None) == _lib.VRL_ERR_ALIGN
-    assert f(4, 10, 32, 0, P, P + 4, None, None) == _lib.VRL_ERR_ALIGN
-    assert f(0, 10, 16, 1, None, None, None, None) == _lib.VRL_OK
-
-
 def test_lmhead_dlogits_argument_errors(lib):
     f = lib.vrl_lmhead_dlogits
     ok = dict(h=P, w=P, dt=_lib.VRL_BF16, T=512, V=1024, K=128, hs=128, ws=128, lab=P, temp=None, lse=P, ent=P, gl=P, gh=P,

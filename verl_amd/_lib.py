@@ -77,8 +77,6 @@ SIGNATURES = {
         [_P, _INT, _I64, _I64, _I64, _P, _P, _P, _P, _P, _P, _P]
         + [_P, _P, _P, _P, _I64, _I64, _F32, _F32, _P, _P, _P, _P, _P, _I64, _P, _P, _P],
     ),
-    "vrl_stream_probe": (_INT, [_P, _P, _I64, _I64, _INT, _P, _P]),
-    "vrl_mfma_probe": (_INT, [_I64, _I64, _INT, _INT, _P, _P, _P, _P]),
     "vrl_strerror": (_c.c_char_p, [_INT]),
     "vrl_last_hip_error": (_c.c_char_p, []),
     "vrl_abi_version": (_INT, []),

@@ -12,8 +12,8 @@
 #include "backward_kernels.h"
 #include "layout_kernels.h"
 #include "lmhead_kernels.h"
-#include "probe_kernels.h"
 #include "rollout_corr_kernels.h"
+#include "row_shapes.h"
 #include "rowscore_kernels.h"
 #include "transpose_kernels.h"
 #include "verify_flat_kernels.h"
@@ -46,35 +46,6 @@ static __device__ __align__(256) float scratch[VRL_STATIC_PARTIALS_MAX * 4];
 
 constexpr int kMaxDevices = 64;
 std::atomic<float*> g_scratch_ptr[kMaxDevices];
-
-// Workgroup shape of the row kernel (wavefronts per row, 128-bit loads per lane
-// and batch), chosen by measurement on MI355X at 8192 x 151936 and 32768 x 152064.
-// Every shape from 1 to 16 wavefronts and 2 to 8 loads lands within 3 % of the
-// others (6.7 to 7.05 TB/s, a plain read of the same rows reaches 7.05); these
-// were on top at both sizes.
-template <int DT>
-struct RowShape;
-template <>
-struct RowShape<VRL_F32> {
-  static constexpr int kWaves = 4, kUnroll = 4;
-};
-template <>
-struct RowShape<VRL_BF16> {
-  static constexpr int kWaves = 8, kUnroll = 2;
-};
-template <>
-struct RowShape<VRL_F16> {
-  static constexpr int kWaves = 8, kUnroll = 2;
-};
-// Shape of a workgroup that reduces one slice of a row (split path).
-constexpr int kSplitWaves = 4;
-constexpr int kSplitUnroll = 2;
-constexpr int kMaxSplits = 64;
-// Shape of the backward workgroup (one per row): wavefronts, 128-bit loads/stores per lane and batch.
-// (measured 5.2-5.3 TB/s of read+write for every shape from 4 to 16 wavefronts, the same as a plain
-// non-temporal copy of the same buffers)
-constexpr int kBackwardWaves = 8;
-constexpr int kBackwardUnroll = 2;
 
 int check_rowscore(const void* logits, int dtype, int64_t n_rows, int64_t vocab, int64_t row_stride,
                    const int64_t* labels, const float* temperature, const float* out_logprob,
@@ -983,59 +954,6 @@ int vrl_fused_score_verify(const void* logits, int dtype, int64_t n_rows, int64_
   return vrl_spec_verify(out_logprob, logp_old, log_u, mask, cu_seqlens, B, T, n_rows, thresh_offset, near_eps,
                          accept, first_reject, prefix_len, near_count, draft_ids, pad_id, out_ids,
                          out_mask, err_flag, nullptr, 0, stream);
-}
-
-int vrl_stream_probe(const void* src, void* dst, int64_t n_rows, int64_t row_bytes, int mode, uint32_t* sink,
-                     void* stream) {
-  if (mode < 0 || mode > 3) return VRL_ERR_ARG;
-  if (n_rows < 0 || row_bytes < 0 || row_bytes % 16 != 0 || n_rows > kMaxGrid) return VRL_ERR_SHAPE;
-  if (n_rows == 0 || row_bytes == 0) return VRL_OK;
-  const bool reads_only = mode == 0 || mode == 3;
-  if (src == nullptr || (!reads_only && dst == nullptr) || (reads_only && sink == nullptr)) return VRL_ERR_NULL;
-  if (!aligned(src, 16) || !aligned(dst, 16) || !aligned(sink, 4)) return VRL_ERR_ALIGN;
-  const dim3 grid(static_cast<unsigned>(n_rows));
-  hipStream_t s = static_cast<hipStream_t>(stream);
-  const int64_t vecs = row_bytes / 16;
-  // the forward / backward row kernels' workgroup shapes for 16-bit logits
-  if (mode == 0)
-    vrl::stream_probe_kernel<RowShape<VRL_BF16>::kWaves, RowShape<VRL_BF16>::kUnroll, false>
-        <<<grid, dim3(RowShape<VRL_BF16>::kWaves * 64), 0, s>>>(static_cast<const vrl::u32x4*>(src), nullptr, vecs,
-                                                                0x9e3779b9u, sink);
-  else if (mode == 3)   // the forward kernel's workgroup shape for 32-bit logits
-    vrl::stream_probe_kernel<RowShape<VRL_F32>::kWaves, RowShape<VRL_F32>::kUnroll, false>
-        <<<grid, dim3(RowShape<VRL_F32>::kWaves * 64), 0, s>>>(static_cast<const vrl::u32x4*>(src), nullptr, vecs,
-                                                               0x9e3779b9u, sink);
-  else if (mode == 1)
-    vrl::stream_probe_kernel<kBackwardWaves, kBackwardUnroll, true><<<grid, dim3(kBackwardWaves * 64), 0, s>>>(
-        static_cast<const vrl::u32x4*>(src), static_cast<vrl::u32x4*>(dst), vecs, 0u, nullptr);
-  else
-    vrl::stream_probe_flat_copy_kernel<<<dim3(512), dim3(256), 0, s>>>(
-        static_cast<const vrl::u32x4*>(src), static_cast<vrl::u32x4*>(dst), n_rows * vecs);
-  return launch_status();
-}
-
-int vrl_mfma_probe(int64_t n_workgroups, int64_t iters, int instruction, int random_operands, float* sink,
-                   int64_t* clocks, int64_t* wall_clock_khz, void* stream) {
-  if (n_workgroups < 0 || iters < 0 || n_workgroups > kMaxGrid) return VRL_ERR_SHAPE;
-  if (instruction != 16 && instruction != 32) return VRL_ERR_ARG;
-  if (wall_clock_khz != nullptr) {
-    int dev = 0, khz = 0;
-    if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&khz, hipDeviceAttributeWallClockRate, dev) != hipSuccess) {
-      launch_status();   // keeps the runtime's message for vrl_last_hip_error
-      return VRL_ERR_HIP;
-    }
-    *wall_clock_khz = khz;
-  }
-  if (n_workgroups == 0) return VRL_OK;
-  if (sink == nullptr) return VRL_ERR_NULL;
-  if (!aligned(sink, 4) || !aligned(clocks, 8)) return VRL_ERR_ALIGN;
-  const dim3 grid(static_cast<unsigned>(n_workgroups));
-  hipStream_t s = static_cast<hipStream_t>(stream);
-  if (instruction == 16)
-    vrl::mfma_probe_kernel<16><<<grid, dim3(512), 0, s>>>(iters, random_operands != 0 ? 1 : 0, sink, clocks);
-  else
-    vrl::mfma_probe_kernel<32><<<grid, dim3(512), 0, s>>>(iters, random_operands != 0 ? 1 : 0, sink, clocks);
-  return launch_status();
 }
 
 const char* vrl_strerror(int status) {
