@@ -199,32 +199,40 @@ int vrl_score_responses_backward(const void* logits, int dtype, int64_t n_rows, 
                                  const float* g_resp_entropy, void* dlogits, int64_t d_row_stride, void* stream);
 
 /*
- * vrl_response_slice — packed per-token values (total_nnz,) -> padded (B, T_out)
+ * vrl_response_slice — packed per-token values (total_nnz, *) -> padded (B, T_out, *)
  * response block: out[b, j] = values[cu_seqlens[b+1] - response_lens[b] - 1 + j]
- * for j < response_lens[b], else 0 (the model output at a position scores the
- * NEXT token, hence the shift by one). `values` has n_tokens entries. Sets
- * VRL_FLAG_SLICE_RANGE and writes a zero row when a sequence has no prompt token,
- * or response_lens[b] is outside [0, T_out]; VRL_FLAG_SEQ_RANGE and a zero row when
+ * for j < response_lens[b], else zeros (the model output at a position scores the
+ * NEXT token, hence the shift by one). A value is a row of row_bytes bytes: the
+ * element size times the product of the trailing dimensions (4 for an fp32 vector,
+ * 2 * K for (total_nnz, K) bf16 top-k log-probs, ...), copied bit for bit, whatever
+ * the element type; the trailing dimensions are not padded
+ * (verl/workers/utils/padding.py:100-101, :133-138: skip_padding = (0, 0) * (values.ndim - 1)).
+ * `values` has n_tokens rows, out B * T_out rows; neither needs more alignment than its element type. Sets
+ * VRL_FLAG_SLICE_RANGE and writes a zero row block when a sequence has no prompt token,
+ * or response_lens[b] is outside [0, T_out]; VRL_FLAG_SEQ_RANGE and a zero row block when
  * the sequence's offsets do not fit n_tokens (see "Sequence space" above).
+ * row_bytes is at most 2^30; T_out * row_bytes at most 2^31 or so (VRL_ERR_SHAPE beyond).
  *
- * Replaces verl/workers/utils/padding.py:97-141 (no_padding_2_padding) for fp32
- * per-token vectors; fixture: tests/models/test_fsdp_no_padding_on_gpu.py:180-201.
+ * Replaces verl/workers/utils/padding.py:97-141 (no_padding_2_padding); fixture:
+ * tests/models/test_fsdp_no_padding_on_gpu.py:180-201.
  */
-int vrl_response_slice(const float* values, const int64_t* cu_seqlens, const int64_t* response_lens,
-                       int64_t B, int64_t n_tokens, int64_t T_out, float* out, int32_t* err_flag, void* stream);
+int vrl_response_slice(const void* values, int64_t row_bytes, const int64_t* cu_seqlens, const int64_t* response_lens,
+                       int64_t B, int64_t n_tokens, int64_t T_out, void* out, int32_t* err_flag, void* stream);
 
 /*
- * vrl_response_pack — packed per-token values (total_nnz,) -> packed response values (sum of response_lens,):
+ * vrl_response_pack — packed per-token values (total_nnz, *) -> packed response values (sum of response_lens, *):
  *   out[out_offsets[b] + j] = values[cu_seqlens[b+1] - response_lens[b] - 1 + j],  j < response_lens[b]
- * out_offsets is the caller's exclusive prefix sum of response_lens (B+1 entries, last = out_total).
+ * with rows of row_bytes bytes as in vrl_response_slice.
+ * out_offsets is the caller's exclusive prefix sum of response_lens (B+1 entries, last = out_total rows).
  * A sequence without a prompt token, a negative length, or a window that is not exactly
- * [out_offsets[b], out_offsets[b+1]) inside the output sets VRL_FLAG_SLICE_RANGE and writes nothing for it;
- * offsets that do not fit the n_tokens entries of `values` set VRL_FLAG_SEQ_RANGE and write nothing for it.
+ * [out_offsets[b], out_offsets[b+1]) inside the output (the last one ending at out_total) sets VRL_FLAG_SLICE_RANGE
+ * and writes nothing for it;
+ * offsets that do not fit the n_tokens rows of `values` set VRL_FLAG_SEQ_RANGE and write nothing for it.
  *
- * Replaces verl/workers/utils/padding.py:194-210 (response_from_nested) for fp32 per-token vectors.
+ * Replaces verl/workers/utils/padding.py:194-210 (response_from_nested).
  */
-int vrl_response_pack(const float* values, const int64_t* cu_seqlens, const int64_t* response_lens,
-                      const int64_t* out_offsets, int64_t B, int64_t n_tokens, int64_t out_total, float* out,
+int vrl_response_pack(const void* values, int64_t row_bytes, const int64_t* cu_seqlens, const int64_t* response_lens,
+                      const int64_t* out_offsets, int64_t B, int64_t n_tokens, int64_t out_total, void* out,
                       int32_t* err_flag, void* stream);
 
 /*

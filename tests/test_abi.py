@@ -139,13 +139,16 @@ def test_split_and_slice_argument_errors(lib):
     assert back(dx=P + 1) == _lib.VRL_ERR_ALIGN
     assert back(n=0, x=None, dx=None, lse=None) == _lib.VRL_OK
 
-    g = lib.vrl_response_slice     # (values, cu, response_lens, B, n_tokens, T_out, out, err_flag, stream)
-    assert g(P, P, P, -1, 9, 4, P, P, None) == _lib.VRL_ERR_SHAPE
-    assert g(P, P, P, 2, -1, 4, P, P, None) == _lib.VRL_ERR_SHAPE
-    assert g(None, P, P, 2, 9, 4, P, P, None) == _lib.VRL_ERR_NULL
-    assert g(P, P, P, 2, 9, 4, P, None, None) == _lib.VRL_ERR_NULL
-    assert g(P, P + 4, P, 2, 9, 4, P, P, None) == _lib.VRL_ERR_ALIGN
-    assert g(None, None, None, 0, 0, 4, None, None, None) == _lib.VRL_OK
+    g = lib.vrl_response_slice     # (values, row_bytes, cu, response_lens, B, n_tokens, T_out, out, err_flag, stream)
+    assert g(P, 4, P, P, -1, 9, 4, P, P, None) == _lib.VRL_ERR_SHAPE
+    assert g(P, 4, P, P, 2, -1, 4, P, P, None) == _lib.VRL_ERR_SHAPE
+    assert g(P, 0, P, P, 2, 9, 4, P, P, None) == _lib.VRL_ERR_SHAPE       # a row holds at least one byte
+    assert g(P, (1 << 30) + 1, P, P, 2, 9, 4, P, P, None) == _lib.VRL_ERR_SHAPE
+    assert g(P, 1 << 20, P, P, 2, 9, 1 << 20, P, P, None) == _lib.VRL_ERR_SHAPE   # a padded row block beyond the grid
+    assert g(None, 4, P, P, 2, 9, 4, P, P, None) == _lib.VRL_ERR_NULL
+    assert g(P, 4, P, P, 2, 9, 4, P, None, None) == _lib.VRL_ERR_NULL
+    assert g(P, 4, P + 4, P, 2, 9, 4, P, P, None) == _lib.VRL_ERR_ALIGN
+    assert g(None, 4, None, None, 0, 0, 4, None, None, None) == _lib.VRL_OK
 
 
 def test_label_logprob_argument_errors_and_flag_values(lib):
@@ -308,16 +311,17 @@ def test_lmhead_dlogits_argument_errors(lib):
 
 
 def test_response_pack_argument_errors(lib):
-    g = lib.vrl_response_pack      # (values, cu, response_lens, out_offsets, B, n_tokens, out_total, out, err_flag, stream)
-    assert g(P, P, P, P, -1, 9, 4, P, P, None) == _lib.VRL_ERR_SHAPE
-    assert g(P, P, P, P, 2, 9, -1, P, P, None) == _lib.VRL_ERR_SHAPE
-    assert g(P, P, P, P, 2, -9, 4, P, P, None) == _lib.VRL_ERR_SHAPE
-    assert g(None, P, P, P, 2, 9, 4, P, P, None) == _lib.VRL_ERR_NULL
-    assert g(P, P, P, None, 2, 9, 4, P, P, None) == _lib.VRL_ERR_NULL
-    assert g(P, P, P, P, 2, 9, 4, None, P, None) == _lib.VRL_ERR_NULL
-    assert g(P, P, P, P, 2, 9, 4, P, None, None) == _lib.VRL_ERR_NULL
-    assert g(P, P, P, P + 4, 2, 9, 4, P, P, None) == _lib.VRL_ERR_ALIGN
-    assert g(None, None, None, None, 0, 0, 0, None, None, None) == _lib.VRL_OK
+    g = lib.vrl_response_pack      # (values, row_bytes, cu, response_lens, out_offsets, B, n_tokens, out_total, out, err_flag, stream)
+    assert g(P, 4, P, P, P, -1, 9, 4, P, P, None) == _lib.VRL_ERR_SHAPE
+    assert g(P, 4, P, P, P, 2, 9, -1, P, P, None) == _lib.VRL_ERR_SHAPE
+    assert g(P, 4, P, P, P, 2, -9, 4, P, P, None) == _lib.VRL_ERR_SHAPE
+    assert g(P, -2, P, P, P, 2, 9, 4, P, P, None) == _lib.VRL_ERR_SHAPE
+    assert g(None, 4, P, P, P, 2, 9, 4, P, P, None) == _lib.VRL_ERR_NULL
+    assert g(P, 4, P, P, None, 2, 9, 4, P, P, None) == _lib.VRL_ERR_NULL
+    assert g(P, 4, P, P, P, 2, 9, 4, None, P, None) == _lib.VRL_ERR_NULL
+    assert g(P, 4, P, P, P, 2, 9, 4, P, None, None) == _lib.VRL_ERR_NULL
+    assert g(P, 4, P, P, P + 4, 2, 9, 4, P, P, None) == _lib.VRL_ERR_ALIGN
+    assert g(None, 4, None, None, None, 0, 0, 0, None, None, None) == _lib.VRL_OK
 
 
 def test_lmhead_argument_errors(lib):

@@ -107,7 +107,7 @@ def test_response_slice_and_pack_hold_bad_offsets_to_the_arrays(dev, case):
     print(f"[bounds] response slice/pack with cu_seqlens={BAD_OFFSETS[case]} over {N} values", flush=True)
     with torch.cuda.device(dev):
         s = _lib.stream_ptr(dev)
-        st = lib.vrl_response_slice(values.data_ptr(), cu.data_ptr(), rl.data_ptr(), B, N, T, out.data_ptr(),
+        st = lib.vrl_response_slice(values.data_ptr(), 4, cu.data_ptr(), rl.data_ptr(), B, N, T, out.data_ptr(),
                                     flag.data_ptr(), s)
         assert st == _lib.VRL_OK
         torch.cuda.synchronize(dev)
@@ -115,12 +115,28 @@ def test_response_slice_and_pack_hold_bad_offsets_to_the_arrays(dev, case):
         assert ar.guards_intact()
         assert torch.isfinite(out).all()            # every output element was written (values or zeros)
         flag.zero_()
-        st = lib.vrl_response_pack(values.data_ptr(), cu.data_ptr(), rl.data_ptr(), out_cu.data_ptr(), B, N, 20,
+        st = lib.vrl_response_pack(values.data_ptr(), 4, cu.data_ptr(), rl.data_ptr(), out_cu.data_ptr(), B, N, 20,
                                    packed.data_ptr(), flag.data_ptr(), s)
         assert st == _lib.VRL_OK
         torch.cuda.synchronize(dev)
         assert int(flag.item()) & _lib.VRL_FLAG_SEQ_RANGE
         assert ar.guards_intact()
+        # rows of several elements ((N, 6) bf16: 12 bytes a row, moved in 4-byte units) between guards of their own
+        flag.zero_()
+        wide = ar.make(N * 6, torch.bfloat16, torch.randn(N * 6, generator=g).bfloat16())
+        wide_out = ar.make(B * T * 6, torch.bfloat16)
+        wide_packed = ar.make(20 * 6, torch.bfloat16)
+        print(f"[bounds] response slice/pack of 12-byte rows with cu_seqlens={BAD_OFFSETS[case]}", flush=True)
+        st = lib.vrl_response_slice(wide.data_ptr(), 12, cu.data_ptr(), rl.data_ptr(), B, N, T, wide_out.data_ptr(),
+                                    flag.data_ptr(), s)
+        assert st == _lib.VRL_OK
+        st = lib.vrl_response_pack(wide.data_ptr(), 12, cu.data_ptr(), rl.data_ptr(), out_cu.data_ptr(), B, N, 20,
+                                   wide_packed.data_ptr(), flag.data_ptr(), s)
+        assert st == _lib.VRL_OK
+        torch.cuda.synchronize(dev)
+        assert int(flag.item()) & _lib.VRL_FLAG_SEQ_RANGE
+        assert ar.guards_intact()
+        assert torch.isfinite(wide_out.float()).all()
     cu_t = torch.tensor(BAD_OFFSETS[case], dtype=torch.int64, device=dev)
     with pytest.raises(ValueError, match="partition"):
         layout.response_slice(values.clone(), cu_t, rl.clone(), T)

@@ -51,8 +51,8 @@ SIGNATURES = {
     "vrl_score_responses": (_INT, [_P, _INT, _I64, _I64, _I64, _P, _P, _P, _P, _P, _I64, _I64, _P, _P, _P, _P, _P, _P, _P]),
     "vrl_score_responses_backward": (
         _INT, [_P, _INT, _I64, _I64, _I64, _P, _P, _P, _P, _P, _I64, _I64, _P, _P, _P, _P, _P, _I64, _P]),
-    "vrl_response_slice": (_INT, [_P, _P, _P, _I64, _I64, _I64, _P, _P, _P]),
-    "vrl_response_pack": (_INT, [_P, _P, _P, _P, _I64, _I64, _I64, _P, _P, _P]),
+    "vrl_response_slice": (_INT, [_P, _I64, _P, _P, _I64, _I64, _I64, _P, _P, _P]),
+    "vrl_response_pack": (_INT, [_P, _I64, _P, _P, _P, _I64, _I64, _I64, _P, _P, _P]),
     "vrl_lmhead_score": (_INT, [_P, _P, _INT, _I64, _I64, _I64, _I64, _I64, _P, _P, _INT, _P, _P, _P, _P, _P, _P]),
     "vrl_lmhead_dlogits": (_INT, [_P, _P, _INT, _I64, _I64, _I64, _I64, _I64, _P, _P, _P, _P, _P, _P, _INT, _P, _I64, _P]),
     "vrl_gemm_nt_plan": (_INT, [_INT, _I64, _I64, _I64, _P]),

@@ -235,6 +235,18 @@ int verify_waves(const int64_t* cu_seqlens, int64_t B, int64_t T) {
   return B <= 4096 ? 16 : 4;
 }
 
+// Response slicing moves rows of `row_bytes` bytes in units of the largest power of two up to 16 that divides the row
+// and the alignment of both arrays.
+constexpr int64_t kMaxRowBytes = int64_t(1) << 30;
+constexpr int64_t kMaxGridY = 65535;
+constexpr int64_t kPackMaxChunks = 64;
+
+int copy_unit(int64_t row_bytes, const void* a, const void* b) {
+  for (int u = 16; u > 1; u >>= 1)
+    if (row_bytes % u == 0 && aligned(a, u) && aligned(b, u)) return u;
+  return 1;
+}
+
 struct LmGrid {
   int64_t tblocks;
   int tiles_per_split;
@@ -693,34 +705,72 @@ int vrl_rollout_corr(const float* old_log_prob, const float* rollout_log_prob, c
 
 int vrl_rollout_corr_num_stats(void) { return vrl::kNumCorrStats; }
 
-int vrl_response_slice(const float* values, const int64_t* cu_seqlens, const int64_t* response_lens,
-                       int64_t B, int64_t n_tokens, int64_t T_out, float* out, int32_t* err_flag, void* stream) {
-  if (B < 0 || T_out < 0 || n_tokens < 0 || B > kMaxGrid) return VRL_ERR_SHAPE;
+int vrl_response_slice(const void* values, int64_t row_bytes, const int64_t* cu_seqlens, const int64_t* response_lens,
+                       int64_t B, int64_t n_tokens, int64_t T_out, void* out, int32_t* err_flag, void* stream) {
+  if (B < 0 || T_out < 0 || n_tokens < 0 || B > kMaxGrid || row_bytes <= 0 || row_bytes > kMaxRowBytes)
+    return VRL_ERR_SHAPE;
   if (B == 0 || T_out == 0) return VRL_OK;
   if ((values == nullptr && n_tokens > 0) || cu_seqlens == nullptr || response_lens == nullptr || out == nullptr ||
       err_flag == nullptr)
     return VRL_ERR_NULL;
-  if (!aligned(values, 4) || !aligned(cu_seqlens, 8) || !aligned(response_lens, 8) || !aligned(out, 4) ||
-      !aligned(err_flag, 4))
-    return VRL_ERR_ALIGN;
-  vrl::response_slice_kernel<<<dim3(static_cast<unsigned>(B)), dim3(256), 0, static_cast<hipStream_t>(stream)>>>(
-      values, cu_seqlens, response_lens, n_tokens, T_out, out, err_flag);
+  if (!aligned(cu_seqlens, 8) || !aligned(response_lens, 8) || !aligned(err_flag, 4)) return VRL_ERR_ALIGN;
+  const int unit = copy_unit(row_bytes, values, out);
+  const int64_t row_units = row_bytes / unit;
+  if (T_out > (int64_t(1) << 62) / row_units) return VRL_ERR_SHAPE;
+  const int64_t chunks = (T_out * row_units + vrl::kSliceChunk - 1) / vrl::kSliceChunk;
+  if (chunks > kMaxGridY) return VRL_ERR_SHAPE;
+  const dim3 grid(static_cast<unsigned>(B), static_cast<unsigned>(chunks));
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const char* v = static_cast<const char*>(values);
+  char* o = static_cast<char*>(out);
+#define VRL_SLICE(U)                                                                                                   \
+  vrl::response_slice_kernel<U><<<grid, dim3(vrl::kSliceThreads), 0, s>>>(v, row_units, cu_seqlens, response_lens,     \
+                                                                          n_tokens, T_out, o, err_flag)
+  switch (unit) {
+    case 16: VRL_SLICE(16); break;
+    case 8: VRL_SLICE(8); break;
+    case 4: VRL_SLICE(4); break;
+    case 2: VRL_SLICE(2); break;
+    default: VRL_SLICE(1); break;
+  }
+#undef VRL_SLICE
   return launch_status();
 }
 
-int vrl_response_pack(const float* values, const int64_t* cu_seqlens, const int64_t* response_lens,
-                      const int64_t* out_offsets, int64_t B, int64_t n_tokens, int64_t out_total, float* out,
+int vrl_response_pack(const void* values, int64_t row_bytes, const int64_t* cu_seqlens, const int64_t* response_lens,
+                      const int64_t* out_offsets, int64_t B, int64_t n_tokens, int64_t out_total, void* out,
                       int32_t* err_flag, void* stream) {
-  if (B < 0 || out_total < 0 || n_tokens < 0 || B > kMaxGrid) return VRL_ERR_SHAPE;
+  if (B < 0 || out_total < 0 || n_tokens < 0 || B > kMaxGrid || row_bytes <= 0 || row_bytes > kMaxRowBytes)
+    return VRL_ERR_SHAPE;
   if (B == 0) return VRL_OK;
   if ((values == nullptr && n_tokens > 0) || cu_seqlens == nullptr || response_lens == nullptr || out_offsets == nullptr ||
       err_flag == nullptr || (out == nullptr && out_total > 0))
     return VRL_ERR_NULL;
-  if (!aligned(values, 4) || !aligned(cu_seqlens, 8) || !aligned(response_lens, 8) || !aligned(out_offsets, 8) ||
-      !aligned(out, 4) || !aligned(err_flag, 4))
+  if (!aligned(cu_seqlens, 8) || !aligned(response_lens, 8) || !aligned(out_offsets, 8) || !aligned(err_flag, 4))
     return VRL_ERR_ALIGN;
-  vrl::response_pack_kernel<<<dim3(static_cast<unsigned>(B)), dim3(256), 0, static_cast<hipStream_t>(stream)>>>(
-      values, cu_seqlens, response_lens, out_offsets, n_tokens, out_total, out, err_flag);
+  const int unit = copy_unit(row_bytes, values, out);
+  const int64_t row_units = row_bytes / unit;
+  // a window cannot be longer than the shorter of the two arrays; more workgroups per sequence than that needs are idle
+  const int64_t longest = out_total < n_tokens ? out_total : n_tokens;
+  if (longest > (int64_t(1) << 62) / row_units) return VRL_ERR_SHAPE;
+  int64_t chunks = (longest * row_units + vrl::kSliceChunk - 1) / vrl::kSliceChunk;
+  if (chunks < 1) chunks = 1;
+  if (chunks > kPackMaxChunks) chunks = kPackMaxChunks;   // the kernel strides over what is left
+  const dim3 grid(static_cast<unsigned>(B), static_cast<unsigned>(chunks));
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const char* v = static_cast<const char*>(values);
+  char* o = static_cast<char*>(out);
+#define VRL_PACK(U)                                                                                                    \
+  vrl::response_pack_kernel<U><<<grid, dim3(vrl::kSliceThreads), 0, s>>>(v, row_units, cu_seqlens, response_lens,      \
+                                                                         out_offsets, n_tokens, out_total, o, err_flag)
+  switch (unit) {
+    case 16: VRL_PACK(16); break;
+    case 8: VRL_PACK(8); break;
+    case 4: VRL_PACK(4); break;
+    case 2: VRL_PACK(2); break;
+    default: VRL_PACK(1); break;
+  }
+#undef VRL_PACK
   return launch_status();
 }
 

@@ -38,23 +38,40 @@ def _slice_messages(what: str, n_tokens: int) -> dict:
     }
 
 
+def _rows(values: torch.Tensor, what: str):
+    """-> (contiguous values, bytes per row of the leading axis, trailing shape)."""
+    if not values.is_cuda:
+        raise RuntimeError(f"values is on {values.device}; verl_amd only runs on the GPU, it has no CPU implementation")
+    if values.dim() < 1:
+        raise ValueError(f"{what}: values must be (total_nnz, *), got a scalar")
+    if values.is_nested or values.is_sparse:
+        raise TypeError(f"{what}: values must be a dense tensor (pass a nested tensor's .values())")
+    trailing = tuple(values.shape[1:])
+    inner = 1
+    for d in trailing:
+        inner *= int(d)
+    if inner == 0:
+        raise ValueError(f"{what}: values has an empty trailing dimension, shape {tuple(values.shape)}")
+    return values.contiguous(), inner * values.element_size(), trailing
+
+
 def response_slice(values: torch.Tensor, cu_seqlens: torch.Tensor, response_lens: torch.Tensor,
                    max_response_len: Optional[int] = None, check=None) -> torch.Tensor:
-    """Packed per-token fp32 ``values`` (total_nnz,) -> ``(B, max_response_len)`` block of response positions.
+    """Packed per-token ``values`` (total_nnz, *) -> ``(B, max_response_len, *)`` block of response positions, in
+    ``values``' dtype (any: the rows are copied bit for bit) with trailing dimensions kept as they are, like the
+    reference's ``no_padding_2_padding`` (verl/workers/utils/padding.py:100-101, :133-138).
 
     Row b holds ``values[end_b - r_b - 1 : end_b - 1]`` (model output is shifted left by one token) padded
     with zeros, where ``end_b = cu_seqlens[b+1]`` and ``r_b = response_lens[b]``. Like the reference it
     requires every sequence to have a prompt token and ``cu_seqlens`` to partition ``values``
     (verl/workers/utils/padding.py:129-130); a violation writes a zero row and raises ValueError, when and how is
     ``check``'s business (verl_amd.errors: None = the mode in force, True = now, False = never, "deferred").
+    With ``max_response_len`` given the call does not synchronise with the device; without it the longest response is
+    read back first, as the reference does (``response_lens.max().item()``, padding.py:117).
     """
     _errors.poll()
-    if not values.is_cuda:
-        raise RuntimeError(f"values is on {values.device}; verl_amd only runs on the GPU, it has no CPU implementation")
-    if values.dim() != 1:
-        raise ValueError(f"values must be 1-D (total_nnz,), got shape {tuple(values.shape)}")
-    dev = values.device
-    v = values.to(torch.float32).contiguous()
+    v, row_bytes, trailing = _rows(values, "response_slice")
+    dev = v.device
     cu = cu_seqlens.to(device=dev, dtype=torch.int64).contiguous()
     rl = response_lens.to(device=dev, dtype=torch.int64).contiguous()
     B = rl.numel()
@@ -63,30 +80,28 @@ def response_slice(values: torch.Tensor, cu_seqlens: torch.Tensor, response_lens
     if max_response_len is None or max_response_len < 0:
         max_response_len = int(rl.max().item()) if B > 0 else 0
     T = int(max_response_len)
-    out = torch.empty((B, T), dtype=torch.float32, device=dev)
+    out = torch.empty((B, T) + trailing, dtype=v.dtype, device=dev)
     flag = torch.zeros(1, dtype=torch.int32, device=dev)
     lib = _lib.load()
     with torch.cuda.device(dev):
-        st = lib.vrl_response_slice(v.data_ptr() if v.numel() else None, cu.data_ptr(), rl.data_ptr(), B, v.numel(), T,
-                                    out.data_ptr(), flag.data_ptr(), _lib.stream_ptr(dev))
+        st = lib.vrl_response_slice(v.data_ptr() if v.numel() else None, row_bytes, cu.data_ptr(), rl.data_ptr(), B,
+                                    v.shape[0], T, out.data_ptr(), flag.data_ptr(), _lib.stream_ptr(dev))
     _lib.check("vrl_response_slice", st)
     if B > 0 and T > 0:
-        _errors.report(flag, _slice_messages("response_slice", v.numel()), check)
+        _errors.report(flag, _slice_messages("response_slice", v.shape[0]), check)
     return out
 
 
 def response_from_packed(values: torch.Tensor, cu_seqlens: torch.Tensor, response_lens: torch.Tensor,
-                         check=None):
-    """Packed per-token fp32 ``values`` (total_nnz,) -> (packed response values ``(sum(response_lens),)``, their
-    ``cu_seqlens`` ``(B+1,)`` int64): sequence b contributes ``values[end_b - r_b - 1 : end_b - 1]``. The packed
-    counterpart of ``response_slice``; the reference does it with a Python loop and ``as_nested_tensor``
-    (verl/workers/utils/padding.py:194-210), to whose ``(values, offsets)`` pair the two results correspond."""
-    if not values.is_cuda:
-        raise RuntimeError(f"values is on {values.device}; verl_amd only runs on the GPU, it has no CPU implementation")
-    if values.dim() != 1:
-        raise ValueError(f"values must be 1-D (total_nnz,), got shape {tuple(values.shape)}")
-    dev = values.device
-    v = values.to(torch.float32).contiguous()
+                         check=None, total_response_tokens: Optional[int] = None):
+    """Packed per-token ``values`` (total_nnz, *) -> (packed response values ``(sum(response_lens), *)`` in the same
+    dtype, their ``cu_seqlens`` ``(B+1,)`` int64): sequence b contributes ``values[end_b - r_b - 1 : end_b - 1]``. The
+    packed counterpart of ``response_slice``; the reference does it with a Python loop and ``as_nested_tensor``
+    (verl/workers/utils/padding.py:194-210), to whose ``(values, offsets)`` pair the two results correspond.
+    ``total_response_tokens`` (= ``sum(response_lens)``, which sizes the result) spares the call its one read-back from
+    the device when the caller knows it; a value that is not the sum is reported like any other inconsistent offsets."""
+    v, row_bytes, trailing = _rows(values, "response_from_packed")
+    dev = v.device
     cu = cu_seqlens.to(device=dev, dtype=torch.int64).contiguous()
     rl = response_lens.to(device=dev, dtype=torch.int64).contiguous()
     B = rl.numel()
@@ -95,17 +110,22 @@ def response_from_packed(values: torch.Tensor, cu_seqlens: torch.Tensor, respons
     out_cu = torch.zeros(B + 1, dtype=torch.int64, device=dev)
     if B > 0:
         out_cu[1:] = torch.cumsum(rl.clamp(min=0), 0)
-    total = int(out_cu[-1].item()) if B > 0 else 0
-    out = torch.empty(total, dtype=torch.float32, device=dev)
+    if total_response_tokens is not None:
+        total = int(total_response_tokens)
+        if total < 0:
+            raise ValueError(f"total_response_tokens must not be negative, got {total}")
+    else:
+        total = int(out_cu[-1].item()) if B > 0 else 0
+    out = torch.empty((total,) + trailing, dtype=v.dtype, device=dev)
     flag = torch.zeros(1, dtype=torch.int32, device=dev)
     lib = _lib.load()
     with torch.cuda.device(dev):
-        st = lib.vrl_response_pack(v.data_ptr() if v.numel() else None, cu.data_ptr(), rl.data_ptr(), out_cu.data_ptr(),
-                                   B, v.numel(), total, out.data_ptr() if total > 0 else None, flag.data_ptr(),
-                                   _lib.stream_ptr(dev))
+        st = lib.vrl_response_pack(v.data_ptr() if v.numel() else None, row_bytes, cu.data_ptr(), rl.data_ptr(),
+                                   out_cu.data_ptr(), B, v.shape[0], total, out.data_ptr() if total > 0 else None,
+                                   flag.data_ptr(), _lib.stream_ptr(dev))
     _lib.check("vrl_response_pack", st)
     if B > 0:
-        _errors.report(flag, _slice_messages("response_from_packed", v.numel()), check)
+        _errors.report(flag, _slice_messages("response_from_packed", v.shape[0]), check)
     return out, out_cu
 
 
