@@ -9,17 +9,16 @@ import pytest
 import torch
 
 from verl_amd.fused_linear import linear_cross_entropy, FusedLinearForPPO, fused_linear_for_ppo
+from oracle import fused_linear as ofl
 
 pytestmark = pytest.mark.gpu
 
 
 def _torch_reference(hidden, weight, labels, temperature):
-    """run_torch_entropy of the reference's test (fp32 GEMM, softmax/logsumexp/cross_entropy)."""
-    logits = torch.matmul(hidden.float(), weight.float().t()) / temperature
-    pd = torch.softmax(logits, dim=-1)
-    entropy = torch.logsumexp(logits, dim=-1) - torch.sum(pd * logits, dim=-1)
-    logprobs = -torch.nn.functional.cross_entropy(logits, labels, reduction="none")
-    return logprobs, entropy
+    """The reference's composition in fp32 (run_torch_entropy of its test, tests/utils/test_linear_cross_entropy.py:97-118),
+    as oracle/fused_linear.py states it; differentiable with respect to hidden and weight."""
+    lp, ent, _ = ofl.forward(hidden, weight, labels, temperature, dtype=torch.float32)
+    return lp, ent
 
 
 @pytest.mark.parametrize("T,D,V,chunk", [(300, 256, 32256, 128), (257, 128, 10007, 512), (64, 64, 151936, 17)])

@@ -9,17 +9,15 @@ import torch
 
 from verl_amd import _lib
 from verl_amd.fused_linear import fused_linear_for_ppo, lm_head_score_mfma
+from oracle import fused_linear as ofl
 
 pytestmark = pytest.mark.gpu
 
 
 def _reference(h, w, ids, temp):
-    z = h.double() @ w.double().t()
-    if temp is not None:
-        z = z / (temp.double().clamp(min=1e-8)[:, None] if isinstance(temp, torch.Tensor) else float(temp))
-    lse = torch.logsumexp(z, -1)
-    lp = z.gather(-1, ids[:, None]).squeeze(-1) - lse
-    ent = lse - (torch.softmax(z, -1) * z).sum(-1)
+    """fp64 value of the reference's forward on these operands (oracle/fused_linear.py, pinned on the CPU by
+    tests/test_oracle_fused_linear.py)."""
+    lp, ent, _ = ofl.forward(h, w, ids, temp, dtype=torch.float64)
     return lp, ent
 
 
@@ -77,19 +75,13 @@ def test_benchmark_shape_against_the_chunked_fp64_composition(dev):
 
 
 def _dlogits_reference(h, w, ids, temp, g_lp, g_h):
-    """fp64 gradient of sum(g_lp * logprob + g_h * entropy) with respect to the logits, by autograd."""
-    z = (h.double() @ w.double().t()).requires_grad_(True)
-    zt = z if temp is None else z / (temp.double().clamp(min=1e-8)[:, None] if isinstance(temp, torch.Tensor) else float(temp))
-    lse = torch.logsumexp(zt, -1)
-    lp = zt.gather(-1, ids[:, None]).squeeze(-1) - lse
-    ent = lse - (torch.softmax(zt, -1) * zt).sum(-1)
-    loss = 0.0
-    if g_lp is not None:
-        loss = loss + (lp * g_lp.double()).sum()
-    if g_h is not None:
-        loss = loss + (ent * g_h.double()).sum()
-    loss.backward()
-    return z.grad, lse.detach(), ent.detach()
+    """fp64 gradient of sum(g_lp * logprob + g_h * entropy) with respect to the logits (closed form of
+    verl/utils/experimental/torch_functional.py:66-78 as oracle/fused_linear.py states it), with the logsumexp and
+    entropy the backward kernel is handed."""
+    z = ofl.logits_of(h, w, temp, dtype=torch.float64)
+    lp, ent, lse = ofl.forward(h, w, ids, temp, dtype=torch.float64)
+    d = ofl.dlogits(z, ids, None if g_lp is None else g_lp.double(), None if g_h is None else g_h.double(), temp)
+    return d, lse, ent
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
