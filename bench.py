@@ -3,7 +3,7 @@
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c2|c3|c4|c1|c5]
     python bench.py --backward [--workload ...]          (the row op's backward kernel)
-    python bench.py --lm-head [--chunk N] [--keep-logits]  (LM head + scoring without the full logits)
+    python bench.py --lm-head [--chunk N] [--keep-logits auto|yes|no]  (LM head + scoring, forward + backward)
     python bench.py --score-responses                     (packed logits -> (B, T) blocks in one launch, and its backward)
     python bench.py --ceilings                            (plain read / copy of the same buffers, matrix-core probe)
 
@@ -452,7 +452,8 @@ def bench_lm_head(args, dev):
     ids = torch.randint(0, V, (T,), generator=g, device=dev)
     g_lp = torch.randn(T, generator=g, device=dev)
     g_h = torch.randn(T, generator=g, device=dev) * 0.01
-    temperature, chunk, keep = 1.5, args.chunk, args.keep_logits
+    temperature, chunk = 1.5, args.chunk
+    keep = {"auto": None, "yes": True, "no": False}[args.keep_logits]
 
     def fwd():
         with torch.no_grad():
@@ -499,17 +500,25 @@ def bench_lm_head(args, dev):
     del zz
     if not (e3 <= 1e-4 and e4 <= 1e-4):   # fp32 sums of exact products on both sides; only the order differs
         raise SystemExit(f"bench: matrix-core LM-head scores disagree with torch (log-prob {e3}, entropy {e4})")
-    def fwd_bwd_mfma():
-        lp, h = fused_linear_for_ppo(hidden, weight, ids, temperature, chunk, False, "mfma")
+    def fwd_bwd_recompute():
+        lp, h = fused_linear_for_ppo(hidden, weight, ids, temperature, chunk, False, "auto")
+        return torch.autograd.grad((lp, h), (hidden, weight), (g_lp, g_h))
+
+    def fwd_bwd_kept():
+        lp, h = fused_linear_for_ppo(hidden, weight, ids, temperature, chunk, True, "auto")
         return torch.autograd.grad((lp, h), (hidden, weight), (g_lp, g_h))
 
     def fwd_bwd_library():
-        lp, h = fused_linear_for_ppo(hidden, weight, ids, temperature, chunk, keep, "library")
+        lp, h = fused_linear_for_ppo(hidden, weight, ids, temperature, chunk, False, "library")
+        return torch.autograd.grad((lp, h), (hidden, weight), (g_lp, g_h))
+
+    def fwd_bwd_library_kept():
+        lp, h = fused_linear_for_ppo(hidden, weight, ids, temperature, chunk, True, "library")
         return torch.autograd.grad((lp, h), (hidden, weight), (g_lp, g_h))
 
     # guard: the paths with this package's matrix-core kernels against the all-library one
     ga = fwd_bwd_library()
-    for gb, which in ((fwd_bwd(), "default"), (fwd_bwd_mfma(), "matrix-core")):
+    for gb, which in ((fwd_bwd_recompute(), "recomputing"), (fwd_bwd_kept(), "kept-logits")):
         for x, y, what in ((ga[0], gb[0], "d hidden"), (ga[1], gb[1], "d weight")):
             err = (x.float() - y.float()).abs().max().item()
             if not err <= 3e-2 * max(x.float().abs().max().item(), 1e-6):
@@ -526,51 +535,114 @@ def bench_lm_head(args, dev):
         return best
 
     t_f, t_f_lib, t_m = timed_pairwise(fwd, fwd_library, fwd_mfma)
-    t_fb, t_fb_lib, t_fb_m = timed_pairwise(fwd_bwd, fwd_bwd_library, fwd_bwd_mfma)
+    t_fb_rec, t_fb_lib, t_fb_kept, t_fb_lib_kept = timed_pairwise(fwd_bwd_recompute, fwd_bwd_library, fwd_bwd_kept,
+                                                                  fwd_bwd_library_kept)
+    from verl_amd import fused_linear as _fl
+    kept_by_default = keep is True or (keep is None and T * V * 2 <= _fl.DEFAULT_KEEP_LOGITS_BYTES)
+    t_fb = t_fb_kept if kept_by_default else t_fb_rec
     wt = torch.empty(D, V, dtype=weight.dtype, device=dev)
     t_tr = timed(lambda: transpose_2d(weight.detach(), wt))
-    # the two products of the backward on one chunk's worth of tokens, own kernel against the library on operands laid
-    # out as the library likes them best (transposed copies made beforehand and not timed)
+    # Kernel by kernel: `launches` calls back to back between one HIP event pair; the library's products beside the
+    # package's own on operands laid out as the library likes them best (transposed copies made beforehand, not timed).
+    from verl_amd import fused_linear as own_fl
     from verl_amd import gemm as own_gemm
+
+    lib = _lib.load()
+    stream = torch.cuda.current_stream(dev).cuda_stream
     n_c = min(chunk, T)
+    flops_c, flops_all = 2.0 * n_c * D * V, 2.0 * T * D * V
+
+    def rec(kernel, what, ms, flops, library_ms=None):
+        r = {"kernel": kernel, "what": what, "avg_kernel_ms": ms, "flops": flops, "tflops": flops / ms / 1e9,
+             "frac": flops / ms / 1e9 / MFMA_BF16_PEAK_TFLOPS}
+        if library_ms is not None:
+            r["library_ms"] = library_ms
+        return r
+
+    def per_launch(fn, n=10):
+        spin_up(fn, 200.0)
+        return batch_time_ms(fn, n, 3)
+
     with torch.no_grad():
         G = (torch.randn(n_c, V, generator=g, device=dev) * 0.01).bfloat16()
-        Hc = hidden.detach()[:n_c]
+        Hd, Wd = hidden.detach(), weight.detach()
+        Hc = Hd[:n_c]
         Ht = transpose_2d(Hc)
         d_h = torch.empty(n_c, D, dtype=torch.bfloat16, device=dev)
         d_w = torch.zeros(V, D, dtype=torch.bfloat16, device=dev)
-        Wd = weight.detach()
-        products = {
-            "tokens": n_c,
-            "d_hidden": {"own_ms": timed(lambda: own_gemm.gemm(Wd, G, x_t=True, out=d_h)) * 1e3,
-                         "library_ms": timed(lambda: torch.matmul(G, wt.t(), out=d_h)) * 1e3},
-            "d_weight_stored": {"own_ms": timed(lambda: own_gemm.gemm(Hc, G, x_t=True, y_t=True, out=d_w)) * 1e3,
-                                "library_ms": timed(lambda: torch.matmul(G.t(), Ht.t(), out=d_w)) * 1e3},
-            "d_weight_accumulated": {"own_ms": timed(lambda: own_gemm.gemm(Hc, G, x_t=True, y_t=True, out=d_w, accumulate=True)) * 1e3,
-                                     "library_ms": timed(lambda: d_w.addmm_(G.t(), Ht.t())) * 1e3},
-            "note": "own: vrl_gemm on W, the hidden states and the gradient buffer as they lie; library: torch.matmul / "
-                    "addmm_ on the transposed copies of W and of the hidden chunk (made beforehand, not timed)",
-        }
-        del G, Ht, d_h, d_w
-    flops_f, flops_fb = 2.0 * T * D * V, 6.0 * T * D * V
+        lp_f, ent_f, lse_f, _ = own_fl._own_forward(Hd, Wd, ids, torch.full((T,), temperature, device=dev), None, "bench")
+        temp_c = torch.full((n_c,), temperature, device=dev)
+        splits_c = lib.vrl_lmhead_plan(n_c, V)
+
+        def dlogits():
+            st = lib.vrl_lmhead_dlogits(Hc.data_ptr(), Wd.data_ptr(), _lib.VRL_BF16, n_c, V, D, D, D, ids.data_ptr(),
+                                        temp_c.data_ptr(), lse_f.data_ptr(), ent_f.data_ptr(), g_lp.data_ptr(),
+                                        g_h.data_ptr(), splits_c, G.data_ptr(), V, stream)
+            _lib.check("vrl_lmhead_dlogits", st)
+
+        kernels = [
+            rec("lmhead_partial_kernel<bf16, false> + lmhead_finish_kernel", f"forward, {T} tokens", t_m * 1e3, flops_all),
+            rec("lmhead_partial_kernel<bf16, true> + lmhead_finish_kernel", f"forward that also writes the logits, {T} tokens",
+                per_launch(lambda: own_fl._own_forward(Hd, Wd, ids, None, None, "bench", keep=True), 5), flops_all),
+            rec("lmhead_dlogits_kernel<bf16>", f"logits formed again, their gradient written, {n_c} tokens", per_launch(dlogits),
+                flops_c),
+        ]
+        G.copy_((torch.randn(n_c, V, generator=g, device=dev) * 0.01).bfloat16())
+        kernels += [
+            rec("lm_gemm_kernel<bf16, 0, true, false>", f"d hidden = G . W, {n_c} tokens",
+                per_launch(lambda: own_gemm.gemm(Wd, G, x_t=True, out=d_h)), flops_c,
+                per_launch(lambda: torch.matmul(G, wt.t(), out=d_h))),
+            rec("lm_gemm_kernel<bf16, 0, true, true>", f"d W = G^T . H stored, {n_c} tokens",
+                per_launch(lambda: own_gemm.gemm(Hc, G, x_t=True, y_t=True, out=d_w)), flops_c,
+                per_launch(lambda: torch.matmul(G.t(), Ht.t(), out=d_w))),
+            rec("lm_gemm_kernel<bf16, 1, true, true>", f"d W += G^T . H accumulated, {n_c} tokens",
+                per_launch(lambda: own_gemm.gemm(Hc, G, x_t=True, y_t=True, out=d_w, accumulate=True)), flops_c,
+                per_launch(lambda: d_w.addmm_(G.t(), Ht.t()))),
+        ]
+        del G, Ht
+        if T > n_c:
+            G8 = (torch.randn(T, V, generator=g, device=dev) * 0.01).bfloat16()
+            H8t = transpose_2d(Hd)
+            d_h8 = torch.empty(T, D, dtype=torch.bfloat16, device=dev)
+            kernels += [
+                rec("lm_gemm_kernel<bf16, 0, true, false>", f"d hidden = G . W, {T} tokens (kept logits)",
+                    per_launch(lambda: own_gemm.gemm(Wd, G8, x_t=True, out=d_h8), 5), flops_all,
+                    per_launch(lambda: torch.matmul(G8, wt.t(), out=d_h8), 5)),
+                rec("lm_gemm_kernel<bf16, 0, true, true>", f"d W = G^T . H stored, {T} tokens (kept logits)",
+                    per_launch(lambda: own_gemm.gemm(Hd, G8, x_t=True, y_t=True, out=d_w), 5), flops_all,
+                    per_launch(lambda: torch.matmul(G8.t(), H8t.t(), out=d_w), 5)),
+            ]
+            del G8, H8t, d_h8
+        del d_h, d_w
+    flops_f = 2.0 * T * D * V
+    executed = (3 if kept_by_default else 4) * flops_f
     ceiling = mfma_ceiling(dev, args.steps)
     return {
-        "metric": "tokens/sec of LM head + scoring, forward + backward, never holding more than one chunk of logits",
+        "metric": "tokens/sec of LM head + scoring, forward + backward",
         "value": T / t_fb, "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": t_fb * 1e3, "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16",
         "data": "synthetic",
-        "config": {"workload": "lm_head_8192x3584_v152064_bf16", "chunk_tokens": chunk, "keep_logits": keep,
-                   "temperature": temperature,
-                   "step": "verl_amd.fused_linear_for_ppo forward + torch.autograd.grad for hidden and weight, default "
-                           "kernels (\"auto\": vrl_lmhead_score forward; backward vrl_lmhead_dlogits, vrl_gemm for d hidden and "
-                           "d W, operands read in place; no library GEMM)"},
+        "config": {"workload": "lm_head_8192x3584_v152064_bf16", "chunk_tokens": chunk, "keep_logits": args.keep_logits,
+                   "logits_kept": kept_by_default, "temperature": temperature,
+                   "step": "verl_amd.fused_linear_for_ppo forward + torch.autograd.grad for hidden and weight with the "
+                           "package's own kernels throughout (no library GEMM): " +
+                           ("forward that also writes the logits, vrl_rowscore_backward over them in place, one vrl_gemm each "
+                            "for d hidden and d W" if kept_by_default else
+                            "vrl_lmhead_score forward; per chunk vrl_lmhead_dlogits and vrl_gemm for d hidden and d W")},
         "forward_ms": t_f * 1e3,
         "forward_tokens_per_s": T / t_f,
-        "roofline": {"bound": "mfma", "achieved": flops_fb / t_fb / 1e12, "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
-                     "frac": flops_fb / t_fb / 1e12 / MFMA_BF16_PEAK_TFLOPS, "traffic": None,
-                     "kernel": "lmhead_partial_kernel<bf16> + lmhead_finish_kernel, lmhead_dlogits_kernel<bf16>, "
-                               "lm_gemm_kernel<bf16> (d hidden, d W)",
+        "roofline": {"bound": "mfma", "achieved": 3 * flops_f / t_fb / 1e12, "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
+                     "frac": 3 * flops_f / t_fb / 1e12 / MFMA_BF16_PEAK_TFLOPS, "traffic": None,
+                     "flops": "algorithmic: 2*T*D*V forward + 4*T*D*V backward",
+                     "executed_flops_frac": executed / t_fb / 1e12 / MFMA_BF16_PEAK_TFLOPS,
+                     "kernel": "whole step; the kernels one by one are under `kernels`",
                      "forward_tflops": flops_f / t_f / 1e12},
+        "kernels": kernels,
+        "paths_forward_backward_ms": {
+            "own kernels, logits kept (default when they fit DEFAULT_KEEP_LOGITS_BYTES)": t_fb_kept * 1e3,
+            "own kernels, logits formed again per chunk (keep_logits=False)": t_fb_rec * 1e3,
+            "library products, logits kept": t_fb_lib_kept * 1e3,
+            "library products, logits formed again per chunk": t_fb_lib * 1e3},
         "single_kernel_forward": {"ms": t_m * 1e3, "tflops": flops_f / t_m / 1e12, "frac_of_mfma_peak": flops_f / t_m / 1e12 / MFMA_BF16_PEAK_TFLOPS,
                                   "kernel": "lmhead_partial_kernel<bf16> + lmhead_finish_kernel (vrl_lmhead_score)",
                                   "parity_guard": {"rows": int(pick.numel()), "max_abs_err_logprob": e3, "max_abs_err_entropy": e4},
@@ -578,16 +650,10 @@ def bench_lm_head(args, dev):
                                   "note": "hand-written MFMA kernel, logits never written"},
         "matrix_core_ceiling": ceiling,
         "all_library": {"forward_ms": t_f_lib * 1e3, "forward_backward_ms": t_fb_lib * 1e3,
+                        "forward_backward_kept_ms": t_fb_lib_kept * 1e3,
                         "kernel": "torch.matmul for every product (kernels=\"library\")"},
-        "matrix_core_backward": {"forward_backward_ms": t_fb_m * 1e3,
-                                 "kernel": "kernels=\"mfma\": the same kernels as the default today",
-                                 "note": "the logits are formed again by the hand-written MFMA kernel and their gradient "
-                                         "is written from registers (no GEMM into the buffer, no pass over it); d hidden "
-                                         "and d W come from the same main loop, which reads W, the hidden states and the "
-                                         "gradient buffer as they lie (transposing LDS reads)"},
-        "backward_products": products,
         "weight_transpose": {"ms": t_tr * 1e3, "gbps": 2.0 * V * D * 2 / t_tr / 1e9, "kernel": "transpose_kernel<2>",
-                             "note": "the copy the all-library backward makes once per call; the default path needs none"},
+                             "note": "the copy the all-library backward makes once per call; the package's own path needs none"},
         "parity_guard": {"rows": 256, "max_abs_err_logprob": e1, "max_abs_err_entropy": e2},
     }
 
@@ -977,7 +1043,8 @@ def main():
     ap.add_argument("--lm-head", action="store_true",
                     help="time the LM head + scoring step (verl_amd.fused_linear) instead of the fused forward step")
     ap.add_argument("--chunk", type=int, default=4096, help="--lm-head: tokens projected at a time")
-    ap.add_argument("--keep-logits", action="store_true", help="--lm-head: keep the logits for the backward")
+    ap.add_argument("--keep-logits", choices=["auto", "yes", "no"], default="auto",
+                    help="--lm-head: keep the logits for the backward (auto: when they fit the package's default budget)")
     ap.add_argument("--ceilings", action="store_true",
                     help="time plain non-temporal read / copy probes with the row kernels' access pattern")
     ap.add_argument("--verify-form", choices=["auto", "two-pass", "per-sequence"], default="auto",
@@ -1043,7 +1110,7 @@ def main():
         lm.steps, lm.warmup = min(args.steps, 5), min(args.warmup, 2)
         rec = bench_lm_head(lm, dev)
         short = compact(rec)
-        short.update({k: rec[k] for k in ("forward_ms", "all_library", "backward_products")})
+        short.update({k: rec[k] for k in ("forward_ms", "all_library", "kernels", "paths_forward_backward_ms")})
         short["single_kernel_forward"] = {k: rec["single_kernel_forward"][k] for k in ("ms", "tflops", "frac_of_mfma_peak",
                                                                                      "frac_of_sustained_mfma_rate")}
         others.append(short)

@@ -262,6 +262,11 @@ int vrl_transpose(const void* src, int elem_size, int64_t rows, int64_t cols, in
  * Requirements checked on the host: n_tokens >= 256, vocab >= 256, hidden_size a multiple of 64, pitches multiples
  * of 8 elements and at most 2^28, n_tokens and vocab at most 2^30, 16-byte aligned operands, 1 <= n_splits <= 64. out_logprob (with labels
  * and err_flag), out_entropy, out_lse: any may be NULL, not all.
+ * logits_out (optional): the logits themselves, sum_k hidden[t, k] * weight[v, k] before the temperature, rounded once to the
+ * operands' type and written to logits_out[t * logits_stride + v] from the registers that hold them (vocab and logits_stride
+ * multiples of 8, 16-byte aligned): for a backward pass that may spend n_tokens * vocab elements of memory instead of
+ * forming the logits again, which then runs vrl_rowscore_backward over them in place (the reference's torch path keeps
+ * them the same way, verl/utils/experimental/torch_functional.py:33-35). The scores are folded from the fp32 values either way.
  *
  * Replaces the reference's fused linear + cross-entropy forward:
  *   verl/utils/kernel/linear_cross_entropy.py:38-85 (LinearCrossEntropy.forward)
@@ -270,7 +275,8 @@ int vrl_transpose(const void* src, int elem_size, int64_t rows, int64_t cols, in
 int vrl_lmhead_score(const void* hidden, const void* weight, int dtype, int64_t n_tokens, int64_t vocab,
                      int64_t hidden_size, int64_t h_stride, int64_t w_stride, const int64_t* labels,
                      const float* temperature, int n_splits, float* partials, float* out_logprob,
-                     float* out_entropy, float* out_lse, int32_t* err_flag, void* stream);
+                     float* out_entropy, float* out_lse, int32_t* err_flag, void* logits_out, int64_t logits_stride,
+                     void* stream);
 /*
  * vrl_lmhead_dlogits — backward counterpart of vrl_lmhead_score: the logits are formed again on the matrix cores,
  * tile by tile, and turned in registers into the gradient with respect to the logits,

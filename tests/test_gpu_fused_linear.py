@@ -34,7 +34,7 @@ def test_fp32_forward_and_backward_match_torch(dev, T, D, V, chunk):
     ref_lp, ref_ent = _torch_reference(hidden, weight, labels, temperature)
     d_ref_h, d_ref_w = torch.autograd.grad((ref_ent, ref_lp), (hidden, weight), (g_ent, g_lp))
 
-    lp, ent = fused_linear_for_ppo(hidden, weight, labels, temperature, chunk_size=chunk)
+    lp, ent = fused_linear_for_ppo(hidden, weight, labels, temperature, chunk_size=chunk, keep_logits=False)
     assert lp.dtype == torch.float32 and lp.shape == (T,) and ent.shape == (T,)
     torch.testing.assert_close(ref_lp, lp, atol=1e-4, rtol=1e-4)
     torch.testing.assert_close(ref_ent, ent, atol=1e-4, rtol=1e-4)
@@ -53,10 +53,10 @@ def test_bf16_module_3d_inputs(dev):
     weight = torch.empty(V, D, device=dev).uniform_(-0.5, 0.5, generator=g).bfloat16().requires_grad_()
     labels = torch.randint(0, V, (B, S), generator=g, device=dev)
     # the default forward keeps the logits in fp32: it sits on the all-fp32 reference
-    d_lp, d_ent = FusedLinearForPPO(chunk_size=64)(hidden, weight, labels, temperature=1.5)
+    d_lp, d_ent = FusedLinearForPPO(chunk_size=64, keep_logits=False)(hidden, weight, labels, temperature=1.5)
     f_lp, f_ent = _torch_reference(hidden.detach().view(-1, D), weight.detach(), labels.view(-1), 1.5)
     assert (d_lp.view(-1) - f_lp).abs().max().item() <= 1e-4 and (d_ent.view(-1) - f_ent).abs().max().item() <= 1e-4
-    mod = FusedLinearForPPO(chunk_size=64, kernels="library")
+    mod = FusedLinearForPPO(chunk_size=64, keep_logits=False, kernels="library")
     lp, ent = mod(hidden, weight, labels, temperature=1.5)
     assert lp.shape == (B, S) and ent.shape == (B, S)
     # the kernels' share, exactly: fp32 math on the bf16 logits the library GEMM produced
@@ -89,7 +89,7 @@ def test_bf16_long_batch_uses_transposed_operands(dev):
     labels = torch.randint(0, V, (T,), generator=g, device=dev)
     g_lp = torch.empty(T, device=dev).uniform_(-1, 1, generator=g)
     g_ent = torch.empty(T, device=dev).uniform_(-0.5, 0.5, generator=g)
-    lp, ent = fused_linear_for_ppo(hidden, weight, labels, 0.9, chunk_size=1000)
+    lp, ent = fused_linear_for_ppo(hidden, weight, labels, 0.9, chunk_size=1000, keep_logits=False)
     d_h, d_w = torch.autograd.grad((ent, lp), (hidden, weight), (g_ent, g_lp))
     lp1, ent1 = fused_linear_for_ppo(hidden, weight, labels, 0.9)          # default chunk: one chunk here
     # the library may sum a product of another height in another order: a bf16 logit can move by one rounding step
@@ -112,7 +112,7 @@ def test_keep_logits_same_results_one_backward(dev, dtype):
     labels = torch.randint(0, V, (T,), generator=g, device=dev)
     g_lp = torch.empty(T, device=dev).uniform_(-1, 1, generator=g)
     g_ent = torch.empty(T, device=dev).uniform_(-0.5, 0.5, generator=g)
-    lp0, ent0 = fused_linear_for_ppo(hidden, weight, labels, 1.3, chunk_size=512)
+    lp0, ent0 = fused_linear_for_ppo(hidden, weight, labels, 1.3, chunk_size=512, keep_logits=False)
     dh0, dw0 = torch.autograd.grad((ent0, lp0), (hidden, weight), (g_ent, g_lp))
     lp1, ent1 = fused_linear_for_ppo(hidden, weight, labels, 1.3, chunk_size=512, keep_logits=True)
     assert torch.equal(lp0, lp1) and torch.equal(ent0, ent1)
@@ -178,7 +178,7 @@ def test_input_checks(dev):
     with pytest.raises(ValueError):
         fused_linear_for_ppo(h, w, ids[:3])
     with pytest.raises(ValueError):
-        fused_linear_for_ppo(h, w, ids, chunk_size=0)
+        fused_linear_for_ppo(h, w, ids, chunk_size=0, keep_logits=False)
     with pytest.raises(IndexError):
         fused_linear_for_ppo(h, w, torch.full((4,), 16, device=dev))
     # the kernels read the ids through a raw device pointer: ids that live on the host are moved, never dereferenced

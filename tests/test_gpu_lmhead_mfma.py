@@ -125,7 +125,7 @@ def test_dlogits_matches_fp64_autograd(dev, dtype, T, V, K, splits):
 def test_backward_products_come_from_the_matrix_core_kernel(dev, kernels):
     """Unless told "library", the backward forms d hidden and d W with vrl_gemm, reading the weight, the hidden states and
     the gradient buffer in place: same tolerances against torch autograd as the other paths, and the launches are
-    counted (two per chunk; with kept logits d hidden only, the single d W product over all tokens is the library's)."""
+    counted (two per chunk; with kept logits one d hidden and one d W product over all tokens)."""
     from verl_amd import gemm
 
     g = torch.Generator(device=dev).manual_seed(78)
@@ -139,7 +139,7 @@ def test_backward_products_come_from_the_matrix_core_kernel(dev, kernels):
     ref_ent = torch.logsumexp(logits, -1) - (torch.softmax(logits, -1) * logits).sum(-1)
     ref_lp = -torch.nn.functional.cross_entropy(logits, labels, reduction="none")
     d_ref_h, d_ref_w = torch.autograd.grad((ref_ent, ref_lp), (hidden, weight), (g_ent, g_lp))
-    for chunk, keep, launches in ((1024, False, 6), (4096, False, 2), (4096, True, 1)):
+    for chunk, keep, launches in ((1024, False, 6), (4096, False, 2), (4096, True, 2)):
         before = gemm.counters["gemm"]
         lp, ent = fused_linear_for_ppo(hidden, weight, labels, 1.5, chunk_size=chunk, keep_logits=keep, kernels=kernels)
         d_h, d_w = torch.autograd.grad((ent, lp), (hidden, weight), (g_ent, g_lp))
@@ -153,8 +153,9 @@ def test_backward_products_come_from_the_matrix_core_kernel(dev, kernels):
 
 
 def test_benchmark_shape_backward_against_fp64(dev):
-    """8192 tokens x 3584 -> 152064 bf16, chunks of 4096 (what bench.py --lm-head times): d hidden and d W of the default
-    path (vrl_lmhead_dlogits + vrl_gemm, two chunks, the second accumulated) against the closed-form gradient in fp64,
+    """8192 tokens x 3584 -> 152064 bf16, chunks of 4096 (what bench.py --lm-head times): d hidden and d W of the
+    recomputing path (vrl_lmhead_dlogits + vrl_gemm, two chunks, the second accumulated) and of the default at this size
+    (logits kept by the forward kernel, vrl_rowscore_backward in place, one product each) against the closed-form gradient in fp64,
     formed 1024 tokens at a time; the all-library path is measured against the same reference beside it. Bar: 2^-7 +
     2^-10 of the largest reference element: a row of either gradient is dominated by its label term, whose factor from
     the gradient buffer is rounded to bf16 once (up to 2^-8 relative) before the product is rounded to bf16 again (2^-8);
@@ -168,9 +169,9 @@ def test_benchmark_shape_backward_against_fp64(dev):
     g_lp = torch.empty(T, device=dev).uniform_(-1, 1, generator=g)
     g_ent = torch.empty(T, device=dev).uniform_(-0.5, 0.5, generator=g)
     got = {}
-    for kernels in ("auto", "library"):
-        lp, ent = fused_linear_for_ppo(h, w, ids, temp, chunk_size=4096, kernels=kernels)
-        got[kernels] = torch.autograd.grad((lp, ent), (h, w), (g_lp, g_ent))
+    for name, kernels, keep in (("auto", "auto", False), ("library", "library", False), ("auto, logits kept", "auto", None)):
+        lp, ent = fused_linear_for_ppo(h, w, ids, temp, chunk_size=4096, keep_logits=keep, kernels=kernels)
+        got[name] = torch.autograd.grad((lp, ent), (h, w), (g_lp, g_ent))
         del lp, ent
     w64 = w.detach().double()
     ref_dw = torch.zeros(V, K, dtype=torch.float64, device=dev)
@@ -211,14 +212,14 @@ def test_fused_linear_with_the_matrix_core_kernels(dev):
     ref_lp = -torch.nn.functional.cross_entropy(logits, labels, reduction="none")
     d_ref_h, d_ref_w = torch.autograd.grad((ref_ent, ref_lp), (hidden, weight), (g_ent, g_lp))
     for chunk in (512, 4096):
-        lp, ent = fused_linear_for_ppo(hidden, weight, labels, 1.5, chunk_size=chunk, kernels="mfma")
+        lp, ent = fused_linear_for_ppo(hidden, weight, labels, 1.5, chunk_size=chunk, keep_logits=False, kernels="mfma")
         torch.testing.assert_close(ref_lp, lp, atol=1e-4, rtol=1e-4)     # the same single kernel with gradients: fp32 logits
         torch.testing.assert_close(ref_ent, ent, atol=1e-4, rtol=1e-4)
         d_h, d_w = torch.autograd.grad((ent, lp), (hidden, weight), (g_ent, g_lp))
         assert d_h.dtype == torch.bfloat16 and d_w.dtype == torch.bfloat16
         torch.testing.assert_close(d_ref_h.float(), d_h.float(), atol=1e-2, rtol=1e-2)
         torch.testing.assert_close(d_ref_w.float(), d_w.float(), atol=1e-2, rtol=1e-2)
-        lp2, ent2 = fused_linear_for_ppo(hidden, weight, labels, 1.5, chunk_size=chunk, kernels="library")
+        lp2, ent2 = fused_linear_for_ppo(hidden, weight, labels, 1.5, chunk_size=chunk, keep_logits=False, kernels="library")
         d_h2, d_w2 = torch.autograd.grad((ent2, lp2), (hidden, weight), (g_ent, g_lp))
         assert (d_h.float() - d_h2.float()).abs().max().item() <= 2e-2 * max(d_h2.float().abs().max().item(), 1e-3)
         assert (d_w.float() - d_w2.float()).abs().max().item() <= 2e-2 * max(d_w2.float().abs().max().item(), 1e-3)
@@ -247,7 +248,7 @@ def test_fused_linear_fp16_model(dev):
     d_ref_h, d_ref_w = torch.autograd.grad((ref_ent, ref_lp), (hidden, weight), (g_ent, g_lp))
     from verl_amd import gemm
     before = gemm.counters["gemm"]
-    lp, ent = fused_linear_for_ppo(hidden, weight, labels, 0.7, chunk_size=256)
+    lp, ent = fused_linear_for_ppo(hidden, weight, labels, 0.7, chunk_size=256, keep_logits=False)
     torch.testing.assert_close(ref_lp, lp, atol=1e-4, rtol=1e-4)
     torch.testing.assert_close(ref_ent, ent, atol=1e-4, rtol=1e-4)
     d_h, d_w = torch.autograd.grad((ent, lp), (hidden, weight), (g_ent, g_lp))
@@ -286,7 +287,7 @@ def test_default_forward_is_the_same_with_and_without_gradients_and_for_any_toke
     with torch.no_grad():
         lp_all, ent_all = fused_linear_for_ppo(h, w, ids, 0.8)
     hg, wg = h.clone().requires_grad_(), w.clone().requires_grad_()
-    lp_g, ent_g = fused_linear_for_ppo(hg, wg, ids, 0.8, chunk_size=256)
+    lp_g, ent_g = fused_linear_for_ppo(hg, wg, ids, 0.8, chunk_size=256, keep_logits=False)
     assert torch.equal(lp_g.detach(), lp_all) and torch.equal(ent_g.detach(), ent_all)
     for lo, hi in ((0, 100), (100, 356), (356, 700), (699, 700)):
         with torch.no_grad():
@@ -375,7 +376,7 @@ def test_matrix_core_entry_points_replay_from_a_graph(dev):
     def call(stream):
         assert lib.vrl_lmhead_score(h.data_ptr(), w.data_ptr(), BF, T, V, K, K, K, ids.data_ptr(), None, splits,
                                     partials.data_ptr(), lp.data_ptr(), ent.data_ptr(), lse.data_ptr(), flag.data_ptr(),
-                                    stream) == 0
+                                    None, 0, stream) == 0
         assert lib.vrl_lmhead_dlogits(h.data_ptr(), w.data_ptr(), BF, T, V, K, K, K, ids.data_ptr(), None, lse.data_ptr(),
                                       ent.data_ptr(), g_lp.data_ptr(), g_ent.data_ptr(), lib.vrl_lmhead_plan(T, V),
                                       G.data_ptr(), V, stream) == 0
@@ -442,3 +443,102 @@ def lib_plan_is_sane():
     lib = _lib.load()
     return (lib.vrl_lmhead_plan(8192, 152064) == 8 and lib.vrl_lmhead_plan(256, 256) == 1
             and 1 <= lib.vrl_lmhead_plan(100000, 151936) <= 64 and lib.vrl_lmhead_plan(256, 151936) == 64)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("T,V,K", [(256, 256, 64), (300, 704, 192), (1000, 304, 64), (2048, 4104, 320), (257, 18992, 512)])
+def test_forward_also_writes_the_logits_when_asked(dev, dtype, T, V, K):
+    """vrl_lmhead_score with logits_out: the scores are bit for bit those of the call without it, and the stored logits are
+    the fp64 products rounded once to the operand type (half an ulp: up to 2^-8 relative for bf16, 2^-11 for fp16, plus the
+    fp32 sum's own error), every element of the (T, V) block and nothing beyond it. Edge tiles in both directions."""
+    lib = _lib.load()
+    g = torch.Generator(device=dev).manual_seed(T + 2 * V + K)
+    h = (torch.randn(T, K, generator=g, device=dev) * 0.5).to(dtype)
+    w = (torch.randn(V, K, generator=g, device=dev) * 0.2).to(dtype)
+    ids = torch.randint(0, V, (T,), generator=g, device=dev)
+    temp = torch.rand(T, generator=g, device=dev) + 0.5
+    code = _lib.VRL_BF16 if dtype == torch.bfloat16 else _lib.VRL_F16
+    splits = lib.vrl_lmhead_plan(T, V)
+    part = torch.empty(T * splits * 4, device=dev)
+    pitch = V + 16
+    outs = []
+    for keep in (False, True):
+        lp, ent, lse = (torch.empty(T, device=dev) for _ in range(3))
+        flag = torch.zeros(1, dtype=torch.int32, device=dev)
+        logits = torch.full((T, pitch), float("nan"), dtype=dtype, device=dev)
+        with torch.cuda.device(dev):
+            st = lib.vrl_lmhead_score(h.data_ptr(), w.data_ptr(), code, T, V, K, K, K, ids.data_ptr(), temp.data_ptr(), splits,
+                                      part.data_ptr(), lp.data_ptr(), ent.data_ptr(), lse.data_ptr(), flag.data_ptr(),
+                                      logits.data_ptr() if keep else None, pitch if keep else 0, _lib.stream_ptr(dev))
+        assert st == _lib.VRL_OK, lib.vrl_strerror(st)
+        outs.append((lp, ent, lse, logits))
+    for a, b in zip(outs[0][:3], outs[1][:3]):
+        assert torch.equal(a, b)
+    logits = outs[1][3]
+    z = ofl.logits_of(h, w, None, dtype=torch.float64)
+    assert torch.isnan(logits[:, V:].float()).all()
+    got = logits[:, :V].double()
+    assert torch.isfinite(got).all()
+    rel = 2.0 ** -8 if dtype == torch.bfloat16 else 2.0 ** -11
+    assert bool(((got - z).abs() <= rel * z.abs() + 2e-6).all()), (got - z).abs().max().item()
+
+
+@pytest.mark.parametrize("T,V,D", [(2304, 32256, 512), (300, 4104, 256), (100, 1000, 320), (4100, 8200, 256)])
+def test_kept_logits_backward_runs_on_the_package_kernels(dev, T, V, D):
+    """keep_logits=True on a 16-bit model: the forward kernel writes the logits, vrl_rowscore_backward turns them into
+    their gradient in place, vrl_gemm forms d hidden and d W once each (counted; no library product except the partial
+    last step of a vocabulary that is not a multiple of 64). Token counts that are not a multiple of 64 or below one
+    256-token block are padded with zero rows. Against fp32 autograd of the reference composition at its own tolerances,
+    and against the recomputing default path."""
+    from verl_amd import gemm
+
+    g = torch.Generator(device=dev).manual_seed(T + V)
+    hidden = torch.empty(T, D, device=dev).uniform_(-0.5, 0.5, generator=g).bfloat16().requires_grad_()
+    weight = torch.empty(V, D, device=dev).uniform_(-0.5, 0.5, generator=g).bfloat16().requires_grad_()
+    labels = torch.randint(0, V, (T,), generator=g, device=dev)
+    g_ent = torch.empty(T, device=dev).uniform_(-0.5, 0.5, generator=g)
+    g_lp = torch.empty(T, device=dev).uniform_(-1, 1, generator=g)
+    r_lp, r_ent, _ = ofl.forward(hidden, weight, labels, 1.5, dtype=torch.float32)
+    d_ref_h, d_ref_w = torch.autograd.grad((r_ent, r_lp), (hidden, weight), (g_ent, g_lp))
+    lp0, ent0 = fused_linear_for_ppo(hidden, weight, labels, 1.5, keep_logits=False)
+    dh0, dw0 = torch.autograd.grad((ent0, lp0), (hidden, weight), (g_ent, g_lp))
+    before = gemm.counters["gemm"]
+    lp, ent = fused_linear_for_ppo(hidden, weight, labels, 1.5, keep_logits=True)
+    assert torch.equal(lp, lp0) and torch.equal(ent, ent0)          # the scores do not depend on keeping the logits
+    assert (lp - r_lp).abs().max().item() <= 1e-4 and (ent - r_ent).abs().max().item() <= 1e-4
+    d_h, d_w = torch.autograd.grad((ent, lp), (hidden, weight), (g_ent, g_lp), retain_graph=True)
+    assert gemm.counters["gemm"] == before + 2
+    torch.testing.assert_close(d_ref_h.float(), d_h.float(), atol=1e-2, rtol=1e-2)
+    torch.testing.assert_close(d_ref_w.float(), d_w.float(), atol=1e-2, rtol=1e-2)
+    torch.testing.assert_close(dh0.float(), d_h.float(), atol=1e-2, rtol=2e-2)
+    torch.testing.assert_close(dw0.float(), d_w.float(), atol=1e-2, rtol=2e-2)
+    with pytest.raises(RuntimeError, match="overwritten by the first backward"):
+        torch.autograd.grad((ent, lp), (hidden, weight), (g_ent, g_lp))
+    # one gradient only, and a single incoming gradient
+    lp, ent = fused_linear_for_ppo(hidden, weight.detach(), labels, 1.5, keep_logits=True)
+    (only_h,) = torch.autograd.grad(lp, hidden, g_lp)
+    lp_r, _, _ = ofl.forward(hidden, weight.detach(), labels, 1.5, dtype=torch.float32)
+    (ref_h,) = torch.autograd.grad(lp_r, hidden, g_lp)
+    torch.testing.assert_close(ref_h.float(), only_h.float(), atol=1e-2, rtol=1e-2)
+
+
+def test_logits_are_kept_by_default_when_they_fit_the_budget(dev, monkeypatch):
+    """keep_logits=None: kept when tokens x vocab x element size fits DEFAULT_KEEP_LOGITS_BYTES (a kept graph can be
+    differentiated once), recomputed chunk by chunk otherwise (any number of times); the scores are the same bits."""
+    from verl_amd import fused_linear as fl
+
+    g = torch.Generator(device=dev).manual_seed(31)
+    T, D, V = 512, 256, 4096
+    hidden = torch.empty(T, D, device=dev).uniform_(-0.5, 0.5, generator=g).bfloat16().requires_grad_()
+    weight = torch.empty(V, D, device=dev).uniform_(-0.5, 0.5, generator=g).bfloat16().requires_grad_()
+    labels = torch.randint(0, V, (T,), generator=g, device=dev)
+    g_lp = torch.empty(T, device=dev).uniform_(-1, 1, generator=g)
+    lp, _ = fused_linear_for_ppo(hidden, weight, labels)
+    torch.autograd.grad(lp, hidden, g_lp, retain_graph=True)
+    with pytest.raises(RuntimeError, match="overwritten by the first backward"):
+        torch.autograd.grad(lp, hidden, g_lp)
+    monkeypatch.setattr(fl, "DEFAULT_KEEP_LOGITS_BYTES", T * V * 2 - 1)
+    lp2, _ = fused_linear_for_ppo(hidden, weight, labels)
+    a = torch.autograd.grad(lp2, hidden, g_lp, retain_graph=True)[0]
+    b = torch.autograd.grad(lp2, hidden, g_lp)[0]
+    assert torch.equal(a, b) and torch.equal(lp, lp2)

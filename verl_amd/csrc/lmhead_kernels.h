@@ -140,8 +140,13 @@ __device__ __forceinline__ LmWork lm_work(int64_t V, int64_t T, int n_splits, in
 // computing wavefront per SIMD the pipe always has a wavefront to issue from: 6.11 against 6.49 ms for the forward at
 // 8192 x 3584 -> 152064 bf16 in one process, with the very same results. The two roles are two instantiations of the
 // walk, chosen by a wave-uniform branch, so each stays straight-line code.
-// EPILOGUE_STORES: on_tile writes to global memory. Stores count in vmcnt like loads but complete in their own order,
-// so the first barrier after on_tile waits for everything.
+// EPILOGUE_STORES != 0: on_tile writes to global memory. Stores count in vmcnt like loads but complete in their own order.
+//   1: the first barrier after on_tile waits for everything (loads and stores).
+//   2: a loading wavefront still waits only until at most its eight newest loads are in flight. Loads complete in the order
+//      they were issued, so once no more than eight operations are outstanding every older load has landed, whatever stores
+//      the epilogue put between them (a store that is still in flight only makes the wait longer, never shorter); a
+//      computing wavefront has no loads to wait for and leaves its stores to drain behind the next tile.
+// Which of the two is faster differs by kernel (1-1.5 % either way, measured per kernel in one process).
 //
 // W_CM / H_CM: that operand is stored contraction-major, M[k][row] with `stride` elements between consecutive k (the
 // layout of the other factor of a product whose contraction runs over the operands' rows, e.g. W itself in G . W).
@@ -149,7 +154,7 @@ __device__ __forceinline__ LmWork lm_work(int64_t V, int64_t T, int n_splits, in
 // In LDS the tile is [k>>3][16-row block][k&7 (^4 for odd k>>3)][16 rows]: a fragment is two transposing reads
 // (ds_read_b64_tr_b16: 16 lanes read 4 k x 16 rows and each receives the 4 k of its row), the 8 k-rows a half
 // wavefront reads fall on distinct banks, and the row block enters the address as a plain offset of 256 bytes.
-template <int DT, bool EPILOGUE_STORES, bool W_CM, bool H_CM, int LOAD_GROUP, int LOAD_PHASE, int H_DELAY, bool LOADER,
+template <int DT, int EPILOGUE_STORES, bool W_CM, bool H_CM, int LOAD_GROUP, int LOAD_PHASE, int H_DELAY, bool LOADER,
           class OnTile>
 __device__ __forceinline__ void lm_walk_tiles_as(const uint16_t* __restrict__ W, const uint16_t* __restrict__ H, int64_t V,
                                                  int64_t K, int64_t w_stride, int64_t h_stride, const LmWork& work,
@@ -333,7 +338,7 @@ __device__ __forceinline__ void lm_walk_tiles_as(const uint16_t* __restrict__ W,
 #pragma unroll
       for (int hf = 0; hf < 2; ++hf) {
         if (hf == 1) {
-          if (EPILOGUE_STORES && after_epilogue) {
+          if (EPILOGUE_STORES == 1 && after_epilogue) {
             asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
           } else if (LOADER) {
             asm volatile("s_waitcnt vmcnt(8) lgkmcnt(0)" ::: "memory");
@@ -395,7 +400,7 @@ __device__ __forceinline__ void lm_walk_tiles_as(const uint16_t* __restrict__ W,
 // single loads one instruction earlier, the gradient kernel single loads three instructions earlier. H_DELAY moves the
 // loading wavefronts' refills of the H fragments that many instructions back, away from the computing wavefronts' (which
 // stay right behind a column's last product): worth 3 % to the d hidden product, nothing or less to the others.
-template <int DT, bool EPILOGUE_STORES, bool W_CM, bool H_CM, int LOAD_GROUP, int LOAD_PHASE, int H_DELAY, class OnTile>
+template <int DT, int EPILOGUE_STORES, bool W_CM, bool H_CM, int LOAD_GROUP, int LOAD_PHASE, int H_DELAY, class OnTile>
 __device__ __forceinline__ void lm_walk_tiles(const uint16_t* __restrict__ W, const uint16_t* __restrict__ H, int64_t V,
                                               int64_t K, int64_t w_stride, int64_t h_stride, const LmWork& work,
                                               char* lds, OnTile&& on_tile) {
@@ -410,11 +415,15 @@ __device__ __forceinline__ void lm_walk_tiles(const uint16_t* __restrict__ W, co
 
 // grid.x = token blocks * n_splits, block = 512, dynamic LDS = kLmLdsBytes. Writes, per (token, split), the online-softmax
 // partial (m, s, t, 0) of the split's vocabulary tiles to partials[(token * n_splits + split) * 4 ...].
-template <int DT>
+// STORE: the logits tile (the plain products, before the temperature) is also written, in the operands' type, to
+// logits_out[tok * l_stride + v] (l_stride and V multiples of 8, 16-byte aligned base): what a backward pass that may
+// spend memory instead of forming the logits again reads (vrl_rowscore_backward over them, in place). The softmax state
+// is folded from the fp32 values all the same, so the scores do not depend on whether the logits are kept.
+template <int DT, bool STORE>
 __global__ __launch_bounds__(kLmWaves * 64, 1) void lmhead_partial_kernel(
     const uint16_t* __restrict__ W, const uint16_t* __restrict__ H, int64_t V, int64_t T, int64_t K, int64_t w_stride,
     int64_t h_stride, const float* __restrict__ temperature, int n_splits, int tiles_per_split,
-    int xcd_map, float* __restrict__ partials) {
+    int xcd_map, float* __restrict__ partials, uint16_t* __restrict__ logits_out, int64_t l_stride) {
   extern __shared__ __attribute__((aligned(1024))) char lds[];  // the operand ring; its start serves the final merge
   float (*red)[256][3] = reinterpret_cast<float (*)[256][3]>(lds);   // [4][256][3], used once the walk is over
 
@@ -436,12 +445,15 @@ __global__ __launch_bounds__(kLmWaves * 64, 1) void lmhead_partial_kernel(
     c[j] = make_scale<false>(temperature, tok).c;   // log2(e) / max(T, 1e-8), exactly what the finishing kernel uses
   }
 
-  lm_walk_tiles<DT, false, false, false, 2, 0, 0>(W, H, V, K, w_stride, h_stride, work, lds, [&](int64_t vt, lm_f32x4 (&acc)[4][8]) {
+  lm_walk_tiles<DT, STORE ? 2 : 0, false, false, 2, 0, 0>(W, H, V, K, w_stride, h_stride, work, lds, [&](int64_t vt, lm_f32x4 (&acc)[4][8]) {
     // fold 16 logits per token column into the running state (maximum first, then the exponentials; nothing is
     // buffered): acc[i][j][v] is vocabulary row tile_row0 + wv*64 + i*16 + 4*(lane>>4) + v of token column j
     const bool edge = (vt + 1) * kLmVocab > V;
     const int64_t vrow0 = (edge ? V - kLmVocab : vt * kLmVocab) + wv * 64 + 4 * (lane >> 4);
     const int64_t vfirst = vt * kLmVocab;   // rows below belong to the tile before
+    // (the row pointer is formed per tile; the empty asm keeps it out of the main loop's registers)
+    int64_t tok0v = work.tok0_ld + wt * 128 + (lane & 15);
+    if constexpr (STORE) asm volatile("" : "+v"(tok0v));
 #pragma unroll
     for (int j = 0; j < 8; ++j) {
       float x[16];
@@ -449,6 +461,22 @@ __global__ __launch_bounds__(kLmWaves * 64, 1) void lmhead_partial_kernel(
       for (int i = 0; i < 4; ++i)
 #pragma unroll
         for (int v = 0; v < 4; ++v) x[i * 4 + v] = acc[i][j][v];
+      if constexpr (STORE) {
+        using O = ElemOut<DT>;
+        if (tok0v + j * 16 >= work.tok0) {   // false for the rows an edge block shares with the block before
+          uint16_t* out = logits_out + (tok0v + j * 16) * l_stride;
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            const int64_t vr = vrow0 + i * 16;   // first of 4 consecutive vocabulary entries (a multiple of 4)
+            if (vr >= vfirst) {
+              uint2 pk;
+              pk.x = O::pack2(x[i * 4], x[i * 4 + 1]);
+              pk.y = O::pack2(x[i * 4 + 2], x[i * 4 + 3]);
+              *reinterpret_cast<uint2*>(out + vr) = pk;
+            }
+          }
+        }
+      }
       if (edge) {
 #pragma unroll
         for (int e = 0; e < 16; ++e) {
@@ -588,7 +616,7 @@ __global__ __launch_bounds__(kLmWaves * 64, 1) void lmhead_dlogits_kernel(
     label[j] = (lab >= 0 && lab < V) ? (int)lab : -1;   // an out-of-range label was reported by the forward pass
   }
 
-  lm_walk_tiles<DT, true, false, false, 1, 3, 0>(W, H, V, K, w_stride, h_stride, work, lds, [&](int64_t vt, lm_f32x4 (&acc)[4][8]) {
+  lm_walk_tiles<DT, 2, false, false, 1, 3, 0>(W, H, V, K, w_stride, h_stride, work, lds, [&](int64_t vt, lm_f32x4 (&acc)[4][8]) {
     // acc[i][j][0..3]: vocabulary entries vr .. vr+3, vr = tile_row0 + wv*64 + i*16 + 4*(lane>>4), of token column j
     const bool edge = (vt + 1) * kLmVocab > V;
     const int vrow0 = (int)(edge ? V - kLmVocab : vt * kLmVocab) + wv * 64 + 4 * (lane >> 4);
@@ -700,7 +728,7 @@ __global__ __launch_bounds__(kLmWaves * 64, 1) void lm_gemm_kernel(
 
   const uint16_t* x0 = X + step0 * kLmK * (X_CM ? x_stride : 1);
   const uint16_t* y0p = Y + step0 * kLmK * (Y_CM ? y_stride : 1);
-  lm_walk_tiles<DT, true, X_CM, Y_CM, 1, 1, (X_CM && !Y_CM) ? 1 : 0>(x0, y0p, g.NX, nsteps * kLmK, x_stride, y_stride, work, lds,
+  lm_walk_tiles<DT, 1, X_CM, Y_CM, 1, 1, (X_CM && !Y_CM) ? 1 : 0>(x0, y0p, g.NX, nsteps * kLmK, x_stride, y_stride, work, lds,
                                       [&](int64_t vt, lm_f32x4 (&acc)[4][8]) {
     // acc[i][j][0..3]: columns x0 .. x0+3 of out, x0 = tile_row0 + wv*64 + i*16 + 4*(lane>>4), of row
     // y = tok0_ld + wt*128 + j*16 + (lane&15)

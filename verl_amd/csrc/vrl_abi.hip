@@ -276,18 +276,19 @@ int raise_lds_limit(const void* kernel, std::atomic<bool>* raised) {
   return VRL_OK;
 }
 
-template <int DT>
+template <int DT, bool STORE>
 int launch_lmhead(const void* hidden, const void* weight, int64_t T, int64_t V, int64_t K, int64_t h_stride,
                   int64_t w_stride, const int64_t* labels, const float* temperature, int n_splits, float* partials,
-                  float* out_logprob, float* out_entropy, float* out_lse, int32_t* err_flag, hipStream_t s) {
+                  float* out_logprob, float* out_entropy, float* out_lse, int32_t* err_flag, void* logits_out,
+                  int64_t l_stride, hipStream_t s) {
   const LmGrid g = lm_grid(T, V, n_splits);
   static std::atomic<bool> raised[kMaxDevices];
-  const int rs = raise_lds_limit(reinterpret_cast<const void*>(vrl::lmhead_partial_kernel<DT>), raised);
+  const int rs = raise_lds_limit(reinterpret_cast<const void*>(vrl::lmhead_partial_kernel<DT, STORE>), raised);
   if (rs != VRL_OK) return rs;
-  vrl::lmhead_partial_kernel<DT><<<dim3(static_cast<unsigned>(g.tblocks * n_splits)), dim3(vrl::kLmWaves * 64),
-                                   vrl::kLmLdsBytes, s>>>(
+  vrl::lmhead_partial_kernel<DT, STORE><<<dim3(static_cast<unsigned>(g.tblocks * n_splits)), dim3(vrl::kLmWaves * 64),
+                                          vrl::kLmLdsBytes, s>>>(
       static_cast<const uint16_t*>(weight), static_cast<const uint16_t*>(hidden), V, T, K, w_stride, h_stride,
-      temperature, n_splits, g.tiles_per_split, g.xcd_map, partials);
+      temperature, n_splits, g.tiles_per_split, g.xcd_map, partials, static_cast<uint16_t*>(logits_out), l_stride);
   vrl::lmhead_finish_kernel<DT><<<dim3(static_cast<unsigned>((T + 3) / 4)), dim3(256), 0, s>>>(
       static_cast<const char*>(weight), static_cast<const char*>(hidden), V, T, K, w_stride, h_stride, labels,
       temperature, n_splits, partials, out_logprob, out_entropy, out_lse, err_flag);
@@ -793,22 +794,28 @@ int vrl_lmhead_plan(int64_t n_tokens, int64_t vocab) {
 int vrl_lmhead_score(const void* hidden, const void* weight, int dtype, int64_t n_tokens, int64_t vocab,
                      int64_t hidden_size, int64_t h_stride, int64_t w_stride, const int64_t* labels,
                      const float* temperature, int n_splits, float* partials, float* out_logprob,
-                     float* out_entropy, float* out_lse, int32_t* err_flag, void* stream) {
+                     float* out_entropy, float* out_lse, int32_t* err_flag, void* logits_out, int64_t logits_stride,
+                     void* stream) {
   const int cs = check_lmhead_shape(dtype, n_tokens, vocab, hidden_size, h_stride, w_stride, n_splits);
   if (cs != VRL_OK) return cs;
-  if (out_logprob == nullptr && out_entropy == nullptr && out_lse == nullptr) return VRL_ERR_ARG;
+  if (out_logprob == nullptr && out_entropy == nullptr && out_lse == nullptr && logits_out == nullptr) return VRL_ERR_ARG;
   if (hidden == nullptr || weight == nullptr || partials == nullptr) return VRL_ERR_NULL;
   if (out_logprob != nullptr && (labels == nullptr || err_flag == nullptr)) return VRL_ERR_NULL;
+  // kept logits: 8-byte stores of 4 consecutive vocabulary entries, so the vocabulary and the pitch must keep them aligned
+  if (logits_out != nullptr && (vocab % 8 != 0 || logits_stride < vocab || logits_stride % 8 != 0 || logits_stride > kLmMaxStride))
+    return VRL_ERR_SHAPE;
   if (!aligned(hidden, 16) || !aligned(weight, 16) || !aligned(labels, 8) || !aligned(temperature, 4) ||
       !aligned(partials, 4) || !aligned(out_logprob, 4) || !aligned(out_entropy, 4) || !aligned(out_lse, 4) ||
-      !aligned(err_flag, 4))
+      !aligned(err_flag, 4) || !aligned(logits_out, 16))
     return VRL_ERR_ALIGN;
   hipStream_t s = static_cast<hipStream_t>(stream);
+#define VRL_LMHEAD_ARGS                                                                                            \
+  hidden, weight, n_tokens, vocab, hidden_size, h_stride, w_stride, labels, temperature, n_splits, partials,        \
+      out_logprob, out_entropy, out_lse, err_flag, logits_out, logits_stride, s
   if (dtype == VRL_BF16)
-    return launch_lmhead<VRL_BF16>(hidden, weight, n_tokens, vocab, hidden_size, h_stride, w_stride, labels, temperature,
-                                   n_splits, partials, out_logprob, out_entropy, out_lse, err_flag, s);
-  return launch_lmhead<VRL_F16>(hidden, weight, n_tokens, vocab, hidden_size, h_stride, w_stride, labels, temperature,
-                                n_splits, partials, out_logprob, out_entropy, out_lse, err_flag, s);
+    return logits_out != nullptr ? launch_lmhead<VRL_BF16, true>(VRL_LMHEAD_ARGS) : launch_lmhead<VRL_BF16, false>(VRL_LMHEAD_ARGS);
+  return logits_out != nullptr ? launch_lmhead<VRL_F16, true>(VRL_LMHEAD_ARGS) : launch_lmhead<VRL_F16, false>(VRL_LMHEAD_ARGS);
+#undef VRL_LMHEAD_ARGS
 }
 
 int vrl_lmhead_dlogits(const void* hidden, const void* weight, int dtype, int64_t n_tokens, int64_t vocab,

@@ -8,13 +8,17 @@ softmax state as it forms them and never writes them (``vrl_lmhead_score``); the
 each chunk's logits again on the matrix cores and writes their gradient into a reusable ``(chunk, vocab)`` buffer
 (``vrl_lmhead_dlogits``), then forms ``d hidden`` and ``d W`` with ``vrl_gemm``, which reads the weight, the hidden states
 and the gradient buffer as they lie (no transposed copies). No library GEMM runs. Peak extra memory is that one buffer, in
-the backward only.
+the backward only. With ``keep_logits=True`` the same forward kernel also writes the logits from its registers, and the
+backward turns them into their gradient in place (``vrl_rowscore_backward``) and forms each of the two products once with
+``vrl_gemm``: a quarter fewer matrix-core flops for ``tokens x vocab`` elements of memory, still without a library GEMM.
 
-Library path (``kernels="library"``, fp32 models, ``keep_logits=True``): per chunk the projection ``hidden @ W^T`` is one
-library GEMM (torch.matmul, i.e. hipBLASLt) into the buffer, and everything after it is the HIP row kernel: forward
-``vrl_rowscore`` (one pass over the chunk's logits), backward ``vrl_rowscore_backward`` writing the gradient over the
-recomputed logits in place, followed by the two GEMMs. The reference does the post-GEMM part with ~10 torch ops per chunk
-(softmax, logsumexp, log_softmax, gather, scatter, ...; :27-79).
+Library path (``kernels="library"``, fp32 models, models the kernels' shape rules do not take): per chunk the projection
+``hidden @ W^T`` is one library GEMM (torch.matmul, i.e. hipBLASLt) into the buffer, and everything after it is the HIP row
+kernel: forward ``vrl_rowscore`` (one pass over the chunk's logits), backward ``vrl_rowscore_backward`` writing the gradient
+over the recomputed logits in place, followed by the two GEMMs. The reference does the post-GEMM part with ~10 torch ops per
+chunk (softmax, logsumexp, log_softmax, gather, scatter, ...; :27-79). fp32 models are served by the library on purpose:
+the fp32 matrix rate of the part (157 TFLOP/s) is what the library already delivers, and no model in verl's recipes runs
+its LM head in fp32.
 """
 
 from __future__ import annotations
@@ -40,20 +44,21 @@ DEFAULT_CHUNK_TOKENS = 4096
 # Which matrix products are this package's own kernels.
 #   "library": every product is torch.matmul (hipBLASLt); the row kernels run over the chunk buffer.
 #   "auto" (default) and "mfma" (the same today): every step runs this package's own matrix-core kernel.
-#              The forward is one kernel that never writes logits (vrl_lmhead_score: 6.1-6.25 ms at 8192 x 3584 ->
-#              152064 bf16 against 6.5 ms for the library GEMM + row kernel, no (chunk, vocab) buffer, logits kept
-#              in fp32), with and without gradients and whatever the number of tokens, so that old (no-grad) and new
-#              (grad) log-probs of the same weights are bit-identical when both calls cut the vocabulary alike (see
-#              DEFAULT_FORWARD_SPLITS) and a few ulps apart otherwise; the backward forms the logits again and writes
-#              their gradient from registers (vrl_lmhead_dlogits, 3.33 ms per 4096 tokens against 3.53 ms for the library
-#              GEMM + row backward) and forms d hidden and d W with vrl_gemm, which reads W, the hidden states and the
-#              gradient buffer in place: the contraction of either product runs over rows of its operands, and the kernel
-#              takes such operands through transposing LDS reads. Per 4096-token chunk d hidden takes 3.3 ms against 3.75 ms
-#              for the library (which also wants a transposed copy of W); d W 3.44 / 3.7 ms stored / accumulated against
-#              3.4 / 3.5 ms for the library on transposed copies (which also needs the copies and a zero fill of d W). keep_logits=True needs the logits in memory and therefore takes the library forward, also
-#              without gradients, and the library's single d W product over all tokens.
+#              The forward is one kernel (vrl_lmhead_score: 6.0-6.25 ms at 8192 x 3584 -> 152064 bf16 against 6.5 ms for the
+#              library GEMM + row kernel, logits kept in fp32), with and without gradients and whatever the number of
+#              tokens, so that old (no-grad) and new (grad) log-probs of the same weights are bit-identical when both calls
+#              cut the vocabulary alike (see DEFAULT_FORWARD_SPLITS) and a few ulps apart otherwise. It never writes the
+#              logits unless keep_logits=True asks for them (they then leave the kernel's registers rounded once).
+#              Without kept logits the backward forms them again and writes their gradient from registers
+#              (vrl_lmhead_dlogits, 3.2-3.3 ms per 4096 tokens against 3.5 ms for the library GEMM + row backward); with
+#              kept logits vrl_rowscore_backward turns them into their gradient in place. d hidden and d W come from
+#              vrl_gemm, which reads W, the hidden states and the gradient buffer in place: the contraction of either
+#              product runs over rows of its operands, and the kernel takes such operands through transposing LDS reads.
+#              Per 4096-token chunk d hidden takes 3.1 ms against 3.75 ms for the library (which also wants a transposed
+#              copy of W); d W 3.4 / 3.7 ms stored / accumulated against 3.3 / 3.5 ms for the library on transposed copies
+#              (which also needs the copies and a zero fill of d W).
 # The environment variable and the ``kernels`` argument select; models the kernels do not take (fp32, a hidden size that is
-# not a multiple of 64, fewer than 256 vocabulary entries) go to the library.
+# not a multiple of 64, fewer than 256 or not a multiple of 8 vocabulary entries) go to the library.
 DEFAULT_KERNELS = os.environ.get("VERL_AMD_LMHEAD_KERNELS", "auto")
 
 # Into how many ranges the single forward kernel cuts the vocabulary. None lets the library plan per call: 8 for every call
@@ -75,13 +80,19 @@ def _mfma_takes_model(hidden: torch.Tensor, weight: torch.Tensor) -> bool:
             and hidden.data_ptr() % 16 == 0 and weight.data_ptr() % 16 == 0)
 
 
-def _own_forward_in_use(kernels: str, keep_logits: bool, hidden: torch.Tensor, weight: torch.Tensor) -> bool:
-    """Whether the forward is vrl_lmhead_score. Decided by the caller's options and by the model only, never by the number
-    of tokens or by whether gradients are recorded: a trainer's old (no-grad) and new (grad) log-probs of the same
-    weights then come from the same kernel whatever the micro-batch sizes are (and from the same summation order when
-    the calls use the same number of vocabulary ranges, see DEFAULT_FORWARD_SPLITS)."""
-    return kernels != "library" and not keep_logits and _mfma_takes_model(hidden, weight)
+def _own_forward_in_use(kernels: str, hidden: torch.Tensor, weight: torch.Tensor) -> bool:
+    """Whether the forward is vrl_lmhead_score. Decided by the ``kernels`` option and by the model only, never by the
+    number of tokens, by ``keep_logits`` or by whether gradients are recorded: a trainer's old (no-grad) and new (grad)
+    log-probs of the same weights then come from the same kernel whatever the micro-batch sizes are (and from the same
+    summation order when the calls use the same number of vocabulary ranges, see DEFAULT_FORWARD_SPLITS)."""
+    return kernels != "library" and _mfma_takes_model(hidden, weight)
 
+
+# keep_logits=None (the default) keeps the logits for the backward when all of them fit this many bytes: on a 288 GB part
+# the 2.5 GB of an 8192 x 152064 bf16 micro-batch are under 1 % of the memory and save a quarter of the matrix-core flops
+# (20.7 ms forward + backward instead of 26.0 ms); a call whose logits are larger recomputes them chunk by chunk as the
+# reference does. The environment variable VERL_AMD_LMHEAD_KEEP_BYTES sets the limit (0: never keep unless asked).
+DEFAULT_KEEP_LOGITS_BYTES = int(os.environ.get("VERL_AMD_LMHEAD_KEEP_BYTES", str(4 << 30)))
 
 # From this many tokens on, one transposed copy of the weight per backward (0.44 ms for 152064 x 3584 bf16) is
 # repaid by the faster `d hidden` product.
@@ -106,15 +117,22 @@ def _padded(x: torch.Tensor, rows: int) -> torch.Tensor:
 def _d_hidden(grad_logits, weight, weight_t, out, own_kernel):
     """out = grad_logits @ weight: this package's matrix-core kernel (``vrl_gemm``, the weight read as it lies) when
     asked for and the shapes allow, the library otherwise (with the transposed copy of the weight when there is one:
-    both operands contiguous along the vocabulary)."""
-    if own_kernel and _own_d_hidden_takes(grad_logits, weight, out):
-        _gemm.gemm(weight, grad_logits, x_t=True, out=out)
+    both operands contiguous along the vocabulary). The kernel contracts in steps of 64: of a vocabulary that is not a
+    multiple of 64 it takes the whole steps and the library adds the last, partial one (fewer than 64 columns)."""
+    V = weight.shape[0]
+    main = V // 64 * 64
+    if own_kernel and main >= 128 and _own_d_hidden_takes(grad_logits[:, :main], weight[:main], out):
+        _gemm.gemm(weight[:main], grad_logits[:, :main], x_t=True, out=out)
+        if main != V:
+            out.addmm_(grad_logits[:, main:], weight[main:])
     else:
         torch.matmul(grad_logits, weight if weight_t is None else weight_t.t(), out=out)
 
 
 def _own_d_hidden_takes(grad_logits, weight, out) -> bool:
-    return _gemm.gemm_takes(weight, grad_logits, True, False) and out.stride(0) % 4 == 0 and out.stride(1) == 1
+    """Everything vrl_gemm checks about the operands of d hidden, so that what it would refuse goes to the library."""
+    return (_gemm.gemm_takes(weight, grad_logits, True, False) and out.stride(0) % 4 == 0 and out.stride(1) == 1
+            and out.data_ptr() % 8 == 0 and out.stride(0) >= weight.shape[1])
 
 
 class _FusedLinearForPPOFunction(torch.autograd.Function):
@@ -130,17 +148,20 @@ class _FusedLinearForPPOFunction(torch.autograd.Function):
         h = torch.empty(T, **f32)
         lse = torch.empty(T, **f32)
         flag = torch.zeros(1, dtype=torch.int32, device=dev)
-        if _own_forward_in_use(kernels, keep_logits, hidden, weight):
+        keep = bool(keep_logits) and T > 0 and (ctx.needs_input_grad[0] or ctx.needs_input_grad[1])
+        ctx.own_kept = False
+        if _own_forward_in_use(kernels, hidden, weight):
             temp_all = None if temperature == 1.0 else torch.full((T,), float(temperature), **f32)
-            lp, h, lse = _own_forward(hidden, weight, input_ids, temp_all, forward_splits, "fused_linear_for_ppo")
+            lp, h, lse, kept = _own_forward(hidden, weight, input_ids, temp_all, forward_splits, "fused_linear_for_ppo",
+                                            keep=keep)
             ctx.save_for_backward(hidden, weight, input_ids, lse, h)
             ctx.temperature = float(temperature)
             ctx.chunk_size = int(chunk_size)
-            ctx.kept_logits = None
+            ctx.kept_logits = kept
+            ctx.own_kept = kept is not None
             return lp.clone(), h.clone()
         temp = None if temperature == 1.0 else torch.full((min(chunk_size, max(T, 1)),), float(temperature), **f32)
         lib = _lib.load()
-        keep = bool(keep_logits) and T > 0 and (ctx.needs_input_grad[0] or ctx.needs_input_grad[1])
         rows = T if keep else min(chunk_size, max(T, 1))
         buf = torch.empty((rows, V), dtype=hidden.dtype, device=dev)
         with torch.cuda.device(dev):
@@ -184,6 +205,30 @@ class _FusedLinearForPPOFunction(torch.autograd.Function):
         d_weight = torch.empty_like(weight) if need_dw else None
         dw_started = False     # whether d_weight holds a partial sum yet
         lib = _lib.load()
+        if kept is not None and ctx.own_kept:
+            # The forward kernel left the logits of all tokens (rows padded to a multiple of 64 with zero hidden states,
+            # whose logits and hence gradients are zero): their gradient is written over them, and each product runs once
+            # over all tokens with this package's kernel, nothing to accumulate.
+            m = kept.shape[0]
+            temp_rows = None if ctx.temperature == 1.0 else torch.full((T,), ctx.temperature, **f32)
+            with torch.cuda.device(dev):
+                st = lib.vrl_rowscore_backward(
+                    kept.data_ptr(), _DTYPE_CODES[hidden.dtype], T, V, kept.stride(0), input_ids.data_ptr(),
+                    _ptr(temp_rows), lse.data_ptr(), h.data_ptr(), _ptr(gl), _ptr(gh), kept.data_ptr(), kept.stride(0),
+                    _lib.stream_ptr(dev))
+            _lib.check("vrl_rowscore_backward", st)
+            if need_dh:
+                out = d_hidden if m == T else torch.empty((m, D), dtype=hidden.dtype, device=dev)
+                _d_hidden(kept, weight, None, out, True)
+                if m != T:
+                    d_hidden.copy_(out[:T])
+            if need_dw:
+                c_h = hidden if m == T else _padded(hidden, m)
+                if _gemm.gemm_takes(c_h, kept, True, True):
+                    _gemm.gemm(c_h, kept, x_t=True, y_t=True, out=d_weight)
+                else:
+                    torch.matmul(kept[:T].t(), hidden, out=d_weight)
+            return d_hidden, d_weight, None, None, None, None, None, None
         # With this package's own kernels every chunk is at least one block of 256 tokens: a smaller chunk size is raised
         # to 256, a short tail joins the chunk before it, and a call with fewer than 256 tokens is padded to one block
         # (zero hidden states and zero incoming gradients give zero rows), so the backward never falls back to logits
@@ -278,8 +323,9 @@ class _FusedLinearForPPOFunction(torch.autograd.Function):
 
 
 def fused_linear_for_ppo(hidden_states: torch.Tensor, vocab_weights: torch.Tensor, input_ids: torch.Tensor,
-                         temperature: float = 1.0, chunk_size: int = DEFAULT_CHUNK_TOKENS, keep_logits: bool = False,
-                         kernels: Optional[str] = None, forward_splits: Optional[int] = None):
+                         temperature: float = 1.0, chunk_size: int = DEFAULT_CHUNK_TOKENS,
+                         keep_logits: Optional[bool] = None, kernels: Optional[str] = None,
+                         forward_splits: Optional[int] = None):
     """(log_probs fp32, entropy fp32) of ``softmax((hidden_states @ vocab_weights.T) / temperature)`` at ``input_ids``.
 
     ``hidden_states`` is ``(tokens, hidden)`` or ``(batch, seq, hidden)`` with ``input_ids`` of the matching leading
@@ -289,8 +335,11 @@ def fused_linear_for_ppo(hidden_states: torch.Tensor, vocab_weights: torch.Tenso
     this GPU rather than the reference's 512.
 
     ``keep_logits=True`` trades memory for time when gradients are needed: the forward keeps all
-    ``tokens x vocab`` logits (2.5 GB for 8192 x 152064 bf16), the backward writes their gradient over them instead of
-    projecting again and forms ``d hidden`` and ``d W`` with one product each. Such a graph can be differentiated once.
+    ``tokens x vocab`` logits (2.5 GB for 8192 x 152064 bf16; written by the same forward kernel from its registers), the
+    backward writes their gradient over them instead of projecting again and forms ``d hidden`` and ``d W`` with one
+    product each. Such a graph can be differentiated once. The scores do not depend on it. ``None`` (the default) keeps
+    them when all of them fit ``DEFAULT_KEEP_LOGITS_BYTES`` (4 GiB unless ``VERL_AMD_LMHEAD_KEEP_BYTES`` says otherwise) and
+    recomputes otherwise; ``False`` never holds more than one chunk of logits, like the reference.
 
     ``kernels`` chooses which matrix products are this package's own kernels: ``"library"`` (none: torch.matmul
     throughout) or ``"auto"`` / ``"mfma"`` (all of them: a forward that is one kernel and never
@@ -334,27 +383,31 @@ def fused_linear_for_ppo(hidden_states: torch.Tensor, vocab_weights: torch.Tenso
     ids = input_ids.reshape(-1).to(device=h2.device, dtype=torch.int64).contiguous()
     w2 = vocab_weights.contiguous()
     needs_grad = torch.is_grad_enabled() and (h2.requires_grad or w2.requires_grad)
-    if not needs_grad and _own_forward_in_use(kernels, keep_logits, h2, w2):
+    if keep_logits is None:
+        keep_logits = needs_grad and h2.shape[0] * w2.shape[0] * h2.element_size() <= DEFAULT_KEEP_LOGITS_BYTES
+    if not needs_grad and _own_forward_in_use(kernels, h2, w2):
         temp = None if float(temperature) == 1.0 else torch.full((h2.shape[0],), float(temperature), dtype=torch.float32,
                                                                   device=h2.device)
         with torch.no_grad():
-            lp, ent, _ = _own_forward(h2, w2, ids, temp, forward_splits, "fused_linear_for_ppo")
+            lp, ent, _, _ = _own_forward(h2, w2, ids, temp, forward_splits, "fused_linear_for_ppo")
         return lp.reshape(lead), ent.reshape(lead)
     lp, ent = _FusedLinearForPPOFunction.apply(h2, w2, ids, float(temperature), int(chunk_size), bool(keep_logits),
                                                kernels, None if forward_splits is None else int(forward_splits))
     return lp.reshape(lead), ent.reshape(lead)
 
 
-def _own_forward(h, w, ids, temp, n_splits, what):
-    """(log-prob, entropy, logsumexp), fp32, of the rows of ``h`` from vrl_lmhead_score. ``temp`` is None or one value per
-    token. The kernels work on blocks of 256 tokens: a shorter input is copied into a zero-padded block first."""
+def _own_forward(h, w, ids, temp, n_splits, what, keep=False):
+    """(log-prob, entropy, logsumexp, kept logits), the first three fp32 per row of ``h``, from vrl_lmhead_score. ``temp``
+    is None or one value per token. The kernels work on blocks of 256 tokens: a shorter input is copied into a zero-padded
+    block first. With ``keep`` the kernel also writes the logits, into a buffer whose rows are padded to a multiple of 64
+    (the step of the contraction of d W): rows past the input hold the logits of zero hidden states, zeros."""
     T, K = h.shape
     V = w.shape[0]
     dev = h.device
     f32 = dict(dtype=torch.float32, device=dev)
     if T == 0:
-        return torch.empty(0, **f32), torch.empty(0, **f32), torch.empty(0, **f32)
-    n = max(T, 256)
+        return torch.empty(0, **f32), torch.empty(0, **f32), torch.empty(0, **f32), None
+    n = max((T + 63) // 64 * 64, 256) if keep else max(T, 256)
     if n != T:
         hp = torch.zeros((n, K), dtype=h.dtype, device=dev)
         hp[:T] = h
@@ -371,14 +424,15 @@ def _own_forward(h, w, ids, temp, n_splits, what):
     lp = torch.empty(n, **f32)
     ent = torch.empty(n, **f32)
     lse = torch.empty(n, **f32)
+    kept = torch.empty((n, V), dtype=h.dtype, device=dev) if keep else None
     flag = torch.zeros(1, dtype=torch.int32, device=dev)
     with torch.cuda.device(dev):
         st = lib.vrl_lmhead_score(h.data_ptr(), w.data_ptr(), _DTYPE_CODES[h.dtype], n, V, K, h.stride(0), w.stride(0),
                                   ids.data_ptr(), _ptr(temp), splits, partials.data_ptr(), lp.data_ptr(), ent.data_ptr(),
-                                  lse.data_ptr(), flag.data_ptr(), _lib.stream_ptr(dev))
+                                  lse.data_ptr(), flag.data_ptr(), _ptr(kept), V if keep else 0, _lib.stream_ptr(dev))
     _lib.check("vrl_lmhead_score", st)
     _errors.report(flag, {_lib.VRL_FLAG_LABEL_OOB: (IndexError, f"{what}: an input id is outside [0, {V})")})
-    return lp[:T], ent[:T], lse[:T]
+    return lp[:T], ent[:T], lse[:T], kept
 
 
 def lm_head_score_mfma(hidden_states: torch.Tensor, vocab_weights: torch.Tensor, input_ids: torch.Tensor,
@@ -422,7 +476,7 @@ def lm_head_score_mfma(hidden_states: torch.Tensor, vocab_weights: torch.Tensor,
             raise ValueError(f"temperature has {temp.numel()} entries, expected one per token ({T})")
     elif float(temperature) != 1.0:
         temp = torch.full((T,), float(temperature), dtype=torch.float32, device=dev)
-    lp, ent, _ = _own_forward(h, w, ids, temp, n_splits, "lm_head_score_mfma")
+    lp, ent, _, _ = _own_forward(h, w, ids, temp, n_splits, "lm_head_score_mfma")
     return lp.reshape(lead), ent.reshape(lead)
 
 
@@ -453,8 +507,8 @@ def linear_cross_entropy(hidden: torch.Tensor, weight: torch.Tensor, labels: tor
 class FusedLinearForPPO(torch.nn.Module):
     """Module form, constructed and called like verl's (verl/utils/experimental/torch_functional.py:211-231)."""
 
-    def __init__(self, chunk_size: int = DEFAULT_CHUNK_TOKENS, keep_logits: bool = False, kernels: Optional[str] = None,
-                 forward_splits: Optional[int] = None):
+    def __init__(self, chunk_size: int = DEFAULT_CHUNK_TOKENS, keep_logits: Optional[bool] = None,
+                 kernels: Optional[str] = None, forward_splits: Optional[int] = None):
         super().__init__()
         self.chunk_size = chunk_size
         self.keep_logits = keep_logits

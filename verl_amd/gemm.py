@@ -29,14 +29,16 @@ def _dims(x: torch.Tensor, y: torch.Tensor, x_t: bool, y_t: bool):
 
 
 def gemm_takes(x: torch.Tensor, y: torch.Tensor, x_t: bool = False, y_t: bool = False) -> bool:
-    """Whether ``gemm`` accepts these operands: 16-bit, >= 256 rows each, contraction a multiple of 64 and >= 128, last
-    axis contiguous, row strides multiples of 8; ``NX`` a multiple of 4, a contraction-major operand's rows a multiple
-    of 8."""
+    """Whether ``gemm`` accepts these operands, i.e. everything ``vrl_gemm`` checks about them: 16-bit, >= 256 rows each,
+    contraction a multiple of 64 and >= 128, last axis contiguous, row strides multiples of 8, 16-byte aligned storage;
+    ``NX`` a multiple of 4, a contraction-major operand's rows a multiple of 8."""
     if not (x.dtype in _DTYPE_CODES and y.dtype == x.dtype and x.dim() == 2 and y.dim() == 2):
         return False
     NX, NY, KX, KY = _dims(x, y, x_t, y_t)
     return (KX == KY and NX >= 256 and NY >= 256 and NX % 4 == 0 and KX % 64 == 0 and KX >= 128
             and x.stride(1) == 1 and y.stride(1) == 1 and x.stride(0) % 8 == 0 and y.stride(0) % 8 == 0
+            and x.stride(0) >= x.shape[1] and y.stride(0) >= y.shape[1]
+            and x.data_ptr() % 16 == 0 and y.data_ptr() % 16 == 0
             and (not x_t or NX % 8 == 0) and (not y_t or NY % 8 == 0))
 
 
