@@ -14,6 +14,12 @@
  *     OR-ed into *err_flag (device int32, caller zeroes it, caller reads it
  *     after synchronising).
  *   - Nothing throws or aborts across this boundary.
+ *   - First calls. The first call of an entry point on a device may touch the runtime beyond a launch: the
+ *     matrix-core entry points (vrl_lmhead_score, vrl_lmhead_dlogits, vrl_gemm / vrl_gemm_nt) raise their kernels' LDS
+ *     limit with hipFuncSetAttribute, once per device and kernel variant (element type, operand layouts, stored /
+ *     accumulated / partial product, logits kept or not), and vrl_rowscore_split_static looks up its scratch array's
+ *     address. Neither is allowed while a stream is being captured into a HIP graph: make each call once, with the
+ *     options that will be captured, before the capture starts. Later calls only enqueue kernels.
  *   - Row space: logits are (n_rows, vocab), row r starts at element
  *     r * row_stride. Per-token arrays (labels, temperature, outputs, and
  *     for verify logp/mask/accept) are indexed by the same r.
@@ -267,6 +273,10 @@ int vrl_transpose(const void* src, int elem_size, int64_t rows, int64_t cols, in
  * multiples of 8, 16-byte aligned): for a backward pass that may spend n_tokens * vocab elements of memory instead of
  * forming the logits again, which then runs vrl_rowscore_backward over them in place (the reference's torch path keeps
  * them the same way, verl/utils/experimental/torch_functional.py:33-35). The scores are folded from the fp32 values either way.
+ *
+ * fp32 operands are refused (VRL_ERR_DTYPE) on purpose: the part's fp32 matrix rate (157 TFLOP/s) is what the library GEMM
+ * already delivers, so an fp32 LM head is served by the library GEMM followed by vrl_rowscore (the Python side does that),
+ * where the reference's Triton loop takes any element type (verl/utils/kernel/kernels.py:183-188).
  *
  * Replaces the reference's fused linear + cross-entropy forward:
  *   verl/utils/kernel/linear_cross_entropy.py:38-85 (LinearCrossEntropy.forward)

@@ -34,6 +34,9 @@ def test_fp32_forward_and_backward_match_torch(dev, T, D, V, chunk):
     ref_lp, ref_ent = _torch_reference(hidden, weight, labels, temperature)
     d_ref_h, d_ref_w = torch.autograd.grad((ref_ent, ref_lp), (hidden, weight), (g_ent, g_lp))
 
+    from verl_amd import gemm
+
+    before = gemm.counters["gemm"]
     lp, ent = fused_linear_for_ppo(hidden, weight, labels, temperature, chunk_size=chunk, keep_logits=False)
     assert lp.dtype == torch.float32 and lp.shape == (T,) and ent.shape == (T,)
     torch.testing.assert_close(ref_lp, lp, atol=1e-4, rtol=1e-4)
@@ -43,6 +46,8 @@ def test_fp32_forward_and_backward_match_torch(dev, T, D, V, chunk):
     torch.testing.assert_close(d_ref_w, d_w, atol=1e-2, rtol=1e-4)
     # much closer than the reference asks for
     assert (d_ref_h - d_h).abs().max().item() <= 2e-4 and (d_ref_w - d_w).abs().max().item() <= 2e-4
+    # an fp32 model is served by the library GEMM + the row kernels on purpose: none of the 16-bit matrix-core products ran
+    assert gemm.counters["gemm"] == before
 
 
 def test_bf16_module_3d_inputs(dev):

@@ -221,3 +221,41 @@ def test_drift_recipes():
     t = synthetic.drift_old_logprobs(base, synthetic.WORKLOADS["c5"], 3)
     # Student-t(3) * 0.3: heavy tails, median absolute deviation 0.3 * 0.765
     assert abs(t.abs().median().item() - 0.3 * 0.7649) < 0.02 and t.abs().max().item() > 3.0
+
+
+def test_deprecated_label_check_switch_still_switches():
+    """Setting verl_amd.torch_functional.LABEL_CHECK (the switch of earlier versions) maps onto verl_amd.errors."""
+    import warnings
+
+    from verl_amd import errors, torch_functional as vf
+
+    before = errors.DEFAULT_MODE
+    try:
+        with warnings.catch_warnings(record=True) as caught:
+            warnings.simplefilter("always")
+            vf.LABEL_CHECK = False
+        assert errors.DEFAULT_MODE == "off" and errors.mode() == "off" and vf.LABEL_CHECK is False
+        assert any(issubclass(w.category, DeprecationWarning) for w in caught)
+        with warnings.catch_warnings():
+            warnings.simplefilter("ignore")
+            vf.LABEL_CHECK = True
+        assert errors.DEFAULT_MODE == "sync" and vf.LABEL_CHECK is True
+    finally:
+        errors.DEFAULT_MODE = before
+
+
+def test_gemm_takes_refuses_what_vrl_gemm_would_refuse():
+    """Operands vrl_gemm rejects (storage that starts off the 16-byte grid, a row stride below the row) must be refused
+    by gemm_takes too, so that callers send them to the library product instead of into an error in mid-backward."""
+    import torch
+
+    from verl_amd import gemm
+
+    x = torch.zeros(512 * 128 + 8, dtype=torch.bfloat16)
+    y = torch.zeros(256 * 128 + 8, dtype=torch.bfloat16)
+    aligned_x, aligned_y = x[:512 * 128].view(512, 128), y[:256 * 128].view(256, 128)
+    assert gemm.gemm_takes(aligned_x, aligned_y)
+    off_x = x[1:512 * 128 + 1].view(512, 128)            # starts 2 bytes into the allocation
+    assert off_x.data_ptr() % 16 != 0 and not gemm.gemm_takes(off_x, aligned_y)
+    assert not gemm.gemm_takes(aligned_x, y[4:256 * 128 + 4].view(256, 128))
+    assert not gemm.gemm_takes(aligned_x.float(), aligned_y.float())

@@ -334,7 +334,8 @@ __device__ __forceinline__ void lm_walk_tiles_as(const uint16_t* __restrict__ W,
       // column, and each is refilled in place with the next half's as soon as it is dead - the second half's from this
       // step's tiles during the first half, the next step's first half from the next tiles during the second. The
       // step's barrier therefore sits between the halves: behind it W(s), H(s) are dead and W(s+1), H(s+1) must have
-      // landed. First half: the four loads of W(s+2) (into the slot H(s-1) left); second half: H(s+2) (slot of W(s)).
+      // landed. First half: the loading wavefronts' eight loads each of W(s+2) (into the slot H(s-1) left); second half: H(s+2)
+      // (slot of W(s)).
 #pragma unroll
       for (int hf = 0; hf < 2; ++hf) {
         if (hf == 1) {

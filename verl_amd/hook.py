@@ -113,6 +113,14 @@ def _memo_clear() -> None:
     _memo_local.memo = None
 
 
+def clear_memo() -> None:
+    """Drop what the calling thread's last shim call left for the other call of its pair. With gradients that record
+    holds the first call's result with its autograd graph, and through it the logits, until the thread's next shim
+    call; a caller that makes an entropy call without the log-prob call that would take the record (or the reverse) and
+    wants the memory back at once calls this."""
+    _memo_clear()
+
+
 _LOGPROB_NAMES = ("logprobs_from_logits", "logprobs_from_logits_v2", "logprobs_from_logits_naive")
 _ENTROPY_NAMES = ("entropy_from_logits", "entropy_from_logits_with_chunking")
 

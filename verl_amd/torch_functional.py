@@ -595,3 +595,27 @@ def score_responses(
     if per_token:
         return r_lp, r_h, t_lp, t_h
     return r_lp, r_h
+
+
+# ``LABEL_CHECK`` was this module's switch for the label check before verl_amd.errors took it over; code that still sets
+# ``verl_amd.torch_functional.LABEL_CHECK = False`` keeps its meaning (no read-back of the error flag, no host
+# synchronisation per direct call) instead of silently losing it.
+import sys as _sys
+import types as _types
+import warnings as _warnings
+
+
+class _ModuleWithLabelCheck(_types.ModuleType):
+    @property
+    def LABEL_CHECK(self) -> bool:
+        return _errors.DEFAULT_MODE != "off"
+
+    @LABEL_CHECK.setter
+    def LABEL_CHECK(self, value) -> None:
+        _warnings.warn("verl_amd.torch_functional.LABEL_CHECK is deprecated: set verl_amd.errors.DEFAULT_MODE "
+                       "('sync', 'deferred' or 'off'), the VERL_AMD_CHECK environment variable or pass check_labels",
+                       DeprecationWarning, stacklevel=2)
+        _errors.DEFAULT_MODE = "sync" if value else "off"
+
+
+_sys.modules[__name__].__class__ = _ModuleWithLabelCheck
