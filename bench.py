@@ -467,6 +467,20 @@ def bench_lm_head(args, dev):
         lp, h = fused_linear_for_ppo(hidden, weight, ids, temperature, chunk, keep)
         return torch.autograd.grad((lp, h), (hidden, weight), (g_lp, g_h))
 
+    if args.own_only:
+        # for a kernel trace of the default call alone: nothing but the package's own path runs
+        spin_up(fwd_bwd, 300.0)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            fwd_bwd()
+        torch.cuda.synchronize()
+        ms = (time.perf_counter() - t0) * 1e3 / args.steps
+        return {"metric": "tokens/sec of LM head + scoring, forward + backward", "value": T / ms * 1e3, "unit": "tokens/s",
+                "ms_per_step": ms, "steps": args.steps, "dtype": "bf16",
+                "config": {"workload": "lm_head_8192x3584_v152064_bf16", "keep_logits": args.keep_logits,
+                           "chunk_tokens": chunk, "step": "fused_linear_for_ppo forward + backward, default kernels only"}}
+
     # guard: first tokens of the library forward against torch in fp32 on the bf16 logits the same GEMM produces
     lp, h = fwd_library()
     z = torch.matmul(hidden[:256].detach(), weight.detach().t()).float() / temperature
@@ -1017,7 +1031,8 @@ def compact(rec: dict) -> dict:
     out.update({k: rec[k] for k in keep if k in rec})
     r = rec["roofline"]
     out["roofline"] = {k: r[k] for k in ("bound", "achieved", "peak", "unit", "frac", "traffic", "kernel", "avg_kernel_ms",
-                                         "algorithmic_bytes_per_launch") if k in r}
+                                         "algorithmic_bytes_per_launch", "timing", "launch_floor_ms",
+                                         "achieved_net_of_launch_floor", "flops", "executed_flops_frac") if k in r}
     return out
 
 
@@ -1045,6 +1060,9 @@ def main():
     ap.add_argument("--chunk", type=int, default=4096, help="--lm-head: tokens projected at a time")
     ap.add_argument("--keep-logits", choices=["auto", "yes", "no"], default="auto",
                     help="--lm-head: keep the logits for the backward (auto: when they fit the package's default budget)")
+    ap.add_argument("--own-only", action="store_true",
+                    help="--lm-head: run the default call (the package's own kernels) alone, without the library paths it "
+                         "is compared with (for a kernel trace)")
     ap.add_argument("--ceilings", action="store_true",
                     help="time plain non-temporal read / copy probes with the row kernels' access pattern")
     ap.add_argument("--verify-form", choices=["auto", "two-pass", "per-sequence"], default="auto",
