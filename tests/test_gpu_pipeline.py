@@ -294,6 +294,54 @@ def test_stock_update_actor_sequence_shares_one_forward_and_one_backward_pass(de
         hook.check_errors()
 
 
+def test_a_pair_that_never_completes_pins_nothing(dev):
+    """With gradients the first call of a pair leaves a per-row vector that carries its autograd graph, and the graph
+    holds the logits. A caller that makes only one call of the pair (entropy without log-probs, or a forward that is
+    never followed by a backward) must get the logits' memory back as soon as it lets go of the result, without
+    another shim call on the thread."""
+    import gc
+    import weakref
+    with _stand_in_verl() as mods:
+        tf = mods["verl.utils.torch_functional"]
+        hook.install()
+        g = torch.Generator(device=dev).manual_seed(5)
+        n, V = 64, 4099
+        lab = torch.randint(0, V, (n,), generator=g, device=dev)
+        leaf = torch.randn(n, V, generator=g, device=dev).requires_grad_(True)
+        for first in ("entropy", "logprob"):
+            logits = leaf * 1.0
+            alive = weakref.ref(logits)
+            res = tf.entropy_from_logits(logits) if first == "entropy" else tf.logprobs_from_logits(logits, lab)
+            assert res.requires_grad
+            del logits
+            gc.collect()
+            assert alive() is not None          # held by the result's graph, as with any differentiable op
+            del res
+            gc.collect()
+            assert alive() is None, first       # ... and by nothing else
+        # the result is kept (as the engine does) and the pair completes: shared as before
+        logits = leaf * 1.0
+        s0 = hook.stats()
+        h = tf.entropy_from_logits(logits)
+        lp = tf.logprobs_from_logits(logits, lab, inplace_backward=False)
+        (h.sum() + lp.sum()).backward()
+        s1 = hook.stats()
+        assert s1["memo_hits"] - s0["memo_hits"] == 1 and s1["backward_passes"] - s0["backward_passes"] == 1
+        # the explicit form
+        logits = leaf * 1.0
+        alive = weakref.ref(logits)
+        res = tf.entropy_from_logits(logits)
+        hook.clear_memo()
+        n0 = hook.stats()["forward_passes"]
+        tf.logprobs_from_logits(logits, lab)
+        assert hook.stats()["forward_passes"] == n0 + 1     # nothing was left to share
+        hook.clear_memo()
+        del logits, res
+        gc.collect()
+        assert alive() is None
+        hook.check_errors()
+
+
 def test_installed_shims_never_synchronise(dev, monkeypatch):
     """The torch.gather the shims replace asserts on the device and returns (verl/utils/torch_functional.py:69): the
     shims must not drain the launch queue either. Fifty calls with every host synchronisation torch offers patched

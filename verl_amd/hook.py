@@ -74,7 +74,7 @@ class _RowMemo:
     """What one pass over a logits tensor left for the other call of the pair."""
 
     __slots__ = ("ref", "version", "ptr", "shape", "stride", "dtype", "stream", "needs_grad", "kind", "entropy", "lse",
-                 "pair")
+                 "pair", "_watch")
 
     def __init__(self, logits, stream, needs_grad, kind, entropy=None, lse=None, pair=None):
         self.ref = weakref.ref(logits)
@@ -89,6 +89,20 @@ class _RowMemo:
         self.entropy = entropy
         self.lse = lse
         self.pair = pair          # grad mode, kind "entropy": the dict the two autograd nodes share
+        self._watch = None
+
+    def release_with(self, result) -> None:
+        """With gradients what is held carries the first call's autograd graph, and through it the logits. Let it go
+        when ``result``, the tensor that call returned, dies: a caller that never makes the second call of the pair then
+        keeps nothing alive beyond its own reference to the result."""
+        self._watch = weakref.finalize(result, self.drop)
+        self._watch.atexit = False
+
+    def drop(self) -> None:
+        self.entropy = self.lse = self.pair = None
+        if self._watch is not None:
+            self._watch.detach()     # (the finalizer holds this record; without it the record dies with its last user)
+            self._watch = None
 
     def matches(self, logits, stream, needs_grad) -> bool:
         return (self.ref() is logits and self.version == logits._version and self.ptr == logits.data_ptr()
@@ -100,24 +114,34 @@ _memo_local = threading.local()   # per thread: a pair of calls is made by one t
 
 
 def _memo_take() -> Optional[_RowMemo]:
+    """The record the thread's last shim call left, which is gone from the thread afterwards; its tensors stay with the
+    returned object until the caller lets go of it."""
     memo = getattr(_memo_local, "memo", None)
     _memo_local.memo = None
+    if memo is not None and memo._watch is not None:
+        memo._watch.detach()
+        memo._watch = None
     return memo
 
 
-def _memo_store(memo: _RowMemo) -> None:
+def _memo_store(memo: _RowMemo, result=None) -> None:
+    _memo_clear()
+    if memo.needs_grad and result is not None:
+        memo.release_with(result)
     _memo_local.memo = memo
 
 
 def _memo_clear() -> None:
+    memo = getattr(_memo_local, "memo", None)
     _memo_local.memo = None
+    if memo is not None:
+        memo.drop()
 
 
 def clear_memo() -> None:
     """Drop what the calling thread's last shim call left for the other call of its pair. With gradients that record
-    holds the first call's result with its autograd graph, and through it the logits, until the thread's next shim
-    call; a caller that makes an entropy call without the log-prob call that would take the record (or the reverse) and
-    wants the memory back at once calls this."""
+    holds a per-row vector with the first call's autograd graph, and through it the logits; it goes by itself at the
+    thread's next shim call or when the tensor that first call returned dies, whichever comes first."""
     _memo_clear()
 
 
@@ -162,11 +186,12 @@ def _memo_serve(name, logits, args, kwargs):
         if needs_grad:
             pair = {}
             h, lse = _amd._EntropyLseFunction.apply(x, None, None, pair)
-            _memo_store(_RowMemo(logits, stream, True, "entropy", lse=lse, pair=pair))
-        else:
-            with torch.no_grad():
-                _, h, _, lse, _ = _amd._forward_2d(x, None, None, False, True, False, True, None)
-            _memo_store(_RowMemo(logits, stream, False, "entropy", lse=lse))
+            out = h.reshape(lead)
+            _memo_store(_RowMemo(logits, stream, True, "entropy", lse=lse, pair=pair), out)
+            return out
+        with torch.no_grad():
+            _, h, _, lse, _ = _amd._forward_2d(x, None, None, False, True, False, True, None)
+        _memo_store(_RowMemo(logits, stream, False, "entropy", lse=lse))
         return h.reshape(lead)
 
     labels = args[0] if args else kwargs.get("labels")
@@ -192,9 +217,10 @@ def _memo_serve(name, logits, args, kwargs):
     else:
         with torch.no_grad():
             lp, h, _, _, flag = _amd._forward_2d(x, lab, None, True, True, False, False, None)
-    _memo_store(_RowMemo(logits, stream, needs_grad, "logprob", entropy=h.reshape(lead)))
+    out = lp.reshape(lead)
+    _memo_store(_RowMemo(logits, stream, needs_grad, "logprob", entropy=h.reshape(lead)), out)
     _errors.report(flag, messages)
-    return lp.reshape(lead)
+    return out
 
 
 _originals: Dict[str, Callable] = {}
