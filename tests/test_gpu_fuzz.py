@@ -155,3 +155,49 @@ def test_random_verify_cases_all_forms_against_the_c_oracle(dev):
                 assert np.array_equal(getattr(res, k).cpu().numpy(), ref[k]), (what, k)
             assert np.array_equal(res.out_ids.cpu().numpy(), ref["out_ids"]), what
             assert np.array_equal(res.out_mask.cpu().numpy().astype(np.uint8), ref["out_mask"]), what
+    print(f"{case + 1} random verify batches")
+
+
+def test_random_response_slices_against_the_oracle(dev):
+    """Seeded random packed batches through vrl_response_slice / vrl_response_pack: every element size the copy units
+    1, 2, 4, 8 and 16 bytes come from, trailing dimensions of odd and even sizes, values that are views off the 16-byte
+    grid, empty responses, responses as long as their sequence allows, a padded length below, at and above the longest
+    response. Bit for bit against the reference's loop (verl/workers/utils/padding.py:133-138, :194-210)."""
+    import os
+
+    from verl_amd import layout
+
+    dtypes = [torch.uint8, torch.int16, torch.bfloat16, torch.float16, torch.float32, torch.int32, torch.int64,
+              torch.float64]
+    rng = np.random.default_rng(int(os.environ.get("VRL_FUZZ_SEED", "20240607")) + 1)
+    for case in range(int(os.environ.get("VRL_FUZZ_CASES", "150"))):
+        g = torch.Generator().manual_seed(int(rng.integers(0, 2**31)))
+        dtype = dtypes[int(rng.integers(0, len(dtypes)))]
+        trailing = [(), (1,), (3,), (4,), (7,), (8,), (5, 3), (64,), (130,)][int(rng.integers(0, 9))]
+        B = int(rng.integers(1, 20))
+        prompt = torch.randint(1, 30, (B,), generator=g)
+        kind = rng.integers(0, 4, size=B)
+        resp = torch.tensor([int({0: 0, 1: 1, 2: rng.integers(0, 40), 3: rng.integers(40, 700)}[k]) for k in kind])
+        cu = torch.zeros(B + 1, dtype=torch.int64)
+        cu[1:] = torch.cumsum(prompt + resp, 0)
+        N = int(cu[-1])
+        inner = int(np.prod(trailing)) if trailing else 1
+        lead = int(rng.integers(0, 5))            # elements the view starts behind its buffer's beginning
+        flat = torch.randint(0, 251, (lead + N * inner,), generator=g).to(dtype)
+        vals = flat[lead:].view((N,) + trailing)
+        longest = int(resp.max())
+        T = max(0, longest + int(rng.integers(-2, 4)))
+        flat_d = flat.to(dev)
+        vals_d = flat_d[lead:].view((N,) + trailing)
+        if T >= longest:
+            got = layout.response_slice(vals_d, cu.to(dev), resp.to(dev), T)
+            ref = scoring.response_slice(vals, prompt.tolist(), resp.tolist(), T)
+            assert got.dtype == dtype and torch.equal(got.cpu(), ref), (case, dtype, trailing, lead)
+        elif T > 0:                                # a response does not fit the block: reported (a block without
+            with pytest.raises(ValueError):        # columns is not looked at)
+                layout.response_slice(vals_d, cu.to(dev), resp.to(dev), T)
+        total = int(resp.sum()) if rng.random() < 0.5 else None
+        packed, packed_cu = layout.response_from_packed(vals_d, cu.to(dev), resp.to(dev), total_response_tokens=total)
+        ref_p, ref_cu = scoring.response_from_nested(vals, cu.tolist(), resp.tolist())
+        assert packed.dtype == dtype and torch.equal(packed.cpu(), ref_p) and torch.equal(packed_cu.cpu(), ref_cu), case
+    print(f"{case + 1} random packed batches sliced and packed")
