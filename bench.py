@@ -1084,6 +1084,8 @@ def main():
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
     if args.lm_head:
+        if args.copy_calibration:
+            copy_calibration(dev)
         print(json.dumps(bench_lm_head(args, dev)), flush=True)
         return
     if args.ceilings:
