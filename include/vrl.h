@@ -42,7 +42,7 @@
 extern "C" {
 #endif
 
-#define VRL_ABI_VERSION 3
+#define VRL_ABI_VERSION 4
 
 /* status codes */
 #define VRL_OK 0
@@ -224,6 +224,20 @@ int vrl_score_responses_backward(const void* logits, int dtype, int64_t n_rows, 
  */
 int vrl_response_slice(const void* values, int64_t row_bytes, const int64_t* cu_seqlens, const int64_t* response_lens,
                        int64_t B, int64_t n_tokens, int64_t T_out, void* out, int32_t* err_flag, void* stream);
+
+/*
+ * vrl_expand_per_sequence — one fp32 value per sequence -> one per token of the packed batch:
+ *   out[t] = values[b]  for  cu_seqlens[b] <= t < cu_seqlens[b+1]
+ * (empty sequences contribute nothing). This is how the engine turns the per-sample temperature into the per-token
+ * one that the scoring entry points take. `values` has B entries, `out` n_tokens. Offsets that are not a partition of
+ * [0, n_tokens] set VRL_FLAG_SEQ_RANGE; a token that no sequence holds gets 0. B = 0 with n_tokens > 0 is
+ * VRL_ERR_SHAPE.
+ *
+ * Replaces verl/utils/torch_functional.py:989-1011 (expand_as_nested: repeat_interleave by the sequence lengths) as
+ * called at verl/workers/engine/fsdp/transformer_impl.py:1158-1162.
+ */
+int vrl_expand_per_sequence(const float* values, const int64_t* cu_seqlens, int64_t B, int64_t n_tokens, float* out,
+                            int32_t* err_flag, void* stream);
 
 /*
  * vrl_response_pack — packed per-token values (total_nnz, *) -> packed response values (sum of response_lens, *):

@@ -134,6 +134,16 @@ def roll_labels(input_ids_rmpad: torch.Tensor) -> torch.Tensor:
     return torch.roll(input_ids_rmpad, shifts=-1, dims=-1)
 
 
+def expand_as_nested_values(per_sequence: torch.Tensor, offsets) -> torch.Tensor:
+    """The per-token values of the reference's ``expand_as_nested(tensor, nested)``: entry b repeated over the
+    tokens of sequence b (``torch.repeat_interleave(tensor, offsets.diff())``). This is how the engine builds
+    ``temperature_rmpad``. verl/utils/torch_functional.py:989-1011; caller fsdp/transformer_impl.py:1158-1162."""
+    offsets = torch.as_tensor(offsets, dtype=torch.int64)
+    assert per_sequence.dim() == 1, "The ndim of tensor must be 1"                      # :1003
+    assert per_sequence.shape[0] == offsets.numel() - 1, "The batch shape must be the same"   # :1000-1002
+    return torch.repeat_interleave(per_sequence, offsets.diff(), dim=0)
+
+
 def response_slice(values: torch.Tensor, prompt_lens, response_lens, max_response_len: int | None = None) -> torch.Tensor:
     """Packed per-token values (total_nnz, ...) -> (B, max_response_len, ...): for each sequence the
     rows [end - resp_len - 1, end - 1) (model output is shifted left by one token), right-padded

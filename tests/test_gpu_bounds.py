@@ -137,7 +137,20 @@ def test_response_slice_and_pack_hold_bad_offsets_to_the_arrays(dev, case):
         assert int(flag.item()) & _lib.VRL_FLAG_SEQ_RANGE
         assert ar.guards_intact()
         assert torch.isfinite(wide_out.float()).all()
+        # one value per sequence spread over the tokens: every token written (a value or 0), nothing else
+        flag.zero_()
+        per_seq = ar.make(B, torch.float32, torch.tensor([0.5, 1.5, 2.5]))
+        per_tok = ar.make(N, torch.float32)
+        print(f"[bounds] expand per sequence with cu_seqlens={BAD_OFFSETS[case]} over {N} tokens", flush=True)
+        st = lib.vrl_expand_per_sequence(per_seq.data_ptr(), cu.data_ptr(), B, N, per_tok.data_ptr(), flag.data_ptr(), s)
+        assert st == _lib.VRL_OK
+        torch.cuda.synchronize(dev)
+        assert int(flag.item()) & _lib.VRL_FLAG_SEQ_RANGE
+        assert ar.guards_intact()
+        assert bool(torch.isin(per_tok, torch.tensor([0.0, 0.5, 1.5, 2.5], device=dev)).all())
     cu_t = torch.tensor(BAD_OFFSETS[case], dtype=torch.int64, device=dev)
+    with pytest.raises(ValueError, match="partition"):
+        layout.expand_per_sequence(per_seq.clone(), cu_t, N)
     with pytest.raises(ValueError, match="partition"):
         layout.response_slice(values.clone(), cu_t, rl.clone(), T)
     with pytest.raises(ValueError, match="partition"):

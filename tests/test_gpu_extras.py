@@ -239,3 +239,44 @@ def test_response_slice_with_known_lengths_does_not_synchronise(dev):
     errors.check_errors()
     assert torch.equal(a.cpu(), scoring.response_slice(vals.cpu(), prompt.tolist(), resp.tolist(), T))
     assert torch.equal(b.cpu(), scoring.response_from_nested(vals.cpu(), cu.tolist(), resp.tolist())[0])
+
+
+def test_expand_per_sequence_matches_the_reference_repeat_interleave(dev):
+    """expand_as_nested (verl/utils/torch_functional.py:989-1011): the per-sample temperature repeated over the tokens
+    of its sequence. Random batches with empty sequences, one sequence, many; known total (no synchronisation) and
+    unknown; and offsets that are not a partition are reported."""
+    g = torch.Generator().manual_seed(77)
+    for B in (1, 2, 7, 300, 5000):
+        lens = torch.randint(0, 40, (B,), generator=g)
+        lens[torch.rand(B, generator=g) < 0.2] = 0
+        if B == 7:
+            lens[3] = 5000
+        cu = torch.zeros(B + 1, dtype=torch.int64)
+        cu[1:] = torch.cumsum(lens, 0)
+        vals = torch.rand(B, generator=g) + 0.3
+        ref = scoring.expand_as_nested_values(vals, cu)
+        got = layout.expand_per_sequence(vals.to(dev), cu.to(dev))
+        assert got.dtype == torch.float32 and torch.equal(got.cpu(), ref), B
+        got = layout.expand_per_sequence(vals.to(dev), cu.to(dev), total_nnz=int(cu[-1]))
+        assert torch.equal(got.cpu(), ref), B
+    # no tokens at all
+    assert layout.expand_per_sequence(torch.ones(3, device=dev), torch.zeros(4, dtype=torch.int64, device=dev)).numel() == 0
+    # with the total known the call does not wait for the device
+    vals_d, cu_d, n = vals.to(dev), cu.to(dev), int(cu[-1])
+    layout.expand_per_sequence(vals_d, cu_d, n, check="deferred")
+    torch.cuda.synchronize(dev)
+    torch.cuda.set_sync_debug_mode("error")
+    try:
+        got = layout.expand_per_sequence(vals_d, cu_d, n, check="deferred")
+    finally:
+        torch.cuda.set_sync_debug_mode("default")
+    errors.check_errors()
+    assert torch.equal(got.cpu(), ref)
+    # offsets that do not partition the tokens
+    for bad in ([1, 3, 6], [0, 4, 3, 6], [0, 3, 5], [0, 3, 9]):
+        with pytest.raises(ValueError):
+            layout.expand_per_sequence(torch.ones(len(bad) - 1, device=dev), torch.tensor(bad, device=dev), 6)
+    with pytest.raises(ValueError):
+        layout.expand_per_sequence(torch.ones(3, device=dev), torch.tensor([0, 3, 6], device=dev), 6)
+    with pytest.raises(RuntimeError):
+        layout.expand_per_sequence(torch.ones(2), torch.tensor([0, 3, 6]), 6)

@@ -91,6 +91,28 @@ def test_random_packed_batches_against_oracle_and_separate_entry_points(dev, dty
         assert torch.equal(r_lp.cpu() == 0, want_lp == 0)
 
 
+def test_one_temperature_per_sequence_is_expanded_like_the_engine_does(dev):
+    """The engine holds one temperature per sample and repeats it over the sample's tokens before dividing
+    (verl/workers/engine/fsdp/transformer_impl.py:1149-1162, expand_as_nested): passing the (B,) tensor gives the
+    same bits as passing the expanded (total_nnz,) one."""
+    g = torch.Generator().manual_seed(31)
+    B, V = 9, 3001
+    prompt = torch.randint(1, 20, (B,), generator=g)
+    resp = torch.randint(0, 30, (B,), generator=g)
+    cu = torch.zeros(B + 1, dtype=torch.int64)
+    cu[1:] = torch.cumsum(prompt + resp, 0)
+    n = int(cu[-1])
+    x = (torch.randn(n, V, generator=g) * 2).bfloat16().to(dev)
+    ids = torch.randint(0, V, (n,), generator=g).to(dev)
+    t_seq = (torch.rand(B, generator=g) + 0.5).to(dev)
+    t_tok = scoring.expand_as_nested_values(t_seq.cpu(), cu).to(dev)
+    T = int(resp.max())
+    a = vf.score_responses(x, cu.to(dev), resp.to(dev), T, input_ids=ids, temperature=t_seq)
+    b = vf.score_responses(x, cu.to(dev), resp.to(dev), T, input_ids=ids, temperature=t_tok)
+    assert torch.equal(a[0], b[0]) and torch.equal(a[1], b[1])
+    assert not torch.equal(a[0], vf.score_responses(x, cu.to(dev), resp.to(dev), T, input_ids=ids)[0])
+
+
 def test_prompt_rows_do_not_matter_without_per_token_outputs(dev):
     """Only rows inside a response window are scored when no per-token vector is asked for: whatever the prompt rows
     hold (here NaN), the blocks are the same."""

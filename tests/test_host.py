@@ -52,7 +52,8 @@ def test_lenience_offset():
 
 def test_package_surface():
     for name in ("logprobs_from_logits", "entropy_from_logits", "entropy_from_logits_with_chunking",
-                 "fused_logprob_entropy", "spec_verify", "fused_score_verify", "truncate_draft", "install", "uninstall"):
+                 "fused_logprob_entropy", "spec_verify", "fused_score_verify", "truncate_draft", "install", "uninstall",
+                 "score_responses", "response_slice", "response_from_packed", "expand_per_sequence"):
         assert callable(getattr(verl_amd, name)), name
 
 

@@ -317,3 +317,32 @@ def test_property_bounds(V, n, scale, seed):
     p = torch.softmax(x.double(), -1)
     direct = -(p * torch.log(p.clamp_min(1e-300))).sum(-1)
     assert np.allclose(c_h, direct.numpy(), atol=1e-9)
+
+
+def test_expand_as_nested_values_is_one_value_per_token_of_its_sequence():
+    """Pinned without the formula: written out by hand for a small batch, by a per-token loop for a random one, and
+    through what it is for (the per-token temperature gives the same scores as scoring each sequence on its own with
+    its scalar temperature)."""
+    t = torch.tensor([0.5, 2.0, 1.25])
+    got = scoring.expand_as_nested_values(t, [0, 2, 2, 5])            # the middle sequence is empty
+    assert got.tolist() == [0.5, 0.5, 1.25, 1.25, 1.25]
+    g = torch.Generator().manual_seed(3)
+    lens = torch.randint(0, 9, (17,), generator=g)
+    cu = torch.zeros(18, dtype=torch.int64)
+    cu[1:] = torch.cumsum(lens, 0)
+    vals = torch.rand(17, generator=g)
+    got = scoring.expand_as_nested_values(vals, cu)
+    assert got.shape == (int(cu[-1]),)
+    for tok in range(int(cu[-1])):
+        b = max(i for i in range(17) if int(cu[i]) <= tok and tok < int(cu[i + 1]))
+        assert got[tok] == vals[b]
+    x = torch.randn(int(cu[-1]), 50, generator=g)
+    lab = torch.randint(0, 50, (int(cu[-1]),), generator=g)
+    lp_all, h_all = scoring.score_fp64(x, lab, got.double())
+    for b in range(17):
+        lo, hi = int(cu[b]), int(cu[b + 1])
+        if hi > lo:
+            lp_b, h_b = scoring.score_fp64(x[lo:hi], lab[lo:hi], torch.full((hi - lo,), float(vals[b]), dtype=torch.float64))
+            assert torch.equal(lp_b, lp_all[lo:hi]) and torch.equal(h_b, h_all[lo:hi])
+    with pytest.raises(AssertionError):
+        scoring.expand_as_nested_values(vals[:-1], cu)

@@ -14,7 +14,7 @@ Setting ``VERL_USE_EXTERNAL_MODULES=verl_amd.plugin`` makes verl import
 from . import rollout_corr
 from .fused_linear import FusedLinearForPPO, fused_linear_for_ppo, linear_cross_entropy, lm_head_score_mfma
 from .hook import install, uninstall
-from .layout import response_slice, roll_labels, transpose_2d
+from .layout import expand_per_sequence, response_from_packed, response_slice, roll_labels, transpose_2d
 from .spec_rl import (
     VerifyResult,
     draw_log_uniforms,
@@ -50,6 +50,8 @@ __all__ = [
     "spec_verify",
     "thresh_offset_from_lenience",
     "truncate_draft",
+    "expand_per_sequence",
+    "response_from_packed",
     "response_slice",
     "roll_labels",
     "transpose_2d",

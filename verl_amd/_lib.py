@@ -32,7 +32,7 @@ VRL_FLAG_LABEL_OOB = 1
 VRL_FLAG_SLICE_RANGE = 2
 VRL_FLAG_SEQ_RANGE = 4
 
-ABI_VERSION = 3
+ABI_VERSION = 4
 
 _c = ctypes
 _P = _c.c_void_p
@@ -53,6 +53,7 @@ SIGNATURES = {
         _INT, [_P, _INT, _I64, _I64, _I64, _P, _P, _P, _P, _P, _I64, _I64, _P, _P, _P, _P, _P, _I64, _P]),
     "vrl_response_slice": (_INT, [_P, _I64, _P, _P, _I64, _I64, _I64, _P, _P, _P]),
     "vrl_response_pack": (_INT, [_P, _I64, _P, _P, _P, _I64, _I64, _I64, _P, _P, _P]),
+    "vrl_expand_per_sequence": (_INT, [_P, _P, _I64, _I64, _P, _P, _P]),
     "vrl_lmhead_score": (_INT, [_P, _P, _INT, _I64, _I64, _I64, _I64, _I64, _P, _P, _INT, _P, _P, _P, _P, _P, _P, _I64, _P]),
     "vrl_lmhead_dlogits": (_INT, [_P, _P, _INT, _I64, _I64, _I64, _I64, _I64, _P, _P, _P, _P, _P, _P, _INT, _P, _I64, _P]),
     "vrl_gemm_nt_plan": (_INT, [_INT, _I64, _I64, _I64, _P]),

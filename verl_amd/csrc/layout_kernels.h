@@ -118,4 +118,31 @@ __global__ __launch_bounds__(kSliceThreads) void response_pack_kernel(
   }
 }
 
+// One value per sequence -> one value per token of the packed batch: out[t] = values[b] for the sequence b that holds
+// token t (cu_seqlens[b] <= t < cu_seqlens[b+1]). One thread per token finds its sequence by bisection over the
+// offsets (every index stays in [0, B], whatever they hold) and writes exactly one element; a token that no sequence
+// holds gets 0 and sets VRL_FLAG_SEQ_RANGE (4), and so do offsets that do not start at 0, end at n_tokens or decrease
+// (threads 0 .. B check one entry each). grid = ceil(max(n_tokens, B + 1) / 256), block = 256, B >= 1.
+__global__ __launch_bounds__(kSliceThreads) void expand_per_sequence_kernel(
+    const float* __restrict__ values, const int64_t* __restrict__ cu_seqlens, int64_t B, int64_t n_tokens,
+    float* __restrict__ out, int32_t* err_flag) {
+  const int64_t t = static_cast<int64_t>(blockIdx.x) * kSliceThreads + threadIdx.x;
+  bool bad = false;
+  if (t <= B) {
+    const int64_t c = cu_seqlens[t];
+    bad = (t == 0 && c != 0) || (t == B && c != n_tokens) || (t < B && cu_seqlens[t + 1] < c);
+  }
+  if (t < n_tokens) {
+    int64_t lo = 0, hi = B;   // the largest b < B with cu_seqlens[b] <= t lies in [lo, hi)
+    while (hi - lo > 1) {
+      const int64_t mid = (lo + hi) >> 1;
+      if (cu_seqlens[mid] <= t) lo = mid; else hi = mid;
+    }
+    const bool held = cu_seqlens[lo] <= t && t < cu_seqlens[lo + 1];
+    out[t] = held ? values[lo] : 0.f;
+    bad = bad || !held;
+  }
+  if (bad) atomicOr(err_flag, 4);
+}
+
 }  // namespace vrl

@@ -738,6 +738,21 @@ int vrl_response_slice(const void* values, int64_t row_bytes, const int64_t* cu_
   return launch_status();
 }
 
+int vrl_expand_per_sequence(const float* values, const int64_t* cu_seqlens, int64_t B, int64_t n_tokens, float* out,
+                            int32_t* err_flag, void* stream) {
+  if (B < 0 || n_tokens < 0 || B > kMaxGrid) return VRL_ERR_SHAPE;
+  if (B == 0) return n_tokens == 0 ? VRL_OK : VRL_ERR_SHAPE;   // tokens, but no sequence to take a value from
+  if (values == nullptr || cu_seqlens == nullptr || err_flag == nullptr || (out == nullptr && n_tokens > 0))
+    return VRL_ERR_NULL;
+  if (!aligned(values, 4) || !aligned(out, 4) || !aligned(cu_seqlens, 8) || !aligned(err_flag, 4)) return VRL_ERR_ALIGN;
+  const int64_t threads = n_tokens > B + 1 ? n_tokens : B + 1;
+  const int64_t blocks = (threads + vrl::kSliceThreads - 1) / vrl::kSliceThreads;
+  if (blocks > kMaxGrid) return VRL_ERR_SHAPE;
+  vrl::expand_per_sequence_kernel<<<dim3(static_cast<unsigned>(blocks)), dim3(vrl::kSliceThreads), 0,
+                                    static_cast<hipStream_t>(stream)>>>(values, cu_seqlens, B, n_tokens, out, err_flag);
+  return launch_status();
+}
+
 int vrl_response_pack(const void* values, int64_t row_bytes, const int64_t* cu_seqlens, const int64_t* response_lens,
                       const int64_t* out_offsets, int64_t B, int64_t n_tokens, int64_t out_total, void* out,
                       int32_t* err_flag, void* stream) {

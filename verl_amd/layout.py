@@ -1,7 +1,8 @@
 """Layout steps either side of the scoring path, on the GPU.
 
 ``roll_labels`` restates the one-line label construction of the reference's engine
-(verl/workers/engine/fsdp/transformer_impl.py:1177); ``response_slice`` replaces the
+(verl/workers/engine/fsdp/transformer_impl.py:1177); ``expand_per_sequence`` builds the per-token temperature from the
+per-sample one (verl/utils/torch_functional.py:989-1011); ``response_slice`` replaces the
 per-sequence Python loop of verl/workers/utils/padding.py:97-141 with one kernel launch;
 ``transpose_2d`` is the bit-exact transposed copy the LM-head backward uses to give the library GEMM
 operands that are contiguous along the contraction axis.
@@ -16,7 +17,7 @@ import torch
 from . import _lib
 from . import errors as _errors
 
-__all__ = ["roll_labels", "response_slice", "response_from_packed", "transpose_2d"]
+__all__ = ["roll_labels", "expand_per_sequence", "response_slice", "response_from_packed", "transpose_2d"]
 
 
 def roll_labels(input_ids_rmpad: torch.Tensor) -> torch.Tensor:
@@ -153,4 +154,42 @@ def transpose_2d(x: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.T
                                out.data_ptr(), out.stride(0) if cols > 1 else rows,
                                _lib.stream_ptr(x.device))
     _lib.check("vrl_transpose", st)
+    return out
+
+
+def expand_per_sequence(values: torch.Tensor, cu_seqlens: torch.Tensor, total_nnz: Optional[int] = None,
+                        check=None) -> torch.Tensor:
+    """One value per sequence ``(B,)`` -> one per token of the packed batch ``(total_nnz,)`` fp32: token t gets
+    ``values[b]`` for ``cu_seqlens[b] <= t < cu_seqlens[b+1]``. The values of the reference's
+    ``expand_as_nested(temperature, input_ids)`` (verl/utils/torch_functional.py:989-1011,
+    ``repeat_interleave`` by the sequence lengths), which is how the engine builds the per-token temperature
+    (verl/workers/engine/fsdp/transformer_impl.py:1158-1162).
+
+    ``total_nnz`` (= ``cu_seqlens[-1]``, which sizes the result) spares the call its read-back from the device when
+    the caller knows it; offsets that are not a partition of ``[0, total_nnz]`` raise ValueError as ``check`` says
+    (verl_amd.errors)."""
+    _errors.poll()
+    if values.dim() != 1:
+        raise ValueError(f"expand_per_sequence: values must have one entry per sequence, got shape {tuple(values.shape)}")
+    if not values.is_cuda:
+        raise RuntimeError(f"values is on {values.device}; verl_amd only runs on the GPU, it has no CPU implementation")
+    dev = values.device
+    v = values.to(dtype=torch.float32).contiguous()
+    cu = cu_seqlens.to(device=dev, dtype=torch.int64).contiguous()
+    B = v.numel()
+    if cu.dim() != 1 or cu.numel() != B + 1:
+        raise ValueError(f"expand_per_sequence: cu_seqlens must have B+1 = {B + 1} entries, got {tuple(cu.shape)}")
+    n = int(cu[-1].item()) if total_nnz is None else int(total_nnz)
+    if n < 0:
+        raise ValueError("expand_per_sequence: total_nnz must not be negative")
+    out = torch.empty(n, dtype=torch.float32, device=dev)
+    flag = torch.zeros(1, dtype=torch.int32, device=dev)
+    lib = _lib.load()
+    with torch.cuda.device(dev):
+        st = lib.vrl_expand_per_sequence(v.data_ptr() if B else None, cu.data_ptr(), B, n,
+                                         out.data_ptr() if n else None, flag.data_ptr(), _lib.stream_ptr(dev))
+    _lib.check("vrl_expand_per_sequence", st)
+    if B > 0:
+        _errors.report(flag, {_lib.VRL_FLAG_SEQ_RANGE: (ValueError, f"expand_per_sequence: cu_seqlens is not a "
+                              f"partition of the {n} tokens (it must start at 0, never decrease and end there)")}, check)
     return out

@@ -533,7 +533,8 @@ def score_responses(
     (verl/workers/engine/fsdp/transformer_impl.py:1177), divide by the temperature (:1357), entropy and log-probs
     (:1364-1399), then ``no_padding_2_padding`` (verl/workers/utils/padding.py:97-141: per sequence take
     ``values[end - r - 1 : end - 1]`` and right-pad with zeros) — done by the row kernel itself: give ``input_ids``
-    (the packed ids, rolled inside the kernel) or ready ``labels``; ``temperature`` is a float or one value per token.
+    (the packed ids, rolled inside the kernel) or ready ``labels``; ``temperature`` is a float, one value per token or one per
+    sequence (expanded over its tokens like ``expand_as_nested``, verl/utils/torch_functional.py:989-1011).
 
     Returns ``(resp_logprob | None, resp_entropy | None)``; with ``per_token`` also the ``(total_nnz,)`` vectors, as
     ``(resp_logprob, resp_entropy, logprob, entropy)``. Without ``per_token`` the logits of tokens outside every
@@ -564,12 +565,16 @@ def score_responses(
         if src.dtype.is_floating_point or src.dtype == torch.bool:
             raise TypeError(f"{what}: labels / input_ids must be an integer tensor, got {src.dtype}")
         lab = src.to(device=dev, dtype=torch.int64).contiguous()
-    temp = _temperature_rows(temperature, (n,), n, dev)
     cu = cu_seqlens.to(device=dev, dtype=torch.int64).contiguous()
     rl = response_lens.to(device=dev, dtype=torch.int64).contiguous()
     B = rl.numel()
     if cu.dim() != 1 or cu.numel() != B + 1:
         raise ValueError(f"{what}: cu_seqlens must have B+1 = {B + 1} entries, got {tuple(cu.shape)}")
+    if isinstance(temperature, torch.Tensor) and temperature.dim() == 1 and temperature.numel() == B and B != n and B > 1:
+        # one value per sample, as the engine holds it (fsdp/transformer_impl.py:1149-1162)
+        from .layout import expand_per_sequence
+        temperature = expand_per_sequence(temperature.to(dev), cu, n, check)
+    temp = _temperature_rows(temperature, (n,), n, dev)
     T = int(max_response_len)
     if T < 0:
         raise ValueError(f"{what}: max_response_len must not be negative")
