@@ -597,7 +597,7 @@ def bench_lm_head(args, dev):
         kernels = [
             rec("lmhead_partial_kernel<bf16, false> + lmhead_finish_kernel", f"forward, {T} tokens", t_m * 1e3, flops_all),
             rec("lmhead_partial_kernel<bf16, true> + lmhead_finish_kernel", f"forward that also writes the logits, {T} tokens",
-                per_launch(lambda: own_fl._own_forward(Hd, Wd, ids, None, None, "bench", keep=True), 5), flops_all),
+                per_launch(lambda: own_fl._own_forward(Hd, Wd, ids, None, None, "bench", keep_rows=T), 5), flops_all),
             rec("lmhead_dlogits_kernel<bf16>", f"logits formed again, their gradient written, {n_c} tokens", per_launch(dlogits),
                 flops_c),
         ]

@@ -287,6 +287,8 @@ int vrl_transpose(const void* src, int elem_size, int64_t rows, int64_t cols, in
  * multiples of 8, 16-byte aligned): for a backward pass that may spend n_tokens * vocab elements of memory instead of
  * forming the logits again, which then runs vrl_rowscore_backward over them in place (the reference's torch path keeps
  * them the same way, verl/utils/experimental/torch_functional.py:33-35). The scores are folded from the fp32 values either way.
+ * Only the first logits_rows tokens' logits are written (1 <= logits_rows <= n_tokens, VRL_ERR_SHAPE otherwise; ignored
+ * without logits_out): a caller with a memory budget keeps what fits and forms the rest again in its backward pass.
  *
  * fp32 operands are refused (VRL_ERR_DTYPE) on purpose: the part's fp32 matrix rate (157 TFLOP/s) is what the library GEMM
  * already delivers, so an fp32 LM head is served by the library GEMM followed by vrl_rowscore (the Python side does that),
@@ -300,7 +302,7 @@ int vrl_lmhead_score(const void* hidden, const void* weight, int dtype, int64_t 
                      int64_t hidden_size, int64_t h_stride, int64_t w_stride, const int64_t* labels,
                      const float* temperature, int n_splits, float* partials, float* out_logprob,
                      float* out_entropy, float* out_lse, int32_t* err_flag, void* logits_out, int64_t logits_stride,
-                     void* stream);
+                     int64_t logits_rows, void* stream);
 /*
  * vrl_lmhead_dlogits — backward counterpart of vrl_lmhead_score: the logits are formed again on the matrix cores,
  * tile by tile, and turned in registers into the gradient with respect to the logits,

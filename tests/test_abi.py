@@ -327,12 +327,12 @@ def test_response_pack_argument_errors(lib):
 def test_lmhead_argument_errors(lib):
     f = lib.vrl_lmhead_score
     ok = dict(h=P, w=P, dt=_lib.VRL_BF16, T=512, V=1024, K=128, hs=128, ws=128, lab=P, temp=None, S=2, part=P, lp=P, ent=P,
-              lse=None, flag=P, logits=None, ls=0)
+              lse=None, flag=P, logits=None, ls=0, lr=0)
 
     def call(**kw):
         a = {**ok, **kw}
         return f(a["h"], a["w"], a["dt"], a["T"], a["V"], a["K"], a["hs"], a["ws"], a["lab"], a["temp"], a["S"], a["part"],
-                 a["lp"], a["ent"], a["lse"], a["flag"], a["logits"], a["ls"], None)
+                 a["lp"], a["ent"], a["lse"], a["flag"], a["logits"], a["ls"], a["lr"], None)
 
     assert call(dt=_lib.VRL_F32) == _lib.VRL_ERR_DTYPE
     assert call(T=255) == _lib.VRL_ERR_SHAPE and call(V=100) == _lib.VRL_ERR_SHAPE
@@ -343,10 +343,12 @@ def test_lmhead_argument_errors(lib):
     assert call(lab=None) == _lib.VRL_ERR_NULL and call(flag=None) == _lib.VRL_ERR_NULL
     assert call(h=P + 8) == _lib.VRL_ERR_ALIGN and call(w=P + 2) == _lib.VRL_ERR_ALIGN
     # kept logits: a pitch that holds a row and keeps 8-byte groups aligned
-    assert call(logits=P, ls=1000) == _lib.VRL_ERR_SHAPE and call(logits=P, ls=1028) == _lib.VRL_ERR_SHAPE
-    assert call(logits=P, ls=1024, V=1020) == _lib.VRL_ERR_SHAPE
-    assert call(logits=P + 8, ls=1024) == _lib.VRL_ERR_ALIGN
-    assert call(lp=None, ent=None, logits=P, ls=1024, h=None) == _lib.VRL_ERR_NULL     # the logits alone are a valid request
+    assert call(logits=P, ls=1000, lr=512) == _lib.VRL_ERR_SHAPE and call(logits=P, ls=1028, lr=512) == _lib.VRL_ERR_SHAPE
+    assert call(logits=P, ls=1024, V=1020, lr=512) == _lib.VRL_ERR_SHAPE
+    assert call(logits=P + 8, ls=1024, lr=512) == _lib.VRL_ERR_ALIGN
+    assert call(lp=None, ent=None, logits=P, ls=1024, lr=256, h=None) == _lib.VRL_ERR_NULL   # the logits alone are a valid request
+    # ... of the first logits_rows tokens, at least one and no more than there are
+    assert call(logits=P, ls=1024, lr=0) == _lib.VRL_ERR_SHAPE and call(logits=P, ls=1024, lr=513) == _lib.VRL_ERR_SHAPE
     assert lib.vrl_lmhead_plan(8192, 152064) == 8 and lib.vrl_lmhead_plan(0, 5) == 1
 
 

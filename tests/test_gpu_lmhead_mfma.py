@@ -376,7 +376,7 @@ def test_matrix_core_entry_points_replay_from_a_graph(dev):
     def call(stream):
         assert lib.vrl_lmhead_score(h.data_ptr(), w.data_ptr(), BF, T, V, K, K, K, ids.data_ptr(), None, splits,
                                     partials.data_ptr(), lp.data_ptr(), ent.data_ptr(), lse.data_ptr(), flag.data_ptr(),
-                                    None, 0, stream) == 0
+                                    None, 0, 0, stream) == 0
         assert lib.vrl_lmhead_dlogits(h.data_ptr(), w.data_ptr(), BF, T, V, K, K, K, ids.data_ptr(), None, lse.data_ptr(),
                                       ent.data_ptr(), g_lp.data_ptr(), g_ent.data_ptr(), lib.vrl_lmhead_plan(T, V),
                                       G.data_ptr(), V, stream) == 0
@@ -469,7 +469,8 @@ def test_forward_also_writes_the_logits_when_asked(dev, dtype, T, V, K):
         with torch.cuda.device(dev):
             st = lib.vrl_lmhead_score(h.data_ptr(), w.data_ptr(), code, T, V, K, K, K, ids.data_ptr(), temp.data_ptr(), splits,
                                       part.data_ptr(), lp.data_ptr(), ent.data_ptr(), lse.data_ptr(), flag.data_ptr(),
-                                      logits.data_ptr() if keep else None, pitch if keep else 0, _lib.stream_ptr(dev))
+                                      logits.data_ptr() if keep else None, pitch if keep else 0, T if keep else 0,
+                                      _lib.stream_ptr(dev))
         assert st == _lib.VRL_OK, lib.vrl_strerror(st)
         outs.append((lp, ent, lse, logits))
     for a, b in zip(outs[0][:3], outs[1][:3]):
@@ -537,8 +538,85 @@ def test_logits_are_kept_by_default_when_they_fit_the_budget(dev, monkeypatch):
     torch.autograd.grad(lp, hidden, g_lp, retain_graph=True)
     with pytest.raises(RuntimeError, match="overwritten by the first backward"):
         torch.autograd.grad(lp, hidden, g_lp)
-    monkeypatch.setattr(fl, "DEFAULT_KEEP_LOGITS_BYTES", T * V * 2 - 1)
+    monkeypatch.setattr(fl, "DEFAULT_KEEP_LOGITS_BYTES", 256 * V * 2 - 1)      # not even one 256-token block
     lp2, _ = fused_linear_for_ppo(hidden, weight, labels)
     a = torch.autograd.grad(lp2, hidden, g_lp, retain_graph=True)[0]
     b = torch.autograd.grad(lp2, hidden, g_lp)[0]
     assert torch.equal(a, b) and torch.equal(lp, lp2)
+
+
+@pytest.mark.parametrize("T,V,D,budget_rows", [(1100, 4104, 256, 600), (2304, 8192, 512, 2303), (1300, 1000, 320, 600),
+                                               (1536, 1024, 256, 1100)])
+def test_a_budget_below_all_logits_keeps_the_leading_blocks(dev, monkeypatch, T, V, D, budget_rows):
+    """keep_logits=None with a budget that holds only some of the logits: the forward kernel writes the logits of the
+    leading tokens, as many whole 256-token blocks as fit and leave whole chunks (vrl_lmhead_score's logits_rows), the
+    backward turns those into their gradient
+    in place and forms the rest again chunk by chunk, adding its share of d W. Same scores as both other paths, gradients
+    within the tolerances those two agree to."""
+    from verl_amd import fused_linear as fl
+    from verl_amd import gemm
+
+    g = torch.Generator(device=dev).manual_seed(T + V)
+    hidden = torch.empty(T, D, device=dev).uniform_(-0.5, 0.5, generator=g).bfloat16().requires_grad_()
+    weight = torch.empty(V, D, device=dev).uniform_(-0.5, 0.5, generator=g).bfloat16().requires_grad_()
+    labels = torch.randint(0, V, (T,), generator=g, device=dev)
+    g_ent = torch.empty(T, device=dev).uniform_(-0.5, 0.5, generator=g)
+    g_lp = torch.empty(T, device=dev).uniform_(-1, 1, generator=g)
+    r_lp, r_ent, _ = ofl.forward(hidden, weight, labels, 1.5, dtype=torch.float32)
+    d_ref_h, d_ref_w = torch.autograd.grad((r_ent, r_lp), (hidden, weight), (g_ent, g_lp))
+    lp0, ent0 = fused_linear_for_ppo(hidden, weight, labels, 1.5, keep_logits=False, chunk_size=512)
+    dh0, dw0 = torch.autograd.grad((ent0, lp0), (hidden, weight), (g_ent, g_lp))
+    monkeypatch.setattr(fl, "DEFAULT_KEEP_LOGITS_BYTES", budget_rows * V * 2)
+    again = -(-(T - budget_rows) // 512) * 512          # what is formed again is whole chunks (of 512 tokens here)
+    kept_rows = max(T - again, 0) // 256 * 256
+    seen = {}
+    real = fl._own_forward
+
+    def spy(*a, **k):
+        out = real(*a, **k)
+        seen["kept"] = None if out[3] is None else tuple(out[3].shape)
+        return out
+
+    monkeypatch.setattr(fl, "_own_forward", spy)
+    lp, ent = fused_linear_for_ppo(hidden, weight, labels, 1.5, chunk_size=512)
+    assert seen["kept"] == (kept_rows, V)
+    assert torch.equal(lp, lp0) and torch.equal(ent, ent0)
+    before = gemm.counters["gemm"]
+    d_h, d_w = torch.autograd.grad((ent, lp), (hidden, weight), (g_ent, g_lp), retain_graph=True)
+    assert gemm.counters["gemm"] > before + 2            # the kept part's two products and the chunks' after them
+    torch.testing.assert_close(d_ref_h.float(), d_h.float(), atol=1e-2, rtol=1e-2)
+    torch.testing.assert_close(d_ref_w.float(), d_w.float(), atol=1e-2, rtol=1e-2)
+    torch.testing.assert_close(dh0.float(), d_h.float(), atol=1e-2, rtol=2e-2)
+    torch.testing.assert_close(dw0.float(), d_w.float(), atol=1e-2, rtol=2e-2)
+    with pytest.raises(RuntimeError, match="overwritten by the first backward"):
+        torch.autograd.grad((ent, lp), (hidden, weight), (g_ent, g_lp))
+
+
+def test_only_the_first_logits_rows_are_written(dev):
+    """vrl_lmhead_score with logits_rows below the token count: those rows hold what the full call writes, the rest of the
+    buffer is untouched, the scores are the same bits."""
+    lib = _lib.load()
+    g = torch.Generator(device=dev).manual_seed(9)
+    T, V, K, rows = 1000, 1032, 128, 512
+    h = torch.empty(T, K, device=dev).uniform_(-0.5, 0.5, generator=g).bfloat16()
+    w = torch.empty(V, K, device=dev).uniform_(-0.5, 0.5, generator=g).bfloat16()
+    ids = torch.randint(0, V, (T,), generator=g, device=dev)
+    splits = 2
+    part = torch.empty(T * splits * 4, device=dev)
+    outs = []
+    for n_rows in (T, rows, 1):
+        lp, ent, lse = (torch.empty(T, device=dev) for _ in range(3))
+        flag = torch.zeros(1, dtype=torch.int32, device=dev)
+        logits = torch.full((T, V), float("nan"), dtype=torch.bfloat16, device=dev)
+        with torch.cuda.device(dev):
+            st = lib.vrl_lmhead_score(h.data_ptr(), w.data_ptr(), _lib.VRL_BF16, T, V, K, K, K, ids.data_ptr(), None, splits,
+                                      part.data_ptr(), lp.data_ptr(), ent.data_ptr(), lse.data_ptr(), flag.data_ptr(),
+                                      logits.data_ptr(), V, n_rows, _lib.stream_ptr(dev))
+        assert st == _lib.VRL_OK, lib.vrl_strerror(st)
+        outs.append((lp, ent, lse, logits))
+    full = outs[0][3]
+    assert torch.isfinite(full.float()).all()
+    for (lp, ent, lse, logits), n_rows in zip(outs[1:], (rows, 1)):
+        assert torch.equal(lp, outs[0][0]) and torch.equal(ent, outs[0][1]) and torch.equal(lse, outs[0][2])
+        assert torch.equal(logits[:n_rows], full[:n_rows])
+        assert torch.isnan(logits[n_rows:].float()).all()

@@ -54,7 +54,8 @@ SIGNATURES = {
     "vrl_response_slice": (_INT, [_P, _I64, _P, _P, _I64, _I64, _I64, _P, _P, _P]),
     "vrl_response_pack": (_INT, [_P, _I64, _P, _P, _P, _I64, _I64, _I64, _P, _P, _P]),
     "vrl_expand_per_sequence": (_INT, [_P, _P, _I64, _I64, _P, _P, _P]),
-    "vrl_lmhead_score": (_INT, [_P, _P, _INT, _I64, _I64, _I64, _I64, _I64, _P, _P, _INT, _P, _P, _P, _P, _P, _P, _I64, _P]),
+    "vrl_lmhead_score": (_INT, [_P, _P, _INT, _I64, _I64, _I64, _I64, _I64, _P, _P, _INT, _P, _P, _P, _P, _P, _P, _I64, _I64,
+                                _P]),
     "vrl_lmhead_dlogits": (_INT, [_P, _P, _INT, _I64, _I64, _I64, _I64, _I64, _P, _P, _P, _P, _P, _P, _INT, _P, _I64, _P]),
     "vrl_gemm_nt_plan": (_INT, [_INT, _I64, _I64, _I64, _P]),
     "vrl_gemm_nt": (_INT, [_P, _P, _INT, _I64, _I64, _I64, _I64, _I64, _P, _I64, _INT, _INT, _P, _P]),

@@ -424,7 +424,7 @@ template <int DT, bool STORE>
 __global__ __launch_bounds__(kLmWaves * 64, 1) void lmhead_partial_kernel(
     const uint16_t* __restrict__ W, const uint16_t* __restrict__ H, int64_t V, int64_t T, int64_t K, int64_t w_stride,
     int64_t h_stride, const float* __restrict__ temperature, int n_splits, int tiles_per_split,
-    int xcd_map, float* __restrict__ partials, uint16_t* __restrict__ logits_out, int64_t l_stride) {
+    int xcd_map, float* __restrict__ partials, uint16_t* __restrict__ logits_out, int64_t l_stride, int64_t l_rows) {
   extern __shared__ __attribute__((aligned(1024))) char lds[];  // the operand ring; its start serves the final merge
   float (*red)[256][3] = reinterpret_cast<float (*)[256][3]>(lds);   // [4][256][3], used once the walk is over
 
@@ -464,7 +464,8 @@ __global__ __launch_bounds__(kLmWaves * 64, 1) void lmhead_partial_kernel(
         for (int v = 0; v < 4; ++v) x[i * 4 + v] = acc[i][j][v];
       if constexpr (STORE) {
         using O = ElemOut<DT>;
-        if (tok0v + j * 16 >= work.tok0) {   // false for the rows an edge block shares with the block before
+        // (false for the rows an edge block shares with the block before, and for tokens whose logits are not kept)
+        if (tok0v + j * 16 >= work.tok0 && tok0v + j * 16 < l_rows) {
           uint16_t* out = logits_out + (tok0v + j * 16) * l_stride;
 #pragma unroll
           for (int i = 0; i < 4; ++i) {
@@ -663,7 +664,8 @@ __global__ __launch_bounds__(kLmWaves * 64, 1) void lmhead_dlogits_kernel(
 //
 // A work item is (y block of 256 rows, `tiles_per_item` x tiles, one of `k_parts` ranges of the contraction). Items
 // are dealt so that the workgroups resident on one XCD together form py x px patches of (y block, x split) pairs of
-// one contraction range and share their operand tiles through its L2; ids past the last patch leave at once.
+// one contraction range and share their operand tiles through its L2; ids past the last patch leave at once, and so do
+// the slots of a patch that lie past the last y block or x split (py and px need not divide their counts).
 // MODE 0 stores the product in the operands' type, MODE 1 adds it to what `out` holds (one rounding, like a GEMM with
 // beta = 1), MODE 2 stores fp32 partial sums at partials[(kp * NY + y) * NX + x] for lm_gemm_reduce_kernel.
 typedef float f32x4 __attribute__((ext_vector_type(4)));
@@ -702,7 +704,7 @@ __global__ __launch_bounds__(kLmWaves * 64, 1) void lm_gemm_kernel(
   const int64_t nyb = (g.NY + kLmTokens - 1) / kLmTokens;
   const int64_t nxt = (g.NX + kLmVocab - 1) / kLmVocab;
   const int64_t nxs = (nxt + g.tiles_per_item - 1) / g.tiles_per_item;
-  const int64_t patches_y = nyb / g.py, patches_x = nxs / g.px;   // the host passes py | nyb and px | nxs
+  const int64_t patches_y = (nyb + g.py - 1) / g.py, patches_x = (nxs + g.px - 1) / g.px;
   const int64_t per_part = patches_y * patches_x;
   const int psize = g.py * g.px;
   const int64_t id = blockIdx.x;
@@ -715,6 +717,7 @@ __global__ __launch_bounds__(kLmWaves * 64, 1) void lm_gemm_kernel(
   const int r = __builtin_amdgcn_readfirstlane((int)(patch % per_part));
   const int yb = __builtin_amdgcn_readfirstlane((int)((r % patches_y) * g.py + within % g.py));
   const int xsplit = __builtin_amdgcn_readfirstlane((int)((r / patches_y) * g.px + within / g.py));
+  if (yb >= nyb || xsplit >= nxs) return;   // a slot of the last row or column of patches that holds no work
 
   LmWork work;
   work.split = kp;

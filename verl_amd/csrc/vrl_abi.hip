@@ -280,7 +280,7 @@ template <int DT, bool STORE>
 int launch_lmhead(const void* hidden, const void* weight, int64_t T, int64_t V, int64_t K, int64_t h_stride,
                   int64_t w_stride, const int64_t* labels, const float* temperature, int n_splits, float* partials,
                   float* out_logprob, float* out_entropy, float* out_lse, int32_t* err_flag, void* logits_out,
-                  int64_t l_stride, hipStream_t s) {
+                  int64_t l_stride, int64_t l_rows, hipStream_t s) {
   const LmGrid g = lm_grid(T, V, n_splits);
   static std::atomic<bool> raised[kMaxDevices];
   const int rs = raise_lds_limit(reinterpret_cast<const void*>(vrl::lmhead_partial_kernel<DT, STORE>), raised);
@@ -288,7 +288,8 @@ int launch_lmhead(const void* hidden, const void* weight, int64_t T, int64_t V, 
   vrl::lmhead_partial_kernel<DT, STORE><<<dim3(static_cast<unsigned>(g.tblocks * n_splits)), dim3(vrl::kLmWaves * 64),
                                           vrl::kLmLdsBytes, s>>>(
       static_cast<const uint16_t*>(weight), static_cast<const uint16_t*>(hidden), V, T, K, w_stride, h_stride,
-      temperature, n_splits, g.tiles_per_split, g.xcd_map, partials, static_cast<uint16_t*>(logits_out), l_stride);
+      temperature, n_splits, g.tiles_per_split, g.xcd_map, partials, static_cast<uint16_t*>(logits_out), l_stride,
+      l_rows);
   vrl::lmhead_finish_kernel<DT><<<dim3(static_cast<unsigned>((T + 3) / 4)), dim3(256), 0, s>>>(
       static_cast<const char*>(weight), static_cast<const char*>(hidden), V, T, K, w_stride, h_stride, labels,
       temperature, n_splits, partials, out_logprob, out_entropy, out_lse, err_flag);
@@ -337,7 +338,7 @@ int check_lmhead_shape(int dtype, int64_t n_tokens, int64_t vocab, int64_t hidde
 // rounds. One workgroup per CU runs at a time (the kernels take all of its LDS).
 struct GemmPlan {
   vrl::LmGemmShape shape;
-  int64_t items;
+  int64_t patches;   // py x px groups of work items, over all contraction ranges
 };
 
 int device_cus() {
@@ -352,10 +353,30 @@ int device_cus() {
   return n;
 }
 
-int largest_divisor_up_to(int64_t n, int limit) {
-  for (int d = limit; d > 1; --d)
-    if (n % d == 0) return d;
-  return 1;
+// The workgroups resident on one XCD form patches of py y blocks x px x splits that walk the contraction in step and
+// share operand tiles through its L2: an X tile is fetched once for the py workgroups that use it, a Y tile once for px,
+// so what leaves L2 is proportional to 1/py + 1/px. Counts that py or px do not divide leave idle slots in the last
+// row or column of patches (those workgroups return at once), which lowers the sharing there; the choice below weighs
+// both by the average number of busy workgroups per patch row and column. py <= 4, px <= 8: 32 CUs per XCD.
+void choose_patch(int64_t nyb, int64_t nxs, int* py_out, int* px_out) {
+  double best = 1e30;
+  int best_py = 1, best_px = 1;
+  for (int py = 1; py <= 4; ++py) {
+    for (int px = 1; px <= 8; ++px) {
+      const double eff_y = static_cast<double>(nyb) / static_cast<double>((nyb + py - 1) / py);
+      const double eff_x = static_cast<double>(nxs) / static_cast<double>((nxs + px - 1) / px);
+      const double slots = static_cast<double>(((nyb + py - 1) / py) * py) * static_cast<double>(((nxs + px - 1) / px) * px);
+      // fetched bytes, and as a tie-break (1e-3 per unit) the share of slots that hold no work
+      const double cost = 1.0 / eff_y + 1.0 / eff_x + 1e-3 * slots / (static_cast<double>(nyb) * static_cast<double>(nxs));
+      if (cost < best - 1e-12) {
+        best = cost;
+        best_py = py;
+        best_px = px;
+      }
+    }
+  }
+  *py_out = best_py;
+  *px_out = best_px;
 }
 
 GemmPlan gemm_plan(int64_t NX, int64_t NY, int64_t K, int forced_parts) {
@@ -386,9 +407,8 @@ GemmPlan gemm_plan(int64_t NX, int64_t NY, int64_t K, int forced_parts) {
   }
   g.steps_per_part = static_cast<int>((g.k_steps + best - 1) / best);
   g.k_parts = static_cast<int>((g.k_steps + g.steps_per_part - 1) / g.steps_per_part);   // no empty range
-  g.py = largest_divisor_up_to(nyb, 4);
-  g.px = largest_divisor_up_to(nxs, 8);
-  p.items = base * g.k_parts;
+  choose_patch(nyb, nxs, &g.py, &g.px);
+  p.patches = ((nyb + g.py - 1) / g.py) * ((nxs + g.px - 1) / g.px) * g.k_parts;
   return p;
 }
 
@@ -397,8 +417,7 @@ int launch_gemm(const void* x, const void* y, const GemmPlan& plan, int64_t x_st
                 int64_t out_stride, int accumulate, float* workspace, hipStream_t s) {
   const vrl::LmGemmShape& g = plan.shape;
   const int psize = g.py * g.px;
-  const int64_t patches = plan.items / psize;
-  const int64_t grid = ((patches + 7) / 8) * 8 * psize;
+  const int64_t grid = ((plan.patches + 7) / 8) * 8 * psize;
   if (grid > kMaxGrid) return VRL_ERR_SHAPE;
   const dim3 gd(static_cast<unsigned>(grid)), bd(vrl::kLmWaves * 64);
   const uint16_t* X = static_cast<const uint16_t*>(x);
@@ -810,10 +829,11 @@ int vrl_lmhead_score(const void* hidden, const void* weight, int dtype, int64_t 
                      int64_t hidden_size, int64_t h_stride, int64_t w_stride, const int64_t* labels,
                      const float* temperature, int n_splits, float* partials, float* out_logprob,
                      float* out_entropy, float* out_lse, int32_t* err_flag, void* logits_out, int64_t logits_stride,
-                     void* stream) {
+                     int64_t logits_rows, void* stream) {
   const int cs = check_lmhead_shape(dtype, n_tokens, vocab, hidden_size, h_stride, w_stride, n_splits);
   if (cs != VRL_OK) return cs;
   if (out_logprob == nullptr && out_entropy == nullptr && out_lse == nullptr && logits_out == nullptr) return VRL_ERR_ARG;
+  if (logits_out != nullptr && (logits_rows < 1 || logits_rows > n_tokens)) return VRL_ERR_SHAPE;
   if (hidden == nullptr || weight == nullptr || partials == nullptr) return VRL_ERR_NULL;
   if (out_logprob != nullptr && (labels == nullptr || err_flag == nullptr)) return VRL_ERR_NULL;
   // kept logits: 8-byte stores of 4 consecutive vocabulary entries, so the vocabulary and the pitch must keep them aligned
@@ -826,7 +846,7 @@ int vrl_lmhead_score(const void* hidden, const void* weight, int dtype, int64_t 
   hipStream_t s = static_cast<hipStream_t>(stream);
 #define VRL_LMHEAD_ARGS                                                                                            \
   hidden, weight, n_tokens, vocab, hidden_size, h_stride, w_stride, labels, temperature, n_splits, partials,        \
-      out_logprob, out_entropy, out_lse, err_flag, logits_out, logits_stride, s
+      out_logprob, out_entropy, out_lse, err_flag, logits_out, logits_stride, logits_rows, s
   if (dtype == VRL_BF16)
     return logits_out != nullptr ? launch_lmhead<VRL_BF16, true>(VRL_LMHEAD_ARGS) : launch_lmhead<VRL_BF16, false>(VRL_LMHEAD_ARGS);
   return logits_out != nullptr ? launch_lmhead<VRL_F16, true>(VRL_LMHEAD_ARGS) : launch_lmhead<VRL_F16, false>(VRL_LMHEAD_ARGS);

@@ -88,10 +88,11 @@ def _own_forward_in_use(kernels: str, hidden: torch.Tensor, weight: torch.Tensor
     return kernels != "library" and _mfma_takes_model(hidden, weight)
 
 
-# keep_logits=None (the default) keeps the logits for the backward when all of them fit this many bytes: on a 288 GB part
-# the 2.5 GB of an 8192 x 152064 bf16 micro-batch are under 1 % of the memory and save a quarter of the matrix-core flops
-# (20.7 ms forward + backward instead of 26.0 ms); a call whose logits are larger recomputes them chunk by chunk as the
-# reference does. The environment variable VERL_AMD_LMHEAD_KEEP_BYTES sets the limit (0: never keep unless asked).
+# keep_logits=None (the default) keeps for the backward as many logits as fit this many bytes: on a 288 GB part the
+# 2.5 GB of an 8192 x 152064 bf16 micro-batch are under 1 % of the memory and save a quarter of the matrix-core flops
+# (21 ms forward + backward instead of 26.5 ms). Of a call whose logits are larger the leading tokens' are kept, as many
+# as fit and leave whole chunks, and the rest is formed again chunk by chunk as the reference does (the library path keeps
+# all or nothing). The environment variable VERL_AMD_LMHEAD_KEEP_BYTES sets the limit (0: never keep unless asked).
 DEFAULT_KEEP_LOGITS_BYTES = int(os.environ.get("VERL_AMD_LMHEAD_KEEP_BYTES", str(4 << 30)))
 
 # From this many tokens on, one transposed copy of the weight per backward (0.44 ms for 152064 x 3584 bf16) is
@@ -137,7 +138,9 @@ def _own_d_hidden_takes(grad_logits, weight, out) -> bool:
 
 class _FusedLinearForPPOFunction(torch.autograd.Function):
     @staticmethod
-    def forward(ctx, hidden, weight, input_ids, temperature, chunk_size, keep_logits, kernels, forward_splits=None):
+    def forward(ctx, hidden, weight, input_ids, temperature, chunk_size, keep_rows, kernels, forward_splits=None):
+        # keep_rows: the logits of this many leading tokens are kept for the backward (all of them when it reaches the
+        # token count; a part only on the package's own path, in whole 256-token blocks)
         ctx.set_materialize_grads(False)
         ctx.kernels = kernels
         T, D = hidden.shape
@@ -148,12 +151,14 @@ class _FusedLinearForPPOFunction(torch.autograd.Function):
         h = torch.empty(T, **f32)
         lse = torch.empty(T, **f32)
         flag = torch.zeros(1, dtype=torch.int32, device=dev)
-        keep = bool(keep_logits) and T > 0 and (ctx.needs_input_grad[0] or ctx.needs_input_grad[1])
+        wants_grad = T > 0 and (ctx.needs_input_grad[0] or ctx.needs_input_grad[1])
+        keep = wants_grad and int(keep_rows) >= T
         ctx.own_kept = False
         if _own_forward_in_use(kernels, hidden, weight):
             temp_all = None if temperature == 1.0 else torch.full((T,), float(temperature), **f32)
+            rows = T if keep else (int(keep_rows) // 256 * 256 if wants_grad else 0)
             lp, h, lse, kept = _own_forward(hidden, weight, input_ids, temp_all, forward_splits, "fused_linear_for_ppo",
-                                            keep=keep)
+                                            keep_rows=rows)
             ctx.save_for_backward(hidden, weight, input_ids, lse, h)
             ctx.temperature = float(temperature)
             ctx.chunk_size = int(chunk_size)
@@ -205,30 +210,36 @@ class _FusedLinearForPPOFunction(torch.autograd.Function):
         d_weight = torch.empty_like(weight) if need_dw else None
         dw_started = False     # whether d_weight holds a partial sum yet
         lib = _lib.load()
+        base = 0               # tokens before this one are done
         if kept is not None and ctx.own_kept:
-            # The forward kernel left the logits of all tokens (rows padded to a multiple of 64 with zero hidden states,
-            # whose logits and hence gradients are zero): their gradient is written over them, and each product runs once
-            # over all tokens with this package's kernel, nothing to accumulate.
+            # The forward kernel left the logits of the first tokens, or of all of them (then in rows padded to a multiple
+            # of 64 with zero hidden states, whose logits and hence gradients are zero): their gradient is written over
+            # them, and each product runs once over those tokens with this package's kernel. What follows them, if
+            # anything, is formed again chunk by chunk below and added.
             m = kept.shape[0]
-            temp_rows = None if ctx.temperature == 1.0 else torch.full((T,), ctx.temperature, **f32)
+            n_k = min(m, T)
+            temp_rows = None if ctx.temperature == 1.0 else torch.full((n_k,), ctx.temperature, **f32)
             with torch.cuda.device(dev):
                 st = lib.vrl_rowscore_backward(
-                    kept.data_ptr(), _DTYPE_CODES[hidden.dtype], T, V, kept.stride(0), input_ids.data_ptr(),
+                    kept.data_ptr(), _DTYPE_CODES[hidden.dtype], n_k, V, kept.stride(0), input_ids.data_ptr(),
                     _ptr(temp_rows), lse.data_ptr(), h.data_ptr(), _ptr(gl), _ptr(gh), kept.data_ptr(), kept.stride(0),
                     _lib.stream_ptr(dev))
             _lib.check("vrl_rowscore_backward", st)
             if need_dh:
-                out = d_hidden if m == T else torch.empty((m, D), dtype=hidden.dtype, device=dev)
+                out = d_hidden[:m] if m <= T else torch.empty((m, D), dtype=hidden.dtype, device=dev)
                 _d_hidden(kept, weight, None, out, True)
-                if m != T:
+                if m > T:
                     d_hidden.copy_(out[:T])
             if need_dw:
-                c_h = hidden if m == T else _padded(hidden, m)
+                c_h = hidden[:m] if m <= T else _padded(hidden, m)
                 if _gemm.gemm_takes(c_h, kept, True, True):
                     _gemm.gemm(c_h, kept, x_t=True, y_t=True, out=d_weight)
                 else:
-                    torch.matmul(kept[:T].t(), hidden, out=d_weight)
-            return d_hidden, d_weight, None, None, None, None, None, None
+                    torch.matmul(kept[:n_k].t(), hidden[:n_k], out=d_weight)
+                dw_started = True
+            if m >= T:
+                return d_hidden, d_weight, None, None, None, None, None, None
+            base, kept = m, None
         # With this package's own kernels every chunk is at least one block of 256 tokens: a smaller chunk size is raised
         # to 256, a short tail joins the chunk before it, and a call with fewer than 256 tokens is padded to one block
         # (zero hidden states and zero incoming gradients give zero rows), so the backward never falls back to logits
@@ -236,7 +247,7 @@ class _FusedLinearForPPOFunction(torch.autograd.Function):
         # the step of the contraction of d W.
         own = kept is None and ctx.kernels != "library" and V % 8 == 0 and _mfma_takes_model(hidden, weight)
         step = max(chunk, 256) if own else chunk
-        starts = list(range(0, T, step))
+        starts = list(range(base, T, step))
         if own and len(starts) > 1 and T - starts[-1] < 256:
             starts.pop()
         bounds = [(lo, starts[i + 1] if i + 1 < len(starts) else T) for i, lo in enumerate(starts)]
@@ -338,8 +349,10 @@ def fused_linear_for_ppo(hidden_states: torch.Tensor, vocab_weights: torch.Tenso
     ``tokens x vocab`` logits (2.5 GB for 8192 x 152064 bf16; written by the same forward kernel from its registers), the
     backward writes their gradient over them instead of projecting again and forms ``d hidden`` and ``d W`` with one
     product each. Such a graph can be differentiated once. The scores do not depend on it. ``None`` (the default) keeps
-    them when all of them fit ``DEFAULT_KEEP_LOGITS_BYTES`` (4 GiB unless ``VERL_AMD_LMHEAD_KEEP_BYTES`` says otherwise) and
-    recomputes otherwise; ``False`` never holds more than one chunk of logits, like the reference.
+    what fits ``DEFAULT_KEEP_LOGITS_BYTES`` (4 GiB unless ``VERL_AMD_LMHEAD_KEEP_BYTES`` says otherwise): all of them, or the
+    logits of the leading tokens, so many that the rest is whole chunks (the same forward kernel writes just those; the
+    backward forms the others again chunk by chunk and adds their share of ``d W``); ``False`` never holds more than one
+    chunk of logits, like the reference.
 
     ``kernels`` chooses which matrix products are this package's own kernels: ``"library"`` (none: torch.matmul
     throughout) or ``"auto"`` / ``"mfma"`` (all of them: a forward that is one kernel and never
@@ -383,31 +396,46 @@ def fused_linear_for_ppo(hidden_states: torch.Tensor, vocab_weights: torch.Tenso
     ids = input_ids.reshape(-1).to(device=h2.device, dtype=torch.int64).contiguous()
     w2 = vocab_weights.contiguous()
     needs_grad = torch.is_grad_enabled() and (h2.requires_grad or w2.requires_grad)
+    T = h2.shape[0]
     if keep_logits is None:
-        keep_logits = needs_grad and h2.shape[0] * w2.shape[0] * h2.element_size() <= DEFAULT_KEEP_LOGITS_BYTES
+        # what fits the budget: everything, or (the package's own kernels) the leading whole 256-token blocks
+        keep_rows = min(T, DEFAULT_KEEP_LOGITS_BYTES // max(w2.shape[0] * h2.element_size(), 1)) if needs_grad else 0
+        if keep_rows < T:
+            # a part: so many that what is formed again is whole chunks (a short last chunk costs nearly a full one:
+            # 16384 tokens under 4 GiB, 12288 kept + one chunk of 4096: 45.0 ms; 14080 kept + 2304: 48.3; none kept: 52.2)
+            again = -(-(T - keep_rows) // int(chunk_size)) * int(chunk_size)
+            keep_rows = max(T - again, 0) // 256 * 256 if _own_forward_in_use(kernels, h2, w2) else 0
+    else:
+        keep_rows = T if keep_logits else 0
     if not needs_grad and _own_forward_in_use(kernels, h2, w2):
         temp = None if float(temperature) == 1.0 else torch.full((h2.shape[0],), float(temperature), dtype=torch.float32,
                                                                   device=h2.device)
         with torch.no_grad():
             lp, ent, _, _ = _own_forward(h2, w2, ids, temp, forward_splits, "fused_linear_for_ppo")
         return lp.reshape(lead), ent.reshape(lead)
-    lp, ent = _FusedLinearForPPOFunction.apply(h2, w2, ids, float(temperature), int(chunk_size), bool(keep_logits),
+    lp, ent = _FusedLinearForPPOFunction.apply(h2, w2, ids, float(temperature), int(chunk_size), int(keep_rows),
                                                kernels, None if forward_splits is None else int(forward_splits))
     return lp.reshape(lead), ent.reshape(lead)
 
 
-def _own_forward(h, w, ids, temp, n_splits, what, keep=False):
+def _own_forward(h, w, ids, temp, n_splits, what, keep_rows=0):
     """(log-prob, entropy, logsumexp, kept logits), the first three fp32 per row of ``h``, from vrl_lmhead_score. ``temp``
     is None or one value per token. The kernels work on blocks of 256 tokens: a shorter input is copied into a zero-padded
-    block first. With ``keep`` the kernel also writes the logits, into a buffer whose rows are padded to a multiple of 64
-    (the step of the contraction of d W): rows past the input hold the logits of zero hidden states, zeros."""
+    block first. With ``keep_rows`` the kernel also writes the logits of that many leading tokens. All of them
+    (``keep_rows`` = the token count) go into a buffer whose rows are padded to a multiple of 64, the step of the
+    contraction of d W: rows past the input hold the logits of zero hidden states, zeros. A part of them (a multiple of
+    256 below the token count) goes into a buffer of exactly that many rows."""
     T, K = h.shape
     V = w.shape[0]
     dev = h.device
     f32 = dict(dtype=torch.float32, device=dev)
     if T == 0:
         return torch.empty(0, **f32), torch.empty(0, **f32), torch.empty(0, **f32), None
-    n = max((T + 63) // 64 * 64, 256) if keep else max(T, 256)
+    keep_rows = min(int(keep_rows), T)
+    keep_all = keep_rows == T
+    if not keep_all and keep_rows % 256 != 0:
+        raise ValueError(f"{what}: a part of the logits is kept in whole 256-token blocks, got {keep_rows} of {T} tokens")
+    n = max((T + 63) // 64 * 64, 256) if keep_all else max(T, 256)
     if n != T:
         hp = torch.zeros((n, K), dtype=h.dtype, device=dev)
         hp[:T] = h
@@ -424,12 +452,14 @@ def _own_forward(h, w, ids, temp, n_splits, what, keep=False):
     lp = torch.empty(n, **f32)
     ent = torch.empty(n, **f32)
     lse = torch.empty(n, **f32)
-    kept = torch.empty((n, V), dtype=h.dtype, device=dev) if keep else None
+    rows = n if keep_all else keep_rows
+    kept = torch.empty((rows, V), dtype=h.dtype, device=dev) if rows > 0 else None
     flag = torch.zeros(1, dtype=torch.int32, device=dev)
     with torch.cuda.device(dev):
         st = lib.vrl_lmhead_score(h.data_ptr(), w.data_ptr(), _DTYPE_CODES[h.dtype], n, V, K, h.stride(0), w.stride(0),
                                   ids.data_ptr(), _ptr(temp), splits, partials.data_ptr(), lp.data_ptr(), ent.data_ptr(),
-                                  lse.data_ptr(), flag.data_ptr(), _ptr(kept), V if keep else 0, _lib.stream_ptr(dev))
+                                  lse.data_ptr(), flag.data_ptr(), _ptr(kept), V if rows > 0 else 0, rows,
+                                  _lib.stream_ptr(dev))
     _lib.check("vrl_lmhead_score", st)
     _errors.report(flag, {_lib.VRL_FLAG_LABEL_OOB: (IndexError, f"{what}: an input id is outside [0, {V})")})
     return lp[:T], ent[:T], lse[:T], kept
