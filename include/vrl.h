@@ -278,7 +278,10 @@ int vrl_transpose(const void* src, int elem_size, int64_t rows, int64_t cols, in
  * hidden (n_tokens, hidden_size) and weight (vocab, hidden_size) are bf16 or fp16 (dtype as for vrl_rowscore),
  * row-major with row pitches h_stride / w_stride in elements; products are accumulated in fp32 (the logits are
  * NOT rounded to the operand type on the way, unlike a GEMM that writes them out). Forward only.
- * `partials` is caller-owned scratch of n_tokens * n_splits * 4 floats; vrl_lmhead_plan gives n_splits.
+ * `partials` is caller-owned scratch of vrl_lmhead_partials(n_tokens, vocab) floats (12 per token and 768 vocabulary
+ * entries); vrl_lmhead_plan gives n_splits, which only decides how the work is dealt to workgroups: a token's softmax
+ * state is handed over at fixed places of the vocabulary and merged in a fixed order, so its results are the same bits
+ * for any n_splits and any number of tokens in the call.
  * Requirements checked on the host: n_tokens >= 256, vocab >= 256, hidden_size a multiple of 64, pitches multiples
  * of 8 elements and at most 2^28, n_tokens and vocab at most 2^30, 16-byte aligned operands, 1 <= n_splits <= 64. out_logprob (with labels
  * and err_flag), out_entropy, out_lse: any may be NULL, not all.
@@ -351,10 +354,11 @@ int vrl_gemm(const void* x, const void* y, int dtype, int64_t NX, int64_t NY, in
 int vrl_gemm_nt(const void* x, const void* y, int dtype, int64_t NX, int64_t NY, int64_t K, int64_t x_stride,
                 int64_t y_stride, void* out, int64_t out_stride, int accumulate, int k_parts, float* workspace,
                 void* stream);
-/* Vocabulary splits per 256-token block for this shape: enough to give every CU a workgroup, never fewer than 8 (so that
- * every call of 8192 tokens or more cuts the vocabulary alike and gives a token the same bits whatever the call's size),
- * at most 64 and at most one per 256-row vocabulary tile. */
+/* Vocabulary splits per 256-token block for this shape: the number (at most 64) for which the workgroups, one per CU
+ * at a time, finish soonest: rounds of workgroups times the vocabulary tiles of the longest share. Results do not
+ * depend on it. vrl_lmhead_partials: floats of scratch that vrl_lmhead_score needs for this shape. */
 int vrl_lmhead_plan(int64_t n_tokens, int64_t vocab);
+int64_t vrl_lmhead_partials(int64_t n_tokens, int64_t vocab);
 
 /*
  * vrl_rollout_corr — rollout correction on padded (B, T) log-probs in one launch:

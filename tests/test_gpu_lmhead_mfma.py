@@ -307,40 +307,57 @@ def test_default_forward_is_the_same_with_and_without_gradients_and_for_any_toke
     assert not d_h[100:].any()
 
 
-def test_token_results_do_not_depend_on_the_call_when_the_vocabulary_is_cut_alike(dev):
-    """A token's partial softmax states are summed in the order of the vocabulary ranges. Calls of 8192 tokens or more all
-    use 8 ranges: the same token gives the same bits in a call of 8192 and in one of 16640 tokens. Smaller calls are cut
-    finer (here 64 and 32 ranges): a few ulps apart, and bit-identical again once `forward_splits` pins the number."""
+def test_token_results_do_not_depend_on_the_call(dev):
+    """The forward kernel hands a token's softmax state over at fixed places of the vocabulary (every three tiles, per
+    wavefront quarter) and the finishing kernel merges the states in a fixed order: the same token gives the same bits
+    in calls of any size and for any number of splits (which only deals the work to workgroups), with and without
+    gradients. A trainer's old and new log-probs of unchanged weights are therefore bit-identical whatever its
+    micro-batch sizes."""
     g = torch.Generator(device=dev).manual_seed(15)
-    K, V = 64, 16384                                     # 64 vocabulary tiles
+    K, V = 64, 16384 + 264                               # 66 vocabulary tiles, the last one partial
     T = 16640
     h = torch.empty(T, K, device=dev).uniform_(-1.0, 1.0, generator=g).bfloat16()
     w = torch.empty(V, K, device=dev).uniform_(-1.0, 1.0, generator=g).bfloat16()
     ids = torch.randint(0, V, (T,), generator=g, device=dev)
     lib = _lib.load()
-    assert lib.vrl_lmhead_plan(T, V) == 8 and lib.vrl_lmhead_plan(8192, V) == 8 and lib.vrl_lmhead_plan(10 ** 6, V) == 8
-    assert lib.vrl_lmhead_plan(256, V) == 64 and lib.vrl_lmhead_plan(2048, V) == 32
+    plans = {n: lib.vrl_lmhead_plan(n, V) for n in (256, 2048, 8192, 8448, T)}
+    assert len(set(plans.values())) >= 3, plans          # the sizes below are dealt differently
     with torch.no_grad():
         lp_all, ent_all = fused_linear_for_ppo(h, w, ids, 0.9)
-        lp_a, ent_a = fused_linear_for_ppo(h[:8192], w, ids[:8192], 0.9)
-        assert torch.equal(lp_a, lp_all[:8192]) and torch.equal(ent_a, ent_all[:8192])
-        lp_b, ent_b = fused_linear_for_ppo(h[8192:], w, ids[8192:], 0.9)          # 8448 tokens
-        assert torch.equal(lp_b, lp_all[8192:]) and torch.equal(ent_b, ent_all[8192:])
-        # smaller calls, planned: 64 and 32 ranges
-        lp_s, ent_s = fused_linear_for_ppo(h[:256], w, ids[:256], 0.9)
-        lp_m, ent_m = fused_linear_for_ppo(h[:2048], w, ids[:2048], 0.9)
-        for got_lp, got_ent, n in ((lp_s, ent_s, 256), (lp_m, ent_m, 2048)):
-            assert (got_lp - lp_all[:n]).abs().max().item() <= 4e-6 and (got_ent - ent_all[:n]).abs().max().item() <= 4e-6
-        # pinned: the same bits whatever the size of the call
-        pin_all = fused_linear_for_ppo(h, w, ids, 0.9, forward_splits=16)
-        for lo, hi in ((0, 256), (300, 2348), (8000, 16640), (5, 6)):
-            lp_p, ent_p = fused_linear_for_ppo(h[lo:hi], w, ids[lo:hi], 0.9, forward_splits=16)
-            assert torch.equal(lp_p, pin_all[0][lo:hi]) and torch.equal(ent_p, pin_all[1][lo:hi]), (lo, hi)
+        for lo, hi in ((0, 8192), (8192, T), (0, 256), (0, 2048), (300, 2348), (8000, T), (5, 6), (1000, 1300)):
+            lp_p, ent_p = fused_linear_for_ppo(h[lo:hi], w, ids[lo:hi], 0.9)
+            assert torch.equal(lp_p, lp_all[lo:hi]) and torch.equal(ent_p, ent_all[lo:hi]), (lo, hi)
+        for splits in (1, 2, 7, 22, 64):
+            lp_p, ent_p = fused_linear_for_ppo(h[:2048], w, ids[:2048], 0.9, forward_splits=splits)
+            assert torch.equal(lp_p, lp_all[:2048]) and torch.equal(ent_p, ent_all[:2048]), splits
     hg = h[:300].clone().requires_grad_()
-    lp_g, _ = fused_linear_for_ppo(hg, w, ids[:300], 0.9, forward_splits=16)        # and with gradients
-    assert torch.equal(lp_g.detach(), pin_all[0][:300])
+    lp_g, _ = fused_linear_for_ppo(hg, w, ids[:300], 0.9)                            # and with gradients
+    assert torch.equal(lp_g.detach(), lp_all[:300])
+    lp_g, _ = fused_linear_for_ppo(hg, w, ids[:300], 0.9, keep_logits=True)
+    assert torch.equal(lp_g.detach(), lp_all[:300])
     with pytest.raises(ValueError):
         fused_linear_for_ppo(h[:256], w, ids[:256], 0.9, forward_splits=65)
+
+
+def test_the_plan_fills_whole_rounds_of_workgroups(dev):
+    """vrl_lmhead_plan: one workgroup per CU runs at a time, so the splits are chosen to make (rounds of workgroups) x
+    (tiles of the longest share) smallest; every split gets tiles, in whole runs of three."""
+    lib = _lib.load()
+    cus = torch.cuda.get_device_properties(dev).multi_processor_count
+    for T, V in ((8192, 152064), (10240, 152064), (12288, 152064), (256, 152064), (2304, 152064), (4096, 32000),
+                 (100000, 128256), (20000, 1000)):
+        s = lib.vrl_lmhead_plan(T, V)
+        tblocks, runs = -(-T // 256), -(-(-(-V // 256)) // 3)
+        assert 1 <= s <= min(64, runs)
+        share = -(-runs // s)
+        assert -(-runs // share) == s                         # no split without tiles
+
+        def cost(k):
+            return -(-tblocks * k // cus) * (-(-runs // k) * 3 + 2)
+
+        assert cost(s) == min(cost(k) for k in range(1, min(64, runs) + 1)), (T, V, s)
+    assert lib.vrl_lmhead_plan(8192, 152064) == 8 if cus == 256 else True
+    assert lib.vrl_lmhead_partials(8192, 152064) == 198 * 12 * 8192 and lib.vrl_lmhead_partials(0, 5) == 0
 
 
 def test_matrix_core_entry_points_replay_from_a_graph(dev):
@@ -357,7 +374,7 @@ def test_matrix_core_entry_points_replay_from_a_graph(dev):
     g_lp = torch.empty(T, device=dev)
     g_ent = torch.empty(T, device=dev)
     splits = lib.vrl_lmhead_plan(T, V)
-    partials = torch.empty(T * splits * 4, device=dev)
+    partials = torch.empty(int(lib.vrl_lmhead_partials(T, V)), device=dev)
     lp = torch.empty(T, device=dev); ent = torch.empty(T, device=dev); lse = torch.empty(T, device=dev)
     flag = torch.zeros(1, dtype=torch.int32, device=dev)
     G = torch.empty(T, V, dtype=torch.bfloat16, device=dev)
@@ -442,7 +459,7 @@ def test_special_values_and_errors(dev):
 def lib_plan_is_sane():
     lib = _lib.load()
     return (lib.vrl_lmhead_plan(8192, 152064) == 8 and lib.vrl_lmhead_plan(256, 256) == 1
-            and 1 <= lib.vrl_lmhead_plan(100000, 151936) <= 64 and lib.vrl_lmhead_plan(256, 151936) == 64)
+            and 1 <= lib.vrl_lmhead_plan(100000, 151936) <= 64 and lib.vrl_lmhead_plan(256, 151936) == 50)   # 198 runs in shares of 4
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
@@ -459,7 +476,7 @@ def test_forward_also_writes_the_logits_when_asked(dev, dtype, T, V, K):
     temp = torch.rand(T, generator=g, device=dev) + 0.5
     code = _lib.VRL_BF16 if dtype == torch.bfloat16 else _lib.VRL_F16
     splits = lib.vrl_lmhead_plan(T, V)
-    part = torch.empty(T * splits * 4, device=dev)
+    part = torch.empty(int(lib.vrl_lmhead_partials(T, V)), device=dev)
     pitch = V + 16
     outs = []
     for keep in (False, True):
@@ -602,7 +619,7 @@ def test_only_the_first_logits_rows_are_written(dev):
     w = torch.empty(V, K, device=dev).uniform_(-0.5, 0.5, generator=g).bfloat16()
     ids = torch.randint(0, V, (T,), generator=g, device=dev)
     splits = 2
-    part = torch.empty(T * splits * 4, device=dev)
+    part = torch.empty(int(lib.vrl_lmhead_partials(T, V)), device=dev)
     outs = []
     for n_rows in (T, rows, 1):
         lp, ent, lse = (torch.empty(T, device=dev) for _ in range(3))

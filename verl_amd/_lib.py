@@ -61,6 +61,7 @@ SIGNATURES = {
     "vrl_gemm_nt": (_INT, [_P, _P, _INT, _I64, _I64, _I64, _I64, _I64, _P, _I64, _INT, _INT, _P, _P]),
     "vrl_gemm": (_INT, [_P, _P, _INT, _I64, _I64, _I64, _I64, _I64, _INT, _INT, _P, _I64, _INT, _INT, _P, _P]),
     "vrl_lmhead_plan": (_INT, [_I64, _I64]),
+    "vrl_lmhead_partials": (_I64, [_I64, _I64]),
     "vrl_transpose": (_INT, [_P, _INT, _I64, _I64, _I64, _P, _I64, _P]),
     "vrl_rollout_corr": (
         _INT,

@@ -22,7 +22,7 @@
 // lm_gemm_kernel: out (+)= Y . X^T on the same walk, for the two products that follow (d hidden, d W).
 //
 // lmhead_finish_kernel: one wavefront per token forms the label's logit as a dot product in fp32, merges the
-// token's partials over the splits and writes log-prob, entropy and logsumexp (same finish as the row kernel).
+// token's partial states and writes log-prob, entropy and logsumexp (same finish as the row kernel).
 //
 // Roofline: dense bf16 MFMA. 2 * tokens * vocab * hidden flops; HBM traffic is the weight once per XCD group.
 #pragma once
@@ -50,6 +50,11 @@ constexpr int kLmTileBytes = 256 * kLmRowBytes;   // one operand tile in LDS (32
 constexpr int kLmRingSlots = 5;                   // operand tiles resident in LDS
 constexpr int kLmLdsBytes = kLmRingSlots * kLmTileBytes;   // 160 KiB: all of a CU's LDS
 constexpr int kLmMaxSplits = 64;
+// The forward kernel hands over a token's softmax state once per kLmSubTiles vocabulary tiles (and wavefront quarter)
+// instead of once per workgroup: what is summed in which order then depends on the vocabulary alone, not on how its
+// tiles are dealt to workgroups, so a token's results are the same bits whatever the number of tokens or splits of the
+// call. A workgroup's share of the vocabulary is a whole number of such runs.
+constexpr int kLmSubTiles = 3;
 
 template <int DT>
 struct LmFrag;
@@ -420,13 +425,28 @@ __device__ __forceinline__ void lm_walk_tiles(const uint16_t* __restrict__ W, co
 // logits_out[tok * l_stride + v] (l_stride and V multiples of 8, 16-byte aligned base): what a backward pass that may
 // spend memory instead of forming the logits again reads (vrl_rowscore_backward over them, in place). The softmax state
 // is folded from the fp32 values all the same, so the scores do not depend on whether the logits are kept.
+// The two values that meet when x is exchanged between rows of 16 lanes (round 0: row 0 with 1 and row 2 with 3; round 1:
+// the lower with the upper half of the wavefront): every lane of such a pair receives the same two values, out[0] from
+// the lower-numbered row(s) and out[1] from the higher.
+__device__ __forceinline__ void lm_swap_rows(float x, int round, float (&out)[2]) {
+  const unsigned u = __float_as_uint(x);
+  if (round == 0) {
+    const auto r = __builtin_amdgcn_permlane16_swap(u, u, false, false);
+    out[0] = __uint_as_float(r[0]);
+    out[1] = __uint_as_float(r[1]);
+  } else {
+    const auto r = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+    out[0] = __uint_as_float(r[0]);
+    out[1] = __uint_as_float(r[1]);
+  }
+}
+
 template <int DT, bool STORE>
 __global__ __launch_bounds__(kLmWaves * 64, 1) void lmhead_partial_kernel(
     const uint16_t* __restrict__ W, const uint16_t* __restrict__ H, int64_t V, int64_t T, int64_t K, int64_t w_stride,
     int64_t h_stride, const float* __restrict__ temperature, int n_splits, int tiles_per_split,
     int xcd_map, float* __restrict__ partials, uint16_t* __restrict__ logits_out, int64_t l_stride, int64_t l_rows) {
-  extern __shared__ __attribute__((aligned(1024))) char lds[];  // the operand ring; its start serves the final merge
-  float (*red)[256][3] = reinterpret_cast<float (*)[256][3]>(lds);   // [4][256][3], used once the walk is over
+  extern __shared__ __attribute__((aligned(1024))) char lds[];  // the operand ring
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -434,6 +454,7 @@ __global__ __launch_bounds__(kLmWaves * 64, 1) void lmhead_partial_kernel(
   const int wv = wave >> 1;
   const int wt = wave & 1;
   const LmWork work = lm_work(V, T, n_splits, tiles_per_split, xcd_map);
+  const int64_t n_vtiles = (V + kLmVocab - 1) / kLmVocab;
 
   // per-lane softmax state for the 8 token columns this lane sees (16 x 16 blocks: column = lane & 15)
   float m[8], s[8], t[8], c[8];
@@ -446,7 +467,9 @@ __global__ __launch_bounds__(kLmWaves * 64, 1) void lmhead_partial_kernel(
     c[j] = make_scale<false>(temperature, tok).c;   // log2(e) / max(T, 1e-8), exactly what the finishing kernel uses
   }
 
-  lm_walk_tiles<DT, STORE ? 2 : 0, false, false, 2, 0, 0>(W, H, V, K, w_stride, h_stride, work, lds, [&](int64_t vt, lm_f32x4 (&acc)[4][8]) {
+  // (load placement, see lm_walk_tiles: pairs two instructions before a column ends; single loads behind it when the
+  // logits are written too - 6.28 against 6.45 ms and 6.65 against 6.94 ms for the other's choice, one process)
+  lm_walk_tiles<DT, 2, false, false, STORE ? 1 : 2, STORE ? 0 : 2, 0>(W, H, V, K, w_stride, h_stride, work, lds, [&](int64_t vt, lm_f32x4 (&acc)[4][8]) {
     // fold 16 logits per token column into the running state (maximum first, then the exponentials; nothing is
     // buffered): acc[i][j][v] is vocabulary row tile_row0 + wv*64 + i*16 + 4*(lane>>4) + v of token column j
     const bool edge = (vt + 1) * kLmVocab > V;
@@ -511,65 +534,52 @@ __global__ __launch_bounds__(kLmWaves * 64, 1) void lmhead_partial_kernel(
       // one token column at a time: keeps the compiler from pulling the next columns' accumulator copies forward
       __builtin_amdgcn_sched_barrier(0);
     }
-  });
-
-  __syncthreads();   // every wavefront has left the ring: its memory now serves the merge
-  // combine: lanes l, l^16, l^32, l^48 hold the same tokens (other vocabulary rows), then the four vocabulary-quarter
-  // wavefronts of a token half through LDS
+    // End of a run of kLmSubTiles tiles (or of the vocabulary): hand the state over and start afresh. Lanes l, l^16,
+    // l^32, l^48 hold the same tokens (other vocabulary rows): they are combined here, the four vocabulary-quarter
+    // wavefronts and the runs by the finishing kernel. partials[(token * n_runs * 4 + run * 4 + quarter) * 3 + {m, s, t}]:
+    // a token's states lie together for the finishing kernel; here a lane stores 12 bytes per token column.
+    if ((vt + 1) % kLmSubTiles == 0 || vt + 1 == n_vtiles) {
+      const int64_t n_states = ((n_vtiles + kLmSubTiles - 1) / kLmSubTiles) * 4;
+      const int64_t tok_lane = work.tok0_ld + wt * 128 + (lane & 15);
+      float* dst = partials + (tok_lane * n_states + (vt / kLmSubTiles) * 4 + wv) * 3;
 #pragma unroll
-  for (int j = 0; j < 8; ++j) {
-    float M = m[j], S = s[j], Tt = t[j];
+      for (int j = 0; j < 8; ++j) {
+        float M = m[j], S = s[j], Tt = t[j];
+        // rows of 16 lanes pairwise (0 with 1, 2 with 3), then the two halves of the wavefront: the swaps are vector-ALU
+        // instructions (an exchange through the LDS crossbar would wait behind the ring's fragment reads), and every
+        // lane of a pair computes the same merge of the same two states
 #pragma unroll
-    for (int sh = 16; sh <= 32; sh <<= 1) {
-      const float om = __shfl_xor(M, sh);
-      const float os = __shfl_xor(S, sh);
-      const float ot = __shfl_xor(Tt, sh);
-      const float N = __builtin_fmaxf(M, om);
-      float S2 = 0.f, T2 = 0.f;
-      if (N != neg_inf()) {
-        const float a1 = hw_exp2(M - N), a2 = hw_exp2(om - N);
-        const float d1 = (M == neg_inf()) ? 0.f : M - N;
-        const float d2 = (om == neg_inf()) ? 0.f : om - N;
-        S2 = a1 * S + a2 * os;
-        T2 = a1 * (Tt + d1 * S) + a2 * (ot + d2 * os);
-      }
-      M = N;
-      S = S2;
-      Tt = T2;
-    }
-    if (lane < 16) {
-      const int col = wt * 128 + j * 16 + lane;
-      red[wv][col][0] = M;
-      red[wv][col][1] = S;
-      red[wv][col][2] = Tt;
-    }
-  }
-  __syncthreads();
-  if (tid < 256) {
-    const int col = tid;  // 256 token columns
-    const int64_t tok = work.tok0_ld + col;
-    if (tok >= work.tok0) {
-      float M = red[0][col][0];
-#pragma unroll
-      for (int q = 1; q < 4; ++q) M = __builtin_fmaxf(M, red[q][col][0]);
-      float S = 0.f, Tt = 0.f;
-      if (M != neg_inf()) {
-#pragma unroll
-        for (int q = 0; q < 4; ++q) {
-          const float mq = red[q][col][0];
-          const float aq = hw_exp2(mq - M);
-          const float dq = (mq == neg_inf()) ? 0.f : mq - M;
-          S += aq * red[q][col][1];
-          Tt += aq * (red[q][col][2] + dq * red[q][col][1]);
+        for (int round = 0; round < 2; ++round) {
+          float pm[2], ps[2], pt[2];
+          lm_swap_rows(M, round, pm);
+          lm_swap_rows(S, round, ps);
+          lm_swap_rows(Tt, round, pt);
+          const float N = __builtin_fmaxf(pm[0], pm[1]);
+          float S2 = 0.f, T2 = 0.f;
+          if (N != neg_inf()) {
+            const float a1 = hw_exp2(pm[0] - N), a2 = hw_exp2(pm[1] - N);
+            const float d1 = (pm[0] == neg_inf()) ? 0.f : pm[0] - N;
+            const float d2 = (pm[1] == neg_inf()) ? 0.f : pm[1] - N;
+            S2 = a1 * ps[0] + a2 * ps[1];
+            T2 = a1 * (pt[0] + d1 * ps[0]) + a2 * (pt[1] + d2 * ps[1]);
+          }
+          M = N;
+          S = S2;
+          Tt = T2;
         }
+        // (rows that an edge block shares with the block before are that block's to write)
+        if (lane < 16 && tok_lane + j * 16 >= work.tok0) {
+          float* d = dst + static_cast<int64_t>(j * 16) * n_states * 3;
+          d[0] = M;
+          d[1] = S;
+          d[2] = Tt;
+        }
+        m[j] = neg_inf();
+        s[j] = 0.f;
+        t[j] = 0.f;
       }
-      float* p = partials + (tok * n_splits + work.split) * 4;
-      p[0] = M;
-      p[1] = S;
-      p[2] = Tt;
-      p[3] = 0.f;
     }
-  }
+  });
 }
 
 // Backward: dlogits[tok, v] = (g_logprob[tok] * (1[v == label[tok]] - p) - g_entropy[tok] * p * (log p + entropy[tok])) / T[tok]
@@ -833,7 +843,7 @@ __global__ __launch_bounds__(256) void lm_gemm_reduce_kernel(const float* __rest
 template <int DT>
 __global__ __launch_bounds__(256) void lmhead_finish_kernel(
     const char* __restrict__ W, const char* __restrict__ H, int64_t V, int64_t T, int64_t K, int64_t w_stride,
-    int64_t h_stride, const int64_t* __restrict__ labels, const float* __restrict__ temperature, int n_splits,
+    int64_t h_stride, const int64_t* __restrict__ labels, const float* __restrict__ temperature, int n_runs,
     const float* __restrict__ partials, float* __restrict__ out_logprob, float* __restrict__ out_entropy,
     float* __restrict__ out_lse, int32_t* err_flag) {
   using E = Elem<DT>;
@@ -859,24 +869,31 @@ __global__ __launch_bounds__(256) void lmhead_finish_kernel(
       xl = wave_sum(acc);
     }
   }
-  Part p;
-  p.m = neg_inf();
-  p.s = 0.f;
-  p.t = 0.f;
-  p.q = 0.f;
-  if (lane < n_splits) {
-    const float* src = partials + (tok * n_splits + lane) * 4;
-    p.m = src[0];
-    p.s = src[1];
-    p.t = src[2];
-  }
-  const float M = wave_max(p.m);
-  rescale(p, M);
+  // The token's n_runs * 4 states (lmhead_partial_kernel: one per run of vocabulary tiles and wavefront quarter), in an
+  // order that the vocabulary alone fixes: lane l takes states l, l + 64, ...; all are brought to the common maximum,
+  // summed per lane in that order and then over the lanes.
+  const int64_t n_states = static_cast<int64_t>(n_runs) * 4;
+  const float* mine = partials + tok * n_states * 3;
+  float M = neg_inf();
+  for (int64_t i = lane; i < n_states; i += 64) M = __builtin_fmaxf(M, mine[i * 3]);
+  M = wave_max(M);
   Part w;
   w.m = M;
-  w.s = wave_sum(p.s);
-  w.t = wave_sum(p.t);
+  w.s = 0.f;
+  w.t = 0.f;
   w.q = 0.f;
+  for (int64_t i = lane; i < n_states; i += 64) {
+    Part p;
+    p.m = mine[i * 3];
+    p.s = mine[i * 3 + 1];
+    p.t = mine[i * 3 + 2];
+    p.q = 0.f;
+    rescale(p, M);
+    w.s += p.s;
+    w.t += p.t;
+  }
+  w.s = wave_sum(w.s);
+  w.t = wave_sum(w.t);
   if (lane == 0) {
     const Scale<false> sc = make_scale<false>(temperature, tok);
     finalize_row<false, false>(w, xl, label_ok, sc, tok, out_logprob, out_entropy, nullptr, out_lse, err_flag);

@@ -253,11 +253,14 @@ struct LmGrid {
   int xcd_map;
 };
 
-LmGrid lm_grid(int64_t T, int64_t V, int n_splits) {
+// `run` tiles at a time go to a split: kLmSubTiles for the forward kernel, which hands its softmax state over at the
+// ends of such runs, 1 for the gradient kernel, whose results are elementwise.
+LmGrid lm_grid(int64_t T, int64_t V, int n_splits, int run) {
   LmGrid g;
   g.tblocks = (T + vrl::kLmTokens - 1) / vrl::kLmTokens;
   const int64_t vtiles = (V + vrl::kLmVocab - 1) / vrl::kLmVocab;
-  g.tiles_per_split = static_cast<int>((vtiles + n_splits - 1) / n_splits);
+  const int64_t runs = (vtiles + run - 1) / run;
+  g.tiles_per_split = static_cast<int>((runs + n_splits - 1) / n_splits) * run;
   // 8 token blocks x 4 splits per XCD when the grid divides that way (see vrl::lm_work)
   g.xcd_map = (g.tblocks % 8 == 0 && n_splits % 4 == 0 && ((g.tblocks / 8) * (n_splits / 4)) % 8 == 0) ? 1 : 0;
   return g;
@@ -281,7 +284,7 @@ int launch_lmhead(const void* hidden, const void* weight, int64_t T, int64_t V, 
                   int64_t w_stride, const int64_t* labels, const float* temperature, int n_splits, float* partials,
                   float* out_logprob, float* out_entropy, float* out_lse, int32_t* err_flag, void* logits_out,
                   int64_t l_stride, int64_t l_rows, hipStream_t s) {
-  const LmGrid g = lm_grid(T, V, n_splits);
+  const LmGrid g = lm_grid(T, V, n_splits, vrl::kLmSubTiles);
   static std::atomic<bool> raised[kMaxDevices];
   const int rs = raise_lds_limit(reinterpret_cast<const void*>(vrl::lmhead_partial_kernel<DT, STORE>), raised);
   if (rs != VRL_OK) return rs;
@@ -292,7 +295,8 @@ int launch_lmhead(const void* hidden, const void* weight, int64_t T, int64_t V, 
       l_rows);
   vrl::lmhead_finish_kernel<DT><<<dim3(static_cast<unsigned>((T + 3) / 4)), dim3(256), 0, s>>>(
       static_cast<const char*>(weight), static_cast<const char*>(hidden), V, T, K, w_stride, h_stride, labels,
-      temperature, n_splits, partials, out_logprob, out_entropy, out_lse, err_flag);
+      temperature, static_cast<int>((((V + vrl::kLmVocab - 1) / vrl::kLmVocab) + vrl::kLmSubTiles - 1) / vrl::kLmSubTiles),
+      partials, out_logprob, out_entropy, out_lse, err_flag);
   return launch_status();
 }
 
@@ -301,7 +305,7 @@ int launch_lmhead_dlogits(const void* hidden, const void* weight, int64_t T, int
                           int64_t w_stride, const int64_t* labels, const float* temperature, const float* lse,
                           const float* entropy, const float* g_logprob, const float* g_entropy, int n_splits,
                           void* dlogits, int64_t d_stride, hipStream_t s) {
-  const LmGrid g = lm_grid(T, V, n_splits);
+  const LmGrid g = lm_grid(T, V, n_splits, 1);
   static std::atomic<bool> raised[kMaxDevices];
   const int rs = raise_lds_limit(reinterpret_cast<const void*>(vrl::lmhead_dlogits_kernel<DT>), raised);
   if (rs != VRL_OK) return rs;
@@ -813,16 +817,30 @@ int vrl_lmhead_plan(int64_t n_tokens, int64_t vocab) {
   if (n_tokens <= 0 || vocab <= 0) return 1;
   const int64_t tblocks = (n_tokens + vrl::kLmTokens - 1) / vrl::kLmTokens;
   const int64_t vtiles = (vocab + vrl::kLmVocab - 1) / vrl::kLmVocab;
-  int64_t s = (256 + tblocks - 1) / tblocks;  // one workgroup per CU
-  s = ((s + 3) / 4) * 4;                       // groups of 4 splits share an XCD with 8 token blocks
-  // Never fewer than 8: every call of 8192 tokens or more then cuts the vocabulary alike and sums a token's partial
-  // softmax states in the same order, so its results do not depend on how many tokens came with it (more workgroups
-  // than CUs cost nothing: they run in rounds).
-  if (s < 8) s = 8;
-  if (s > vrl::kLmMaxSplits) s = vrl::kLmMaxSplits;
-  if (s > vtiles) s = vtiles;
-  if (s < 1) s = 1;
-  return static_cast<int>(s);
+  const int64_t runs = (vtiles + vrl::kLmSubTiles - 1) / vrl::kLmSubTiles;
+  const int64_t cus = device_cus();
+  // One workgroup per CU runs at a time, so a launch takes (rounds of workgroups) x (tiles of the longest share, plus
+  // about two tiles to fill and drain the ring). The fewest splits among the cheapest: a token's results do not
+  // depend on the choice (see kLmSubTiles), only the time does.
+  int64_t best = 1, best_cost = -1;
+  for (int64_t s = 1; s <= vrl::kLmMaxSplits && s <= runs; ++s) {
+    const int64_t share = (runs + s - 1) / s;
+    if ((runs + share - 1) / share != s) continue;   // this many splits would leave one without a tile
+    const int64_t rounds = (tblocks * s + cus - 1) / cus;
+    const int64_t cost = rounds * (share * vrl::kLmSubTiles + 2);
+    if (best_cost < 0 || cost < best_cost) {
+      best = s;
+      best_cost = cost;
+    }
+  }
+  return static_cast<int>(best);
+}
+
+int64_t vrl_lmhead_partials(int64_t n_tokens, int64_t vocab) {
+  if (n_tokens <= 0 || vocab <= 0) return 0;
+  const int64_t vtiles = (vocab + vrl::kLmVocab - 1) / vrl::kLmVocab;
+  const int64_t runs = (vtiles + vrl::kLmSubTiles - 1) / vrl::kLmSubTiles;
+  return runs * 4 * 3 * n_tokens;   // per token: a (max, sum, weighted sum) state per run and wavefront quarter
 }
 
 int vrl_lmhead_score(const void* hidden, const void* weight, int dtype, int64_t n_tokens, int64_t vocab,

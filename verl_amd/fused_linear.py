@@ -46,8 +46,8 @@ DEFAULT_CHUNK_TOKENS = 4096
 #   "auto" (default) and "mfma" (the same today): every step runs this package's own matrix-core kernel.
 #              The forward is one kernel (vrl_lmhead_score: 6.0-6.25 ms at 8192 x 3584 -> 152064 bf16 against 6.5 ms for the
 #              library GEMM + row kernel, logits kept in fp32), with and without gradients and whatever the number of
-#              tokens, so that old (no-grad) and new (grad) log-probs of the same weights are bit-identical when both calls
-#              cut the vocabulary alike (see DEFAULT_FORWARD_SPLITS) and a few ulps apart otherwise. It never writes the
+#              tokens, and a token's results are the same bits whatever else the call holds, so that old (no-grad) and new
+#              (grad) log-probs of the same weights are bit-identical for any micro-batch sizes. It never writes the
 #              logits unless keep_logits=True asks for them (they then leave the kernel's registers rounded once).
 #              Without kept logits the backward forms them again and writes their gradient from registers
 #              (vrl_lmhead_dlogits, 3.2-3.3 ms per 4096 tokens against 3.5 ms for the library GEMM + row backward); with
@@ -61,11 +61,10 @@ DEFAULT_CHUNK_TOKENS = 4096
 # not a multiple of 64, fewer than 256 or not a multiple of 8 vocabulary entries) go to the library.
 DEFAULT_KERNELS = os.environ.get("VERL_AMD_LMHEAD_KERNELS", "auto")
 
-# Into how many ranges the single forward kernel cuts the vocabulary. None lets the library plan per call: 8 for every call
-# of 8192 tokens or more, more for fewer tokens so that the CUs stay busy. A token's partial softmax states are summed in
-# range order, so two calls give the same bits for a token exactly when they use the same number of ranges: always for
-# calls of >= 8192 tokens, and for any mix of sizes when this is pinned (1..64; `forward_splits` argument, or the
-# environment variable VERL_AMD_LMHEAD_SPLITS). Differently cut calls agree to a few fp32 ulps of the logsumexp.
+# Into how many shares per 256-token block the forward kernel's work is dealt. None lets the library plan per call (the
+# number that finishes soonest on this part's CUs). Results do not depend on it: the kernel hands a token's softmax state
+# over at fixed places of the vocabulary, and the states are merged in a fixed order. `forward_splits` / the environment
+# variable VERL_AMD_LMHEAD_SPLITS (1..64) are for measurements.
 _env_splits = os.environ.get("VERL_AMD_LMHEAD_SPLITS", "")
 DEFAULT_FORWARD_SPLITS = int(_env_splits) if _env_splits.strip() else None
 
@@ -83,8 +82,8 @@ def _mfma_takes_model(hidden: torch.Tensor, weight: torch.Tensor) -> bool:
 def _own_forward_in_use(kernels: str, hidden: torch.Tensor, weight: torch.Tensor) -> bool:
     """Whether the forward is vrl_lmhead_score. Decided by the ``kernels`` option and by the model only, never by the
     number of tokens, by ``keep_logits`` or by whether gradients are recorded: a trainer's old (no-grad) and new (grad)
-    log-probs of the same weights then come from the same kernel whatever the micro-batch sizes are (and from the same
-    summation order when the calls use the same number of vocabulary ranges, see DEFAULT_FORWARD_SPLITS)."""
+    log-probs of the same weights then come from the same kernel, and from the same summation order, whatever the
+    micro-batch sizes are."""
     return kernels != "library" and _mfma_takes_model(hidden, weight)
 
 
@@ -362,10 +361,10 @@ def fused_linear_for_ppo(hidden_states: torch.Tensor, vocab_weights: torch.Tenso
     computed with and without gradients are bit-identical. None takes ``DEFAULT_KERNELS`` ("auto" unless
     ``VERL_AMD_LMHEAD_KERNELS`` says otherwise).
 
-    ``forward_splits`` pins the number of vocabulary ranges of that forward (1..64; None: planned per call, 8 for every
-    call of 8192 tokens or more, ``DEFAULT_FORWARD_SPLITS`` / ``VERL_AMD_LMHEAD_SPLITS`` override). Calls with the same
-    number of ranges give a token the same bits whatever else is in the call; a trainer whose micro-batches can be
-    smaller than 8192 tokens and that wants old and new log-probs of unchanged weights to be bit-identical pins it.
+    ``forward_splits`` sets into how many shares per 256-token block that forward's work is dealt (1..64; None: planned
+    per call; ``DEFAULT_FORWARD_SPLITS`` / ``VERL_AMD_LMHEAD_SPLITS`` override). It changes the time only: a token gets the
+    same bits for any value and in calls of any size, so a trainer's old and new log-probs of unchanged weights are
+    bit-identical whatever its micro-batches.
     """
     kernels = DEFAULT_KERNELS if kernels is None else kernels
     if kernels not in ("auto", "library", "mfma"):
@@ -448,7 +447,7 @@ def _own_forward(h, w, ids, temp, n_splits, what, keep_rows=0):
         h, ids, temp = hp, ip, tp
     lib = _lib.load()
     splits = lib.vrl_lmhead_plan(n, V) if n_splits is None else min(int(n_splits), (V + 255) // 256)
-    partials = torch.empty(n * splits * 4, **f32)
+    partials = torch.empty(int(lib.vrl_lmhead_partials(n, V)), **f32)
     lp = torch.empty(n, **f32)
     ent = torch.empty(n, **f32)
     lse = torch.empty(n, **f32)
