@@ -603,13 +603,13 @@ def bench_lm_head(args, dev):
         ]
         G.copy_((torch.randn(n_c, V, generator=g, device=dev) * 0.01).bfloat16())
         kernels += [
-            rec("lm_gemm_kernel<bf16, 0, true, false>", f"d hidden = G . W, {n_c} tokens",
+            rec("lm_gemm_kernel<bf16, W contraction-major> (+ lm_gemm_reduce_kernel when the contraction is cut)", f"d hidden = G . W, {n_c} tokens",
                 per_launch(lambda: own_gemm.gemm(Wd, G, x_t=True, out=d_h)), flops_c,
                 per_launch(lambda: torch.matmul(G, wt.t(), out=d_h))),
-            rec("lm_gemm_kernel<bf16, 0, true, true>", f"d W = G^T . H stored, {n_c} tokens",
+            rec("lm_gemm_kernel<bf16, stored, both contraction-major>", f"d W = G^T . H stored, {n_c} tokens",
                 per_launch(lambda: own_gemm.gemm(Hc, G, x_t=True, y_t=True, out=d_w)), flops_c,
                 per_launch(lambda: torch.matmul(G.t(), Ht.t(), out=d_w))),
-            rec("lm_gemm_kernel<bf16, 1, true, true>", f"d W += G^T . H accumulated, {n_c} tokens",
+            rec("lm_gemm_kernel<bf16, accumulated, both contraction-major>", f"d W += G^T . H accumulated, {n_c} tokens",
                 per_launch(lambda: own_gemm.gemm(Hc, G, x_t=True, y_t=True, out=d_w, accumulate=True)), flops_c,
                 per_launch(lambda: d_w.addmm_(G.t(), Ht.t()))),
         ]
@@ -619,10 +619,10 @@ def bench_lm_head(args, dev):
             H8t = transpose_2d(Hd)
             d_h8 = torch.empty(T, D, dtype=torch.bfloat16, device=dev)
             kernels += [
-                rec("lm_gemm_kernel<bf16, 0, true, false>", f"d hidden = G . W, {T} tokens (kept logits)",
+                rec("lm_gemm_kernel<bf16, W contraction-major> (+ lm_gemm_reduce_kernel when the contraction is cut)", f"d hidden = G . W, {T} tokens (kept logits)",
                     per_launch(lambda: own_gemm.gemm(Wd, G8, x_t=True, out=d_h8), 5), flops_all,
                     per_launch(lambda: torch.matmul(G8, wt.t(), out=d_h8), 5)),
-                rec("lm_gemm_kernel<bf16, 0, true, true>", f"d W = G^T . H stored, {T} tokens (kept logits)",
+                rec("lm_gemm_kernel<bf16, stored, both contraction-major>", f"d W = G^T . H stored, {T} tokens (kept logits)",
                     per_launch(lambda: own_gemm.gemm(Hd, G8, x_t=True, y_t=True, out=d_w), 5), flops_all,
                     per_launch(lambda: torch.matmul(G8.t(), H8t.t(), out=d_w), 5)),
             ]

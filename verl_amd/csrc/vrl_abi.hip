@@ -399,15 +399,23 @@ GemmPlan gemm_plan(int64_t NX, int64_t NY, int64_t K, int forced_parts) {
   int best = 1;
   if (forced_parts > 0) {
     best = forced_parts;
-  } else if (base * 10 < 7LL * cus) {
-    // Too few output tiles for the CUs: cut the contraction until ~85 % of them have a workgroup. More than that does
-    // not pay: the part is power-bound on this loop, idle CUs raise the clock of the busy ones, and every cut costs a
-    // pass over fp32 partial sums (measured at 4096 x 152064 -> 3584: 224 workgroups 3.75 ms, 1792 in 8 ranges 3.82).
-    const int64_t want = (85LL * cus + 99) / 100;
-    int64_t parts = (want + base - 1) / base;
-    if (parts > 16) parts = 16;
-    while (parts > 1 && g.k_steps / parts < 32) --parts;
-    best = static_cast<int>(parts);
+  } else {
+    // One workgroup per CU runs at a time, so a product takes (rounds of workgroups) x (contraction steps of a range, plus
+    // a few to fill and drain the ring); cutting the contraction into ranges fills a last, nearly empty round at the
+    // price of a pass over fp32 partial sums (a fixed cost and 8 bytes per output element and range, in units of a
+    // 1.45 us step). Fitted to d hidden at 3584 <- 152064, one process: 8192 tokens 6.33 ms in 4 ranges against 6.63 in
+    // one, 14080 tokens 11.6 in 6 against 13.4, 16384 tokens 12.9 in 2 against 14.6; 4096 tokens level (3.26 - 3.29).
+    double best_cost = 0.0;
+    for (int parts : {1, 2, 3, 4, 6, 8}) {
+      if (parts > 1 && g.k_steps / parts < 32) break;
+      const double rounds = static_cast<double>((base * parts + cus - 1) / cus);
+      double cost = rounds * static_cast<double>((g.k_steps + parts - 1) / parts + 4);
+      if (parts > 1) cost += 60.0 + 1.2e-6 * static_cast<double>(parts) * static_cast<double>(NX) * static_cast<double>(NY);
+      if (parts == 1 || cost < best_cost) {
+        best_cost = cost;
+        best = parts;
+      }
+    }
   }
   g.steps_per_part = static_cast<int>((g.k_steps + best - 1) / best);
   g.k_parts = static_cast<int>((g.k_steps + g.steps_per_part - 1) / g.steps_per_part);   // no empty range
