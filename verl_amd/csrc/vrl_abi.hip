@@ -411,7 +411,7 @@ GemmPlan gemm_plan(int64_t NX, int64_t NY, int64_t K, int forced_parts) {
       const double rounds = static_cast<double>((base * parts + cus - 1) / cus);
       double cost = rounds * static_cast<double>((g.k_steps + parts - 1) / parts + 4);
       if (parts > 1) cost += 60.0 + 1.2e-6 * static_cast<double>(parts) * static_cast<double>(NX) * static_cast<double>(NY);
-      if (parts == 1 || cost < best_cost) {
+      if (parts == 1 || cost < 0.95 * best_cost) {   // more ranges only for a gain that is worth their scratch
         best_cost = cost;
         best = parts;
       }
