@@ -740,7 +740,8 @@ def bench_ceilings(args, dev):
         src = torch.empty(rows * row_bytes // 2, dtype=torch.int16, device=dev).fill_(5)
         small = rows * row_bytes < (1 << 30)
         modes = ((3, "non-temporal read, 32-bit row shape", 1),) if small else (
-            (0, "non-temporal read", 1), (1, "non-temporal copy", 2),
+            (0, "non-temporal read", 1), (4, "non-temporal read, 1024 workgroups walking the whole buffer", 1),
+            (1, "non-temporal copy", 2),
             (2, "non-temporal copy, 512 workgroups walking the whole buffer", 2))
         for mode, what, factor in modes:
             if mode in (1, 2) and rows * row_bytes > (8 << 30):

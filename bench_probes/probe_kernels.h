@@ -77,6 +77,31 @@ __global__ __launch_bounds__(256) void stream_probe_flat_copy_kernel(const u32x4
   }
 }
 
+// The read-only counterpart: the same walk, the data XOR-folded instead of stored (*sink is written only if the fold
+// equals a constant, which it does not). Whether rows matter to a read stream at all.
+__global__ __launch_bounds__(256) void stream_probe_flat_read_kernel(const u32x4* __restrict__ src, int64_t nvec,
+                                                                     uint32_t magic, uint32_t* sink) {
+  constexpr int U = 8;
+  const int64_t stride = static_cast<int64_t>(gridDim.x) * 256 * U;
+  int64_t base = (static_cast<int64_t>(blockIdx.x) * 256 + (threadIdx.x >> 6) * 64) * U + (threadIdx.x & 63);
+  uint32_t fold = 0;
+  for (; base + (U - 1) * 64 < nvec; base += stride) {
+    u32x4 v[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) v[u] = __builtin_nontemporal_load(src + base + u * 64);
+#pragma unroll
+    for (int u = 0; u < U; ++u) fold ^= v[u].x ^ v[u].y ^ v[u].z ^ v[u].w;
+  }
+  for (int u = 0; u < U; ++u) {
+    const int64_t k = base + u * 64;
+    if (k < nvec) {
+      const u32x4 v = __builtin_nontemporal_load(src + k);
+      fold ^= v.x ^ v.y ^ v.z ^ v.w;
+    }
+  }
+  if (fold == magic) *sink = fold;
+}
+
 // Matrix-core probe: what the part sustains on bf16 matrix instructions with nothing else in the way. 512 threads per
 // workgroup (two wavefronts per SIMD, like the LM-head kernels), every wavefront issues `iters` rounds of the products
 // of a 64 x 128 wavefront tile over 16 contraction elements on register operands. `random_operands` fills the

@@ -22,6 +22,7 @@ extern "C" {
  *   mode 2: the same copy by 512 workgroups walking the buffer as a whole, 8 KiB per wavefront and trip (the fastest
  *           read+write stream found on MI355X; what no row-shaped read+write kernel can exceed)
  *   mode 3: mode 0 with the workgroup shape the forward kernel uses for 32-bit logits (4 wavefronts, 4 loads in flight)
+ *   mode 4: mode 0 by 1024 workgroups walking the buffer as a whole (whether one workgroup per row costs a read stream anything)
  */
 int vrl_stream_probe(const void* src, void* dst, int64_t n_rows, int64_t row_bytes, int mode, uint32_t* sink,
                      void* stream);

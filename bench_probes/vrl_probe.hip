@@ -23,10 +23,10 @@ extern "C" {
 
 int vrl_stream_probe(const void* src, void* dst, int64_t n_rows, int64_t row_bytes, int mode, uint32_t* sink,
                      void* stream) {
-  if (mode < 0 || mode > 3) return VRL_ERR_ARG;
+  if (mode < 0 || mode > 4) return VRL_ERR_ARG;
   if (n_rows < 0 || row_bytes < 0 || row_bytes % 16 != 0 || n_rows > kMaxGrid) return VRL_ERR_SHAPE;
   if (n_rows == 0 || row_bytes == 0) return VRL_OK;
-  const bool reads_only = mode == 0 || mode == 3;
+  const bool reads_only = mode == 0 || mode == 3 || mode == 4;
   if (src == nullptr || (!reads_only && dst == nullptr) || (reads_only && sink == nullptr)) return VRL_ERR_NULL;
   if (!aligned(src, 16) || !aligned(dst, 16) || !aligned(sink, 4)) return VRL_ERR_ALIGN;
   const dim3 grid(static_cast<unsigned>(n_rows));
@@ -44,6 +44,9 @@ int vrl_stream_probe(const void* src, void* dst, int64_t n_rows, int64_t row_byt
   else if (mode == 1)
     vrl::stream_probe_kernel<kBackwardWaves, kBackwardUnroll, true><<<grid, dim3(kBackwardWaves * 64), 0, s>>>(
         static_cast<const vrl::u32x4*>(src), static_cast<vrl::u32x4*>(dst), vecs, 0u, nullptr);
+  else if (mode == 4)
+    vrl::stream_probe_flat_read_kernel<<<dim3(1024), dim3(256), 0, s>>>(static_cast<const vrl::u32x4*>(src),
+                                                                        n_rows * vecs, 0x9e3779b9u, sink);
   else
     vrl::stream_probe_flat_copy_kernel<<<dim3(512), dim3(256), 0, s>>>(
         static_cast<const vrl::u32x4*>(src), static_cast<vrl::u32x4*>(dst), n_rows * vecs);
