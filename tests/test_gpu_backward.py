@@ -176,3 +176,54 @@ def test_fp32_peaked_rows_at_low_temperature_stay_as_close_to_fp64_as_torch(dev)
     e_torch = (g32.double() - g64).abs().max().item()
     e_ours = (ours.double() - g64).abs().max().item()
     assert e_ours <= 2.0 * e_torch + 2e-6, (e_ours, e_torch)
+
+
+@pytest.mark.parametrize("dtype,n,V", [(torch.bfloat16, 1100, 32760), (torch.float32, 1100, 16388),
+                                       (torch.float16, 600, 65544)])
+def test_rows_back_to_back_take_the_walk_without_rows_with_the_same_bits(dev, dtype, n, V):
+    """Contiguous rows of 64 MiB or more are differentiated by workgroups that walk them as one array
+    (rowscore_backward_flat_kernel), every other input by one workgroup per row: same arithmetic per element, so the same
+    bits. Rows here are no multiple of a wavefront's 512-vector trip, so trips straddle rows; labels sit on the first and
+    last element of rows and on both sides of vector borders; also in place."""
+    from verl_amd import _lib
+
+    lib = _lib.load()
+    code = {torch.float32: _lib.VRL_F32, torch.bfloat16: _lib.VRL_BF16, torch.float16: _lib.VRL_F16}[dtype]
+    g = torch.Generator(device=dev).manual_seed(n + V)
+    x = (torch.randn(n, V, generator=g, device=dev) * 3).to(dtype)
+    assert x.numel() * x.element_size() >= (1 << 26)
+    lab = torch.randint(0, V, (n,), generator=g, device=dev)
+    per_vec = 16 // x.element_size()
+    lab[:8] = torch.tensor([0, V - 1, per_vec - 1, per_vec, V - per_vec, V - per_vec - 1, 1, V // 2], device=dev)
+    temp = torch.rand(n, generator=g, device=dev) + 0.5
+    lse = torch.logsumexp(x.float() / temp[:, None], -1)
+    ent = torch.rand(n, generator=g, device=dev) * 4
+    gl = torch.randn(n, generator=g, device=dev)
+    gh = torch.randn(n, generator=g, device=dev)
+    wide = torch.zeros(n, V + 2 * per_vec, dtype=dtype, device=dev)        # the same rows with a pitch: one workgroup per row
+    wide[:, :V] = x
+    out_flat = torch.empty_like(x)
+    out_rows = torch.zeros_like(wide)
+    stream = _lib.stream_ptr(dev)
+    with torch.cuda.device(dev):
+        for src, dst in ((x, out_flat), (wide, out_rows)):
+            st = lib.vrl_rowscore_backward(src.data_ptr(), code, n, V, src.stride(0), lab.data_ptr(), temp.data_ptr(),
+                                           lse.data_ptr(), ent.data_ptr(), gl.data_ptr(), gh.data_ptr(), dst.data_ptr(),
+                                           dst.stride(0), stream)
+            assert st == _lib.VRL_OK
+        bits = torch.int16 if x.element_size() == 2 else torch.int32
+        assert torch.equal(out_flat.view(bits), out_rows[:, :V].contiguous().view(bits))
+        assert not bool(out_rows[:, V:].any())
+        # the label term landed where it belongs: the gradient of the log-prob alone sums to g / T * (1 - 1) = 0 per row
+        st = lib.vrl_rowscore_backward(x.data_ptr(), code, n, V, V, lab.data_ptr(), temp.data_ptr(), lse.data_ptr(), None,
+                                       gl.data_ptr(), None, out_flat.data_ptr(), V, stream)
+        assert st == _lib.VRL_OK
+        sums = out_flat.double().sum(-1)
+        tol = 2e-2 if dtype != torch.float32 else 1e-4
+        assert bool((sums.abs() <= tol * (gl.abs().double() / temp.double() + 1)).all()), sums.abs().max().item()
+        # in place
+        y = x.clone()
+        st = lib.vrl_rowscore_backward(y.data_ptr(), code, n, V, V, lab.data_ptr(), temp.data_ptr(), lse.data_ptr(),
+                                       ent.data_ptr(), gl.data_ptr(), gh.data_ptr(), y.data_ptr(), V, stream)
+        assert st == _lib.VRL_OK
+        assert torch.equal(y.view(bits), out_rows[:, :V].contiguous().view(bits))
