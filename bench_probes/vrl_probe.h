@@ -19,8 +19,8 @@ extern "C" {
  * vrl_rowscore's kernel does.
  *   mode 0: read only (the data is XOR-folded; *sink is written only if the fold equals a constant)  -> forward ceiling
  *   mode 1: read src, write dst (n_rows * row_bytes each, not overlapping)                           -> backward ceiling
- *   mode 2: the same copy by 512 workgroups walking the buffer as a whole, 8 KiB per wavefront and trip (the fastest
- *           read+write stream found on MI355X; what no row-shaped read+write kernel can exceed)
+ *   mode 2: the same copy by 512 workgroups walking the buffer as a whole, 8 KiB per wavefront and trip (faster than
+ *           mode 1 on MI355X; no bound either: the row-op backward in many short workgroups is faster again)
  *   mode 3: mode 0 with the workgroup shape the forward kernel uses for 32-bit logits (4 wavefronts, 4 loads in flight)
  *   mode 4: mode 0 by 1024 workgroups walking the buffer as a whole (whether one workgroup per row costs a read stream anything)
  */
