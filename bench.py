@@ -288,7 +288,7 @@ def bench_backward(args, dev, workload=None):
                    "step": "vrl_rowscore_backward through the C ABI (gradients of log-prob and entropy)"},
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                      "frac": achieved / HBM_PEAK_GBPS, "traffic": MEASURED_BACKWARD_TRAFFIC_BYTES.get(workload),
-                     "kernel": "rowscore_backward_kernel", "avg_kernel_ms": avg_ms,
+                     "kernel": "rowscore_backward_flat_kernel", "avg_kernel_ms": avg_ms,
                      "algorithmic_bytes_per_launch": bytes_launch},
     }
 
