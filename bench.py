@@ -223,8 +223,8 @@ class Step:
         return rec
 
 
-# HBM bytes per launch of rowscore_backward_kernel from rocprofv3 --pmc (FETCH_SIZE, WRITE_SIZE; same scaling as above).
-MEASURED_BACKWARD_TRAFFIC_BYTES = {"c3": 4981794581}   # profiles/rowscore_backward_kernel_hbm_counters_c3.md
+# HBM bytes per launch of rowscore_backward_flat_kernel from rocprofv3 --pmc (FETCH_SIZE, WRITE_SIZE; same scaling as above).
+MEASURED_BACKWARD_TRAFFIC_BYTES = {"c3": 4981856312}   # profiles/rowscore_backward_kernels_hbm_counters_c3.md
 # profiles/score_responses_kernel_hbm_counters_c3_packed.md (forward, backward), for the packed micro-batch bench_score_responses builds
 MEASURED_SCORE_RESPONSES_TRAFFIC_BYTES = (1676672404, 4168192835)
 
