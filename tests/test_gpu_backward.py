@@ -179,7 +179,9 @@ def test_fp32_peaked_rows_at_low_temperature_stay_as_close_to_fp64_as_torch(dev)
 
 
 @pytest.mark.parametrize("dtype,n,V", [(torch.bfloat16, 1100, 32760), (torch.float32, 1100, 16388),
-                                       (torch.float16, 600, 65544)])
+                                       (torch.float16, 600, 65544),
+                                       # rows of 513 vectors, one more than a wavefront's trip: nearly every trip holds two rows
+                                       (torch.bfloat16, 8300, 4104), (torch.float32, 8300, 2052)])
 def test_rows_back_to_back_take_the_walk_without_rows_with_the_same_bits(dev, dtype, n, V):
     """Contiguous rows of 64 MiB or more are differentiated by workgroups that walk them as one array
     (rowscore_backward_flat_kernel), every other input by one workgroup per row: same arithmetic per element, so the same
