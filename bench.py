@@ -226,7 +226,7 @@ class Step:
 # HBM bytes per launch of rowscore_backward_flat_kernel from rocprofv3 --pmc (FETCH_SIZE, WRITE_SIZE; same scaling as above).
 MEASURED_BACKWARD_TRAFFIC_BYTES = {"c3": 4981856312}   # profiles/rowscore_backward_kernels_hbm_counters_c3.md
 # profiles/score_responses_kernel_hbm_counters_c3_packed.md (forward, backward), for the packed micro-batch bench_score_responses builds
-MEASURED_SCORE_RESPONSES_TRAFFIC_BYTES = (1676672404, 4168192835)
+MEASURED_SCORE_RESPONSES_TRAFFIC_BYTES = (1676672404, 4167119102)
 
 
 def bench_backward(args, dev, workload=None):
@@ -1003,7 +1003,7 @@ def bench_score_responses(args, dev, steps, warmup):
     bwd_bytes = n_resp * (w.V * 2 + 8 + 16) + n * w.V * 2 + (B + 1) * 8 + B * 8
     # the counters were read at this very micro-batch (5515 response rows of 8192); another one has no measured traffic
     measured = MEASURED_SCORE_RESPONSES_TRAFFIC_BYTES if (n, n_resp, B) == (8192, 5515, 4) else (None, None)
-    backward = {"avg_kernel_ms": bwd_ms, "kernel": "score_responses_backward_kernel",
+    backward = {"avg_kernel_ms": bwd_ms, "kernel": "score_responses_backward_flat_kernel",
                 "algorithmic_bytes_per_launch": bwd_bytes, "achieved_gbps": bwd_bytes / (bwd_ms * 1e-3) / 1e9,
                 "traffic": measured[1],
                 "all_rows_backward_bytes": n * (w.V * 4 + 8 + 16),

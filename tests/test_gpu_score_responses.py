@@ -339,3 +339,72 @@ def test_c3_micro_batch_full_size(dev):
                                        torch.full((rows.numel(),), 0.9))
     assert (lp[rows.to(dev)].cpu() - ref_lp).abs().max().item() <= 2e-3
     assert (h[rows.to(dev)].cpu() - ref_h).abs().max().item() <= 2e-3
+
+
+@pytest.mark.parametrize("dtype,V", [(torch.bfloat16, 32760), (torch.float32, 16388)])
+def test_gradient_of_back_to_back_rows_takes_the_walk_without_rows_with_the_same_bits(dev, dtype, V):
+    """64 MiB or more of contiguous logits from at most 64 sequences: the gradient is written by workgroups that walk
+    the rows as one array (score_responses_backward_flat_kernel) instead of one workgroup per row. Same bits as the
+    per-row kernel (run here on the same rows with a pitch), zeros for every row outside a response window, and with
+    inconsistent offsets nothing outside the gradient's own array is touched."""
+    from _guards import Arena
+
+    lib = _lib.load()
+    code = _lib.VRL_BF16 if dtype == torch.bfloat16 else _lib.VRL_F32
+    per_vec = 16 // torch.empty((), dtype=dtype).element_size()
+    lens = torch.tensor([300, 1, 250, 2, 348, 199])          # a one-token sequence and one with a one-token response among them
+    resp = torch.tensor([120, 0, 249, 1, 100, 0])
+    B, T = len(lens), 260
+    cu = torch.zeros(B + 1, dtype=torch.int64)
+    cu[1:] = torch.cumsum(lens, 0)
+    N = int(cu[-1])
+    g = torch.Generator(device=dev).manual_seed(V)
+    x = (torch.randn(N, V, generator=g, device=dev) * 2.5).to(dtype)
+    assert x.numel() * x.element_size() >= (1 << 26)
+    ids = torch.randint(0, V, (N,), generator=g, device=dev)
+    temp = torch.rand(N, generator=g, device=dev) + 0.5
+    r_lp, r_h, r_lse = (torch.empty(B, T, device=dev) for _ in range(3))
+    g_lp = torch.randn(B, T, generator=g, device=dev)
+    g_h = torch.randn(B, T, generator=g, device=dev)
+    flag = torch.zeros(1, dtype=torch.int32, device=dev)
+    cu_d, rl_d = cu.to(dev), resp.to(dev)
+    wide = torch.zeros(N, V + 2 * per_vec, dtype=dtype, device=dev)
+    wide[:, :V] = x
+    out_flat = torch.full_like(x, float("nan"))
+    out_rows = torch.full_like(wide, float("nan"))
+    stream = _lib.stream_ptr(dev)
+    with torch.cuda.device(dev):
+        st = lib.vrl_score_responses(x.data_ptr(), code, N, V, V, None, ids.data_ptr(), temp.data_ptr(), cu_d.data_ptr(),
+                                     rl_d.data_ptr(), B, T, None, None, r_lp.data_ptr(), r_h.data_ptr(), r_lse.data_ptr(),
+                                     flag.data_ptr(), stream)
+        assert st == _lib.VRL_OK
+        for src, dst in ((x, out_flat), (wide, out_rows)):
+            st = lib.vrl_score_responses_backward(src.data_ptr(), code, N, V, src.stride(0), None, ids.data_ptr(),
+                                                  temp.data_ptr(), cu_d.data_ptr(), rl_d.data_ptr(), B, T, r_lse.data_ptr(),
+                                                  r_h.data_ptr(), g_lp.data_ptr(), g_h.data_ptr(), dst.data_ptr(),
+                                                  dst.stride(0), stream)
+            assert st == _lib.VRL_OK
+    torch.cuda.synchronize(dev)
+    assert int(flag.item()) == 0
+    bits = torch.int16 if dtype == torch.bfloat16 else torch.int32
+    assert torch.equal(out_flat.view(bits), out_rows[:, :V].contiguous().view(bits))
+    in_window = torch.zeros(N, dtype=torch.bool)
+    for b in range(B):
+        end, r = int(cu[b + 1]), int(resp[b])
+        in_window[end - r - 1:end - 1] = True
+    assert not bool(out_flat[~in_window.to(dev)].any()) and bool(out_flat[in_window.to(dev)].any(-1).all())
+    # inconsistent offsets: the gradient array between guard regions
+    for offsets in ([0, 300, 301, 551, 553, 5000, N], [5, 301, 551, 553, 900, 1000, N], [0, 800, 400, 551, 553, 900, N],
+                    [-50, 301, 551, 553, 900, 1000, N], [0, 301, 2 ** 40, 551, 900, 1000, N]):
+        ar = Arena(dev)
+        grad = ar.make(N * V, dtype)
+        bad = torch.tensor(offsets, dtype=torch.int64, device=dev)
+        with torch.cuda.device(dev):
+            st = lib.vrl_score_responses_backward(x.data_ptr(), code, N, V, V, None, ids.data_ptr(), temp.data_ptr(),
+                                                  bad.data_ptr(), rl_d.data_ptr(), B, T, r_lse.data_ptr(), r_h.data_ptr(),
+                                                  g_lp.data_ptr(), g_h.data_ptr(), grad.data_ptr(), V, stream)
+        assert st == _lib.VRL_OK
+        torch.cuda.synchronize(dev)
+        assert ar.guards_intact(), offsets
+        assert torch.isfinite(grad.float()).all(), offsets        # every element of the gradient was written
+        del ar, grad

@@ -251,11 +251,11 @@ constexpr int kFlatBackwardThreads = 256;
 constexpr int kFlatBackwardUnroll = 8;
 constexpr int64_t kFlatBackwardTripVecs = 64 * kFlatBackwardUnroll;   // per wavefront and trip
 
-template <int DT, bool EXACT = (DT == 0)>
-__global__ __launch_bounds__(kFlatBackwardThreads) void rowscore_backward_flat_kernel(
-    const void* logits, int64_t n_rows, int64_t vocab, const int64_t* __restrict__ labels,
-    const float* __restrict__ temperature, const float* __restrict__ lse, const float* __restrict__ entropy,
-    const float* __restrict__ g_logprob, const float* __restrict__ g_entropy, void* dlogits) {
+// The walk itself. row_constants(r, &label, &active) gives the gradient's constants of row r (wave-uniform r; called by
+// the whole wavefront): `active` false means the row's gradient is zero and its logits are not to be read.
+template <int DT, class RowConstants>
+__device__ __forceinline__ void backward_flat_walk(const void* logits, int64_t n_rows, int64_t vocab, void* dlogits,
+                                                   RowConstants&& row_constants) {
   using E = Elem<DT>;
   using O = ElemOut<DT>;
   constexpr int PV = E::kPerVec;
@@ -273,28 +273,17 @@ __global__ __launch_bounds__(kFlatBackwardThreads) void rowscore_backward_flat_k
   int64_t base = (static_cast<int64_t>(blockIdx.x) * (kFlatBackwardThreads / 64) + wave) * kFlatBackwardTripVecs;
   int64_t row = base / row_vecs, rem = base % row_vecs;   // the trip's first vector: vector `rem` of row `row`
 
-  auto constants = [&](int64_t r, int64_t* label) {
-    float T = 1.f;
-    if (temperature != nullptr) {
-      T = temperature[r];
-      T = (T < kMinTemperature) ? kMinTemperature : T;
-    }
-    const float gl = (g_logprob != nullptr) ? g_logprob[r] : 0.f;
-    const float gh = (g_entropy != nullptr) ? g_entropy[r] : 0.f;
-    const float H = (g_entropy != nullptr) ? entropy[r] : 0.f;
-    *label = (g_logprob != nullptr) ? labels[r] : -1;   // one outside [0, vocab) matches nothing
-    return make_row_grad<EXACT>(T, lse[r], H, gl, gh);
-  };
-
   for (; base < nvec; base += stride) {
     int64_t label0, label1;
-    const auto f0 = constants(row, &label0);
-    const auto f1 = constants(row + 1 < n_rows ? row + 1 : row, &label1);
+    bool active0, active1;
+    const auto f0 = row_constants(row, &label0, &active0);
+    const auto f1 = row_constants(row + 1 < n_rows ? row + 1 : row, &label1, &active1);
     u32x4 v[U];
 #pragma unroll
     for (int u = 0; u < U; ++u) {
       const int64_t k = base + u * 64 + lane;
-      v[u] = (k < nvec) ? __builtin_nontemporal_load(vin + k) : u32x4{0u, 0u, 0u, 0u};
+      const bool active = (rem + u * 64 + lane >= row_vecs) ? active1 : active0;
+      v[u] = (k < nvec && active) ? __builtin_nontemporal_load(vin + k) : u32x4{0u, 0u, 0u, 0u};
     }
 #pragma unroll
     for (int u = 0; u < U; ++u) {
@@ -313,7 +302,9 @@ __global__ __launch_bounds__(kFlatBackwardThreads) void rowscore_backward_flat_k
         for (int i = 0; i < PV; ++i)
           if (i == rel) x[i] += f.lab;
       }
-      if (k < nvec) __builtin_nontemporal_store(O::pack(x), vout + k);
+      u32x4 y = O::pack(x);
+      if (!(second ? active1 : active0)) y = u32x4{0u, 0u, 0u, 0u};
+      if (k < nvec) __builtin_nontemporal_store(y, vout + k);
     }
     row += stride_rows;
     rem += stride_rem;
@@ -322,6 +313,72 @@ __global__ __launch_bounds__(kFlatBackwardThreads) void rowscore_backward_flat_k
       ++row;
     }
   }
+}
+
+template <int DT, bool EXACT = (DT == 0)>
+__global__ __launch_bounds__(kFlatBackwardThreads) void rowscore_backward_flat_kernel(
+    const void* logits, int64_t n_rows, int64_t vocab, const int64_t* __restrict__ labels,
+    const float* __restrict__ temperature, const float* __restrict__ lse, const float* __restrict__ entropy,
+    const float* __restrict__ g_logprob, const float* __restrict__ g_entropy, void* dlogits) {
+  backward_flat_walk<DT>(logits, n_rows, vocab, dlogits, [&](int64_t r, int64_t* label, bool* active) {
+    float T = 1.f;
+    if (temperature != nullptr) {
+      T = temperature[r];
+      T = (T < kMinTemperature) ? kMinTemperature : T;
+    }
+    const float gl = (g_logprob != nullptr) ? g_logprob[r] : 0.f;
+    const float gh = (g_entropy != nullptr) ? g_entropy[r] : 0.f;
+    const float H = (g_entropy != nullptr) ? entropy[r] : 0.f;
+    *label = (g_logprob != nullptr) ? labels[r] : -1;   // one outside [0, vocab) matches nothing
+    *active = true;
+    return make_row_grad<EXACT>(T, lse[r], H, gl, gh);
+  });
+}
+
+// The gradient of score_responses_kernel in the same form, for batches of at most 64 sequences (a wavefront finds a
+// row's sequence with one pair of loads per lane and a ballot instead of a bisection per trip): rows outside every
+// response window, and rows of sequences that fail validation, are written as zeros without being read, like
+// score_responses_backward_kernel below, and the rows inside get the same bits as there.
+template <int DT, bool EXACT = (DT == 0)>
+__global__ __launch_bounds__(kFlatBackwardThreads) void score_responses_backward_flat_kernel(
+    const void* logits, int64_t n_rows, int64_t vocab, const int64_t* __restrict__ labels,
+    const int64_t* __restrict__ input_ids, const float* __restrict__ temperature,
+    const int64_t* __restrict__ cu_seqlens, const int64_t* __restrict__ response_lens, int64_t B, int64_t T_out,
+    const float* __restrict__ resp_lse, const float* __restrict__ resp_entropy,
+    const float* __restrict__ g_resp_logprob, const float* __restrict__ g_resp_entropy, void* dlogits) {
+  const int lane = threadIdx.x & 63;
+  backward_flat_walk<DT>(logits, n_rows, vocab, dlogits, [&](int64_t r, int64_t* label, bool* active) {
+    *label = -1;
+    *active = false;
+    bool hit = false;
+    if (lane < B) hit = cu_seqlens[lane] <= r && r < cu_seqlens[lane + 1];
+    const unsigned long long holders = __ballot(hit);
+    int64_t at = 0;
+    if (holders != 0ull) {
+      const int64_t b = __builtin_ctzll(holders);
+      int why = 0;
+      const ResponseWindow w = response_window(cu_seqlens, response_lens, b, B, n_rows, T_out, &why);
+      const int64_t col = r - w.first;
+      if (w.ok && col >= 0 && col < w.resp) {
+        *active = true;
+        at = b * T_out + col;
+      }
+    }
+    float T = 1.f, gl = 0.f, gh = 0.f, H = 0.f, l = 0.f;
+    if (*active) {
+      if (temperature != nullptr) {
+        T = temperature[r];
+        T = (T < kMinTemperature) ? kMinTemperature : T;
+      }
+      gl = (g_resp_logprob != nullptr) ? g_resp_logprob[at] : 0.f;
+      gh = (g_resp_entropy != nullptr) ? g_resp_entropy[at] : 0.f;
+      H = (g_resp_entropy != nullptr) ? resp_entropy[at] : 0.f;
+      l = resp_lse[at];
+      if (g_resp_logprob != nullptr)
+        *label = (input_ids != nullptr) ? input_ids[r + 1 < n_rows ? r + 1 : 0] : labels[r];
+    }
+    return make_row_grad<EXACT>(T, l, H, gl, gh);
+  });
 }
 
 // Backward of score_responses_kernel (rowscore_kernels.h). grid.x = n_rows, block = WAVES*64. Row r finds its

@@ -577,6 +577,28 @@ int vrl_score_responses(const void* logits, int dtype, int64_t n_rows, int64_t v
   return launch_status();
 }
 
+// The backward walk without rows (rowscore_backward_flat_kernel), for inputs of at least 2^22 vectors (64 MiB; below
+// that one workgroup per row is as fast). Many short workgroups beat few long ones: at 8192 x 151936 bf16 512 workgroups
+// take 936 us, 4096 922, 16384 883, 32768 885, one per trip (75970) 907, against 949 us for one workgroup per row;
+// 2048 x 128256 fp32: 378, 375, 357, 347, 346 against 421 us.
+constexpr int64_t kFlatBackwardGrid = 32768;
+constexpr int64_t kFlatBackwardMinVecs = int64_t(1) << 22;
+
+
+// Workgroups for that walk, or 0 when the rows do not lie back to back on 16-byte boundaries, are shorter than a
+// wavefront's trip, or are too few.
+int64_t flat_backward_grid(const void* logits, const void* dlogits, int64_t n_rows, int64_t vocab, int64_t row_stride,
+                           int64_t d_row_stride, int64_t esize) {
+  const int64_t per_vec = 16 / esize;
+  if (row_stride != vocab || d_row_stride != vocab || vocab % per_vec != 0 ||
+      vocab / per_vec < vrl::kFlatBackwardTripVecs || !aligned(logits, 16) || !aligned(dlogits, 16) ||
+      n_rows * (vocab / per_vec) < kFlatBackwardMinVecs)
+    return 0;
+  constexpr int64_t wg_vecs = (vrl::kFlatBackwardThreads / 64) * vrl::kFlatBackwardTripVecs;
+  const int64_t trips = (n_rows * (vocab / per_vec) + wg_vecs - 1) / wg_vecs;
+  return trips < kFlatBackwardGrid ? trips : kFlatBackwardGrid;
+}
+
 int vrl_score_responses_backward(const void* logits, int dtype, int64_t n_rows, int64_t vocab, int64_t row_stride,
                                  const int64_t* labels, const int64_t* input_ids, const float* temperature,
                                  const int64_t* cu_seqlens, const int64_t* response_lens, int64_t B, int64_t T_out,
@@ -599,9 +621,26 @@ int vrl_score_responses_backward(const void* logits, int dtype, int64_t n_rows, 
       !aligned(temperature, 4) || !aligned(cu_seqlens, 8) || !aligned(response_lens, 8) || !aligned(resp_lse, 4) ||
       !aligned(resp_entropy, 4) || !aligned(g_resp_logprob, 4) || !aligned(g_resp_entropy, 4))
     return VRL_ERR_ALIGN;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  // few sequences (a wavefront looks a row's sequence up with one ballot) and rows back to back: the walk without rows
+  const int64_t flat = B <= 64 ? flat_backward_grid(logits, dlogits, n_rows, vocab, row_stride, d_row_stride,
+                                                    static_cast<int64_t>(esize)) : 0;
+  if (flat > 0) {
+    const dim3 fg(static_cast<unsigned>(flat)), fb(vrl::kFlatBackwardThreads);
+#define VRL_SRBF_ARGS                                                                                                 \
+  logits, n_rows, vocab, labels, input_ids, temperature, cu_seqlens, response_lens, B, T_out, resp_lse, resp_entropy, \
+      g_resp_logprob, g_resp_entropy, dlogits
+    if (dtype == VRL_F32)
+      vrl::score_responses_backward_flat_kernel<VRL_F32><<<fg, fb, 0, s>>>(VRL_SRBF_ARGS);
+    else if (dtype == VRL_BF16)
+      vrl::score_responses_backward_flat_kernel<VRL_BF16><<<fg, fb, 0, s>>>(VRL_SRBF_ARGS);
+    else
+      vrl::score_responses_backward_flat_kernel<VRL_F16><<<fg, fb, 0, s>>>(VRL_SRBF_ARGS);
+#undef VRL_SRBF_ARGS
+    return launch_status();
+  }
   const dim3 grid(static_cast<unsigned>(n_rows));
   const dim3 block(kBackwardWaves * 64);
-  hipStream_t s = static_cast<hipStream_t>(stream);
 #define VRL_SRB_ARGS                                                                                                  \
   logits, n_rows, vocab, row_stride, labels, input_ids, temperature, cu_seqlens, response_lens, B, T_out, resp_lse, \
       resp_entropy, g_resp_logprob, g_resp_entropy, dlogits, d_row_stride
@@ -676,13 +715,6 @@ int vrl_rowscore_split_static(const void* logits, int dtype, int64_t n_rows, int
   return launch_status();
 }
 
-// The backward walk without rows (rowscore_backward_flat_kernel), for inputs of at least 2^22 vectors (64 MiB; below
-// that one workgroup per row is as fast). Many short workgroups beat few long ones: at 8192 x 151936 bf16 512 workgroups
-// take 936 us, 4096 922, 16384 883, 32768 885, one per trip (75970) 907, against 949 us for one workgroup per row;
-// 2048 x 128256 fp32: 378, 375, 357, 347, 346 against 421 us.
-constexpr int64_t kFlatBackwardGrid = 32768;
-constexpr int64_t kFlatBackwardMinVecs = int64_t(1) << 22;
-
 int vrl_rowscore_backward(const void* logits, int dtype, int64_t n_rows, int64_t vocab, int64_t row_stride,
                           const int64_t* labels, const float* temperature, const float* lse,
                           const float* entropy, const float* g_logprob, const float* g_entropy,
@@ -701,14 +733,10 @@ int vrl_rowscore_backward(const void* logits, int dtype, int64_t n_rows, int64_t
     return VRL_ERR_ALIGN;
   const dim3 grid(static_cast<unsigned>(n_rows));
   hipStream_t s = static_cast<hipStream_t>(stream);
-  // Rows that lie back to back on 16-byte boundaries, enough of them to keep a fixed grid busy: the walk without rows.
-  const int64_t per_vec = 16 / static_cast<int64_t>(esize);
-  if (row_stride == vocab && d_row_stride == vocab && vocab % per_vec == 0 &&
-      vocab / per_vec >= vrl::kFlatBackwardTripVecs && aligned(logits, 16) && aligned(dlogits, 16) &&
-      n_rows * (vocab / per_vec) >= kFlatBackwardMinVecs) {
-    constexpr int64_t wg_vecs = (vrl::kFlatBackwardThreads / 64) * vrl::kFlatBackwardTripVecs;
-    const int64_t trips = (n_rows * (vocab / per_vec) + wg_vecs - 1) / wg_vecs;
-    const dim3 fg(static_cast<unsigned>(trips < kFlatBackwardGrid ? trips : kFlatBackwardGrid)), fb(vrl::kFlatBackwardThreads);
+  // Rows that lie back to back on 16-byte boundaries, enough of them: the walk without rows.
+  const int64_t flat = flat_backward_grid(logits, dlogits, n_rows, vocab, row_stride, d_row_stride, static_cast<int64_t>(esize));
+  if (flat > 0) {
+    const dim3 fg(static_cast<unsigned>(flat)), fb(vrl::kFlatBackwardThreads);
     if (dtype == VRL_F32)
       vrl::rowscore_backward_flat_kernel<VRL_F32><<<fg, fb, 0, s>>>(logits, n_rows, vocab, labels, temperature, lse, entropy,
                                                                    g_logprob, g_entropy, dlogits);
