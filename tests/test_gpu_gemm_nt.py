@@ -26,7 +26,10 @@ def _check(out, x, y, base=None, ulps=1.0):
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
-@pytest.mark.parametrize("NX,NY,K", [(256, 256, 128), (512, 256, 192), (260, 300, 256), (768, 1024, 4096), (3584, 512, 1024)])
+@pytest.mark.parametrize("NX,NY,K", [(256, 256, 128), (512, 256, 192), (260, 300, 256), (768, 1024, 4096), (3584, 512, 1024),
+                                     # more than 8 patches of work items with smaller ones at both edges: whole patches go
+                                     # to the XCDs, the last few are dealt item by item
+                                     (3584, 3008, 384), (2304, 2816, 192)])
 def test_product_against_fp64(dev, dtype, NX, NY, K):
     g = torch.Generator(device=dev).manual_seed(NX + NY + K)
     x = (torch.randn(NX, K, generator=g, device=dev) * 0.5).to(dtype)

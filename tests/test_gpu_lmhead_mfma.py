@@ -353,7 +353,7 @@ def test_the_plan_fills_whole_rounds_of_workgroups(dev):
         assert -(-runs // share) == s                         # no split without tiles
 
         def cost(k):
-            return -(-tblocks * k // cus) * (-(-runs // k) * 3 + 2)
+            return -(-tblocks * k // cus) * (2 * -(-runs // k) * 3 + 1)
 
         assert cost(s) == min(cost(k) for k in range(1, min(64, runs) + 1)), (T, V, s)
     assert lib.vrl_lmhead_plan(8192, 152064) == 8 if cus == 256 else True

@@ -76,37 +76,59 @@ struct LmFrag<2> {
 constexpr int kLmWaves = 8;                       // wavefronts per workgroup: 4 vocabulary quarters x 2 token halves
 
 // Which (token block, vocabulary split) a workgroup serves. Hardware deals workgroups round-robin over the 8 XCDs
-// (id % 8); the 32 that are resident on one XCD together should share operands through its L2: 8 token blocks x 4
-// splits per XCD (each W slice read by 8 workgroups, each H slice by 4) when the grid has that shape (xcd_map), plain
-// order otherwise.
+// (id % 8) and each XCD starts its share in id order, 32 at a time (one per CU: the kernels take a CU's LDS). Two
+// things follow. Every XCD must get the same number of workgroups that have work, or the launch waits for the fullest
+// one (a grid with idle ids spread through it took up to twice as long). And the 32 that are resident on one XCD
+// together should share operands through its L2. So the pairs are put in one order in which neighbours share - 8
+// splits of one token block, then of the next block, ... then the next 8 splits - and that order is dealt 32
+// consecutive pairs (4 token blocks x 8 splits) to an XCD at a time; what is left after the last whole round of 256 is
+// cut into 8 equal runs. Only ids at the very end of the grid are idle (split < 0), and such a workgroup returns before
+// any barrier. (Other shapes of 32 - 8 x 4, 16 x 2, 32 x 1 - measured the same to 3 % slower.)
+constexpr int kXcds = 8;
+constexpr int kXcdCus = 32;
+
 struct LmWork {
-  int split;
+  int split;         // < 0: nothing to do
   int64_t tok0;      // first token of the block
   int64_t tok0_ld;   // first token of the 256 rows that are loaded (an edge block is moved back so all rows exist)
   int64_t vt_begin;  // vocabulary tiles [vt_begin, vt_end)
   int64_t vt_end;
 };
 
-__device__ __forceinline__ LmWork lm_work(int64_t V, int64_t T, int n_splits, int tiles_per_split, int xcd_map) {
-  LmWork w;
-  int64_t tb;
-  const int64_t tblocks = (T + kLmTokens - 1) / kLmTokens;
-  const int64_t id = blockIdx.x;
-  if (xcd_map) {
-    const int x = (int)(id & 7);
-    const int64_t local = id >> 3;            // 0 .. tblocks*n_splits/8
-    const int64_t tgroups = tblocks / 8;      // groups of 8 token blocks
-    // super index over (tgroup, sgroup) pairs: 8 consecutive ones run at a time (one per XCD)
-    const int64_t super = (local / 32) * 8 + x;
-    const int64_t within = local % 32;
-    const int64_t tg = super % tgroups;
-    const int sg = (int)(super / tgroups);
-    tb = tg * 8 + (within & 7);
-    w.split = sg * 4 + (int)(within >> 3);
-  } else {
-    w.split = (int)(id % n_splits);
-    tb = id / n_splits;
+// Workgroups to launch for n_pairs (token block, split) pairs; the host and the kernels agree through this.
+__host__ __device__ inline int64_t lm_dealt_grid(int64_t n_pairs) {
+  const int64_t round = kXcds * kXcdCus;
+  const int64_t full = (n_pairs / round) * round;
+  return full + (n_pairs - full + kXcds - 1) / kXcds * kXcds;
+}
+
+// Position of workgroup `id` in the shared order, or -1.
+__device__ __forceinline__ int64_t lm_dealt_position(int64_t id, int64_t n_pairs) {
+  const int64_t round = kXcds * kXcdCus;
+  const int64_t full = (n_pairs / round) * round;
+  const int x = (int)(id & (kXcds - 1));
+  if (id < full) {
+    const int64_t local = id / kXcds;
+    return ((local / kXcdCus) * kXcds + x) * kXcdCus + local % kXcdCus;
   }
+  const int64_t per = (n_pairs - full + kXcds - 1) / kXcds;
+  const int64_t k = full + x * per + (id - full) / kXcds;
+  return k < n_pairs ? k : -1;
+}
+
+constexpr int kLmDealSplits = 8;
+
+__device__ __forceinline__ LmWork lm_work(int64_t V, int64_t T, int n_splits, int tiles_per_split) {
+  LmWork w;
+  const int64_t tblocks = (T + kLmTokens - 1) / kLmTokens;
+  const int64_t k = lm_dealt_position(blockIdx.x, tblocks * n_splits);
+  // columns of kLmDealSplits splits (the last one narrower), one after another; in a column, token block by token block
+  const int64_t col = k / (tblocks * kLmDealSplits);
+  const int64_t in_col = k - col * tblocks * kLmDealSplits;
+  const int rest = n_splits - (int)col * kLmDealSplits;
+  const int width = rest < kLmDealSplits ? rest : kLmDealSplits;
+  const int64_t tb = in_col / width;
+  w.split = k < 0 ? -1 : (int)(col * kLmDealSplits + in_col % width);
   w.tok0 = tb * kLmTokens;
   w.tok0_ld = w.tok0 + kLmTokens <= T ? w.tok0 : T - kLmTokens;
   const int64_t n_vtiles = (V + kLmVocab - 1) / kLmVocab;
@@ -445,7 +467,7 @@ template <int DT, bool STORE>
 __global__ __launch_bounds__(kLmWaves * 64, 1) void lmhead_partial_kernel(
     const uint16_t* __restrict__ W, const uint16_t* __restrict__ H, int64_t V, int64_t T, int64_t K, int64_t w_stride,
     int64_t h_stride, const float* __restrict__ temperature, int n_splits, int tiles_per_split,
-    int xcd_map, float* __restrict__ partials, uint16_t* __restrict__ logits_out, int64_t l_stride, int64_t l_rows) {
+    float* __restrict__ partials, uint16_t* __restrict__ logits_out, int64_t l_stride, int64_t l_rows) {
   extern __shared__ __attribute__((aligned(1024))) char lds[];  // the operand ring
 
   const int tid = threadIdx.x;
@@ -453,7 +475,8 @@ __global__ __launch_bounds__(kLmWaves * 64, 1) void lmhead_partial_kernel(
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int wv = wave >> 1;
   const int wt = wave & 1;
-  const LmWork work = lm_work(V, T, n_splits, tiles_per_split, xcd_map);
+  const LmWork work = lm_work(V, T, n_splits, tiles_per_split);
+  if (work.split < 0) return;   // the whole workgroup: an idle slot of the grid
   const int64_t n_vtiles = (V + kLmVocab - 1) / kLmVocab;
 
   // per-lane softmax state for the 8 token columns this lane sees (16 x 16 blocks: column = lane & 15)
@@ -592,7 +615,7 @@ __global__ __launch_bounds__(kLmWaves * 64, 1) void lmhead_dlogits_kernel(
     const uint16_t* __restrict__ W, const uint16_t* __restrict__ H, int64_t V, int64_t T, int64_t K, int64_t w_stride,
     int64_t h_stride, const int64_t* __restrict__ labels, const float* __restrict__ temperature,
     const float* __restrict__ lse, const float* __restrict__ entropy, const float* __restrict__ g_logprob,
-    const float* __restrict__ g_entropy, int n_splits, int tiles_per_split, int xcd_map, uint16_t* __restrict__ dlogits,
+    const float* __restrict__ g_entropy, int n_splits, int tiles_per_split, uint16_t* __restrict__ dlogits,
     int64_t d_stride) {
   extern __shared__ __attribute__((aligned(1024))) char lds[];  // the operand ring
   using O = ElemOut<DT>;
@@ -601,7 +624,8 @@ __global__ __launch_bounds__(kLmWaves * 64, 1) void lmhead_dlogits_kernel(
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int wv = wave >> 1;
   const int wt = wave & 1;
-  const LmWork work = lm_work(V, T, n_splits, tiles_per_split, xcd_map);
+  const LmWork work = lm_work(V, T, n_splits, tiles_per_split);
+  if (work.split < 0) return;   // the whole workgroup: an idle slot of the grid
 
   // the row constants of the 8 token columns this lane sees (16 x 16 blocks: column = lane & 15)
   RowGrad f[8];
@@ -673,9 +697,9 @@ __global__ __launch_bounds__(kLmWaves * 64, 1) void lmhead_dlogits_kernel(
 // store of out[y][x..x+3]), Y its token side.
 //
 // A work item is (y block of 256 rows, `tiles_per_item` x tiles, one of `k_parts` ranges of the contraction). Items
-// are dealt so that the workgroups resident on one XCD together form py x px patches of (y block, x split) pairs of
-// one contraction range and share their operand tiles through its L2; ids past the last patch leave at once, and so do
-// the slots of a patch that lie past the last y block or x split (py and px need not divide their counts).
+// are grouped in py x px patches of (y block, x split) pairs of one contraction range, which share their operand tiles,
+// and the patches are dealt to the XCDs (see the kernel); py and px need not divide their counts, the patches at the far
+// edges are smaller.
 // MODE 0 stores the product in the operands' type, MODE 1 adds it to what `out` holds (one rounding, like a GEMM with
 // beta = 1), MODE 2 stores fp32 partial sums at partials[(kp * NY + y) * NX + x] for lm_gemm_reduce_kernel.
 typedef float f32x4 __attribute__((ext_vector_type(4)));
@@ -714,20 +738,37 @@ __global__ __launch_bounds__(kLmWaves * 64, 1) void lm_gemm_kernel(
   const int64_t nyb = (g.NY + kLmTokens - 1) / kLmTokens;
   const int64_t nxt = (g.NX + kLmVocab - 1) / kLmVocab;
   const int64_t nxs = (nxt + g.tiles_per_item - 1) / g.tiles_per_item;
-  const int64_t patches_y = (nyb + g.py - 1) / g.py, patches_x = (nxs + g.px - 1) / g.px;
-  const int64_t per_part = patches_y * patches_x;
+  // Patches of py y blocks x px x splits of one contraction range (smaller at the far edges), range by range, columns
+  // of patches one after another. Whole rows of 8 patches go one patch to an XCD, whose 32 CUs then walk the contraction
+  // in step on shared operand tiles; the fewer than 8 patches left at the end are dealt item by item over the XCDs
+  // instead, so that every XCD ends with about the same number of items (a launch waits for the fullest one). A patch
+  // has py * px slots; those past its items are idle, and such a workgroup returns before any barrier.
   const int psize = g.py * g.px;
+  const int patches_y = (int)((nyb + g.py - 1) / g.py), patches_x = (int)((nxs + g.px - 1) / g.px);
+  const int64_t per_part = (int64_t)patches_y * patches_x;
+  const int64_t n_patches = per_part * g.k_parts;
+  const int64_t dealt_whole = (n_patches / kXcds) * kXcds * psize;   // ids that take whole patches
   const int64_t id = blockIdx.x;
-  const int64_t local = id >> 3;
-  const int64_t patch = (local / psize) * 8 + (id & 7);
-  if (patch >= per_part * g.k_parts) return;   // the whole workgroup, before any barrier
+  int64_t patch;
+  int within;
+  if (id < dealt_whole) {
+    const int64_t local = id / kXcds;
+    patch = (local / psize) * kXcds + (id & (kXcds - 1));
+    within = (int)(local % psize);
+  } else {
+    patch = (n_patches / kXcds) * kXcds + (id - dealt_whole) / psize;
+    within = (int)((id - dealt_whole) % psize);
+  }
+  if (patch >= n_patches) return;   // the whole workgroup
   // (64-bit divisions run on the vector ALUs; readfirstlane brings their uniform results back to scalar registers)
-  const int within = __builtin_amdgcn_readfirstlane((int)(local % psize));
   const int kp = __builtin_amdgcn_readfirstlane((int)(patch / per_part));
   const int r = __builtin_amdgcn_readfirstlane((int)(patch % per_part));
-  const int yb = __builtin_amdgcn_readfirstlane((int)((r % patches_y) * g.py + within % g.py));
-  const int xsplit = __builtin_amdgcn_readfirstlane((int)((r / patches_y) * g.px + within / g.py));
-  if (yb >= nyb || xsplit >= nxs) return;   // a slot of the last row or column of patches that holds no work
+  const int row = r % patches_y, col = r / patches_y;
+  const int height = (int)nyb - row * g.py < g.py ? (int)nyb - row * g.py : g.py;
+  const int width = (int)nxs - col * g.px < g.px ? (int)nxs - col * g.px : g.px;
+  if (within >= height * width) return;   // an idle slot of an edge patch
+  const int yb = __builtin_amdgcn_readfirstlane(row * g.py + within % height);
+  const int xsplit = __builtin_amdgcn_readfirstlane(col * g.px + within / height);
 
   LmWork work;
   work.split = kp;

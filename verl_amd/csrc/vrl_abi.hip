@@ -250,7 +250,7 @@ int copy_unit(int64_t row_bytes, const void* a, const void* b) {
 struct LmGrid {
   int64_t tblocks;
   int tiles_per_split;
-  int xcd_map;
+  int64_t grid;    // workgroups, the idle ones at its end included
 };
 
 // `run` tiles at a time go to a split: kLmSubTiles for the forward kernel, which hands its softmax state over at the
@@ -261,8 +261,7 @@ LmGrid lm_grid(int64_t T, int64_t V, int n_splits, int run) {
   const int64_t vtiles = (V + vrl::kLmVocab - 1) / vrl::kLmVocab;
   const int64_t runs = (vtiles + run - 1) / run;
   g.tiles_per_split = static_cast<int>((runs + n_splits - 1) / n_splits) * run;
-  // 8 token blocks x 4 splits per XCD when the grid divides that way (see vrl::lm_work)
-  g.xcd_map = (g.tblocks % 8 == 0 && n_splits % 4 == 0 && ((g.tblocks / 8) * (n_splits / 4)) % 8 == 0) ? 1 : 0;
+  g.grid = vrl::lm_dealt_grid(g.tblocks * n_splits);
   return g;
 }
 
@@ -288,10 +287,10 @@ int launch_lmhead(const void* hidden, const void* weight, int64_t T, int64_t V, 
   static std::atomic<bool> raised[kMaxDevices];
   const int rs = raise_lds_limit(reinterpret_cast<const void*>(vrl::lmhead_partial_kernel<DT, STORE>), raised);
   if (rs != VRL_OK) return rs;
-  vrl::lmhead_partial_kernel<DT, STORE><<<dim3(static_cast<unsigned>(g.tblocks * n_splits)), dim3(vrl::kLmWaves * 64),
+  vrl::lmhead_partial_kernel<DT, STORE><<<dim3(static_cast<unsigned>(g.grid)), dim3(vrl::kLmWaves * 64),
                                           vrl::kLmLdsBytes, s>>>(
       static_cast<const uint16_t*>(weight), static_cast<const uint16_t*>(hidden), V, T, K, w_stride, h_stride,
-      temperature, n_splits, g.tiles_per_split, g.xcd_map, partials, static_cast<uint16_t*>(logits_out), l_stride,
+      temperature, n_splits, g.tiles_per_split, partials, static_cast<uint16_t*>(logits_out), l_stride,
       l_rows);
   vrl::lmhead_finish_kernel<DT><<<dim3(static_cast<unsigned>((T + 3) / 4)), dim3(256), 0, s>>>(
       static_cast<const char*>(weight), static_cast<const char*>(hidden), V, T, K, w_stride, h_stride, labels,
@@ -309,10 +308,10 @@ int launch_lmhead_dlogits(const void* hidden, const void* weight, int64_t T, int
   static std::atomic<bool> raised[kMaxDevices];
   const int rs = raise_lds_limit(reinterpret_cast<const void*>(vrl::lmhead_dlogits_kernel<DT>), raised);
   if (rs != VRL_OK) return rs;
-  vrl::lmhead_dlogits_kernel<DT><<<dim3(static_cast<unsigned>(g.tblocks * n_splits)), dim3(vrl::kLmWaves * 64),
+  vrl::lmhead_dlogits_kernel<DT><<<dim3(static_cast<unsigned>(g.grid)), dim3(vrl::kLmWaves * 64),
                                    vrl::kLmLdsBytes, s>>>(
       static_cast<const uint16_t*>(weight), static_cast<const uint16_t*>(hidden), V, T, K, w_stride, h_stride, labels,
-      temperature, lse, entropy, g_logprob, g_entropy, n_splits, g.tiles_per_split, g.xcd_map,
+      temperature, lse, entropy, g_logprob, g_entropy, n_splits, g.tiles_per_split,
       static_cast<uint16_t*>(dlogits), d_stride);
   return launch_status();
 }
@@ -332,7 +331,8 @@ int check_lmhead_shape(int dtype, int64_t n_tokens, int64_t vocab, int64_t hidde
       h_stride < hidden_size || w_stride < hidden_size || h_stride % 8 != 0 || w_stride % 8 != 0 ||
       n_splits < 1 || n_splits > vrl::kLmMaxSplits)
     return VRL_ERR_SHAPE;
-  if (((n_tokens + vrl::kLmTokens - 1) / vrl::kLmTokens) * n_splits > kMaxGrid || (n_tokens + 3) / 4 > kMaxGrid)
+  if (vrl::lm_dealt_grid(((n_tokens + vrl::kLmTokens - 1) / vrl::kLmTokens) * n_splits) > kMaxGrid ||
+      (n_tokens + 3) / 4 > kMaxGrid)
     return VRL_ERR_SHAPE;
   return VRL_OK;
 }
@@ -359,9 +359,9 @@ int device_cus() {
 
 // The workgroups resident on one XCD form patches of py y blocks x px x splits that walk the contraction in step and
 // share operand tiles through its L2: an X tile is fetched once for the py workgroups that use it, a Y tile once for px,
-// so what leaves L2 is proportional to 1/py + 1/px. Counts that py or px do not divide leave idle slots in the last
-// row or column of patches (those workgroups return at once), which lowers the sharing there; the choice below weighs
-// both by the average number of busy workgroups per patch row and column. py <= 4, px <= 8: 32 CUs per XCD.
+// so what leaves L2 is proportional to 1/py + 1/px. Counts that py or px do not divide leave smaller patches in the
+// last row or column, which lowers the sharing there; the choice below weighs both by the average number of
+// workgroups per patch row and column. py <= 4, px <= 8: 32 CUs per XCD.
 void choose_patch(int64_t nyb, int64_t nxs, int* py_out, int* px_out) {
   double best = 1e30;
   int best_py = 1, best_px = 1;
@@ -428,8 +428,7 @@ template <int DT, bool X_CM, bool Y_CM>
 int launch_gemm(const void* x, const void* y, const GemmPlan& plan, int64_t x_stride, int64_t y_stride, void* out,
                 int64_t out_stride, int accumulate, float* workspace, hipStream_t s) {
   const vrl::LmGemmShape& g = plan.shape;
-  const int psize = g.py * g.px;
-  const int64_t grid = ((plan.patches + 7) / 8) * 8 * psize;
+  const int64_t grid = (plan.patches * g.py * g.px + 7) / 8 * 8;   // a slot per item of a full patch
   if (grid > kMaxGrid) return VRL_ERR_SHAPE;
   const dim3 gd(static_cast<unsigned>(grid)), bd(vrl::kLmWaves * 64);
   const uint16_t* X = static_cast<const uint16_t*>(x);
@@ -882,14 +881,15 @@ int vrl_lmhead_plan(int64_t n_tokens, int64_t vocab) {
   const int64_t runs = (vtiles + vrl::kLmSubTiles - 1) / vrl::kLmSubTiles;
   const int64_t cus = device_cus();
   // One workgroup per CU runs at a time, so a launch takes (rounds of workgroups) x (tiles of the longest share, plus
-  // about two tiles to fill and drain the ring). The fewest splits among the cheapest: a token's results do not
-  // depend on the choice (see kLmSubTiles), only the time does.
+  // about half a tile to start a workgroup and fill and drain its ring; with two tiles the choices at 12288 and 20000
+  // tokens were 8 % and 4 % slower than what this picks). The fewest splits among the cheapest: a token's results do
+  // not depend on the choice (see kLmSubTiles), only the time does.
   int64_t best = 1, best_cost = -1;
   for (int64_t s = 1; s <= vrl::kLmMaxSplits && s <= runs; ++s) {
     const int64_t share = (runs + s - 1) / s;
     if ((runs + share - 1) / share != s) continue;   // this many splits would leave one without a tile
     const int64_t rounds = (tblocks * s + cus - 1) / cus;
-    const int64_t cost = rounds * (share * vrl::kLmSubTiles + 2);
+    const int64_t cost = rounds * (2 * share * vrl::kLmSubTiles + 1);   // in half tiles
     if (best_cost < 0 || cost < best_cost) {
       best = s;
       best_cost = cost;
