@@ -490,9 +490,9 @@ __global__ __launch_bounds__(kLmWaves * 64, 1) void lmhead_partial_kernel(
     c[j] = make_scale<false>(temperature, tok).c;   // log2(e) / max(T, 1e-8), exactly what the finishing kernel uses
   }
 
-  // (load placement, see lm_walk_tiles: pairs two instructions before a column ends; single loads behind it when the
-  // logits are written too - 6.28 against 6.45 ms and 6.65 against 6.94 ms for the other's choice, one process)
-  lm_walk_tiles<DT, 2, false, false, STORE ? 1 : 2, STORE ? 0 : 2, 0>(W, H, V, K, w_stride, h_stride, work, lds, [&](int64_t vt, lm_f32x4 (&acc)[4][8]) {
+  // (load placement, see lm_walk_tiles: single loads right behind a column's last matrix instruction. Pairs of loads
+  // measured 2 % faster to 5 % slower from one build to the next, single loads anywhere in the column within 1 %.)
+  lm_walk_tiles<DT, 2, false, false, 1, 0, 0>(W, H, V, K, w_stride, h_stride, work, lds, [&](int64_t vt, lm_f32x4 (&acc)[4][8]) {
     // fold 16 logits per token column into the running state (maximum first, then the exponentials; nothing is
     // buffered): acc[i][j][v] is vocabulary row tile_row0 + wv*64 + i*16 + 4*(lane>>4) + v of token column j
     const bool edge = (vt + 1) * kLmVocab > V;
