@@ -424,8 +424,8 @@ __device__ __forceinline__ void lm_walk_tiles_as(const uint16_t* __restrict__ W,
 // LOAD_GROUP / LOAD_PHASE place the loading wavefronts' eight loads of a half: LOAD_GROUP (1 or 2) of them together
 // behind every 4 * LOAD_GROUP matrix instructions, LOAD_PHASE instructions before the end of such a run (0 = behind the
 // last product of a column, where the H fragment is refilled too). The kernels differ by 1-3 % in which placement suits
-// them (a sweep per kernel at 8192 / 4096 x 3584 <-> 152064 bf16): the forward takes pairs at phase 0, the two products
-// single loads one instruction earlier, the gradient kernel single loads three instructions earlier. H_DELAY moves the
+// them (a sweep per kernel at 8192 / 4096 x 3584 <-> 152064 bf16): the forward takes single loads at phase 0, the two
+// products single loads one instruction earlier, the gradient kernel single loads three instructions earlier. H_DELAY moves the
 // loading wavefronts' refills of the H fragments that many instructions back, away from the computing wavefronts' (which
 // stay right behind a column's last product): worth 3 % to the d hidden product, nothing or less to the others.
 template <int DT, int EPILOGUE_STORES, bool W_CM, bool H_CM, int LOAD_GROUP, int LOAD_PHASE, int H_DELAY, class OnTile>
