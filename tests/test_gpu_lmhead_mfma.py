@@ -330,6 +330,11 @@ def test_token_results_do_not_depend_on_the_call(dev):
         for splits in (1, 2, 7, 22, 64):
             lp_p, ent_p = fused_linear_for_ppo(h[:2048], w, ids[:2048], 0.9, forward_splits=splits)
             assert torch.equal(lp_p, lp_all[:2048]) and torch.equal(ent_p, ent_all[:2048]), splits
+        # 65 token blocks: (block, split) pairs past the last whole round of 256 workgroups are dealt in 8 equal runs, and
+        # the last group of 8 splits is narrower
+        for splits in (5, 13, 22):
+            lp_p, ent_p = fused_linear_for_ppo(h, w, ids, 0.9, forward_splits=splits)
+            assert torch.equal(lp_p, lp_all) and torch.equal(ent_p, ent_all), splits
     hg = h[:300].clone().requires_grad_()
     lp_g, _ = fused_linear_for_ppo(hg, w, ids[:300], 0.9)                            # and with gradients
     assert torch.equal(lp_g.detach(), lp_all[:300])
