@@ -392,8 +392,10 @@ GemmPlan gemm_plan(int64_t NX, int64_t NY, int64_t K, int forced_parts) {
   const int64_t nyb = (NY + vrl::kLmTokens - 1) / vrl::kLmTokens;
   const int64_t nxt = (NX + vrl::kLmVocab - 1) / vrl::kLmVocab;
   const int cus = device_cus();
-  // x tiles per workgroup: 2 when that still leaves 8 rounds of work (halves the share of pipeline fill and drain)
-  g.tiles_per_item = (nxt % 2 == 0 && nyb * (nxt / 2) >= 8LL * cus) ? 2 : 1;
+  // x tiles per workgroup: 2 when that still leaves 8 rounds of work and a tile is at most 64 contraction steps (halves
+  // the share of pipeline fill and drain; from 128 steps on the coarser items cost more in the last, partly filled round
+  // than they save: d W at 8192 tokens 6.46 against 6.59 ms with one tile per item, the same at 4096)
+  g.tiles_per_item = (nxt % 2 == 0 && nyb * (nxt / 2) >= 8LL * cus && g.k_steps <= 64) ? 2 : 1;
   const int64_t nxs = (nxt + g.tiles_per_item - 1) / g.tiles_per_item;
   const int64_t base = nyb * nxs;
   int best = 1;
